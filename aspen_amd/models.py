@@ -1,0 +1,339 @@
+"""Model descriptions (Darknet-style ``.cfg`` text) and seeded synthetic tensors.
+
+The cfg dialect is the one the reference parses (reference
+``src/darknet_parser.c:410-486``): ``[net]`` is the input layer, ``parent=`` /
+``from=`` are relative layer offsets, ``M/K/n_head/n_embd/masked`` describe the
+transformer layers.  The generators below emit that text from the network's
+arithmetic description, so any depth/width can be produced for tests.
+
+Synthetic tensors come from a counter-based splitmix64 stream so that the same
+(seed, tensor id, element index) gives the same float on every machine and for
+every consumer (the HIP library, the CPU oracle, the reference build).
+Tensors are produced in PyTorch element order -- the order the reference's
+weight file holds (reference ``src/apu_file_io.c:240-262``).
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, List, Tuple
+
+import numpy as np
+
+# ----------------------------------------------------------------------------
+# cfg generators
+# ----------------------------------------------------------------------------
+
+
+def _conv(filters, size, stride, pad, act, parent=None):
+    s = "[convolutional]\n"
+    if parent is not None:
+        s += f"parent={parent}\n"
+    s += f"filters={filters}\nsize={size}\nstride={stride}\npad={pad}\nactivation={act}\n\n"
+    return s
+
+
+def resnet50_cfg(height=224, width=224, classes=1000, widths=(64, 128, 256, 512),
+                 blocks=(3, 4, 6, 3), stem=64) -> str:
+    """ResNet-50 v1.5 (stride 2 on the 3x3 conv); head = 7x7 avgpool + 1x1 conv."""
+    s = f"[net]\nheight={height}\nwidth={width}\nchannels=3\n\n"
+    s += _conv(stem, 7, 2, 3, "relu")
+    s += "[maxpool]\nsize=3\nstride=2\npad=1\n\n"
+    for stage, (w, nb) in enumerate(zip(widths, blocks)):
+        for b in range(nb):
+            stride = 2 if (b == 0 and stage > 0) else 1
+            s += _conv(w, 1, 1, 0, "relu")
+            s += _conv(w, 3, stride, 1, "relu")
+            s += _conv(4 * w, 1, 1, 0, "linear")
+            if b == 0:
+                s += _conv(4 * w, 1, stride, 0, "linear", parent=-4)
+                s += "[shortcut]\nfrom=-2\nactivation=relu\n\n"
+            else:
+                s += "[shortcut]\nfrom=-4\nactivation=relu\n\n"
+    final_hw = height // 32
+    s += f"[avgpool]\nsize={final_hw}\nstride=1\n\n"
+    s += _conv(classes, 1, 1, 0, "linear")
+    return s
+
+
+def vgg16_cfg(height=224, width=224, classes=1000,
+              plan=(64, 64, "M", 128, 128, "M", 256, 256, 256, "M", 512, 512, 512, "M", 512, 512, 512, "M"),
+              fc=(4096, 4096)) -> str:
+    s = f"[net]\nheight={height}\nwidth={width}\nchannels=3\n\n"
+    for p in plan:
+        if p == "M":
+            s += "[maxpool]\nsize=2\nstride=2\n\n"
+        else:
+            s += _conv(p, 3, 1, 1, "relu")
+    for f in fc:
+        s += f"[connected]\noutput={f}\nactivation=relu\n\n"
+    s += f"[connected]\noutput={classes}\nactivation=linear\n\n"
+    return s
+
+
+def _attn_block(n_embd, n_head, masked):
+    hd = n_embd // n_head
+    s = ""
+    for parent in (None, -2, -3):  # Key, Query, Value all read the block input
+        s += "[matmul]\n"
+        if parent is not None:
+            s += f"parent={parent}\n"
+        s += f"M={n_embd}\nn_head={n_head}\nn_embd={n_embd}\n\n"
+    s += f"[attention_k]\nparent=-2\nfrom=-3\nM=1\nK={hd}\nn_head={n_head}\nn_embd={n_embd}\n"
+    if masked:
+        s += "masked=1\n"
+    s += "\n"
+    s += f"[attention_v]\nfrom=-2\nM={n_embd}\nn_head={n_head}\nn_embd={n_embd}\n\n"
+    s += f"[matmul]\nM={n_embd}\n\n"
+    return s
+
+
+def bert_cfg(n_layer=12, n_embd=768, n_head=12, ffn=3072) -> str:
+    """Post-LN encoder: K,Q,V -> attn_k -> attn_v -> proj -> +x -> LN -> FFN -> +x -> LN."""
+    s = f"[net]\nM={n_embd}\nheight=1\nfilters={n_embd}\n\n"
+    for _ in range(n_layer):
+        s += _attn_block(n_embd, n_head, masked=False)
+        s += f"[shortcut]\nfrom=-7\nM={n_embd}\n\n"
+        s += f"[layernorm]\nM={n_embd}\n\n"
+        s += f"[matmul]\nM={ffn}\nactivation=gelu\n\n"
+        s += f"[matmul]\nM={n_embd}\n\n"
+        s += f"[shortcut]\nfrom=-3\nM={n_embd}\n\n"
+        s += f"[layernorm]\nM={n_embd}\n\n"
+    return s
+
+
+def gpt2_cfg(n_layer=12, n_embd=768, n_head=12, ffn=3072) -> str:
+    """Pre-LN causal decoder; no final LN, no LM head (as the reference's cfg)."""
+    s = f"[net]\nM={n_embd}\nheight=1\nfilters={n_embd}\n\n"
+    for _ in range(n_layer):
+        s += f"[layernorm]\nM={n_embd}\n\n"
+        s += _attn_block(n_embd, n_head, masked=True)
+        s += f"[shortcut]\nfrom=-8\nM={n_embd}\n\n"
+        s += f"[layernorm]\nM={n_embd}\n\n"
+        s += f"[matmul]\nM={ffn}\nactivation=gelu_acc\n\n"
+        s += f"[matmul]\nM={n_embd}\n\n"
+        s += f"[shortcut]\nfrom=-4\nM={n_embd}\n\n"
+    return s
+
+
+def custom_cifar_cfg() -> str:
+    """The small CIFAR-10 net of the reference's third example (conv5/pool/conv3/pool/3 FC)."""
+    s = "[net]\nheight=32\nwidth=32\nchannels=3\n\n"
+    s += _conv(32, 5, 1, 2, "relu") + "[maxpool]\nsize=2\nstride=2\n\n"
+    s += _conv(64, 3, 1, 1, "relu") + "[maxpool]\nsize=2\nstride=2\n\n"
+    s += "[connected]\noutput=256\nactivation=relu\n\n[connected]\noutput=128\nactivation=relu\n\n"
+    s += "[connected]\noutput=10\nactivation=linear\n\n"
+    return s
+
+
+# ----------------------------------------------------------------------------
+# cfg -> layer list (host-side mirror of the parser, used to size synthetic tensors)
+# ----------------------------------------------------------------------------
+
+_TYPES = {
+    "[net]": "input", "[network]": "input", "[conv]": "conv", "[convolutional]": "conv",
+    "[shortcut]": "residual", "[max]": "maxpool", "[maxpool]": "maxpool", "[avg]": "avgpool",
+    "[avgpool]": "avgpool", "[conn]": "fc", "[connected]": "fc", "[soft]": "softmax",
+    "[softmax]": "softmax", "[matmul]": "matmul", "[attention_k]": "attn_k",
+    "[attention_v]": "attn_v", "[layernorm]": "layernorm",
+}
+
+
+def parse_cfg(text: str) -> List[Dict]:
+    """Layer dictionaries with resolved parents and in/out shapes
+    (reference ``src/darknet_parser.c:455-486`` and ``src/input_parser.c:35-127``)."""
+    layers: List[Dict] = []
+    cur = None
+    for raw in text.splitlines():
+        line = raw.strip()
+        if not line or line[0] in "#;":
+            continue
+        if line.startswith("["):
+            if line not in _TYPES:
+                cur = None  # unsupported sections are dropped
+                continue
+            cur = {"type": _TYPES[line], "opts": {}}
+            layers.append(cur)
+        elif cur is not None and "=" in line:
+            k, v = line.split("=", 1)
+            cur["opts"][k.strip()] = v.strip()
+    for i, L in enumerate(layers):
+        o = L["opts"]
+        gi = lambda k, d=0: int(o.get(k, d))
+        L["idx"] = i
+        L["act"] = o.get("activation", "none")
+        L["p0"] = None if L["type"] == "input" else (i + gi("parent") if gi("parent") else i - 1)
+        L["p1"] = i + gi("from") if gi("from") else None
+        L["size"], L["stride"], L["pad"] = gi("size"), max(gi("stride"), 1), gi("pad")
+        L["M"], L["K"] = gi("M"), gi("K")
+        L["n_head"], L["n_embd"], L["masked"] = gi("n_head"), gi("n_embd"), gi("masked")
+        if L["type"] == "input":
+            if L["M"]:
+                L["C"], L["H"], L["W"] = L["M"], 1, 0
+            else:
+                L["C"], L["H"], L["W"] = gi("channels"), gi("height"), gi("width")
+            continue
+        P = layers[L["p0"]]
+        L["inC"], L["inH"], L["inW"] = P["C"], P["H"], P["W"]
+        t = L["type"]
+        if t == "conv":
+            L["C"] = gi("filters")
+            L["H"] = (P["H"] + 2 * L["pad"] - (L["size"] - 1) - 1) // L["stride"] + 1
+            L["W"] = (P["W"] + 2 * L["pad"] - (L["size"] - 1) - 1) // L["stride"] + 1
+        elif t in ("maxpool", "avgpool"):
+            L["C"] = P["C"]
+            L["H"] = (P["H"] + 2 * L["pad"] - (L["size"] - 1) - 1) // L["stride"] + 1
+            L["W"] = (P["W"] + 2 * L["pad"] - (L["size"] - 1) - 1) // L["stride"] + 1
+        elif t == "fc":
+            L["C"], L["H"], L["W"] = gi("output") or gi("filters"), 1, 1
+        elif t == "softmax":
+            L["C"], L["H"], L["W"] = P["C"], 1, 1
+        elif t == "residual":
+            L["C"], L["H"], L["W"] = (L["M"], 1, 0) if L["M"] else (P["C"], P["H"], P["W"])
+        elif t in ("matmul", "layernorm", "attn_v"):
+            L["C"], L["H"], L["W"] = L["M"], 1, 0
+            if t == "matmul":
+                L["K"] = P["M"] if P["type"] != "input" else P["C"]
+        elif t == "attn_k":
+            L["C"], L["H"], L["W"] = 0, 1, 0  # rows = seq_len, known at graph build
+            L["K"] = L["n_embd"] // L["n_head"]
+    return layers
+
+
+# ----------------------------------------------------------------------------
+# deterministic tensors
+# ----------------------------------------------------------------------------
+
+_U64 = np.uint64
+_GOLD = _U64(0x9E3779B97F4A7C15)
+
+
+def _mix(x: np.ndarray) -> np.ndarray:
+    with np.errstate(over="ignore"):
+        z = x + _GOLD
+        z = (z ^ (z >> _U64(30))) * _U64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> _U64(27))) * _U64(0x94D049BB133111EB)
+        return z ^ (z >> _U64(31))
+
+
+def _stream(seed: int, tensor_id: int, n: int, lane: int) -> np.ndarray:
+    """n uniform floats in [0,1) with 24 random bits each (exactly representable in fp32)."""
+    with np.errstate(over="ignore"):
+        base = _mix(np.array([seed], dtype=_U64) * _U64(0xD1342543DE82EF95)
+                    + _U64(tensor_id) * _U64(0xA0761D6478BD642F) + _U64(lane))
+        z = _mix(base + np.arange(n, dtype=_U64) * _GOLD)
+    return ((z >> _U64(40)).astype(np.float64) * (1.0 / (1 << 24))).astype(np.float32)
+
+
+def uniform(seed: int, tensor_id: int, shape) -> np.ndarray:
+    n = int(np.prod(shape))
+    return _stream(seed, tensor_id, n, 0).reshape(shape)
+
+
+def normal(seed: int, tensor_id: int, shape, std: float, mean: float = 0.0) -> np.ndarray:
+    n = int(np.prod(shape))
+    u1 = _stream(seed, tensor_id, n, 1).astype(np.float64)
+    u2 = _stream(seed, tensor_id, n, 2).astype(np.float64)
+    r = np.sqrt(-2.0 * np.log(1.0 - u1))  # 1-u1 in (0,1]
+    z = r * np.cos(2.0 * math.pi * u2)
+    return (mean + std * z).astype(np.float32).reshape(shape)
+
+
+Tensor = Tuple[int, str, np.ndarray]  # (1-based weighted-layer index, "WEIGHT"/"BIAS", data)
+
+
+def synth_weights(layers: List[Dict], seed: int, style: str) -> List[Tensor]:
+    """style "he": conv/FC ~ N(0, 2/fan_in), bias ~ N(0, 0.01^2) (stands in for folded BN);
+    style "gpt": matmul W,b ~ N(0, 0.02^2), layernorm w = 1 + N(0, 0.02^2), b ~ N(0, 0.02^2)."""
+    out: List[Tensor] = []
+    widx = 0
+    for L in layers:
+        t = L["type"]
+        if t not in ("conv", "fc", "matmul", "layernorm"):
+            continue
+        widx += 1
+        tid = 2 * widx
+        if t == "conv":
+            shp = (L["C"], L["inC"], L["size"], L["size"])
+            fan = L["inC"] * L["size"] * L["size"]
+        elif t == "fc":
+            shp = (L["C"], L["inC"], L["inH"], L["inW"])
+            fan = L["inC"] * L["inH"] * L["inW"]
+        elif t == "matmul":
+            shp = (L["M"], L["K"])
+            fan = L["K"]
+        else:
+            shp = (L["M"],)
+            fan = 1
+        if t == "layernorm":
+            w = normal(seed, tid, shp, 0.02, 1.0)
+            b = normal(seed, tid + 1, shp, 0.02)
+        elif style == "he":
+            w = normal(seed, tid, shp, math.sqrt(2.0 / fan))
+            b = normal(seed, tid + 1, (shp[0],), 0.01)
+        elif style == "gpt":
+            w = normal(seed, tid, shp, 0.02)
+            b = normal(seed, tid + 1, (shp[0],), 0.02)
+        else:
+            raise ValueError(style)
+        out.append((widx, "WEIGHT", w))
+        out.append((widx, "BIAS", b))
+    return out
+
+
+def write_aspen_data(path: str, tensors: List[Tensor]) -> None:
+    """``ASPEN_DATA`` weight file (format: reference ``src/apu_file_io.c:48-432``)."""
+    with open(path, "wb") as f:
+        f.write(b"ASPEN_DATA\n")
+        for widx, kind, arr in tensors:
+            raw = np.ascontiguousarray(arr, dtype=np.float32).tobytes()
+            f.write(f"LAYER:{widx}\nTENSOR_TYPE:{kind}\nDATA_SIZE:{len(raw)}\nDATA_START:\n".encode())
+            f.write(raw)
+            f.write(b"DATA_END\nLAYER_END\n")
+
+
+# ----------------------------------------------------------------------------
+# the five benchmark configurations
+# ----------------------------------------------------------------------------
+
+CONFIGS = {
+    # name: (cfg generator, weight style, batch, seq, seed, transformer input kind)
+    "resnet50_b1": (resnet50_cfg, "he", 1, 0, 101, None),
+    "resnet50_b32": (resnet50_cfg, "he", 32, 0, 101, None),
+    "vgg16_b32": (vgg16_cfg, "he", 32, 0, 202, None),
+    "resnet50_b16": (resnet50_cfg, "he", 16, 0, 101, None),
+    "vgg16_b16": (vgg16_cfg, "he", 16, 0, 202, None),
+    "bert_base_b8_s128": (bert_cfg, "gpt", 8, 128, 303, "embeddings"),
+    "gpt2_b4_s512": (gpt2_cfg, "gpt", 4, 512, 404, "token_ids"),
+}
+
+
+def make_config(name: str):
+    """(cfg text, parsed layers, weight tensors, dense input, batch, seq) of a named configuration."""
+    gen, style, batch, seq, seed, kind = CONFIGS[name]
+    cfg = gen()
+    layers = parse_cfg(cfg)
+    return cfg, layers, synth_weights(layers, seed, style), synth_input(layers, seed, batch, seq, kind), batch, seq
+
+
+def synth_input(layers: List[Dict], seed: int, batch: int, seq: int, kind: str = "token_ids") -> np.ndarray:
+    """Dense network input in the layout ``rpool_add_nasm_raw_input`` takes:
+    NHWC for images (uniform [0,1)), ``[batch][seq][M]`` for transformers.
+
+    Transformer kind "embeddings": rows ~ N(0, 0.02^2) fed directly.  Kind
+    "token_ids": ids uniform in [0, 50257) select rows of a seeded N(0, 0.02^2) table (wte) and a position
+    table (wpe) is added; the lookup happens here, outside the graph, because
+    the reference graph starts at the float matrix (its cfg has no embedding)."""
+    L0 = layers[0]
+    if L0["M"]:
+        M = L0["M"]
+        if kind == "embeddings":
+            return normal(seed, 1_000_004, (batch, seq, M), 0.02)
+        ids = (uniform(seed, 1_000_001, (batch, seq)).astype(np.float64) * 50257).astype(np.int64)
+        # wte rows generated on demand: row r = normal stream with tensor id derived from r
+        uniq, inv = np.unique(ids, return_inverse=True)
+        rows = np.stack([normal(seed, 2_000_000 + int(r), (M,), 0.02) for r in uniq])
+        wpe = normal(seed, 1_000_002, (seq, M), 0.02)
+        x = rows[inv.reshape(-1)].reshape(batch, seq, M) + wpe[None]
+        return np.ascontiguousarray(x, dtype=np.float32)
+    nchw = uniform(seed, 1_000_003, (batch, L0["C"], L0["H"], L0["W"]))
+    return np.ascontiguousarray(nchw.transpose(0, 2, 3, 1))

@@ -1,0 +1,126 @@
+/*
+ * aspen_hip.h -- flat C ABI of the gfx950 tile kernels and the device-side dataflow engine.
+ *
+ * This is the boundary the C host library (and any other host runtime) binds: plain pointers,
+ * sizes and POD descriptors, no C++ or framework types.  It replaces the reference's internal
+ * kernel seam
+ *     void tiled_X (ninst_t *ninst, dse_t *dse)          reference include/kernels.h:35-46
+ *     switch (layer->type) in dse_schedule               reference src/dse.c:39-79
+ *     SGEMM_KERNEL* (M,N,K,A,lda,B,ldb,C,ldc)            reference include/kernels.h:15-33
+ * and the scheduler / ready-pool protocol around it
+ *     dse_schedule, update_children_*                    reference src/dse.c:20-108, :363-401
+ *     rpool_push_ninsts / rpool_fetch_ninsts             reference src/rpool.c:611-685
+ *     push_first_layer_to_rpool                          reference src/dse.c:443-470
+ *
+ * Data contract (same as the reference's out_mat, reference src/apu_nasm.c:950-1017):
+ * an activation is a matrix of N columns x M rows stored column by column with a stride of `ld`
+ * floats (NHWC with a padded channel run).  Padding rows [M, ld) are zero and are never written.
+ * All pointers inside aspen_hip_layer_t are DEVICE pointers obtained from aspen_hip_alloc.
+ *
+ * Every function returns 0 on success and a non-zero HIP error code otherwise (the text is
+ * available from aspen_hip_last_error); allocation returns NULL on failure.
+ */
+#ifndef ASPEN_AMD_ASPEN_HIP_H
+#define ASPEN_AMD_ASPEN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* One k-chunk (4 consecutive floats of the implicit-GEMM K axis) of a conv / FC layer:
+   where it sits relative to the top-left input pixel of an output position. */
+typedef struct aspen_hip_ktab_t
+{
+    int32_t offset;      /* (kh*IW + kw)*ld_in + ic, in floats */
+    uint16_t kh, kw;     /* tap; kh >= 0x4000 marks a chunk beyond the real K (reads as zero) */
+} aspen_hip_ktab_t;
+
+/* GEMM tile shapes (rows of the weight matrix x activation columns per workgroup). */
+enum { ASPEN_HIP_GEMM_128x128 = 0, ASPEN_HIP_GEMM_64x128 = 1, ASPEN_HIP_GEMM_64x64 = 2, ASPEN_HIP_NUM_GEMM_VARIANTS };
+
+/* Per-layer descriptor: everything one tile needs, so a tile is (layer, tile index).
+   Replaces the fields the reference's tiled_* read through ninst->ldata->layer
+   (reference include/nasm.h:28-66, include/apu.h:33-43). */
+typedef struct aspen_hip_layer_t
+{
+    int32_t type;            /* LAYER_TYPE of aspen.h */
+    int32_t act;             /* LAYER_ACT of aspen.h */
+    int32_t variant;         /* GEMM tile shape for contraction layers */
+    int32_t direct;          /* 1: B operand is read in place (1x1 stride-1 conv / matmul, K % 32 == 0) */
+    uint32_t M, N, ld;       /* output rows, columns, stride */
+    uint32_t tile_m, tile_n; /* tile extent in rows / columns */
+    uint32_t tiles_m, tiles_n;
+    uint32_t ninst_start;    /* engine-wide index of this layer's first tile */
+    uint32_t num_ninst;
+    uint32_t K, Kp;          /* contraction length, padded to a multiple of 32 */
+    uint32_t ld0, ld1;       /* strides of the parents */
+    uint32_t IH, IW, IC, OH, OW, KH, KW, stride, pad;
+    uint32_t heads, seq, hd, masked;
+    uint32_t reserved;
+    float *out;
+    const float *in0;        /* PARENT_0 */
+    const float *in1;        /* PARENT_1 */
+    const float *weight;     /* [roundup(M,128)][Kp] row-major, zero padded; layernorm: gamma[M] */
+    const float *bias;       /* [M] or NULL */
+    const aspen_hip_ktab_t *ktab; /* Kp/4 entries, NULL when direct */
+} aspen_hip_layer_t;
+
+typedef struct aspen_hip_graph_t aspen_hip_graph_t;
+
+/* ---- device, memory, transfers --------------------------------------------------------------- */
+int aspen_hip_init (void);
+const char *aspen_hip_last_error (void);
+/* compute units, engine clock (kHz), HBM bytes, device name */
+int aspen_hip_device_info (int *num_cu, int *clock_khz, size_t *mem_bytes, char *name, int name_len);
+void *aspen_hip_alloc (size_t bytes);            /* zero-filled device memory */
+void aspen_hip_free (void *ptr);
+int aspen_hip_h2d (void *dst, const void *src, size_t bytes);
+int aspen_hip_d2h (void *dst, const void *src, size_t bytes);
+/* strided copies: `rows` runs of `width` bytes, pitches in bytes */
+int aspen_hip_h2d_2d (void *dst, size_t dpitch, const void *src, size_t spitch, size_t width, size_t rows);
+int aspen_hip_d2h_2d (void *dst, size_t dpitch, const void *src, size_t spitch, size_t width, size_t rows);
+int aspen_hip_zero (void *dst, size_t bytes);
+
+/* ---- graph ----------------------------------------------------------------------------------- */
+/* Uploads a tile graph.  ninst_layer[i] = layer of tile i; num_parents[i] = its dependency count;
+   children of tile i are child_idx[child_off[i] .. child_off[i+1]).  roots = tiles with no parent
+   left once the input layer counts as complete.  (reference: ninst_t, include/nasm.h:50-66) */
+aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *layers, uint32_t num_layers,
+    const uint32_t *ninst_layer, const uint32_t *num_parents, const uint32_t *child_off,
+    const uint32_t *child_idx, uint32_t num_ninst, const uint32_t *roots, uint32_t num_roots);
+void aspen_hip_graph_destroy (aspen_hip_graph_t *graph);
+
+/* ---- execution (all asynchronous on the library's stream) -------------------------------------- */
+/* One launch per layer, layers [first, last] in index order: the per-operator baseline and the
+   per-kernel profiling mode. */
+int aspen_hip_run_layers (aspen_hip_graph_t *graph, uint32_t first_layer, uint32_t last_layer);
+/* Barrier-free execution: re-arms the dependency counters and the ready queue, then one persistent
+   kernel of `workgroups` workgroups (0 = two per compute unit) pops ready tiles until all are done.
+   spin_limit bounds every wait on the ready queue (0 = default); a wait that exceeds it raises the
+   abort flag, all workgroups exit and aspen_hip_sync returns ASPEN_HIP_ERR_STALLED. */
+int aspen_hip_run_dataflow (aspen_hip_graph_t *graph, uint32_t workgroups, uint64_t spin_limit);
+#define ASPEN_HIP_ERR_STALLED 0x7001
+int aspen_hip_sync (void);
+/* 1 when everything enqueued so far has finished, 0 when still running */
+int aspen_hip_idle (void);
+/* Tiles executed / executed-twice / executed-before-ready counters of the last dataflow run. */
+int aspen_hip_dataflow_stats (aspen_hip_graph_t *graph, uint32_t *executed, uint32_t *double_runs, uint32_t *abort_flag);
+
+/* ---- timing ------------------------------------------------------------------------------------- */
+/* HIP events on the library's stream: record into slot [0,16), elapsed between two recorded slots. */
+int aspen_hip_event_record (int slot);
+int aspen_hip_event_elapsed_ms (int slot_begin, int slot_end, float *ms);
+
+/* ---- plain SGEMM seam (reference include/kernels.h:15-33 on device pointers) -------------------- */
+/* C[n*ldc + m] = act(bias[m] + sum_k A[m*lda + k] * B[n*ldb + k]); A row-major [M][K] (not packed),
+   lda/ldb/ldc multiples of 4, K a multiple of 32. */
+int aspen_hip_sgemm (uint32_t M, uint32_t N, uint32_t K, const float *A, uint32_t lda, const float *B,
+    uint32_t ldb, float *C, uint32_t ldc, const float *bias, int act);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ASPEN_AMD_ASPEN_HIP_H */
