@@ -1,0 +1,430 @@
+// Host side of the flat C ABI (include/aspen_hip.h): device setup, memory, graph upload, the
+// per-layer launch path and the persistent dataflow engine.
+//
+// The dataflow engine is the device-side counterpart of the reference's scheduler:
+//   ready pool  (reference src/rpool.c:611-685)  -> one ticket queue in HBM, a slot per tile
+//   dse_schedule (reference src/dse.c:20-108)    -> loop of a persistent workgroup
+//   update_children (reference src/dse.c:363-401)-> atomic decrement of the children's dependency
+//                                                   counters; the last parent publishes the child
+//   push_first_layer_to_rpool (src/dse.c:443)    -> arm kernel seeds the queue with the root tiles
+#include <hip/hip_runtime.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include "tile_kernels.h"
+
+#define QUEUE_EMPTY 0xffffffffu
+#define NUM_EVENTS 16
+#define DEFAULT_SPIN_LIMIT (1ull << 26)
+
+struct aspen_hip_graph_t
+{
+    uint32_t num_layers, num_ninst, num_roots, num_edges;
+    aspen_hip_layer_t *h_layers;
+    aspen_hip_layer_t *d_layers;
+    uint32_t *d_ninst_layer, *d_num_parents, *d_child_off, *d_child_idx, *d_roots;
+    uint32_t *d_dep;        // remaining-parent counters, re-armed before every dataflow run
+    uint32_t *d_queue;      // ready queue: slot t is written once, by whoever makes a tile ready
+    uint32_t *d_state;      // [0] pop tickets, [1] push cursor, [2] tiles done, [3] abort flag, [4] double-run count
+    uint32_t *d_ran;        // per-tile execution count (sanity: every tile exactly once)
+};
+
+static hipStream_t g_stream = nullptr;
+static hipEvent_t g_events[NUM_EVENTS];
+static int g_inited = 0;
+static int g_num_cu = 0;
+static char g_err[512] = "";
+
+static int fail (hipError_t e, const char *what)
+{
+    snprintf (g_err, sizeof (g_err), "%s: %s", what, hipGetErrorString (e));
+    fprintf (stderr, "aspen_hip: %s\n", g_err);
+    return (int)e;
+}
+#define CHECK(call) do { hipError_t e_ = (call); if (e_ != hipSuccess) return fail (e_, #call); } while (0)
+
+// ------------------------------------------------------------------------------------------------
+// kernels
+// ------------------------------------------------------------------------------------------------
+
+// Per-layer launch: workgroup -> tile with contiguous tile ranges per XCD (workgroups are dealt to
+// the 8 XCDs round-robin), so tiles that share activation rows meet in the same L2.
+__global__ void __launch_bounds__ (WG_THREADS, 2) layer_kernel (const aspen_hip_layer_t *layers, uint32_t l)
+{
+    extern __shared__ __align__ (16) float smem[];
+    const aspen_hip_layer_t &L = layers[l];
+    const uint32_t nt = gridDim.x, bid = blockIdx.x;
+    const uint32_t xcd = bid & 7, local = bid >> 3, chunk = nt >> 3, rem = nt & 7;
+    const uint32_t t = xcd * chunk + (xcd < rem ? xcd : rem) + local;
+    run_tile (L, t, smem);
+}
+
+// Re-arm: counters back to the parent counts, queue emptied and seeded with the roots.
+__global__ void arm_kernel (uint32_t *dep, const uint32_t *num_parents, uint32_t *queue, uint32_t *ran,
+    const uint32_t *roots, uint32_t num_ninst, uint32_t num_roots, uint32_t *state)
+{
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < num_ninst)
+    {
+        dep[i] = num_parents[i];
+        queue[i] = i < num_roots ? roots[i] : QUEUE_EMPTY;
+        ran[i] = 0;
+    }
+    if (i == 0) { state[0] = 0; state[1] = num_roots; state[2] = 0; state[3] = 0; state[4] = 0; }
+}
+
+struct dataflow_args_t
+{
+    const aspen_hip_layer_t *layers;
+    const uint32_t *ninst_layer, *child_off, *child_idx;
+    uint32_t *dep, *queue, *state, *ran;
+    uint32_t num_ninst;
+    unsigned long long spin_limit;
+};
+
+__global__ void __launch_bounds__ (WG_THREADS, 2) dataflow_kernel (dataflow_args_t a)
+{
+    extern __shared__ __align__ (16) float smem[];
+    __shared__ uint32_t s_tile;
+    for (;;)
+    {
+        if (threadIdx.x == 0)
+        {
+            uint32_t id = QUEUE_EMPTY;
+            const uint32_t ticket = atomicAdd (&a.state[0], 1u);
+            if (ticket < a.num_ninst)
+            {
+                unsigned long long spins = 0;
+                for (;;)
+                {
+                    id = __hip_atomic_load (&a.queue[ticket], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+                    if (id != QUEUE_EMPTY) break;
+                    if (__hip_atomic_load (&a.state[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+                    if (++spins > a.spin_limit)
+                    {
+                        __hip_atomic_store (&a.state[3], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep (8);
+                }
+            }
+            s_tile = id;
+        }
+        __syncthreads ();
+        const uint32_t id = s_tile;
+        if (id == QUEUE_EMPTY) return;          // all tickets taken, or aborted
+        // make the parents' tiles (written by other XCDs) visible to every wave of this workgroup
+        __builtin_amdgcn_fence (__ATOMIC_ACQUIRE, "agent");
+
+        const aspen_hip_layer_t &L = a.layers[a.ninst_layer[id]];
+        run_tile (L, id - L.ninst_start, smem);
+
+        // publish this tile, then count down the children
+        __builtin_amdgcn_fence (__ATOMIC_RELEASE, "agent");
+        __syncthreads ();
+        const uint32_t c0 = a.child_off[id], c1 = a.child_off[id + 1];
+        for (uint32_t c = c0 + threadIdx.x; c < c1; c += WG_THREADS)
+        {
+            const uint32_t child = a.child_idx[c];
+            const uint32_t before = __hip_atomic_fetch_sub (&a.dep[child], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+            if (before == 1u)
+            {
+                const uint32_t slot = atomicAdd (&a.state[1], 1u);
+                __hip_atomic_store (&a.queue[slot], child, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        if (threadIdx.x == 0)
+        {
+            if (atomicAdd (&a.ran[id], 1u) != 0) atomicAdd (&a.state[4], 1u);
+            atomicAdd (&a.state[2], 1u);
+        }
+        __syncthreads ();
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// device, memory
+// ------------------------------------------------------------------------------------------------
+extern "C" int aspen_hip_init (void)
+{
+    if (g_inited) return 0;
+    int count = 0;
+    CHECK (hipGetDeviceCount (&count));
+    if (count < 1) { snprintf (g_err, sizeof (g_err), "no HIP device"); return -1; }
+    CHECK (hipSetDevice (0));
+    hipDeviceProp_t prop;
+    CHECK (hipGetDeviceProperties (&prop, 0));
+    g_num_cu = prop.multiProcessorCount;
+    CHECK (hipStreamCreate (&g_stream));
+    for (int i = 0; i < NUM_EVENTS; i++) CHECK (hipEventCreate (&g_events[i]));
+    CHECK (hipFuncSetAttribute ((const void *)layer_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
+    CHECK (hipFuncSetAttribute ((const void *)dataflow_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
+    g_inited = 1;
+    return 0;
+}
+
+extern "C" const char *aspen_hip_last_error (void) { return g_err; }
+
+extern "C" int aspen_hip_device_info (int *num_cu, int *clock_khz, size_t *mem_bytes, char *name, int name_len)
+{
+    if (aspen_hip_init ()) return -1;
+    hipDeviceProp_t prop;
+    CHECK (hipGetDeviceProperties (&prop, 0));
+    if (num_cu) *num_cu = prop.multiProcessorCount;
+    if (clock_khz) *clock_khz = prop.clockRate;
+    if (mem_bytes) *mem_bytes = prop.totalGlobalMem;
+    if (name && name_len > 0) { strncpy (name, prop.name, name_len - 1); name[name_len - 1] = 0; }
+    return 0;
+}
+
+extern "C" void *aspen_hip_alloc (size_t bytes)
+{
+    if (aspen_hip_init ()) return nullptr;
+    void *p = nullptr;
+    if (bytes == 0) bytes = 256;
+    hipError_t e = hipMalloc (&p, bytes + 256);      // slack: edge tiles may read (never write) a few floats past a row
+    if (e != hipSuccess) { fail (e, "hipMalloc"); return nullptr; }
+    e = hipMemsetAsync (p, 0, bytes + 256, g_stream);
+    if (e == hipSuccess) e = hipStreamSynchronize (g_stream);
+    if (e != hipSuccess) { fail (e, "hipMemset"); (void)hipFree (p); return nullptr; }
+    return p;
+}
+
+extern "C" void aspen_hip_free (void *ptr) { if (ptr) (void)hipFree (ptr); }
+
+extern "C" int aspen_hip_h2d (void *dst, const void *src, size_t bytes)
+{
+    if (aspen_hip_init ()) return -1;
+    CHECK (hipMemcpyAsync (dst, src, bytes, hipMemcpyHostToDevice, g_stream));
+    CHECK (hipStreamSynchronize (g_stream));
+    return 0;
+}
+extern "C" int aspen_hip_d2h (void *dst, const void *src, size_t bytes)
+{
+    if (aspen_hip_init ()) return -1;
+    CHECK (hipMemcpyAsync (dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
+    CHECK (hipStreamSynchronize (g_stream));
+    return 0;
+}
+extern "C" int aspen_hip_h2d_2d (void *dst, size_t dpitch, const void *src, size_t spitch, size_t width, size_t rows)
+{
+    if (aspen_hip_init ()) return -1;
+    CHECK (hipMemcpy2DAsync (dst, dpitch, src, spitch, width, rows, hipMemcpyHostToDevice, g_stream));
+    CHECK (hipStreamSynchronize (g_stream));
+    return 0;
+}
+extern "C" int aspen_hip_d2h_2d (void *dst, size_t dpitch, const void *src, size_t spitch, size_t width, size_t rows)
+{
+    if (aspen_hip_init ()) return -1;
+    CHECK (hipMemcpy2DAsync (dst, dpitch, src, spitch, width, rows, hipMemcpyDeviceToHost, g_stream));
+    CHECK (hipStreamSynchronize (g_stream));
+    return 0;
+}
+extern "C" int aspen_hip_zero (void *dst, size_t bytes)
+{
+    if (aspen_hip_init ()) return -1;
+    CHECK (hipMemsetAsync (dst, 0, bytes, g_stream));
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+// graph
+// ------------------------------------------------------------------------------------------------
+template <class T> static T *upload (const T *src, size_t n)
+{
+    T *d = (T *)aspen_hip_alloc ((n ? n : 1) * sizeof (T));
+    if (d && n && aspen_hip_h2d (d, src, n * sizeof (T))) { aspen_hip_free (d); return nullptr; }
+    return d;
+}
+
+static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
+{
+    const char *why = nullptr;
+    if (L.type == INPUT_LAYER) return 0;
+    if (!L.out || !L.in0) why = "missing buffers";
+    else if (L.ld % 4 || L.ld0 % 4 || (L.in1 && L.ld1 % 4)) why = "strides must be multiples of 4 floats";
+    else if (L.tiles_m == 0 || L.tiles_n == 0 || L.num_ninst != L.tiles_m * L.tiles_n) why = "tile grid";
+    else if (L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER)
+    {
+        const uint32_t bm = L.variant == ASPEN_HIP_GEMM_128x128 ? 128 : 64, bn = L.variant == ASPEN_HIP_GEMM_64x64 ? 64 : 128;
+        if (!L.weight) why = "missing weight";
+        else if (L.Kp == 0 || L.Kp % GEMM_BK) why = "Kp must be a positive multiple of 32";
+        else if (L.tile_m != bm || L.tile_n != bn) why = "tile extent does not match the GEMM variant";
+        else if ((uint64_t)L.tiles_m * bm < L.M || (uint64_t)L.tiles_n * bn < L.N) why = "tile grid does not cover the matrix";
+        else if (!L.direct && !L.ktab) why = "missing k-chunk table";
+        else if (L.direct && (L.ld0 < L.Kp)) why = "direct operand shorter than Kp";
+    }
+    else if (L.type == K_ATTENTION_LAYER)
+    {
+        if (!L.in1 || L.hd == 0 || L.hd % GEMM_BK || L.heads == 0 || L.seq == 0) why = "attention geometry";
+        else if (L.ld < L.seq || L.ld % GEMM_BK) why = "probability stride must be a multiple of 32 covering seq";
+        else if (L.tile_n != 128 || L.tiles_m != 1) why = "K-attention tiles are 128 queries x all keys";
+    }
+    else if (L.type == V_ATTENTION_LAYER)
+    {
+        if (!L.in1 || L.hd == 0 || L.heads == 0 || L.seq == 0) why = "attention geometry";
+        else if (L.tile_n != 128 || L.tile_m > 64 || L.hd % L.tile_m) why = "V-attention tiles are 128 queries x <=64 channels of one head";
+        else if (L.ld0 % GEMM_BK || L.ld0 < L.seq) why = "probability stride must be a multiple of 32 covering seq";
+    }
+    else if (L.type == RESIDUAL_LAYER) { if (!L.in1) why = "missing second parent"; }
+    else if (L.type == LAYERNORM_LAYER) { if (!L.weight) why = "missing gamma"; }
+    if (why)
+    {
+        snprintf (g_err, sizeof (g_err), "layer %u rejected: %s", idx, why);
+        fprintf (stderr, "aspen_hip: %s\n", g_err);
+        return -1;
+    }
+    return 0;
+}
+
+extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *layers, uint32_t num_layers,
+    const uint32_t *ninst_layer, const uint32_t *num_parents, const uint32_t *child_off,
+    const uint32_t *child_idx, uint32_t num_ninst, const uint32_t *roots, uint32_t num_roots)
+{
+    if (aspen_hip_init ()) return nullptr;
+    for (uint32_t l = 0; l < num_layers; l++)
+        if (check_layer (layers[l], l)) return nullptr;
+    // host-side sanity of the dependency structure: every index in range, counts consistent
+    const uint32_t num_edges = child_off[num_ninst];
+    {
+        uint32_t *seen = (uint32_t *)calloc (num_ninst ? num_ninst : 1, sizeof (uint32_t));
+        bool ok = true;
+        for (uint32_t e = 0; e < num_edges && ok; e++) { if (child_idx[e] >= num_ninst) ok = false; else seen[child_idx[e]]++; }
+        for (uint32_t i = 0; i < num_ninst && ok; i++) if (seen[i] != num_parents[i] || ninst_layer[i] >= num_layers) ok = false;
+        for (uint32_t r = 0; r < num_roots && ok; r++) if (roots[r] >= num_ninst || num_parents[roots[r]] != 0) ok = false;
+        free (seen);
+        if (!ok) { snprintf (g_err, sizeof (g_err), "inconsistent dependency arrays"); fprintf (stderr, "aspen_hip: %s\n", g_err); return nullptr; }
+    }
+    aspen_hip_graph_t *g = (aspen_hip_graph_t *)calloc (1, sizeof (aspen_hip_graph_t));
+    g->num_layers = num_layers; g->num_ninst = num_ninst; g->num_roots = num_roots; g->num_edges = num_edges;
+    g->h_layers = (aspen_hip_layer_t *)malloc (sizeof (aspen_hip_layer_t) * num_layers);
+    memcpy (g->h_layers, layers, sizeof (aspen_hip_layer_t) * num_layers);
+    g->d_layers = upload (layers, num_layers);
+    g->d_ninst_layer = upload (ninst_layer, num_ninst);
+    g->d_num_parents = upload (num_parents, num_ninst);
+    g->d_child_off = upload (child_off, (size_t)num_ninst + 1);
+    g->d_child_idx = upload (child_idx, num_edges);
+    g->d_roots = upload (roots, num_roots);
+    g->d_dep = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
+    g->d_queue = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
+    g->d_ran = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
+    g->d_state = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * 16);
+    if (!g->d_layers || !g->d_ninst_layer || !g->d_num_parents || !g->d_child_off || !g->d_child_idx || !g->d_roots
+        || !g->d_dep || !g->d_queue || !g->d_ran || !g->d_state)
+    {
+        aspen_hip_graph_destroy (g);
+        return nullptr;
+    }
+    return g;
+}
+
+extern "C" void aspen_hip_graph_destroy (aspen_hip_graph_t *g)
+{
+    if (!g) return;
+    (void)hipStreamSynchronize (g_stream);
+    aspen_hip_free (g->d_layers); aspen_hip_free (g->d_ninst_layer); aspen_hip_free (g->d_num_parents);
+    aspen_hip_free (g->d_child_off); aspen_hip_free (g->d_child_idx); aspen_hip_free (g->d_roots);
+    aspen_hip_free (g->d_dep); aspen_hip_free (g->d_queue); aspen_hip_free (g->d_ran); aspen_hip_free (g->d_state);
+    free (g->h_layers);
+    free (g);
+}
+
+// ------------------------------------------------------------------------------------------------
+// execution
+// ------------------------------------------------------------------------------------------------
+extern "C" int aspen_hip_run_layers (aspen_hip_graph_t *g, uint32_t first_layer, uint32_t last_layer)
+{
+    if (!g || first_layer > last_layer || last_layer >= g->num_layers) { snprintf (g_err, sizeof (g_err), "run_layers: bad range"); return -1; }
+    for (uint32_t l = first_layer; l <= last_layer; l++)
+    {
+        const aspen_hip_layer_t &L = g->h_layers[l];
+        if (L.type == INPUT_LAYER || L.num_ninst == 0) continue;
+        hipLaunchKernelGGL (layer_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, g->d_layers, l);
+        CHECK (hipGetLastError ());
+    }
+    return 0;
+}
+
+extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups, uint64_t spin_limit)
+{
+    if (!g) { snprintf (g_err, sizeof (g_err), "run_dataflow: null graph"); return -1; }
+    if (g->num_ninst == 0) return 0;
+    if (workgroups == 0) workgroups = 2 * (uint32_t)g_num_cu;
+    hipLaunchKernelGGL (arm_kernel, dim3 ((g->num_ninst + 255) / 256), dim3 (256), 0, g_stream,
+        g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->num_ninst, g->num_roots, g->d_state);
+    CHECK (hipGetLastError ());
+    dataflow_args_t a;
+    a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx;
+    a.dep = g->d_dep; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran;
+    a.num_ninst = g->num_ninst; a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
+    hipLaunchKernelGGL (dataflow_kernel, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);
+    CHECK (hipGetLastError ());
+    return 0;
+}
+
+extern "C" int aspen_hip_sync (void)
+{
+    if (aspen_hip_init ()) return -1;
+    CHECK (hipStreamSynchronize (g_stream));
+    return 0;
+}
+
+extern "C" int aspen_hip_idle (void)
+{
+    if (aspen_hip_init ()) return -1;
+    return hipStreamQuery (g_stream) == hipSuccess ? 1 : 0;
+}
+
+extern "C" int aspen_hip_dataflow_stats (aspen_hip_graph_t *g, uint32_t *executed, uint32_t *double_runs, uint32_t *abort_flag)
+{
+    if (!g) return -1;
+    uint32_t st[8];
+    if (aspen_hip_d2h (st, g->d_state, sizeof (st))) return -1;
+    if (executed) *executed = st[2];
+    if (abort_flag) *abort_flag = st[3];
+    if (double_runs) *double_runs = st[4];
+    return 0;
+}
+
+extern "C" int aspen_hip_event_record (int slot)
+{
+    if (aspen_hip_init ()) return -1;
+    if (slot < 0 || slot >= NUM_EVENTS) return -1;
+    CHECK (hipEventRecord (g_events[slot], g_stream));
+    return 0;
+}
+
+extern "C" int aspen_hip_event_elapsed_ms (int a, int b, float *ms)
+{
+    if (a < 0 || a >= NUM_EVENTS || b < 0 || b >= NUM_EVENTS || !ms) return -1;
+    CHECK (hipEventSynchronize (g_events[b]));
+    CHECK (hipEventElapsedTime (ms, g_events[a], g_events[b]));
+    return 0;
+}
+
+extern "C" int aspen_hip_sgemm (uint32_t M, uint32_t N, uint32_t K, const float *A, uint32_t lda, const float *B,
+    uint32_t ldb, float *C, uint32_t ldc, const float *bias, int act)
+{
+    if (aspen_hip_init ()) return -1;
+    if (K == 0 || K % GEMM_BK || lda % 4 || ldb % 4 || ldc % 4 || lda < K || ldb < K || ldc < M)
+    { snprintf (g_err, sizeof (g_err), "sgemm: K must be a multiple of 32, strides multiples of 4"); return -1; }
+    // weight rows are read in blocks of 64 without a row clamp: stage A into a zero-padded copy
+    const uint32_t Mp = (M + 127) / 128 * 128;
+    float *Ap = (float *)aspen_hip_alloc ((size_t)Mp * K * sizeof (float));
+    if (!Ap) return -1;
+    CHECK (hipMemcpy2DAsync (Ap, (size_t)K * 4, A, (size_t)lda * 4, (size_t)K * 4, M, hipMemcpyDeviceToDevice, g_stream));
+    aspen_hip_layer_t L;
+    memset (&L, 0, sizeof (L));
+    L.type = MATMUL_LAYER; L.act = act; L.variant = ASPEN_HIP_GEMM_64x64; L.direct = 1;
+    L.M = M; L.N = N; L.ld = ldc; L.tile_m = 64; L.tile_n = 64;
+    L.tiles_m = (M + 63) / 64; L.tiles_n = (N + 63) / 64; L.num_ninst = L.tiles_m * L.tiles_n;
+    L.K = K; L.Kp = K; L.ld0 = ldb; L.out = C; L.in0 = B; L.weight = Ap; L.bias = bias;
+    aspen_hip_layer_t *dL = upload (&L, 1);
+    if (!dL) { aspen_hip_free (Ap); return -1; }
+    hipLaunchKernelGGL (layer_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, dL, 0u);
+    hipError_t e = hipGetLastError ();
+    if (e == hipSuccess) e = hipStreamSynchronize (g_stream);
+    aspen_hip_free (dL); aspen_hip_free (Ap);
+    if (e != hipSuccess) return fail (e, "sgemm launch");
+    return 0;
+}

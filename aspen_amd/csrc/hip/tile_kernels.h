@@ -1,0 +1,523 @@
+// Device-side tile arithmetic for gfx950 (MI355X): one function per tile class, each executed by one
+// 256-thread workgroup (4 wavefronts of 64) on one output tile.  Shared by the per-layer launch
+// kernel and the persistent dataflow kernel.
+//
+// Semantics follow the reference's per-ninst operators (reference src/tiled_kernels.c):
+//   contraction tiles  tiled_conv2d :161, tiled_matmul :299, tiled_fully_connected :502
+//                      (zero -> accumulate over K -> + bias -> activation)
+//   tiled_residual :613, tiled_maxpool2d :411, tiled_avgpool2d :456, tiled_layernorm :743,
+//   tiled_softmax :640, tiled_k_attention :784, tiled_v_attention :934
+//   activation formulas: naive_activate, reference src/naive_kernels.c:11-57
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "aspen.h"
+#include "aspen_hip.h"
+
+typedef float floatx16 __attribute__ ((ext_vector_type (16)));
+
+#define WG_THREADS 256
+#define GEMM_BK 32            // K floats staged per iteration: one 128-byte line per operand row
+#define LDS_ROW 36            // floats per staged row: 32 + 4 padding -> conflict-free 128-bit reads
+#define GEMM_SMEM_FLOATS (2 * (128 + 128) * LDS_ROW)
+#define GEMM_SMEM_BYTES (GEMM_SMEM_FLOATS * 4)
+
+__device__ __forceinline__ float4 ld4 (const float *p) { return *reinterpret_cast<const float4 *> (p); }
+__device__ __forceinline__ void st4 (float *p, float4 v) { *reinterpret_cast<float4 *> (p) = v; }
+
+__device__ __forceinline__ float activate (float x, int act)
+{
+    switch (act)
+    {
+    case RELU:          return x > 0 ? x : 0;
+    case LEAKY_RELU:    return x > 0 ? x : (float)(0.1 * (double)x);
+    case ELU:           return x > 0 ? x : (float)(0.1 * (exp ((double)x) - 1));
+    case SELU:          return x > 0 ? (float)(1.0507 * (double)x) : (float)(1.0507 * 1.67326 * (exp ((double)x) - 1));
+    case SIGMOID:       return (float)(1 / (1 + exp (-(double)x)));
+    case TANH:          return (float)tanh ((double)x);
+    case GELU:          return (float)(0.5 * (double)x * (double)(1 + erff (x * 0.7071067811865475f)));
+    case GELU_ACCURATE: return (float)(0.5 * (double)x * (double)(1 + tanhf (0.7978845608028654f * (float)((double)x + 0.044715 * (double)x * (double)x * (double)x))));
+    default:            return x;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Operand loaders.  A loader fetches this thread's share of one GEMM_BK-wide K slice into registers
+// (load) and later parks it in LDS as [row][LDS_ROW] (store), so the global loads of slice i+1 fly
+// while the matrix cores work on slice i.
+// ---------------------------------------------------------------------------------------------
+
+// Rows are K-contiguous in memory: weights [M][Kp], matmul / 1x1-conv activations, Q and K rows.
+template <int ROWS> struct RowLoader
+{
+    static constexpr int R = ROWS / 32;
+    const float *ptr[R];
+    uint32_t chunk, row0;
+    __device__ __forceinline__ void init (const float *base, uint32_t first_row, uint32_t max_row, uint32_t ld, uint32_t tid)
+    {
+        chunk = tid & 7; row0 = tid >> 3;
+        #pragma unroll
+        for (int i = 0; i < R; i++)
+        {
+            uint32_t r = first_row + row0 + 32 * i;
+            r = r < max_row ? r : max_row;          // clamp: rows past the edge re-read the last row, never stored
+            ptr[i] = base + (size_t)r * ld + chunk * 4;
+        }
+    }
+    __device__ __forceinline__ void load (int it, float4 (&v)[R])
+    {
+        #pragma unroll
+        for (int i = 0; i < R; i++) v[i] = ld4 (ptr[i] + it * GEMM_BK);
+    }
+    __device__ __forceinline__ void store (float *lds, const float4 (&v)[R])
+    {
+        #pragma unroll
+        for (int i = 0; i < R; i++) st4 (lds + (row0 + 32 * i) * LDS_ROW + chunk * 4, v[i]);
+    }
+};
+
+// Implicit-GEMM activation operand of conv / FC: row n = output position (b, oh, ow); the K axis runs
+// over (kh, kw, ic) and is resolved through the layer's k-chunk table.  Replaces the reference's
+// pointer table + panel gather (prepare_input / load_im2col_ptr, reference src/tiled_kernels.c:3-159).
+template <int ROWS> struct ConvLoader
+{
+    static constexpr int R = ROWS / 32;
+    const float *in;
+    const aspen_hip_ktab_t *ktab;
+    int32_t base[R], ih0[R], iw0[R];
+    uint32_t IH, IW, chunk, row0;
+    __device__ __forceinline__ void init (const aspen_hip_layer_t &L, uint32_t first_row, uint32_t tid)
+    {
+        in = L.in0; ktab = L.ktab; IH = L.IH; IW = L.IW;
+        chunk = tid & 7; row0 = tid >> 3;
+        const uint32_t ohw = L.OH * L.OW;
+        #pragma unroll
+        for (int i = 0; i < R; i++)
+        {
+            uint32_t n = first_row + row0 + 32 * i;
+            n = n < L.N ? n : L.N - 1;
+            uint32_t b = n / ohw, rem = n - b * ohw, oh = rem / L.OW, ow = rem - oh * L.OW;
+            ih0[i] = (int32_t)(oh * L.stride) - (int32_t)L.pad;
+            iw0[i] = (int32_t)(ow * L.stride) - (int32_t)L.pad;
+            base[i] = ((int32_t)(b * L.IH) + ih0[i]) * (int32_t)L.IW * (int32_t)L.ld0 + iw0[i] * (int32_t)L.ld0;
+        }
+    }
+    __device__ __forceinline__ void load (int it, float4 (&v)[R])
+    {
+        const aspen_hip_ktab_t e = ktab[it * 8 + chunk];
+        #pragma unroll
+        for (int i = 0; i < R; i++)
+        {
+            const bool ok = (uint32_t)(ih0[i] + (int32_t)e.kh) < IH && (uint32_t)(iw0[i] + (int32_t)e.kw) < IW;
+            v[i] = ok ? ld4 (in + (ptrdiff_t)(base[i] + e.offset)) : make_float4 (0.f, 0.f, 0.f, 0.f);
+        }
+    }
+    __device__ __forceinline__ void store (float *lds, const float4 (&v)[R])
+    {
+        #pragma unroll
+        for (int i = 0; i < R; i++) st4 (lds + (row0 + 32 * i) * LDS_ROW + chunk * 4, v[i]);
+    }
+};
+
+// K-strided operand (V of attention: rows = channels, K axis = sequence position with stride ld):
+// read 64 channels x 32 positions with 128-bit loads along the channels, transpose into LDS.
+struct TransLoader64
+{
+    static constexpr int R = 2;
+    const float *ptr[2];
+    uint32_t c4, s0, ld, klen;
+    bool live;
+    // valid_rows: channels of this tile that exist; klen: length of the K axis (positions >= klen read as zero)
+    __device__ __forceinline__ void init (const float *base, uint32_t ld_, uint32_t valid_rows, uint32_t klen_, uint32_t tid)
+    {
+        ld = ld_; klen = klen_; c4 = tid & 15; s0 = tid >> 4; live = c4 * 4 < valid_rows;
+        ptr[0] = base + (size_t)s0 * ld + c4 * 4;
+        ptr[1] = base + (size_t)(s0 + 16) * ld + c4 * 4;
+    }
+    __device__ __forceinline__ void load (int it, float4 (&v)[2])
+    {
+        const float4 z = make_float4 (0.f, 0.f, 0.f, 0.f);
+        const uint32_t s = it * GEMM_BK + s0;
+        v[0] = (live && s < klen) ? ld4 (ptr[0] + (size_t)it * GEMM_BK * ld) : z;
+        v[1] = (live && s + 16 < klen) ? ld4 (ptr[1] + (size_t)it * GEMM_BK * ld) : z;
+    }
+    __device__ __forceinline__ void store (float *lds, const float4 (&v)[2])
+    {
+        #pragma unroll
+        for (int i = 0; i < 2; i++)
+        {
+            float *d = lds + (c4 * 4) * LDS_ROW + s0 + 16 * i;
+            d[0] = v[i].x; d[LDS_ROW] = v[i].y; d[2 * LDS_ROW] = v[i].z; d[3 * LDS_ROW] = v[i].w;
+        }
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// fp32 MFMA core.  Workgroup tile = BM weight rows x BN activation rows; WM x WN wavefronts, each
+// owning (BM/WM) x (BN/WN) built from 32x32 v_mfma_f32_32x32x2_f32 blocks.  The activation row is
+// the MFMA row index and the weight row the MFMA column, so each accumulator register holds 32
+// consecutive output channels of one output column: stores are 128-byte coalesced.
+// LDS is double buffered: one barrier per K slice.
+// ---------------------------------------------------------------------------------------------
+template <int BM, int BN, int WM, int WN, class ALoader, class BLoader>
+__device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kiters, float *smem,
+    floatx16 (&acc)[BN / WN / 32][BM / WM / 32], int ar, int br)
+{
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int STAGE = (BM + BN) * LDS_ROW;
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);
+    const uint32_t frag = (lane & 31) * LDS_ROW + (lane >> 5) * 4;
+    (void)ar; (void)br;
+
+    #pragma unroll
+    for (int i = 0; i < TN; i++)
+        #pragma unroll
+        for (int j = 0; j < TM; j++)
+            #pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+    float4 areg[ALoader::R], breg[BLoader::R];
+    al.load (0, areg); bl.load (0, breg);
+    al.store (smem, areg); bl.store (smem + BM * LDS_ROW, breg);
+    __syncthreads ();
+
+    for (int it = 0; it < kiters; it++)
+    {
+        float *As = smem + (it & 1) * STAGE, *Bs = As + BM * LDS_ROW;
+        const bool more = it + 1 < kiters;
+        if (more) { al.load (it + 1, areg); bl.load (it + 1, breg); }
+        #pragma unroll
+        for (int kk = 0; kk < GEMM_BK / 8; kk++)
+        {
+            float4 af[TM], bf[TN];
+            #pragma unroll
+            for (int j = 0; j < TM; j++) af[j] = ld4 (As + (wm0 + j * 32) * LDS_ROW + frag + kk * 8);
+            #pragma unroll
+            for (int i = 0; i < TN; i++) bf[i] = ld4 (Bs + (wn0 + i * 32) * LDS_ROW + frag + kk * 8);
+            #pragma unroll
+            for (int i = 0; i < TN; i++)
+                #pragma unroll
+                for (int j = 0; j < TM; j++)
+                {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[i].x, af[j].x, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[i].y, af[j].y, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[i].z, af[j].z, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[i].w, af[j].w, acc[i][j], 0, 0, 0);
+                }
+        }
+        if (more)
+        {
+            float *An = smem + ((it + 1) & 1) * STAGE;
+            al.store (An, areg); bl.store (An + BM * LDS_ROW, breg);
+        }
+        __syncthreads ();
+    }
+}
+
+// Accumulator register v of MFMA block (i, j) holds output (row n, channel m):
+//   n = wn0 + 32 i + 8 (v / 4) + 4 (lane / 32) + v % 4,   m = wm0 + 32 j + lane % 32
+#define ACC_N(wn0, i, v, lane) ((wn0) + 32 * (i) + 8 * ((v) >> 2) + 4 * ((lane) >> 5) + ((v) & 3))
+
+// conv / FC / matmul tile
+template <int BM, int BN, int WM, int WN>
+__device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, float *smem)
+{
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t m0 = tm * BM, n0 = tn * BN;
+    floatx16 acc[TN][TM];
+    RowLoader<BM> al;
+    al.init (L.weight, m0, 0xffffffffu, L.Kp, tid);
+    const int kiters = (int)(L.Kp / GEMM_BK);
+    if (L.direct)
+    {
+        RowLoader<BN> bl;
+        bl.init (L.in0, n0, L.N - 1, L.ld0, tid);
+        gemm_core<BM, BN, WM, WN> (al, bl, kiters, smem, acc, 0, 0);
+    }
+    else
+    {
+        ConvLoader<BN> bl;
+        bl.init (L, n0, tid);
+        gemm_core<BM, BN, WM, WN> (al, bl, kiters, smem, acc, 0, 0);
+    }
+    const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);
+    const int act = L.act;
+    #pragma unroll
+    for (int j = 0; j < TM; j++)
+    {
+        const uint32_t m = m0 + wm0 + 32 * j + (lane & 31);
+        if (m >= L.M) continue;
+        const float b = L.bias ? L.bias[m] : 0.f;
+        #pragma unroll
+        for (int i = 0; i < TN; i++)
+            #pragma unroll
+            for (int v = 0; v < 16; v++)
+            {
+                const uint32_t n = n0 + ACC_N (wn0, i, v, lane);
+                if (n < L.N) L.out[(size_t)n * L.ld + m] = activate (acc[i][j][v] + b, act);
+            }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Bandwidth tiles: 128-bit accesses, a tile = tile_n whole columns.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float4 act4 (float4 v, int act)
+{
+    v.x = activate (v.x, act); v.y = activate (v.y, act); v.z = activate (v.z, act); v.w = activate (v.w, act);
+    return v;
+}
+
+__device__ __forceinline__ void tile_residual (const aspen_hip_layer_t &L, uint32_t tn)
+{
+    const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N), M4 = L.ld >> 2;
+    const uint32_t total = (n1 - n0) * M4;
+    for (uint32_t i = threadIdx.x; i < total; i += WG_THREADS)
+    {
+        const uint32_t c = i / M4, m = (i - c * M4) * 4;
+        const size_t n = n0 + c;
+        float4 a = ld4 (L.in0 + n * L.ld0 + m), b = ld4 (L.in1 + n * L.ld1 + m);
+        a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+        st4 (L.out + n * L.ld + m, act4 (a, L.act));
+    }
+}
+
+template <bool IS_MAX>
+__device__ __forceinline__ void tile_pool (const aspen_hip_layer_t &L, uint32_t tn)
+{
+    const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N), M4 = L.ld >> 2;
+    const uint32_t total = (n1 - n0) * M4, ohw = L.OH * L.OW;
+    const float inv = 1.0f / (float)(L.KH * L.KW);
+    for (uint32_t i = threadIdx.x; i < total; i += WG_THREADS)
+    {
+        const uint32_t c = i / M4, m = (i - c * M4) * 4, n = n0 + c;
+        const uint32_t b = n / ohw, rem = n - b * ohw, oh = rem / L.OW, ow = rem - oh * L.OW;
+        float4 r = IS_MAX ? make_float4 (-INFINITY, -INFINITY, -INFINITY, -INFINITY) : make_float4 (0.f, 0.f, 0.f, 0.f);
+        for (uint32_t kh = 0; kh < L.KH; kh++)
+        {
+            const int ih = (int)(oh * L.stride + kh) - (int)L.pad;
+            if ((uint32_t)ih >= L.IH) continue;
+            for (uint32_t kw = 0; kw < L.KW; kw++)
+            {
+                const int iw = (int)(ow * L.stride + kw) - (int)L.pad;
+                if ((uint32_t)iw >= L.IW) continue;
+                const float4 x = ld4 (L.in0 + ((size_t)(b * L.IH + ih) * L.IW + iw) * L.ld0 + m);
+                if (IS_MAX) { r.x = r.x >= x.x ? r.x : x.x; r.y = r.y >= x.y ? r.y : x.y; r.z = r.z >= x.z ? r.z : x.z; r.w = r.w >= x.w ? r.w : x.w; }
+                else { r.x += x.x; r.y += x.y; r.z += x.z; r.w += x.w; }
+            }
+        }
+        if (!IS_MAX) { r.x *= inv; r.y *= inv; r.z *= inv; r.w *= inv; }
+        r = act4 (r, L.act);
+        // keep the zero padding rows [M, ld) intact
+        if (m + 4 > L.M) { if (m + 0 >= L.M) r.x = 0.f; if (m + 1 >= L.M) r.y = 0.f; if (m + 2 >= L.M) r.z = 0.f; if (m + 3 >= L.M) r.w = 0.f; }
+        st4 (L.out + (size_t)n * L.ld + m, r);
+    }
+}
+
+__device__ __forceinline__ float wave_sum (float v)
+{
+    #pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor (v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max (float v)
+{
+    #pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf (v, __shfl_xor (v, o, 64));
+    return v;
+}
+
+// one wavefront per column: mean and E[x^2] in one pass, eps 1e-6f
+__device__ __forceinline__ void tile_layernorm (const aspen_hip_layer_t &L, uint32_t tn)
+{
+    const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N);
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, M4 = L.M >> 2;
+    for (uint32_t n = n0 + wave; n < n1; n += WG_THREADS / 64)
+    {
+        const float *x = L.in0 + (size_t)n * L.ld0;
+        float s = 0.f, q = 0.f;
+        for (uint32_t m = lane; m < M4; m += 64)
+        {
+            const float4 v = ld4 (x + m * 4);
+            s += v.x + v.y + v.z + v.w;
+            q += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        }
+        for (uint32_t m = M4 * 4 + lane; m < L.M; m += 64) { const float v = x[m]; s += v; q += v * v; }
+        s = wave_sum (s); q = wave_sum (q);
+        const float mean = s / (float)L.M;
+        float var = q / (float)L.M - mean * mean;
+        const float rstd = 1.0f / sqrtf (var + 1e-6f);
+        float *o = L.out + (size_t)n * L.ld;
+        for (uint32_t m = lane; m < M4; m += 64)
+        {
+            const float4 v = ld4 (x + m * 4), g = ld4 (L.weight + m * 4);
+            float4 r;
+            r.x = (v.x - mean) * rstd * g.x; r.y = (v.y - mean) * rstd * g.y;
+            r.z = (v.z - mean) * rstd * g.z; r.w = (v.w - mean) * rstd * g.w;
+            if (L.bias) { const float4 b = ld4 (L.bias + m * 4); r.x += b.x; r.y += b.y; r.z += b.z; r.w += b.w; }
+            st4 (o + m * 4, r);
+        }
+        for (uint32_t m = M4 * 4 + lane; m < L.M; m += 64)
+            o[m] = (x[m] - mean) * rstd * L.weight[m] + (L.bias ? L.bias[m] : 0.f);
+    }
+}
+
+// one wavefront per column: max-subtracted softmax over the rows
+__device__ __forceinline__ void tile_softmax (const aspen_hip_layer_t &L, uint32_t tn)
+{
+    const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N);
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (uint32_t n = n0 + wave; n < n1; n += WG_THREADS / 64)
+    {
+        const float *x = L.in0 + (size_t)n * L.ld0;
+        float *o = L.out + (size_t)n * L.ld;
+        float mx = -INFINITY;
+        for (uint32_t m = lane; m < L.M; m += 64) mx = fmaxf (mx, x[m]);
+        mx = wave_max (mx);
+        float s = 0.f;
+        for (uint32_t m = lane; m < L.M; m += 64) { const float e = expf (x[m] - mx); o[m] = e; s += e; }
+        s = wave_sum (s);
+        for (uint32_t m = lane; m < L.M; m += 64) o[m] = o[m] / s;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Attention tiles.
+// K tile: one (batch, head) x 128 queries x all keys.  scores = K.Q on the matrix cores, 128 keys at
+// a time; causal mask (-1e10 before the 1/sqrt(hd) scale), exp without max subtraction and the row
+// sums are fused into the epilogue; a second sweep over the tile's own output divides by the sums.
+// in0 = Query matrix, in1 = Key matrix (reference cfg: parent = Query, from = Key).
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, uint32_t tn, float *smem)
+{
+    constexpr int BM = 128, BN = 128, WM = 2, WN = 2, TM = 2, TN = 2;
+    __shared__ float rowsum[BN];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t S = L.seq, qtiles = (S + BN - 1) / BN;
+    const uint32_t bh = tn / qtiles, q0 = (tn - bh * qtiles) * BN;
+    const uint32_t b = bh / L.heads, h = bh - b * L.heads;
+    const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);
+    const float *Q = L.in0 + (size_t)b * S * L.ld0 + h * L.hd;
+    const float *Kmat = L.in1 + (size_t)b * S * L.ld1 + h * L.hd;
+    float *out = L.out + (size_t)bh * S * L.ld;          // column (b*H + h)*S + q, rows = keys
+    const float scale = 1.0f / sqrtf ((float)L.hd);
+    if (tid < BN) rowsum[tid] = 0.f;
+    float part[TN][16];
+    #pragma unroll
+    for (int i = 0; i < TN; i++)
+        #pragma unroll
+        for (int v = 0; v < 16; v++) part[i][v] = 0.f;
+
+    const int kiters = (int)(L.hd / GEMM_BK);
+    for (uint32_t k0 = 0; k0 < S; k0 += BM)
+    {
+        floatx16 acc[TN][TM];
+        RowLoader<BM> al; al.init (Kmat, k0, S - 1, L.ld1, tid);
+        RowLoader<BN> bl; bl.init (Q, q0, S - 1, L.ld0, tid);
+        gemm_core<BM, BN, WM, WN> (al, bl, kiters, smem, acc, 0, 0);
+        #pragma unroll
+        for (int j = 0; j < TM; j++)
+        {
+            const uint32_t key = k0 + wm0 + 32 * j + (lane & 31);
+            #pragma unroll
+            for (int i = 0; i < TN; i++)
+                #pragma unroll
+                for (int v = 0; v < 16; v++)
+                {
+                    const uint32_t q = q0 + ACC_N (wn0, i, v, lane);
+                    float s = acc[i][j][v];
+                    if (L.masked && key > q) s = -1e10f;
+                    const float e = expf (s * scale);
+                    if (key < S && q < S) { out[(size_t)q * L.ld + key] = e; part[i][v] += e; }
+                }
+        }
+    }
+    // row sums: 32 lanes of a half-wave hold 32 different keys of the same query
+    #pragma unroll
+    for (int i = 0; i < TN; i++)
+        #pragma unroll
+        for (int v = 0; v < 16; v++)
+        {
+            float s = part[i][v];
+            #pragma unroll
+            for (int o = 16; o > 0; o >>= 1) s += __shfl_xor (s, o, 64);
+            if ((lane & 31) == 0) atomicAdd (&rowsum[ACC_N (wn0, i, v, lane)], s);
+        }
+    __syncthreads ();
+    const uint32_t nq = min ((uint32_t)BN, S - q0);
+    const uint32_t S4 = S >> 2;
+    if ((S & 3) == 0)
+        for (uint32_t i = tid; i < nq * S4; i += WG_THREADS)
+        {
+            const uint32_t r = i / S4, c = (i - r * S4) * 4;
+            float *p = out + (size_t)(q0 + r) * L.ld + c;
+            const float inv = rowsum[r];
+            float4 v = ld4 (p);
+            v.x /= inv; v.y /= inv; v.z /= inv; v.w /= inv;
+            st4 (p, v);
+        }
+    else
+        for (uint32_t i = tid; i < nq * S; i += WG_THREADS)
+        {
+            const uint32_t r = i / S, c = i - r * S;
+            out[(size_t)(q0 + r) * L.ld + c] /= rowsum[r];
+        }
+    __syncthreads ();
+}
+
+// V tile: one (batch, head-slice of <= 64 channels) x 128 queries:
+// out[b*S + q][h*hd + j] = sum_s P[(b*H + h)*S + q][s] * V[b*S + s][h*hd + j].
+// in0 = probabilities (K-attention output), in1 = Value matrix.
+__device__ __forceinline__ void tile_v_attention (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, float *smem)
+{
+    constexpr int BM = 64, BN = 128, WM = 2, WN = 2, TM = 1, TN = 2;
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t S = L.seq, qtiles = (S + BN - 1) / BN;
+    const uint32_t b = tn / qtiles, q0 = (tn - b * qtiles) * BN;
+    const uint32_t m0 = tm * L.tile_m, h = m0 / L.hd;
+    const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);
+    const float *P = L.in0 + (size_t)(b * L.heads + h) * S * L.ld0;
+    const float *V = L.in1 + (size_t)b * S * L.ld1 + m0;
+    floatx16 acc[TN][TM];
+    TransLoader64 al; al.init (V, L.ld1, L.tile_m, S, tid);
+    RowLoader<BN> bl; bl.init (P, q0, S - 1, L.ld0, tid);   // P's stride is a multiple of 32 with zero padding
+    gemm_core<BM, BN, WM, WN> (al, bl, (int)((S + GEMM_BK - 1) / GEMM_BK), smem, acc, 0, 0);
+    const uint32_t mm = wm0 + (lane & 31);
+    if (mm < L.tile_m)
+        #pragma unroll
+        for (int i = 0; i < TN; i++)
+            #pragma unroll
+            for (int v = 0; v < 16; v++)
+            {
+                const uint32_t q = q0 + ACC_N (wn0, i, v, lane);
+                if (q < S) L.out[(size_t)(b * S + q) * L.ld + m0 + mm] = acc[i][0][v];
+            }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Dispatch: the device-side counterpart of the switch in the reference's dse_schedule
+// (reference src/dse.c:39-79).  `t` = tile index inside the layer, row-tile fastest
+// (reference src/apu_nasm.c:1218-1224).
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ void run_tile (const aspen_hip_layer_t &L, uint32_t t, float *smem)
+{
+    const uint32_t tn = t / L.tiles_m, tm = t - tn * L.tiles_m;
+    switch (L.type)
+    {
+    case CONV_LAYER: case FC_LAYER: case MATMUL_LAYER:
+        if (L.variant == ASPEN_HIP_GEMM_128x128) tile_contraction<128, 128, 2, 2> (L, tn, tm, smem);
+        else if (L.variant == ASPEN_HIP_GEMM_64x128) tile_contraction<64, 128, 2, 2> (L, tn, tm, smem);
+        else tile_contraction<64, 64, 2, 2> (L, tn, tm, smem);
+        break;
+    case RESIDUAL_LAYER:    tile_residual (L, tn); break;
+    case MAXPOOL_LAYER:     tile_pool<true> (L, tn); break;
+    case AVGPOOL_LAYER:     tile_pool<false> (L, tn); break;
+    case LAYERNORM_LAYER:   tile_layernorm (L, tn); break;
+    case SOFTMAX_LAYER:     tile_softmax (L, tn); break;
+    case K_ATTENTION_LAYER: tile_k_attention (L, tn, smem); break;
+    case V_ATTENTION_LAYER: tile_v_attention (L, tn, tm, smem); break;
+    default: break;
+    }
+}

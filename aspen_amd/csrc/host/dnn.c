@@ -1,0 +1,289 @@
+/*
+ * dnn.c -- model object: creation, ASPEN_DATA weight files, device-side weight layout.
+ *
+ * Counterpart of the reference's apu_create_dnn / apu_load_dnn_data_from_file
+ * (reference src/apu.c:6-43, src/apu_file_io.c:48-432).  The reference repacks weights into
+ * [M/8][K][8] for its 8-row AVX2 micro-kernel; here the device copy is [roundup(M,128)][Kp]
+ * row-major with the K axis laid out as (tap, channel padded to 4) so that every 128-bit load of
+ * the implicit-GEMM kernel stays inside one tap, zero padded to a multiple of 32.
+ */
+#include <math.h>
+#include "internal.h"
+
+static void alloc_tensor (aspen_tensor_t *t, size_t n)
+{
+    t->num_elements = n;
+    t->data = calloc (n ? n : 1, sizeof (float));
+}
+
+/* deterministic stand-in for the reference's rand()-based +-0.3 fill (reference src/apu.c:345-354,
+   :419-421): weights a model has before any file is loaded */
+static void fill_uniform (aspen_tensor_t *t, uint64_t *state, float range)
+{
+    for (size_t i = 0; i < t->num_elements; i++)
+    {
+        *state = *state * 6364136223846793005ull + 1442695040888963407ull;
+        t->data[i] = ((float)((*state >> 40) & 0xffffff) / 16777216.0f - 0.5f) * 2.0f * range;
+    }
+}
+
+static void create_layer_tensors (aspen_layer_t *L, uint64_t *rng)
+{
+    const unsigned int *p = L->params;
+    switch (L->type)
+    {
+    case CONV_LAYER:    L->gemm_m = p[OUT_C]; L->gemm_k = p[WEIGHT_H] * p[WEIGHT_W] * p[IN_C]; break;
+    case FC_LAYER:      L->gemm_m = p[OUT_C]; L->gemm_k = p[IN_H] * p[IN_W] * p[IN_C]; break;
+    case MATMUL_LAYER:  L->gemm_m = p[MAT_M]; L->gemm_k = p[MAT_K]; break;
+    case LAYERNORM_LAYER: L->gemm_m = p[MAT_M]; L->gemm_k = 1; break;
+    default: return;
+    }
+    alloc_tensor (&L->weight, (size_t)L->gemm_m * L->gemm_k);
+    alloc_tensor (&L->bias, L->gemm_m);
+    fill_uniform (&L->weight, rng, 0.3f);
+    fill_uniform (&L->bias, rng, 0.3f);
+}
+
+aspen_dnn_t *apu_create_dnn (char *input_path, char *data_path)
+{
+    if (input_path == NULL) { ERROR_PRTF ("apu_create_dnn: input_path is NULL\n"); return NULL; }
+    aspen_dnn_t *dnn = aspen_parse_cfg (input_path);
+    if (dnn == NULL) return NULL;
+    uint64_t rng = 0x5851f42d4c957f2dull;
+    for (unsigned int i = 0; i < dnn->num_layers; i++)
+        create_layer_tensors (&dnn->layers[i], &rng);
+    if (data_path != NULL)
+        aspen_load_weight_file (dnn, data_path);   /* a missing or broken file only prints, as in the reference */
+    return dnn;
+}
+
+void apu_destroy_dnn (aspen_dnn_t *dnn)
+{
+    if (dnn == NULL) return;
+    if (dnn->ref_nasms != 0)
+    {
+        ERROR_PRTF ("Cannot destroy dnn %s with %d nasms still referencing it.\n", dnn->name, dnn->ref_nasms);
+        return;
+    }
+    for (unsigned int i = 0; i < dnn->num_layers; i++)
+    {
+        aspen_layer_t *L = &dnn->layers[i];
+        free (L->weight.data); free (L->bias.data);
+        aspen_hip_free (L->d_weight); aspen_hip_free (L->d_bias); aspen_hip_free (L->d_ktab);
+    }
+    free (dnn->layers);
+    free (dnn);
+}
+
+/* ---------------------------------------------------------------------------------------------- */
+/* ASPEN_DATA reader                                                                               */
+/* ---------------------------------------------------------------------------------------------- */
+static char *expect_line (FILE *fp, char *buf, size_t len, const char *tag, int eof_ok)
+{
+    if (fgets (buf, (int)len, fp) == NULL)
+    {
+        if (!eof_ok) ERROR_PRTF ("ASPEN DNN file parse error: Unexpected EOF.\n");
+        return NULL;
+    }
+    buf[strcspn (buf, "\n")] = 0;
+    char *p = buf;
+    while (*p == ' ' || *p == '\t') p++;
+    if (strncmp (p, tag, strlen (tag)) != 0)
+    {
+        ERROR_PRTF ("Wrong ASPEN DNN file format: expected \"%s\", got \"%s\"\n", tag, p);
+        return NULL;
+    }
+    return p + strlen (tag);
+}
+
+/* PyTorch [O][C][H][W] -> GEMM order [O][(h*W + w)*C + c] */
+static void ochw_to_ohwc (const float *src, float *dst, unsigned int O, unsigned int C, unsigned int H, unsigned int W)
+{
+    for (unsigned int o = 0; o < O; o++)
+        for (unsigned int c = 0; c < C; c++)
+            for (unsigned int h = 0; h < H; h++)
+                for (unsigned int w = 0; w < W; w++)
+                    dst[((size_t)o * H * W + (size_t)h * W + w) * C + c] = src[(((size_t)o * C + c) * H + h) * W + w];
+}
+
+static void invalidate_device (aspen_layer_t *L)
+{
+    aspen_hip_free (L->d_weight); aspen_hip_free (L->d_bias); aspen_hip_free (L->d_ktab);
+    L->d_weight = NULL; L->d_bias = NULL; L->d_ktab = NULL;
+}
+
+int aspen_load_weight_file (aspen_dnn_t *dnn, const char *path)
+{
+    FILE *fp = fopen (path, "rb");
+    if (fp == NULL) { ERROR_PRTF ("ASPEN DNN file %s not found.\n", path); return -1; }
+    char line[MAX_STRING_LEN];
+    float *bn[3] = {NULL, NULL, NULL};   /* var, mean, weight */
+    int rc = -1;
+    char *p;
+    if (expect_line (fp, line, sizeof (line), "ASPEN_DATA", 0) == NULL) goto done;
+    p = expect_line (fp, line, sizeof (line), "LAYER:", 0);
+    while (p != NULL)
+    {
+        const int file_layer = atoi (p);
+        aspen_layer_t *L = NULL;
+        int weighted = 0;
+        for (unsigned int i = 0; i < dnn->num_layers && L == NULL; i++)
+        {
+            LAYER_TYPE t = dnn->layers[i].type;
+            if (t == CONV_LAYER || t == FC_LAYER || t == MATMUL_LAYER || t == LAYERNORM_LAYER)
+                if (++weighted == file_layer) L = &dnn->layers[i];
+        }
+        if (L == NULL) { ERROR_PRTF ("ASPEN DNN file %s parse error: Invalid file LAYER %d.\n", path, file_layer); goto done; }
+        if ((p = expect_line (fp, line, sizeof (line), "TENSOR_TYPE:", 0)) == NULL) goto done;
+        char kind[32];
+        strncpy (kind, p, sizeof (kind) - 1); kind[sizeof (kind) - 1] = 0;
+        if ((p = expect_line (fp, line, sizeof (line), "DATA_SIZE:", 0)) == NULL) goto done;
+        const size_t bytes = (size_t)atoll (p);
+        if (expect_line (fp, line, sizeof (line), "DATA_START:", 0) == NULL) goto done;
+        float *buf = malloc (bytes ? bytes : 1);
+        if (buf == NULL || fread (buf, 1, bytes, fp) != bytes)
+        {
+            ERROR_PRTF ("ASPEN DNN file %s parse error: Failed to read data.\n", path);
+            free (buf);
+            goto done;
+        }
+        if (expect_line (fp, line, sizeof (line), "DATA_END", 0) == NULL) { free (buf); goto done; }
+        const unsigned int *q = L->params;
+        if (strcmp (kind, "WEIGHT") == 0)
+        {
+            if (bytes != L->weight.num_elements * sizeof (float))
+            {
+                ERROR_PRTF ("ASPEN DNN file %s parse error: Layer %u WEIGHT_TENSOR size mismatch. Tensor: %zu, File: %zu.\n",
+                    path, L->layer_idx, L->weight.num_elements * sizeof (float), bytes);
+                free (buf);
+                goto done;
+            }
+            if (L->type == CONV_LAYER) ochw_to_ohwc (buf, L->weight.data, q[OUT_C], q[IN_C], q[WEIGHT_H], q[WEIGHT_W]);
+            else if (L->type == FC_LAYER) ochw_to_ohwc (buf, L->weight.data, q[OUT_C], q[IN_C], q[IN_H], q[IN_W]);
+            else memcpy (L->weight.data, buf, bytes);
+            invalidate_device (L);
+            free (buf);
+        }
+        else if (strcmp (kind, "BIAS") == 0)
+        {
+            if (bytes != L->bias.num_elements * sizeof (float))
+            {
+                ERROR_PRTF ("ASPEN DNN file %s parse error: Layer %u BIAS_TENSOR size mismatch: Tensor: %zu, File: %zu.\n",
+                    path, L->layer_idx, L->bias.num_elements * sizeof (float), bytes);
+                free (buf);
+                goto done;
+            }
+            memcpy (L->bias.data, buf, bytes);
+            invalidate_device (L);
+            free (buf);
+        }
+        else if (strcmp (kind, "BN_VAR") == 0 || strcmp (kind, "BN_MEAN") == 0 || strcmp (kind, "BN_WEIGHT") == 0)
+        {
+            const int slot = kind[3] == 'V' ? 0 : kind[3] == 'M' ? 1 : 2;
+            if (bn[slot] != NULL || bytes != L->gemm_m * sizeof (float))
+            {
+                ERROR_PRTF ("ASPEN DNN file %s parse error: Duplicate or mis-sized %s.\n", path, kind);
+                free (buf);
+                goto done;
+            }
+            bn[slot] = buf;
+        }
+        else if (strcmp (kind, "INPUT") == 0 || strcmp (kind, "OUTPUT") == 0)
+            free (buf);
+        else
+        {
+            ERROR_PRTF ("ASPEN DNN file %s file layer %d parse error: Invalid TENSOR_TYPE %s.\n", path, file_layer, kind);
+            free (buf);
+            goto done;
+        }
+        if (bn[0] && bn[1] && bn[2])
+        {
+            /* fold inference batch norm into weight and bias, eps 1e-5 (reference src/util.c:259-276) */
+            const double eps = 1e-5;
+            for (unsigned int o = 0; o < L->gemm_m; o++)
+            {
+                const float s = bn[2][o] / sqrtf (bn[0][o] + eps);
+                for (unsigned int k = 0; k < L->gemm_k; k++) L->weight.data[(size_t)o * L->gemm_k + k] *= s;
+                L->bias.data[o] = L->bias.data[o] - bn[2][o] * bn[1][o] / sqrtf (bn[0][o] + eps);
+            }
+            for (int i = 0; i < 3; i++) { free (bn[i]); bn[i] = NULL; }
+            invalidate_device (L);
+        }
+        if (expect_line (fp, line, sizeof (line), "LAYER_END", 0) == NULL) goto done;
+        p = expect_line (fp, line, sizeof (line), "LAYER:", 1);
+    }
+    rc = 0;
+done:
+    for (int i = 0; i < 3; i++) free (bn[i]);
+    fclose (fp);
+    return rc;
+}
+
+/* ---------------------------------------------------------------------------------------------- */
+/* device layout                                                                                    */
+/* ---------------------------------------------------------------------------------------------- */
+static unsigned int round_up (unsigned int v, unsigned int to) { return (v + to - 1) / to * to; }
+
+/* Uploads weight / bias / k-chunk table of one layer for a parent whose column stride is parent_ld
+   floats.  Idempotent; re-run after the weights changed. */
+int aspen_layer_to_device (aspen_layer_t *L, unsigned int parent_ld)
+{
+    if (L->weight.data == NULL) return 0;
+    if (L->d_weight != NULL && L->dev_in_ld == parent_ld) return 0;
+    invalidate_device (L);
+    const unsigned int *p = L->params;
+    if (L->type == LAYERNORM_LAYER)
+    {
+        L->d_weight = aspen_hip_alloc (L->gemm_m * sizeof (float));
+        L->d_bias = aspen_hip_alloc (L->gemm_m * sizeof (float));
+        if (!L->d_weight || !L->d_bias) return -1;
+        L->dev_in_ld = parent_ld;
+        return aspen_hip_h2d (L->d_weight, L->weight.data, L->gemm_m * sizeof (float))
+            || aspen_hip_h2d (L->d_bias, L->bias.data, L->gemm_m * sizeof (float));
+    }
+    unsigned int taps, ic, kw_count, in_w;
+    if (L->type == CONV_LAYER) { taps = p[WEIGHT_H] * p[WEIGHT_W]; ic = p[IN_C]; kw_count = p[WEIGHT_W]; in_w = p[IN_W]; }
+    else if (L->type == FC_LAYER) { taps = p[IN_H] * p[IN_W]; ic = p[IN_C]; kw_count = p[IN_W]; in_w = p[IN_W]; }
+    else { taps = 1; ic = p[MAT_K]; kw_count = 1; in_w = 1; }
+    const unsigned int icp = round_up (ic, 4);
+    const unsigned int kp = round_up (taps * icp, 32);
+    const unsigned int mp = round_up (L->gemm_m, 128);
+    float *staged = calloc ((size_t)mp * kp, sizeof (float));
+    if (staged == NULL) return -1;
+    for (unsigned int m = 0; m < L->gemm_m; m++)
+        for (unsigned int t = 0; t < taps; t++)
+            memcpy (staged + (size_t)m * kp + (size_t)t * icp, L->weight.data + (size_t)m * L->gemm_k + (size_t)t * ic, ic * sizeof (float));
+    L->d_weight = aspen_hip_alloc ((size_t)mp * kp * sizeof (float));
+    int rc = L->d_weight ? aspen_hip_h2d (L->d_weight, staged, (size_t)mp * kp * sizeof (float)) : -1;
+    free (staged);
+    if (rc) return rc;
+    L->d_bias = aspen_hip_alloc (L->gemm_m * sizeof (float));
+    if (!L->d_bias || aspen_hip_h2d (L->d_bias, L->bias.data, L->gemm_m * sizeof (float))) return -1;
+    /* k-chunk table: chunk c covers K positions [4c, 4c+4) = tap (4c / icp), channels (4c % icp).. */
+    aspen_hip_ktab_t *tab = calloc (kp / 4, sizeof (aspen_hip_ktab_t));
+    for (unsigned int c = 0; c < kp / 4; c++)
+    {
+        const unsigned int tap = (c * 4) / icp, ch = (c * 4) % icp;
+        if (tap >= taps) { tab[c].offset = 0; tab[c].kh = 0x4000; tab[c].kw = 0; continue; }
+        const unsigned int kh = tap / kw_count, kw = tap % kw_count;
+        tab[c].offset = (int32_t)((kh * in_w + kw) * parent_ld + ch);
+        tab[c].kh = (uint16_t)kh; tab[c].kw = (uint16_t)kw;
+    }
+    L->d_ktab = aspen_hip_alloc (kp / 4 * sizeof (aspen_hip_ktab_t));
+    rc = L->d_ktab ? aspen_hip_h2d (L->d_ktab, tab, kp / 4 * sizeof (aspen_hip_ktab_t)) : -1;
+    free (tab);
+    L->dev_kp = kp; L->dev_icp = icp; L->dev_in_ld = parent_ld;
+    return rc;
+}
+
+void apu_save_dnn_to_file (aspen_dnn_t *dnn, char *filename)
+{
+    (void)dnn;
+    ERROR_PRTF ("apu_save_dnn_to_file (%s): the .aspen container is not implemented in this build.\n", filename ? filename : "NULL");
+}
+
+aspen_dnn_t *apu_load_dnn_from_file (char *filename)
+{
+    ERROR_PRTF ("apu_load_dnn_from_file (%s): the .aspen container is not implemented in this build.\n", filename ? filename : "NULL");
+    return NULL;
+}

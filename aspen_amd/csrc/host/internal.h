@@ -1,0 +1,120 @@
+/*
+ * internal.h -- data model of the C host library behind include/aspen.h.
+ *
+ * The reference keeps the same three levels (reference include/apu.h:14-43, include/nasm.h:7-66):
+ * dnn (layers + weights), nasm (per-layer runtime data + tiles), ninst (one tile).  The layouts
+ * here are this library's own: activations live in one device arena per nasm, tiles are implicit
+ * (layer, index) pairs, and dependencies are flat CSR arrays ready for upload.
+ */
+#ifndef ASPEN_AMD_INTERNAL_H
+#define ASPEN_AMD_INTERNAL_H
+
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include "aspen.h"
+#include "aspen_hip.h"
+
+#define ERROR_PRTF(...) do { fprintf (stderr, "\033[0;31m(%s:%d) ", __FILE__, __LINE__); fprintf (stderr, __VA_ARGS__); fprintf (stderr, "\033[0m"); } while (0)
+
+struct aspen_tensor_t
+{
+    size_t num_elements;
+    float *data;
+};
+
+struct aspen_layer_t
+{
+    aspen_dnn_t *dnn;
+    unsigned int layer_idx;
+    LAYER_TYPE type;
+    LAYER_ACT activation;
+    int parent_idx[NUM_PARENT_ELEMENTS];     /* layer index or -1 */
+    unsigned int params[NUM_PARAM_ELEMENTS];
+    /* host weights in GEMM order: [M][K], K = (kh, kw, ic) for conv, (h, w, c) for FC, plain for
+       matmul (the reference's K order, src/apu.c:16,25,34, without its 8-row interleave) */
+    aspen_tensor_t weight, bias;
+    unsigned int gemm_m, gemm_k;              /* rows / contraction length of `weight` */
+    /* device copies, created on first use */
+    float *d_weight, *d_bias;
+    aspen_hip_ktab_t *d_ktab;
+    unsigned int dev_kp, dev_icp, dev_in_ld;  /* padded K, padded channels per tap, parent stride assumed */
+};
+
+struct aspen_dnn_t
+{
+    char name[MAX_STRING_LEN];
+    unsigned int element_size;
+    aspen_layer_t *layers;
+    unsigned int num_layers;
+    unsigned int ref_nasms;
+};
+
+struct nasm_ldata_t
+{
+    nasm_t *nasm;
+    aspen_layer_t *layer;
+    int parent_ldata_idx[NUM_PARENT_ELEMENTS];
+    unsigned int out_mat_dims[2];            /* [OUT_W] columns, [OUT_H] rows */
+    unsigned int out_mat_stride;
+    size_t out_mat_offset;                   /* floats from the start of the arena */
+    unsigned int tile_dims[2];
+    unsigned int tiles_w, tiles_h;
+    unsigned int num_ninst, ninst_start;
+    int variant;
+    uint64_t flops;                          /* 2*M*N*K for contraction layers, 64-bit */
+};
+
+struct nasm_t
+{
+    unsigned int nasm_id;
+    aspen_dnn_t *dnn;
+    unsigned int batch_size, tr_seq_len, min_ninst_per_ldata;
+    nasm_ldata_t *ldata_arr;
+    unsigned int num_ldata;
+    unsigned int num_ninst;
+    uint64_t total_flops;
+    /* dependency graph over tiles (CSR) */
+    uint32_t *ninst_ldata;                   /* tile -> ldata index */
+    uint32_t *num_parents;
+    uint32_t *child_off, *child_idx;
+    uint32_t num_edges;
+    /* device state */
+    size_t arena_floats;
+    float *d_arena;
+    rpool_t *rpool;                          /* pool this nasm is attached to */
+    int armed;                               /* input present and counters to be re-armed at the next run */
+    int completed;
+};
+
+#define RPOOL_MAX_NASMS 64
+struct rpool_t
+{
+    nasm_t *nasms[RPOOL_MAX_NASMS];
+    unsigned int num_nasms;
+    unsigned int ref_dses;
+    aspen_hip_graph_t *graph;                /* merged device graph of all attached nasms */
+    int graph_dirty;
+    int running;
+};
+
+struct dse_group_t
+{
+    unsigned int num_dses;
+    rpool_t *rpool;
+    int mode;                                /* 0 = one launch per layer, 1 = persistent dataflow kernel */
+    unsigned int workgroups;
+};
+
+/* cfg.c */
+aspen_dnn_t *aspen_parse_cfg (const char *path);
+/* dnn.c */
+int aspen_layer_to_device (aspen_layer_t *layer, unsigned int parent_ld);
+int aspen_load_weight_file (aspen_dnn_t *dnn, const char *path);
+/* nasm.c */
+int aspen_nasm_to_device (nasm_t *nasm);
+int aspen_nasm_fill_device_layers (nasm_t *nasm, aspen_hip_layer_t *dst, uint32_t ninst_base);
+unsigned int aspen_ld_for_rows (unsigned int rows);
+
+#endif

@@ -1,0 +1,482 @@
+/*
+ * nasm.c -- tile graph: per-layer matrices, GPU tile policy, analytic tile-to-tile dependencies.
+ *
+ * Counterpart of the reference's graph builder (reference src/apu_nasm.c):
+ *   get_out_mat_info :950        -> matrix shape per layer (rows = channels, columns = batch x positions)
+ *   get_ninst_tile_dims :1025,
+ *   init_nasm_ldata :1062        -> tile policy; here sized for 256 compute units and the MFMA tile
+ *                                   shapes instead of 64 x 12 CPU tiles
+ *   ninst_find_parent :49-466    -> dependencies; the reference visits every output element times its
+ *                                   receptive field, here each tile's parents follow from interval
+ *                                   arithmetic on its column / row range
+ *   apu_create_nasm :682, apu_create_transformer_nasm :715, apu_reset_nasm :753, apu_destroy_nasm :936
+ */
+#include "internal.h"
+
+static unsigned int nasm_counter = 0;
+
+static unsigned int cdiv (unsigned int a, unsigned int b) { return (a + b - 1) / b; }
+static unsigned int umin (unsigned int a, unsigned int b) { return a < b ? a : b; }
+static unsigned int umax (unsigned int a, unsigned int b) { return a > b ? a : b; }
+
+/* column stride for a matrix with `rows` rows: 16-byte aligned columns, zero padded */
+unsigned int aspen_ld_for_rows (unsigned int rows) { return cdiv (rows, 4) * 4; }
+
+static int is_contraction (LAYER_TYPE t) { return t == CONV_LAYER || t == FC_LAYER || t == MATMUL_LAYER; }
+
+/* matrix shape, flop count (reference src/apu_nasm.c:950-1023) */
+static int set_out_mat (nasm_t *nasm, nasm_ldata_t *ld)
+{
+    const aspen_layer_t *L = ld->layer;
+    const unsigned int *p = L->params;
+    const unsigned int B = nasm->batch_size, S = nasm->tr_seq_len;
+    uint64_t flop_per_out = 1;
+    switch (L->type)
+    {
+    case CONV_LAYER:
+        flop_per_out = 2ull * p[WEIGHT_H] * p[WEIGHT_W] * p[IN_C];
+        ld->out_mat_dims[OUT_H] = p[OUT_C]; ld->out_mat_dims[OUT_W] = p[OUT_H] * p[OUT_W] * B;
+        break;
+    case FC_LAYER:
+        flop_per_out = 2ull * p[IN_C] * p[IN_H] * p[IN_W];
+        ld->out_mat_dims[OUT_H] = p[OUT_C]; ld->out_mat_dims[OUT_W] = B;
+        break;
+    case MAXPOOL_LAYER: case AVGPOOL_LAYER:
+        flop_per_out = (uint64_t)p[WEIGHT_H] * p[WEIGHT_W];
+        ld->out_mat_dims[OUT_H] = p[OUT_C]; ld->out_mat_dims[OUT_W] = p[OUT_H] * p[OUT_W] * B;
+        break;
+    case INPUT_LAYER: case RESIDUAL_LAYER:
+        if (S != 0) { ld->out_mat_dims[OUT_H] = p[MAT_M]; ld->out_mat_dims[OUT_W] = S * B; }
+        else { ld->out_mat_dims[OUT_H] = p[OUT_C]; ld->out_mat_dims[OUT_W] = p[OUT_H] * p[OUT_W] * B; }
+        break;
+    case SOFTMAX_LAYER:
+        ld->out_mat_dims[OUT_H] = p[OUT_C]; ld->out_mat_dims[OUT_W] = B;
+        break;
+    case MATMUL_LAYER:
+        flop_per_out = 2ull * p[MAT_K];
+        ld->out_mat_dims[OUT_H] = p[MAT_M]; ld->out_mat_dims[OUT_W] = S * B;
+        break;
+    case K_ATTENTION_LAYER:
+        flop_per_out = 2ull * p[NUM_HIDDEN] / p[NUM_HEAD];
+        ld->out_mat_dims[OUT_H] = S; ld->out_mat_dims[OUT_W] = S * p[NUM_HEAD] * B;
+        break;
+    case V_ATTENTION_LAYER:
+        flop_per_out = 2ull * S;
+        ld->out_mat_dims[OUT_H] = p[MAT_M]; ld->out_mat_dims[OUT_W] = S * B;
+        break;
+    case LAYERNORM_LAYER:
+        ld->out_mat_dims[OUT_H] = p[MAT_M]; ld->out_mat_dims[OUT_W] = S * B;
+        break;
+    default:
+        ERROR_PRTF ("ERROR) Unsupported layer type %d\n", (int)L->type);
+        return -1;
+    }
+    if (ld->out_mat_dims[OUT_H] == 0 || ld->out_mat_dims[OUT_W] == 0)
+    {
+        ERROR_PRTF ("layer %u has an empty output matrix (transformer graphs need a sequence length: use apu_create_transformer_nasm)\n", L->layer_idx);
+        return -1;
+    }
+    ld->flops = flop_per_out * ld->out_mat_dims[OUT_H] * ld->out_mat_dims[OUT_W];
+    ld->out_mat_stride = aspen_ld_for_rows (ld->out_mat_dims[OUT_H]);
+    if (L->type == K_ATTENTION_LAYER)
+        ld->out_mat_stride = cdiv (S, 32) * 32;     /* the V tile streams it 32 keys at a time */
+    return 0;
+}
+
+/* Tile policy.  min_ninst = wanted tiles per layer (the knob of apu_create_nasm): the largest tile
+   shape that still yields that many tiles is taken, so big layers get 128 x 128 MFMA tiles and
+   small ones are cut finer to keep all compute units busy. */
+static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
+{
+    const aspen_layer_t *L = ld->layer;
+    const unsigned int M = ld->out_mat_dims[OUT_H], N = ld->out_mat_dims[OUT_W];
+    const unsigned int want = nasm->min_ninst_per_ldata;
+    ld->variant = 0;
+    if (L->type == INPUT_LAYER)
+    {
+        ld->tile_dims[OUT_H] = M; ld->tile_dims[OUT_W] = N; ld->tiles_h = ld->tiles_w = 0; ld->num_ninst = 0;
+        return 0;
+    }
+    if (is_contraction (L->type))
+    {
+        static const unsigned int bm[ASPEN_HIP_NUM_GEMM_VARIANTS] = {128, 64, 64}, bn[ASPEN_HIP_NUM_GEMM_VARIANTS] = {128, 128, 64};
+        int v = M <= 64 ? ASPEN_HIP_GEMM_64x128 : ASPEN_HIP_GEMM_128x128;
+        while (v < ASPEN_HIP_GEMM_64x64 && cdiv (M, bm[v]) * cdiv (N, bn[v]) < want) v++;
+        if (N <= 64) v = ASPEN_HIP_GEMM_64x64;
+        ld->variant = v;
+        ld->tile_dims[OUT_H] = bm[v]; ld->tile_dims[OUT_W] = bn[v];
+    }
+    else if (L->type == K_ATTENTION_LAYER)
+    {
+        const unsigned int S = nasm->tr_seq_len, hd = L->params[NUM_HIDDEN] / L->params[NUM_HEAD];
+        if (hd % 32 != 0) { ERROR_PRTF ("layer %u: head size %u must be a multiple of 32\n", L->layer_idx, hd); return -1; }
+        ld->tile_dims[OUT_H] = M; ld->tile_dims[OUT_W] = 128;
+        ld->tiles_h = 1; ld->tiles_w = (N / S) * cdiv (S, 128);
+        ld->num_ninst = ld->tiles_w;
+        return 0;
+    }
+    else if (L->type == V_ATTENTION_LAYER)
+    {
+        const unsigned int S = nasm->tr_seq_len, hd = L->params[NUM_HIDDEN] / L->params[NUM_HEAD];
+        if (hd * L->params[NUM_HEAD] != M || (hd > 64 && hd % 64 != 0) || hd % 4 != 0)
+        { ERROR_PRTF ("layer %u: unsupported head geometry (M %u, heads %u)\n", L->layer_idx, M, L->params[NUM_HEAD]); return -1; }
+        ld->tile_dims[OUT_H] = umin (hd, 64); ld->tile_dims[OUT_W] = 128;
+        ld->tiles_h = M / ld->tile_dims[OUT_H]; ld->tiles_w = (N / S) * cdiv (S, 128);
+        ld->num_ninst = ld->tiles_h * ld->tiles_w;
+        return 0;
+    }
+    else
+    {
+        /* bandwidth tiles: whole columns; start from 128 columns (the GEMM column tile, so edges
+           line up) and halve until there are enough tiles */
+        unsigned int tn = 128;
+        if (L->type == SOFTMAX_LAYER || L->type == LAYERNORM_LAYER) tn = 32;
+        while (tn > 4 && cdiv (N, tn) < want) tn /= 2;
+        while (tn < 1024 && (uint64_t)tn * ld->out_mat_stride < 16384 && cdiv (N, tn * 2) >= 2 * want) tn *= 2;
+        ld->tile_dims[OUT_H] = M; ld->tile_dims[OUT_W] = tn;
+    }
+    ld->tiles_h = cdiv (M, ld->tile_dims[OUT_H]);
+    ld->tiles_w = cdiv (N, ld->tile_dims[OUT_W]);
+    ld->num_ninst = ld->tiles_h * ld->tiles_w;
+    return 0;
+}
+
+/* ---- tile geometry ---------------------------------------------------------------------------- */
+/* Attention layers tile every sequence separately (a tile never crosses a (batch, head) block). */
+static unsigned int seq_block (const nasm_ldata_t *ld)
+{
+    LAYER_TYPE t = ld->layer->type;
+    return (t == K_ATTENTION_LAYER || t == V_ATTENTION_LAYER) ? ld->nasm->tr_seq_len : 0;
+}
+
+static unsigned int col_tile_of (const nasm_ldata_t *ld, unsigned int col)
+{
+    const unsigned int S = seq_block (ld), tw = ld->tile_dims[OUT_W];
+    if (S == 0) return col / tw;
+    return (col / S) * cdiv (S, tw) + (col % S) / tw;
+}
+
+static void tile_range (const nasm_ldata_t *ld, unsigned int t, unsigned int *c0, unsigned int *c1, unsigned int *r0, unsigned int *r1)
+{
+    const unsigned int tn = t / ld->tiles_h, tm = t % ld->tiles_h;      /* row tile fastest (reference src/apu_nasm.c:1218-1224) */
+    const unsigned int S = seq_block (ld), tw = ld->tile_dims[OUT_W];
+    if (S == 0) { *c0 = tn * tw; *c1 = umin (*c0 + tw, ld->out_mat_dims[OUT_W]); }
+    else
+    {
+        const unsigned int per = cdiv (S, tw), blk = tn / per, q0 = (tn % per) * tw;
+        *c0 = blk * S + q0; *c1 = blk * S + umin (q0 + tw, S);
+    }
+    *r0 = tm * ld->tile_dims[OUT_H]; *r1 = umin (*r0 + ld->tile_dims[OUT_H], ld->out_mat_dims[OUT_H]);
+}
+
+void aspen_nasm_tile_range_internal (const nasm_ldata_t *ld, unsigned int t, unsigned int *r)
+{
+    tile_range (ld, t, &r[0], &r[1], &r[2], &r[3]);
+}
+
+typedef struct { uint32_t *v; size_t n, cap; } u32vec;
+static void push (u32vec *a, uint32_t x)
+{
+    if (a->n == a->cap) { a->cap = a->cap ? a->cap * 2 : 1024; a->v = realloc (a->v, a->cap * sizeof (uint32_t)); }
+    a->v[a->n++] = x;
+}
+
+/* all tiles of `pl` that overlap columns [c0, c1) x rows [r0, r1) become parents */
+static void add_parents (const nasm_ldata_t *pl, unsigned int c0, unsigned int c1, unsigned int r0, unsigned int r1, u32vec *out)
+{
+    if (pl->num_ninst == 0 || c1 <= c0 || r1 <= r0) return;   /* the input layer is complete from the start */
+    c1 = umin (c1, pl->out_mat_dims[OUT_W]); r1 = umin (r1, pl->out_mat_dims[OUT_H]);
+    const unsigned int t0 = col_tile_of (pl, c0), t1 = col_tile_of (pl, c1 - 1);
+    const unsigned int m0 = r0 / pl->tile_dims[OUT_H], m1 = (r1 - 1) / pl->tile_dims[OUT_H];
+    for (unsigned int t = t0; t <= t1; t++)
+        for (unsigned int m = m0; m <= m1; m++)
+            push (out, pl->ninst_start + t * pl->tiles_h + m);
+}
+
+/* parents of tile t of layer ld (semantics: reference src/apu_nasm.c:49-466) */
+static void find_parents (const nasm_t *nasm, const nasm_ldata_t *ld, unsigned int t, u32vec *out)
+{
+    const aspen_layer_t *L = ld->layer;
+    const unsigned int *p = L->params;
+    const nasm_ldata_t *p0 = ld->parent_ldata_idx[PARENT_0] >= 0 ? &nasm->ldata_arr[ld->parent_ldata_idx[PARENT_0]] : NULL;
+    const nasm_ldata_t *p1 = ld->parent_ldata_idx[PARENT_1] >= 0 ? &nasm->ldata_arr[ld->parent_ldata_idx[PARENT_1]] : NULL;
+    unsigned int c0, c1, r0, r1;
+    tile_range (ld, t, &c0, &c1, &r0, &r1);
+    const unsigned int S = nasm->tr_seq_len;
+    switch (L->type)
+    {
+    case CONV_LAYER: case MAXPOOL_LAYER: case AVGPOOL_LAYER:
+    {
+        const unsigned int ohw = p[OUT_H] * p[OUT_W], ihw = p[IN_H] * p[IN_W];
+        const unsigned int pr0 = L->type == CONV_LAYER ? 0 : r0, pr1 = L->type == CONV_LAYER ? p0->out_mat_dims[OUT_H] : r1;
+        for (unsigned int b = c0 / ohw; b <= (c1 - 1) / ohw; b++)
+        {
+            const unsigned int first = umax (c0, b * ohw) - b * ohw, last = umin (c1, (b + 1) * ohw) - 1 - b * ohw;
+            const unsigned int oh0 = first / p[OUT_W], oh1 = last / p[OUT_W];
+            int ih_lo = (int)(oh0 * p[STRIDE]) - (int)p[PADDING], ih_hi = (int)(oh1 * p[STRIDE]) - (int)p[PADDING] + (int)p[WEIGHT_H] - 1;
+            int iw_lo = 0, iw_hi = (int)p[IN_W] - 1;
+            if (oh0 == oh1)
+            {
+                iw_lo = (int)((first % p[OUT_W]) * p[STRIDE]) - (int)p[PADDING];
+                iw_hi = (int)((last % p[OUT_W]) * p[STRIDE]) - (int)p[PADDING] + (int)p[WEIGHT_W] - 1;
+            }
+            if (ih_lo < 0) ih_lo = 0;
+            if (iw_lo < 0) iw_lo = 0;
+            if (ih_hi > (int)p[IN_H] - 1) ih_hi = (int)p[IN_H] - 1;
+            if (iw_hi > (int)p[IN_W] - 1) iw_hi = (int)p[IN_W] - 1;
+            if (ih_hi < ih_lo || iw_hi < iw_lo) continue;             /* window entirely in the padding */
+            add_parents (p0, b * ihw + ih_lo * p[IN_W] + iw_lo, b * ihw + ih_hi * p[IN_W] + iw_hi + 1, pr0, pr1, out);
+        }
+        break;
+    }
+    case FC_LAYER:
+    {
+        const unsigned int ihw = p[IN_H] * p[IN_W];
+        add_parents (p0, c0 * ihw, c1 * ihw, 0, p0->out_mat_dims[OUT_H], out);
+        break;
+    }
+    case MATMUL_LAYER: case LAYERNORM_LAYER: case SOFTMAX_LAYER:
+        add_parents (p0, c0, c1, 0, p0->out_mat_dims[OUT_H], out);
+        break;
+    case RESIDUAL_LAYER:
+        add_parents (p0, c0, c1, r0, r1, out);
+        add_parents (p1, c0, c1, r0, r1, out);
+        break;
+    case K_ATTENTION_LAYER:
+    {
+        const unsigned int H = p[NUM_HEAD], hd = p[NUM_HIDDEN] / H;
+        const unsigned int bh = c0 / S, b = bh / H, h = bh % H, q0 = c0 % S, q1 = q0 + (c1 - c0);
+        add_parents (p0, b * S + q0, b * S + q1, h * hd, (h + 1) * hd, out);    /* Query columns of this tile */
+        add_parents (p1, b * S, (b + 1) * S, h * hd, (h + 1) * hd, out);        /* every Key of the sequence */
+        break;
+    }
+    case V_ATTENTION_LAYER:
+    {
+        const unsigned int H = p[NUM_HEAD], hd = p[NUM_HIDDEN] / H;
+        const unsigned int b = c0 / S, h = r0 / hd, q0 = c0 % S, q1 = q0 + (c1 - c0);
+        add_parents (p0, (b * H + h) * S + q0, (b * H + h) * S + q1, 0, S, out); /* probability rows */
+        add_parents (p1, b * S, (b + 1) * S, r0, r1, out);                       /* every Value of the sequence */
+        break;
+    }
+    default: break;
+    }
+}
+
+static int cmp_u32 (const void *a, const void *b)
+{
+    uint32_t x = *(const uint32_t *)a, y = *(const uint32_t *)b;
+    return x < y ? -1 : x > y;
+}
+
+static int build_graph (nasm_t *nasm)
+{
+    const uint32_t n = nasm->num_ninst;
+    nasm->ninst_ldata = calloc (n ? n : 1, sizeof (uint32_t));
+    nasm->num_parents = calloc (n ? n : 1, sizeof (uint32_t));
+    nasm->child_off = calloc ((size_t)n + 2, sizeof (uint32_t));
+    u32vec edges_parent = {0}, edges_child = {0}, tmp = {0};
+    for (unsigned int l = 0; l < nasm->num_ldata; l++)
+    {
+        const nasm_ldata_t *ld = &nasm->ldata_arr[l];
+        for (unsigned int t = 0; t < ld->num_ninst; t++)
+        {
+            const uint32_t id = ld->ninst_start + t;
+            nasm->ninst_ldata[id] = l;
+            tmp.n = 0;
+            find_parents (nasm, ld, t, &tmp);
+            qsort (tmp.v, tmp.n, sizeof (uint32_t), cmp_u32);
+            uint32_t prev = 0xffffffffu;
+            for (size_t i = 0; i < tmp.n; i++)
+            {
+                if (tmp.v[i] == prev) continue;         /* the two parents of a shortcut may be the same tile */
+                prev = tmp.v[i];
+                if (prev >= id) { ERROR_PRTF ("tile %u depends on a later tile %u\n", id, prev); return -1; }
+                push (&edges_parent, prev); push (&edges_child, id);
+                nasm->num_parents[id]++;
+                nasm->child_off[prev + 1]++;
+            }
+        }
+    }
+    for (uint32_t i = 0; i < n; i++) nasm->child_off[i + 1] += nasm->child_off[i];
+    nasm->num_edges = (uint32_t)edges_parent.n;
+    nasm->child_idx = calloc (edges_parent.n ? edges_parent.n : 1, sizeof (uint32_t));
+    uint32_t *cursor = calloc (n ? n : 1, sizeof (uint32_t));
+    for (size_t e = 0; e < edges_parent.n; e++)
+    {
+        const uint32_t pnt = edges_parent.v[e];
+        nasm->child_idx[nasm->child_off[pnt] + cursor[pnt]++] = edges_child.v[e];
+    }
+    free (cursor); free (edges_parent.v); free (edges_child.v); free (tmp.v);
+    return 0;
+}
+
+static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned int batch, unsigned int seq)
+{
+    if (dnn == NULL) { ERROR_PRTF ("apu_create_nasm: dnn is NULL\n"); return NULL; }
+    if (min_ninst < 1) { ERROR_PRTF ("ERROR: min_ninst_per_ldata should be at least 1\n"); return NULL; }
+    nasm_t *nasm = calloc (1, sizeof (nasm_t));
+    nasm->dnn = dnn; nasm->nasm_id = nasm_counter++;
+    nasm->batch_size = batch > 0 ? batch : 1;
+    nasm->tr_seq_len = seq; nasm->min_ninst_per_ldata = min_ninst;
+    nasm->num_ldata = dnn->num_layers;
+    nasm->ldata_arr = calloc (nasm->num_ldata, sizeof (nasm_ldata_t));
+    size_t arena = 0;
+    unsigned int total = 0;
+    int bad = 0;
+    for (unsigned int l = 0; l < nasm->num_ldata && !bad; l++)
+    {
+        nasm_ldata_t *ld = &nasm->ldata_arr[l];
+        ld->nasm = nasm; ld->layer = &dnn->layers[l];
+        for (int k = 0; k < NUM_PARENT_ELEMENTS; k++) ld->parent_ldata_idx[k] = ld->layer->parent_idx[k];
+        if (set_out_mat (nasm, ld) || set_tiles (nasm, ld)) { bad = 1; break; }
+        for (int k = PARENT_0; k <= PARENT_1; k++)
+        {
+            if (ld->parent_ldata_idx[k] < 0) continue;
+            const nasm_ldata_t *pl = &nasm->ldata_arr[ld->parent_ldata_idx[k]];
+            /* shortcut parents must have this layer's shape (reference src/tiled_kernels.c:613-638 reads both at the same (h, w)) */
+            if (ld->layer->type == RESIDUAL_LAYER && (pl->out_mat_dims[OUT_H] != ld->out_mat_dims[OUT_H] || pl->out_mat_dims[OUT_W] != ld->out_mat_dims[OUT_W]))
+            { ERROR_PRTF ("layer %u: shortcut parents differ in shape\n", l); bad = 1; }
+        }
+        ld->out_mat_offset = arena;
+        arena += ((size_t)ld->out_mat_stride * ld->out_mat_dims[OUT_W] + 63) / 64 * 64;    /* 256-byte aligned matrices */
+        ld->ninst_start = total;
+        total += ld->num_ninst;
+        nasm->total_flops += ld->flops;
+    }
+    nasm->arena_floats = arena;
+    nasm->num_ninst = total;
+    if (!bad && build_graph (nasm)) bad = 1;
+    if (bad) { dnn->ref_nasms++; apu_destroy_nasm (nasm); return NULL; }
+    dnn->ref_nasms++;
+    return nasm;
+}
+
+nasm_t *apu_create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst_per_ldata, unsigned int batch_size)
+{
+    return create_nasm (dnn, min_ninst_per_ldata, batch_size, 0);
+}
+
+nasm_t *apu_create_transformer_nasm (aspen_dnn_t *dnn, unsigned int min_ninst_per_ldata, unsigned int batch_size, unsigned int seq_num)
+{
+    return create_nasm (dnn, min_ninst_per_ldata, batch_size, seq_num);
+}
+
+/* The reference searches min_ninst by timing 50-iteration runs (reference src/apu_nasm.c:601-639);
+   this build uses the fixed policy "two tiles per compute unit". */
+#define DEFAULT_MIN_NINST 512
+nasm_t *apu_generate_nasm (aspen_dnn_t *dnn, unsigned int batch_size, unsigned int num_iter)
+{
+    (void)num_iter;
+    return create_nasm (dnn, DEFAULT_MIN_NINST, batch_size, 0);
+}
+nasm_t *apu_generate_transformer_nasm (aspen_dnn_t *dnn, unsigned int batch_size, unsigned int seq_num, unsigned int num_iter)
+{
+    (void)num_iter;
+    return create_nasm (dnn, DEFAULT_MIN_NINST, batch_size, seq_num);
+}
+
+void apu_destroy_nasm (nasm_t *nasm)
+{
+    if (nasm == NULL) return;
+    if (nasm->rpool != NULL)
+    {
+        rpool_t *rp = nasm->rpool;
+        for (unsigned int i = 0; i < rp->num_nasms; i++)
+            if (rp->nasms[i] == nasm)
+            {
+                memmove (&rp->nasms[i], &rp->nasms[i + 1], (rp->num_nasms - i - 1) * sizeof (nasm_t *));
+                rp->num_nasms--;
+                rp->graph_dirty = 1;
+                break;
+            }
+    }
+    aspen_hip_free (nasm->d_arena);
+    free (nasm->ninst_ldata); free (nasm->num_parents); free (nasm->child_off); free (nasm->child_idx);
+    free (nasm->ldata_arr);
+    nasm->dnn->ref_nasms--;
+    free (nasm);
+}
+
+void apu_reset_nasm (nasm_t *nasm)
+{
+    if (nasm == NULL) return;
+    nasm->completed = 0;
+    nasm->armed = 1;
+}
+
+nasm_t *apu_load_nasm_from_file (char *filename, aspen_dnn_t *dnn)
+{
+    (void)dnn;
+    ERROR_PRTF ("apu_load_nasm_from_file (%s): .nasm files describe the reference's CPU tile grid and are not read by this build; use apu_create_nasm.\n", filename ? filename : "NULL");
+    return NULL;
+}
+
+void apu_save_nasm_to_file (nasm_t *nasm, char *filename)
+{
+    (void)nasm;
+    ERROR_PRTF ("apu_save_nasm_to_file (%s): not implemented in this build.\n", filename ? filename : "NULL");
+}
+
+/* ---- device ------------------------------------------------------------------------------------ */
+int aspen_nasm_to_device (nasm_t *nasm)
+{
+    if (nasm->d_arena == NULL)
+    {
+        nasm->d_arena = aspen_hip_alloc (nasm->arena_floats * sizeof (float));
+        if (nasm->d_arena == NULL) return -1;
+    }
+    for (unsigned int l = 0; l < nasm->num_ldata; l++)
+    {
+        nasm_ldata_t *ld = &nasm->ldata_arr[l];
+        if (ld->parent_ldata_idx[PARENT_0] < 0) continue;
+        if (aspen_layer_to_device (ld->layer, nasm->ldata_arr[ld->parent_ldata_idx[PARENT_0]].out_mat_stride)) return -1;
+    }
+    return 0;
+}
+
+/* Device descriptors of all layers, tile indices shifted by ninst_base (position inside a merged graph). */
+int aspen_nasm_fill_device_layers (nasm_t *nasm, aspen_hip_layer_t *dst, uint32_t ninst_base)
+{
+    for (unsigned int l = 0; l < nasm->num_ldata; l++)
+    {
+        const nasm_ldata_t *ld = &nasm->ldata_arr[l];
+        const aspen_layer_t *L = ld->layer;
+        const unsigned int *p = L->params;
+        aspen_hip_layer_t *d = &dst[l];
+        memset (d, 0, sizeof (*d));
+        d->type = L->type; d->act = L->activation; d->variant = ld->variant;
+        d->M = ld->out_mat_dims[OUT_H]; d->N = ld->out_mat_dims[OUT_W]; d->ld = ld->out_mat_stride;
+        d->tile_m = ld->tile_dims[OUT_H]; d->tile_n = ld->tile_dims[OUT_W];
+        d->tiles_m = ld->tiles_h; d->tiles_n = ld->tiles_w;
+        d->ninst_start = ninst_base + ld->ninst_start; d->num_ninst = ld->num_ninst;
+        d->out = nasm->d_arena + ld->out_mat_offset;
+        if (ld->parent_ldata_idx[PARENT_0] >= 0)
+        {
+            const nasm_ldata_t *pl = &nasm->ldata_arr[ld->parent_ldata_idx[PARENT_0]];
+            d->in0 = nasm->d_arena + pl->out_mat_offset; d->ld0 = pl->out_mat_stride;
+        }
+        if (ld->parent_ldata_idx[PARENT_1] >= 0)
+        {
+            const nasm_ldata_t *pl = &nasm->ldata_arr[ld->parent_ldata_idx[PARENT_1]];
+            d->in1 = nasm->d_arena + pl->out_mat_offset; d->ld1 = pl->out_mat_stride;
+        }
+        d->weight = L->d_weight; d->bias = L->d_bias; d->ktab = L->d_ktab;
+        d->K = L->gemm_k; d->Kp = L->dev_kp;
+        d->IH = p[IN_H]; d->IW = p[IN_W]; d->IC = p[IN_C]; d->OH = p[OUT_H]; d->OW = p[OUT_W];
+        d->KH = p[WEIGHT_H]; d->KW = p[WEIGHT_W]; d->stride = p[STRIDE]; d->pad = p[PADDING];
+        if (L->type == FC_LAYER) { d->KH = p[IN_H]; d->KW = p[IN_W]; d->OH = 1; d->OW = 1; d->stride = 1; d->pad = 0; }
+        if (L->type == MATMUL_LAYER) { d->IH = d->IW = d->OH = d->OW = d->KH = d->KW = d->stride = 1; d->pad = 0; d->IC = p[MAT_K]; }
+        if (is_contraction (L->type))
+        {
+            const int pointwise = L->type == MATMUL_LAYER
+                || (L->type == CONV_LAYER && p[WEIGHT_H] == 1 && p[WEIGHT_W] == 1 && p[STRIDE] == 1 && p[PADDING] == 0)
+                || (L->type == FC_LAYER && p[IN_H] == 1 && p[IN_W] == 1);
+            d->direct = pointwise && (d->IC % 32 == 0) && d->ld0 >= d->Kp;
+        }
+        if (L->type == K_ATTENTION_LAYER || L->type == V_ATTENTION_LAYER)
+        {
+            d->heads = p[NUM_HEAD]; d->seq = nasm->tr_seq_len; d->hd = p[NUM_HIDDEN] / p[NUM_HEAD]; d->masked = p[MASKED];
+        }
+    }
+    return 0;
+}

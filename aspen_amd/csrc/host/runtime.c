@@ -1,0 +1,351 @@
+/*
+ * runtime.c -- ready pool, scheduling-engine group and result read-out on top of the device engine.
+ *
+ * Same call protocol as the reference (reference main.c:105-151):
+ *   rpool_init -> dse_group_init -> dse_group_set_rpool -> rpool_add_nasm[_raw_input]
+ *   loop { rpool_reset_queue; rpool_reset_nasm; dse_group_run; dse_wait_for_nasm_completion; dse_group_stop }
+ *   dse_get_nasm_result
+ * The reference's pool of mutex-guarded queues and its DSE pthreads (reference src/rpool.c,
+ * src/dse.c) live on the device here: the ready queue and the dependency counters are arrays in
+ * HBM and the "engines" are the persistent workgroups of one kernel; this file only arms and
+ * launches them.  Every nasm attached to a pool runs in the same launch, its tiles interleaved
+ * with the others' in one queue (co-scheduled networks, reference examples/2).
+ */
+#include "internal.h"
+
+/* ---- ready pool -------------------------------------------------------------------------------- */
+rpool_t *rpool_init (void)
+{
+    rpool_t *rp = calloc (1, sizeof (rpool_t));
+    rp->graph_dirty = 1;
+    return rp;
+}
+
+void rpool_destroy (rpool_t *rpool)
+{
+    if (rpool == NULL) return;
+    if (rpool->ref_dses > 0)
+    {
+        ERROR_PRTF ("Cannot destroy rpool with %u dses still referencing it.\n", rpool->ref_dses);
+        return;
+    }
+    aspen_hip_sync ();
+    for (unsigned int i = 0; i < rpool->num_nasms; i++) rpool->nasms[i]->rpool = NULL;
+    aspen_hip_graph_destroy (rpool->graph);
+    free (rpool);
+}
+
+static int attach (rpool_t *rpool, nasm_t *nasm)
+{
+    if (nasm->rpool == rpool) return 0;
+    if (nasm->rpool != NULL) { ERROR_PRTF ("nasm %u is already attached to another rpool\n", nasm->nasm_id); return -1; }
+    if (rpool->num_nasms == RPOOL_MAX_NASMS) { ERROR_PRTF ("rpool is full (%d nasms)\n", RPOOL_MAX_NASMS); return -1; }
+    rpool->nasms[rpool->num_nasms++] = nasm;
+    nasm->rpool = rpool;
+    rpool->graph_dirty = 1;
+    return 0;
+}
+
+void rpool_add_nasm_raw_input (rpool_t *rpool, nasm_t *nasm, void *input_data)
+{
+    if (rpool == NULL) { ERROR_PRTF ("ERROR: rpool_add_nasm_raw_input: rpool is NULL.\n"); return; }
+    if (nasm == NULL) { ERROR_PRTF ("ERROR: rpool_add_nasm_raw_input: nasm is NULL.\n"); return; }
+    if (aspen_nasm_to_device (nasm)) { ERROR_PRTF ("ERROR: rpool_add_nasm_raw_input: device setup failed: %s\n", aspen_hip_last_error ()); return; }
+    if (attach (rpool, nasm)) return;
+    if (input_data != NULL)
+    {
+        /* dense columns -> strided columns of layer 0 (reference copy_buffer_to_ldata_out_mat, src/apu_nasm.c:809) */
+        const nasm_ldata_t *ld = &nasm->ldata_arr[0];
+        const size_t H = ld->out_mat_dims[OUT_H], W = ld->out_mat_dims[OUT_W];
+        aspen_hip_sync ();
+        if (aspen_hip_h2d_2d (nasm->d_arena + ld->out_mat_offset, ld->out_mat_stride * sizeof (float),
+                input_data, H * sizeof (float), H * sizeof (float), W))
+            ERROR_PRTF ("ERROR: rpool_add_nasm_raw_input: input upload failed: %s\n", aspen_hip_last_error ());
+    }
+    nasm->armed = 1;
+    nasm->completed = 0;
+}
+
+void rpool_add_nasm (rpool_t *rpool, nasm_t *nasm, char *input_filename)
+{
+    if (rpool == NULL || nasm == NULL) { ERROR_PRTF ("ERROR: rpool_add_nasm: NULL argument.\n"); return; }
+    const nasm_ldata_t *ld = &nasm->ldata_arr[0];
+    const unsigned int *p = ld->layer->params;
+    const size_t H = ld->out_mat_dims[OUT_H], W = ld->out_mat_dims[OUT_W], n = H * W;
+    float *file = calloc (n, sizeof (float)), *dense = calloc (n, sizeof (float));
+    if (input_filename != NULL)
+    {
+        FILE *fp = fopen (input_filename, "rb");
+        if (fp == NULL || fread (file, sizeof (float), n, fp) != n)
+        {
+            ERROR_PRTF ("Error: Failed to read %zu floats from file %s.\n", n, input_filename);
+            if (fp) fclose (fp);
+            free (file); free (dense);
+            return;
+        }
+        fclose (fp);
+    }
+    if (nasm->tr_seq_len == 0)
+    {
+        /* image files are NCHW (reference aspen_load_input_NHWC, src/apu.c:638) */
+        const size_t C = p[OUT_C], HW = (size_t)p[OUT_H] * p[OUT_W];
+        for (size_t b = 0; b < nasm->batch_size; b++)
+            for (size_t c = 0; c < C; c++)
+                for (size_t i = 0; i < HW; i++)
+                    dense[(b * HW + i) * C + c] = file[(b * C + c) * HW + i];
+    }
+    else
+        memcpy (dense, file, n * sizeof (float));
+    rpool_add_nasm_raw_input (rpool, nasm, dense);
+    free (file); free (dense);
+}
+
+void rpool_reset_queue (rpool_t *rpool)
+{
+    /* the device queue is rebuilt by the arm kernel of the next run; nothing is kept between runs */
+    (void)rpool;
+}
+
+void rpool_reset_nasm (rpool_t *rpool, nasm_t *nasm)
+{
+    if (rpool == NULL || nasm == NULL) return;
+    if (nasm->rpool != rpool)
+    {
+        ERROR_PRTF ("ERROR: rpool_reset_nasm: nasm \"%s_nasm_%d\" is not in rpool.\n", nasm->dnn->name, nasm->nasm_id);
+        return;
+    }
+    apu_reset_nasm (nasm);
+}
+
+/* merged device graph of every nasm in the pool: layer and tile indices shifted, roots interleaved */
+static int rebuild_graph (rpool_t *rp)
+{
+    aspen_hip_sync ();
+    aspen_hip_graph_destroy (rp->graph);
+    rp->graph = NULL;
+    uint32_t layers = 0, ninst = 0, edges = 0;
+    for (unsigned int i = 0; i < rp->num_nasms; i++)
+    {
+        layers += rp->nasms[i]->num_ldata; ninst += rp->nasms[i]->num_ninst; edges += rp->nasms[i]->num_edges;
+    }
+    if (layers == 0) { rp->graph_dirty = 0; return 0; }
+    aspen_hip_layer_t *L = calloc (layers, sizeof (aspen_hip_layer_t));
+    uint32_t *nl = calloc (ninst + 1, sizeof (uint32_t)), *np = calloc (ninst + 1, sizeof (uint32_t));
+    uint32_t *co = calloc ((size_t)ninst + 2, sizeof (uint32_t)), *ci = calloc (edges + 1, sizeof (uint32_t));
+    uint32_t *roots = calloc (ninst + 1, sizeof (uint32_t));
+    uint32_t lbase = 0, nbase = 0, ebase = 0, nroots = 0;
+    int rc = 0;
+    for (unsigned int i = 0; i < rp->num_nasms && !rc; i++)
+    {
+        nasm_t *g = rp->nasms[i];
+        if (aspen_nasm_to_device (g)) { rc = -1; break; }
+        aspen_nasm_fill_device_layers (g, L + lbase, nbase);
+        for (uint32_t t = 0; t < g->num_ninst; t++)
+        {
+            nl[nbase + t] = lbase + g->ninst_ldata[t];
+            np[nbase + t] = g->num_parents[t];
+            co[nbase + t] = ebase + g->child_off[t];
+        }
+        for (uint32_t e = 0; e < g->num_edges; e++) ci[ebase + e] = nbase + g->child_idx[e];
+        lbase += g->num_ldata; nbase += g->num_ninst; ebase += g->num_edges;
+    }
+    co[ninst] = edges;
+    /* roots of the attached graphs taken in turns, so co-scheduled networks start together */
+    if (!rc)
+    {
+        uint32_t cursor[RPOOL_MAX_NASMS] = {0}, base[RPOOL_MAX_NASMS];
+        uint32_t b = 0;
+        for (unsigned int i = 0; i < rp->num_nasms; i++) { base[i] = b; b += rp->nasms[i]->num_ninst; }
+        int progress = 1;
+        while (progress)
+        {
+            progress = 0;
+            for (unsigned int i = 0; i < rp->num_nasms; i++)
+            {
+                nasm_t *g = rp->nasms[i];
+                while (cursor[i] < g->num_ninst && g->num_parents[cursor[i]] != 0) cursor[i]++;
+                if (cursor[i] < g->num_ninst) { roots[nroots++] = base[i] + cursor[i]++; progress = 1; }
+            }
+        }
+        rp->graph = aspen_hip_graph_create (L, layers, nl, np, co, ci, ninst, roots, nroots);
+        if (rp->graph == NULL) rc = -1;
+    }
+    free (L); free (nl); free (np); free (co); free (ci); free (roots);
+    rp->graph_dirty = rc != 0;
+    return rc;
+}
+
+/* ---- scheduling engines ------------------------------------------------------------------------ */
+dse_group_t *dse_group_init (unsigned int num_dse)
+{
+    dse_group_t *g = calloc (1, sizeof (dse_group_t));
+    g->num_dses = num_dse;
+    g->mode = 1;
+    const char *m = getenv ("ASPEN_GPU_MODE");           /* "layers" = one launch per layer, "dataflow" = persistent kernel */
+    if (m != NULL && strcmp (m, "layers") == 0) g->mode = 0;
+    const char *w = getenv ("ASPEN_GPU_WORKGROUPS");
+    g->workgroups = w ? (unsigned int)atoi (w) : 0;
+    return g;
+}
+
+void dse_group_set_rpool (dse_group_t *dse_group, rpool_t *rpool)
+{
+    if (dse_group == NULL) { ERROR_PRTF ("ERROR: dse_group_set_rpool: dse_group is NULL\n"); return; }
+    if (rpool == NULL) { ERROR_PRTF ("ERROR: dse_group_set_rpool: rpool is NULL\n"); return; }
+    if (dse_group->rpool != NULL) dse_group->rpool->ref_dses -= dse_group->num_dses;
+    dse_group->rpool = rpool;
+    rpool->ref_dses += dse_group->num_dses;
+}
+
+void dse_group_destroy (dse_group_t *dse_group)
+{
+    if (dse_group == NULL) return;
+    aspen_hip_sync ();
+    if (dse_group->rpool != NULL) dse_group->rpool->ref_dses -= dse_group->num_dses;
+    free (dse_group);
+}
+
+void dse_group_run (dse_group_t *dse_group)
+{
+    if (dse_group == NULL) { ERROR_PRTF ("ERROR: dse_group_run: dse_group is NULL\n"); return; }
+    rpool_t *rp = dse_group->rpool;
+    if (rp == NULL) { ERROR_PRTF ("ERROR: dse_group_run: no rpool set\n"); return; }
+    int armed = 0;
+    for (unsigned int i = 0; i < rp->num_nasms; i++) armed |= rp->nasms[i]->armed;
+    if (!armed) return;                                    /* nothing ready: the engines idle, as in the reference */
+    if (rp->graph_dirty && rebuild_graph (rp)) { ERROR_PRTF ("ERROR: dse_group_run: graph upload failed: %s\n", aspen_hip_last_error ()); return; }
+    if (rp->graph == NULL) return;
+    int rc;
+    if (dse_group->mode == 0)
+    {
+        uint32_t layers = 0;
+        for (unsigned int i = 0; i < rp->num_nasms; i++) layers += rp->nasms[i]->num_ldata;
+        rc = aspen_hip_run_layers (rp->graph, 0, layers - 1);
+    }
+    else
+        rc = aspen_hip_run_dataflow (rp->graph, dse_group->workgroups, 0);
+    if (rc) { ERROR_PRTF ("ERROR: dse_group_run: launch failed: %s\n", aspen_hip_last_error ()); return; }
+    for (unsigned int i = 0; i < rp->num_nasms; i++) { rp->nasms[i]->armed = 0; rp->nasms[i]->completed = 2; }   /* 2 = in flight */
+    rp->running = 1;
+}
+
+static void finish (rpool_t *rp)
+{
+    if (rp == NULL || !rp->running) return;
+    if (aspen_hip_sync ()) ERROR_PRTF ("ERROR: device run failed: %s\n", aspen_hip_last_error ());
+    uint32_t executed = 0, twice = 0, aborted = 0;
+    rp->running = 0;
+    for (unsigned int i = 0; i < rp->num_nasms; i++)
+        if (rp->nasms[i]->completed == 2) rp->nasms[i]->completed = 1;
+    (void)executed; (void)twice; (void)aborted;
+}
+
+void dse_group_stop (dse_group_t *dse_group)
+{
+    if (dse_group == NULL) { ERROR_PRTF ("ERROR: dse_group_stop: dse_group is NULL\n"); return; }
+    finish (dse_group->rpool);
+}
+
+void dse_wait_for_nasm_completion (nasm_t *nasm)
+{
+    if (nasm == NULL) return;
+    if (nasm->completed == 2) finish (nasm->rpool);
+}
+
+unsigned int dse_check_nasm_completion (nasm_t *nasm)
+{
+    if (nasm == NULL) return 0;
+    if (nasm->completed == 2 && aspen_hip_idle () == 1) finish (nasm->rpool);
+    return nasm->completed == 1;
+}
+
+void dse_group_run_until_nasm_completion (dse_group_t *dse_group, nasm_t *nasm)
+{
+    dse_group_run (dse_group);
+    dse_wait_for_nasm_completion (nasm);
+    dse_group_stop (dse_group);
+}
+
+/* ---- results ------------------------------------------------------------------------------------ */
+/* Layer output as a dense tensor in the caller's dimension order (reference get_ldata_output,
+   src/apu.c:227-297): stride padding stripped, native order (batch, positions..., channels) permuted. */
+ssize_t dse_get_ldata_result (nasm_t *nasm, unsigned int ldata_idx, LAYER_PARAMS *order, void **out_ptr)
+{
+    if (nasm == NULL || ldata_idx >= nasm->num_ldata) { ERROR_PRTF ("Error in get_ldata_output: ldata is NULL.\n"); return -1; }
+    if (out_ptr == NULL) { ERROR_PRTF ("Error in get_ldata_output: out_ptr is NULL.\n"); return -1; }
+    if (nasm->d_arena == NULL) { ERROR_PRTF ("Error in get_ldata_output: nasm has not been run.\n"); return -1; }
+    if (nasm->completed == 2) finish (nasm->rpool);
+    const nasm_ldata_t *ld = &nasm->ldata_arr[ldata_idx];
+    const aspen_layer_t *L = ld->layer;
+    const size_t H = ld->out_mat_dims[OUT_H], W = ld->out_mat_dims[OUT_W];
+    float *dense = malloc (H * W * sizeof (float));
+    if (dense == NULL) return -1;
+    if (aspen_hip_d2h_2d (dense, H * sizeof (float), nasm->d_arena + ld->out_mat_offset,
+            ld->out_mat_stride * sizeof (float), H * sizeof (float), W))
+    {
+        ERROR_PRTF ("Error in get_ldata_output: download failed: %s\n", aspen_hip_last_error ());
+        free (dense);
+        return -1;
+    }
+    /* native dimension list, slowest first */
+    LAYER_PARAMS native[4];
+    size_t dim[NUM_PARAM_ELEMENTS] = {0};
+    int nd;
+    const unsigned int *p = L->params;
+    const int matrix = nasm->tr_seq_len != 0;
+    if (L->type == K_ATTENTION_LAYER)
+    {
+        nd = 4; native[0] = BATCH; native[1] = NUM_HEAD; native[2] = MAT_N; native[3] = MAT_M;
+        dim[BATCH] = nasm->batch_size; dim[NUM_HEAD] = p[NUM_HEAD]; dim[MAT_N] = nasm->tr_seq_len; dim[MAT_M] = H;
+    }
+    else if (matrix)
+    {
+        nd = 3; native[0] = BATCH; native[1] = MAT_N; native[2] = MAT_M;
+        dim[BATCH] = nasm->batch_size; dim[MAT_N] = nasm->tr_seq_len; dim[MAT_M] = H;
+    }
+    else if (L->type == FC_LAYER || L->type == SOFTMAX_LAYER)
+    {
+        nd = 2; native[0] = BATCH; native[1] = OUT_C;
+        dim[BATCH] = nasm->batch_size; dim[OUT_C] = H;
+    }
+    else
+    {
+        nd = 4; native[0] = BATCH; native[1] = OUT_H; native[2] = OUT_W; native[3] = OUT_C;
+        dim[BATCH] = nasm->batch_size; dim[OUT_H] = p[OUT_H]; dim[OUT_W] = p[OUT_W]; dim[OUT_C] = H;
+    }
+    /* the first nd entries of `order` must be a permutation of the native dimensions */
+    int valid = order != NULL;
+    for (int i = 0; i < nd && valid; i++)
+    {
+        int found = 0;
+        for (int j = 0; j < nd; j++) found |= native[j] == order[i];
+        for (int j = 0; j < i; j++) if (order[j] == order[i]) found = 0;
+        valid = found;
+    }
+    if (!valid) { *out_ptr = dense; return (ssize_t)(H * W * sizeof (float)); }   /* native order */
+    size_t nstride[NUM_PARAM_ELEMENTS] = {0}, s = 1;
+    for (int i = nd - 1; i >= 0; i--) { nstride[native[i]] = s; s *= dim[native[i]]; }
+    float *out = calloc (H * W, sizeof (float));
+    size_t idx[4] = {0, 0, 0, 0};
+    for (size_t o = 0; o < H * W; o++)
+    {
+        size_t src = 0;
+        for (int i = 0; i < nd; i++) src += idx[i] * nstride[order[i]];
+        out[o] = dense[src];
+        for (int i = nd - 1; i >= 0; i--) { if (++idx[i] < dim[order[i]]) break; idx[i] = 0; }
+    }
+    free (dense);
+    *out_ptr = out;
+    return (ssize_t)(H * W * sizeof (float));
+}
+
+ssize_t dse_get_nasm_result (nasm_t *nasm, LAYER_PARAMS *order, void **out_ptr)
+{
+    if (nasm == NULL) return -1;
+    return dse_get_ldata_result (nasm, nasm->num_ldata - 1, order, out_ptr);
+}
+
+void aspen_flush_dynamic_memory (void)
+{
+    /* activations live in per-nasm arenas that are freed with the nasm; there is no allocator cache to flush */
+}

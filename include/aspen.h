@@ -5,7 +5,7 @@
  * same function names, argument meaning and ownership rules; enum numbering is
  * kept because callers pass LAYER_PARAMS arrays (output dimension order) by
  * value.  All structs are opaque here; no caller in the reference touches a
- * field (reference main.c, examples/*).
+ * field (reference main.c and the examples directory).
  *
  * Each declaration cites the reference declaration it replaces.
  */

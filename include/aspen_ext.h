@@ -1,0 +1,44 @@
+/*
+ * aspen_ext.h -- additions to the public API that have no counterpart in the reference: engine mode
+ * selection, introspection of the tile graph (used by the tests and the benchmark) and run statistics.
+ */
+#ifndef ASPEN_AMD_ASPEN_EXT_H
+#define ASPEN_AMD_ASPEN_EXT_H
+
+#include <stdint.h>
+#include "aspen.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* 0: one kernel launch per layer (layer-synchronous); 1: persistent dataflow kernel (default).
+   The environment variable ASPEN_GPU_MODE=layers|dataflow sets the initial value. */
+void aspen_dse_group_set_mode (dse_group_t *dse_group, int mode);
+/* persistent workgroups of the dataflow kernel; 0 = two per compute unit */
+void aspen_dse_group_set_workgroups (dse_group_t *dse_group, unsigned int workgroups);
+
+unsigned int aspen_nasm_num_ldata (nasm_t *nasm);
+unsigned int aspen_nasm_num_ninst (nasm_t *nasm);
+unsigned int aspen_nasm_num_edges (nasm_t *nasm);
+uint64_t aspen_nasm_total_flops (nasm_t *nasm);
+/* info[0..11] = type, activation, rows, columns, stride, num_ninst, tile_rows, tile_columns,
+   parent0, parent1 (0xffffffff = none), first tile index, GEMM variant */
+void aspen_nasm_ldata_info (nasm_t *nasm, unsigned int ldata_idx, unsigned int *info);
+uint64_t aspen_nasm_ldata_flops (nasm_t *nasm, unsigned int ldata_idx);
+/* dependency graph in CSR form; pointers stay valid until the nasm is destroyed */
+void aspen_nasm_graph (nasm_t *nasm, const uint32_t **ninst_ldata, const uint32_t **num_parents,
+    const uint32_t **child_off, const uint32_t **child_idx);
+/* column / row range [c0, c1) x [r0, r1) of one tile */
+void aspen_nasm_tile_range (nasm_t *nasm, unsigned int ninst_idx, unsigned int *range);
+
+/* counters of the last dataflow run of the pool: tiles executed, tiles executed more than once,
+   abort flag (a wait on the ready queue hit its spin limit).  Returns 0 on success. */
+int aspen_rpool_run_stats (rpool_t *rpool, uint32_t *executed, uint32_t *double_runs, uint32_t *aborted);
+/* tiles in the pool's merged graph */
+unsigned int aspen_rpool_num_ninst (rpool_t *rpool);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

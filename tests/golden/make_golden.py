@@ -27,7 +27,7 @@ MICRO = {
     # name: (cfg, style, batch, seq, seed, kind)
     "custom_b3": (M.custom_cifar_cfg(), "he", 3, 0, 7, None),
     "resnet_mini_b2": (M.resnet50_cfg(64, 64, 10, (16, 32, 64, 128), (1, 2, 1, 1), 16), "he", 2, 0, 8, None),
-    "vgg_mini_b5": (M.vgg16_cfg(32, 32, 10, (8, "M", 16, "M", 64, 64, "M"), (96,)), "he", 5, 0, 9, None),
+    "vgg_mini_b5": (M.vgg16_cfg(32, 32, 10, (8, "M", 16, "M", 64, 64, "M"), (128,)), "he", 5, 0, 9, None),
     "bert_mini_b2_s24": (M.bert_cfg(2, 128, 2, 256), "gpt", 2, 24, 10, "embeddings"),
     "gpt_mini_b2_s20": (M.gpt2_cfg(2, 128, 2, 256), "gpt", 2, 20, 11, "token_ids"),
 }

@@ -1,0 +1,111 @@
+"""GPU parity: the HIP library (through the C ABI) against the compiled-reference fixtures and the
+CPU oracle, per layer, relative L2 <= 1e-4 and identical argmax."""
+import os
+
+import numpy as np
+import pytest
+
+from aspen_amd import api, models as M
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("mode", [api.MODE_LAYERS, api.MODE_DATAFLOW], ids=["layers", "dataflow"])
+@pytest.mark.parametrize("name", list(H.micro_cases()))
+def test_micro_nets_match_reference_fixture(gpu, name, mode):
+    """Full per-layer tensors of small nets, as produced by the compiled reference."""
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()[name])
+    gold = np.load(os.path.join(H.GOLDEN, f"micro_{name}.npz"))
+    net = H.GpuNet(cfg, tens, batch, seq, min_ninst=8, mode=mode)
+    print(f"case {name} mode {mode} tiles {net.nasm.num_ninst}", flush=True)
+    net.run(x)
+    try:
+        for l in range(net.nasm.num_ldata):
+            ref = gold[f"layer{l}"]
+            got = net.layer(l)
+            assert got.shape == ref.shape, (l, got.shape, ref.shape)
+            err = H.rel_l2(got, ref)
+            assert err <= H.REL_L2_TOL, f"layer {l} ({layers[l]['type']}): rel L2 {err:.3g}"
+        assert (net.layer(net.nasm.num_ldata - 1).argmax(1) == gold[f"layer{net.nasm.num_ldata - 1}"].argmax(1)).all()
+        if mode == api.MODE_DATAFLOW:
+            st = net.rpool.run_stats()
+            assert st == {"executed": net.nasm.num_ninst, "double_runs": 0, "aborted": 0}, st
+    finally:
+        net.close()
+
+
+@pytest.mark.parametrize("name", list(H.micro_cases()))
+def test_micro_nets_match_oracle(gpu, name):
+    """Same nets against the CPU oracle (full tensors), dataflow engine with few workgroups so that
+    tiles of several layers are in flight together."""
+    from oracle import cpu
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()[name])
+    outs = cpu.run_network(layers, tens, x, batch, seq)
+    net = H.GpuNet(cfg, tens, batch, seq, min_ninst=32, mode=api.MODE_DATAFLOW, workgroups=24)
+    print(f"case {name} tiles {net.nasm.num_ninst}", flush=True)
+    try:
+        for rep in range(3):          # re-arm and run again: results must not depend on the previous run
+            net.run(x if rep == 0 else None)
+            st = net.rpool.run_stats()
+            assert st == {"executed": net.nasm.num_ninst, "double_runs": 0, "aborted": 0}, st
+        for l in range(net.nasm.num_ldata):
+            err = H.rel_l2(net.layer(l), outs[l])
+            assert err <= H.REL_L2_TOL, f"layer {l} ({layers[l]['type']}): rel L2 {err:.3g}"
+    finally:
+        net.close()
+
+
+FULL = ["resnet50_b1", "resnet50_b32", "vgg16_b32", "bert_base_b8_s128", "gpt2_b4_s512"]
+
+
+@pytest.mark.parametrize("name", FULL)
+def test_full_config_matches_reference_summary(gpu, name):
+    """The five benchmark configurations at full size against the summaries written by the compiled
+    reference: per layer sampled relative L2, norm and sum; identical argmax per image / token."""
+    cfg, layers, tens, x, batch, seq = H.full_config(name)
+    gold = np.load(os.path.join(H.GOLDEN, f"{name}.npz"))
+    net = H.GpuNet(cfg, tens, batch, seq, mode=api.MODE_DATAFLOW)
+    print(f"config {name} tiles {net.nasm.num_ninst} edges {net.nasm.num_edges}", flush=True)
+    try:
+        net.run(x)
+        st = net.rpool.run_stats()
+        assert st == {"executed": net.nasm.num_ninst, "double_runs": 0, "aborted": 0}, st
+        worst = H.check_against_summary(net, gold, layers, name)
+        print(f"config {name}: worst sampled rel L2 {worst:.3g}", flush=True)
+    finally:
+        net.close()
+
+
+def test_co_inference_resnet50_vgg16_b16(gpu):
+    """ResNet-50 batch 16 and VGG-16 batch 16 in one ready pool / one engine launch; each must equal
+    its solo-run reference summary."""
+    nets = []
+    pool = api.RPool()
+    dse = api.DseGroup(1, api.MODE_DATAFLOW)
+    dse.set_rpool(pool)
+    try:
+        for name in ("resnet50_b16", "vgg16_b16"):
+            cfg, layers, tens, x, batch, seq = H.full_config(name)
+            net = H.GpuNet(cfg, tens, batch, seq)
+            net.rpool.destroy()            # the shared pool replaces the private one
+            net.rpool = pool
+            pool.add_nasm_raw_input(net.nasm, x)
+            nets.append((name, net, layers))
+        print("co-inference tiles", sum(n.nasm.num_ninst for _, n, _ in nets), flush=True)
+        dse.run()
+        for _, net, _ in nets:
+            dse.wait(net.nasm)
+        dse.stop()
+        st = pool.run_stats()
+        assert st == {"executed": sum(n.nasm.num_ninst for _, n, _ in nets), "double_runs": 0, "aborted": 0}, st
+        for name, net, layers in nets:
+            gold = np.load(os.path.join(H.GOLDEN, f"{name}.npz"))
+            H.check_against_summary(net, gold, layers, name)
+    finally:
+        for _, net, _ in nets:
+            net.dse.destroy()
+            net.nasm.destroy()
+            net.dnn.destroy()
+        dse.destroy()
+        pool.destroy()
