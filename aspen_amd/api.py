@@ -15,7 +15,7 @@ from typing import Optional, Sequence
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libaspen_amd.so")
+LIB_PATH = os.environ.get("ASPEN_AMD_LIB", os.path.join(_HERE, "libaspen_amd.so"))
 
 # enum values of include/aspen.h
 (OUT_W, OUT_H, OUT_C, BATCH, IN_W, IN_H, IN_C, WEIGHT_W, WEIGHT_H, SUB_C, STRIDE, PADDING, DILATION, GROUPS,
@@ -86,6 +86,7 @@ def lib() -> C.CDLL:
         "aspen_nasm_tile_range": (None, [_vp, C.c_uint, C.POINTER(C.c_uint)]),
         "aspen_rpool_run_stats": (C.c_int, [_vp, _u32p, _u32p, _u32p]),
         "aspen_rpool_num_ninst": (C.c_uint, [_vp]),
+        "aspen_rpool_profile_layers": (C.c_int, [_vp, C.c_uint, _fp]),
         # aspen_hip.h
         "aspen_hip_init": (C.c_int, []),
         "aspen_hip_last_error": (C.c_char_p, []),
@@ -232,6 +233,13 @@ class RPool:
         if lib().aspen_rpool_run_stats(self.h, C.byref(a), C.byref(b), C.byref(c)):
             raise RuntimeError("no dataflow run to report on")
         return {"executed": a.value, "double_runs": b.value, "aborted": c.value}
+
+    def profile_layers(self, num_layers: int, iters: int = 5) -> np.ndarray:
+        """Per-layer kernel time in ms (layer-launch mode, HIP events); the pool must have run once."""
+        ms = np.zeros(num_layers, dtype=np.float32)
+        if lib().aspen_rpool_profile_layers(self.h, iters, ms.ctypes.data_as(_fp)):
+            raise RuntimeError("profile_layers failed: " + lib().aspen_hip_last_error().decode())
+        return ms
 
     def destroy(self):
         if self.h:

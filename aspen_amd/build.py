@@ -26,7 +26,10 @@ def _run(cmd):
     subprocess.check_call(cmd)
 
 
-def build(verbose: bool = True) -> str:
+def build(verbose: bool = True, extra_hip_flags=(), lib_path: str = LIB, obj_dir: str = OBJ) -> str:
+    """Compiles the host C files and the HIP file and links them; extra_hip_flags / lib_path / obj_dir
+    let an experiment build a differently configured copy next to the product library."""
+    OBJ, LIB = obj_dir, lib_path
     os.makedirs(OBJ, exist_ok=True)
     inc = ["-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(HERE, "csrc", "hip"),
            "-I" + os.path.join(HERE, "csrc", "host")]
@@ -37,7 +40,7 @@ def build(verbose: bool = True) -> str:
         objs.append(o)
     for src in sorted(glob.glob(os.path.join(HERE, "csrc", "hip", "*.hip"))):
         o = os.path.join(OBJ, os.path.basename(src)[:-4] + ".o")
-        _run(["hipcc"] + HIP_FLAGS + inc + ["-c", src, "-o", o])
+        _run(["hipcc"] + HIP_FLAGS + list(extra_hip_flags) + inc + ["-c", src, "-o", o])
         objs.append(o)
     _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
          + ["-Wl,-rpath,/opt/rocm/lib", "-lm"])

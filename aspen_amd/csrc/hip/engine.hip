@@ -86,59 +86,71 @@ __global__ void __launch_bounds__ (WG_THREADS, 2) dataflow_kernel (dataflow_args
 {
     extern __shared__ __align__ (16) float smem[];
     __shared__ uint32_t s_tile;
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (;;)
     {
-        if (threadIdx.x == 0)
+        // ---- pop: wavefront 0 takes a ticket and waits for that queue slot to be filled.  The wait
+        // polls with relaxed loads (an acquire here would invalidate this XCD's L2 on every poll);
+        // one acquire fence follows once the tile is known.
+        if (wave == 0)
         {
             uint32_t id = QUEUE_EMPTY;
-            const uint32_t ticket = atomicAdd (&a.state[0], 1u);
-            if (ticket < a.num_ninst)
+            if (lane == 0)
             {
-                unsigned long long spins = 0;
-                for (;;)
+                const uint32_t ticket = atomicAdd (&a.state[0], 1u);
+                if (ticket < a.num_ninst)
                 {
-                    id = __hip_atomic_load (&a.queue[ticket], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
-                    if (id != QUEUE_EMPTY) break;
-                    if (__hip_atomic_load (&a.state[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
-                    if (++spins > a.spin_limit)
+                    unsigned long long spins = 0;
+                    for (;;)
                     {
-                        __hip_atomic_store (&a.state[3], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        break;
+                        id = __hip_atomic_load (&a.queue[ticket], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if (id != QUEUE_EMPTY) break;
+                        if (__hip_atomic_load (&a.state[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+                        if (++spins > a.spin_limit)
+                        {
+                            __hip_atomic_store (&a.state[3], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            break;
+                        }
+                        __builtin_amdgcn_s_sleep (4);
                     }
-                    __builtin_amdgcn_s_sleep (8);
                 }
+                s_tile = id;
             }
-            s_tile = id;
+            // parents' tiles were written by other XCDs: drop stale lines before anyone reads them
+            __builtin_amdgcn_fence (__ATOMIC_ACQUIRE, "agent");
         }
         __syncthreads ();
         const uint32_t id = s_tile;
         if (id == QUEUE_EMPTY) return;          // all tickets taken, or aborted
-        // make the parents' tiles (written by other XCDs) visible to every wave of this workgroup
-        __builtin_amdgcn_fence (__ATOMIC_ACQUIRE, "agent");
 
         const aspen_hip_layer_t &L = a.layers[a.ninst_layer[id]];
         run_tile (L, id - L.ninst_start, smem);
 
-        // publish this tile, then count down the children
-        __builtin_amdgcn_fence (__ATOMIC_RELEASE, "agent");
+        // ---- publish: every wave waits for its own stores, wavefront 0 then writes the tile back to
+        // memory once (release) and counts down the children with relaxed atomics; whoever takes a
+        // child's counter to zero puts it into the queue.
+        __builtin_amdgcn_fence (__ATOMIC_RELEASE, "workgroup");
         __syncthreads ();
-        const uint32_t c0 = a.child_off[id], c1 = a.child_off[id + 1];
-        for (uint32_t c = c0 + threadIdx.x; c < c1; c += WG_THREADS)
+        if (wave == 0)
         {
-            const uint32_t child = a.child_idx[c];
-            const uint32_t before = __hip_atomic_fetch_sub (&a.dep[child], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-            if (before == 1u)
+            __builtin_amdgcn_fence (__ATOMIC_RELEASE, "agent");
+            const uint32_t c0 = a.child_off[id], c1 = a.child_off[id + 1];
+            for (uint32_t c = c0 + lane; c < c1; c += 64)
             {
-                const uint32_t slot = atomicAdd (&a.state[1], 1u);
-                __hip_atomic_store (&a.queue[slot], child, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+                const uint32_t child = a.child_idx[c];
+                const uint32_t before = __hip_atomic_fetch_sub (&a.dep[child], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (before == 1u)
+                {
+                    const uint32_t slot = atomicAdd (&a.state[1], 1u);
+                    __hip_atomic_store (&a.queue[slot], child, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            if (lane == 0)
+            {
+                if (atomicAdd (&a.ran[id], 1u) != 0) atomicAdd (&a.state[4], 1u);
+                atomicAdd (&a.state[2], 1u);
             }
         }
-        if (threadIdx.x == 0)
-        {
-            if (atomicAdd (&a.ran[id], 1u) != 0) atomicAdd (&a.state[4], 1u);
-            atomicAdd (&a.state[2], 1u);
-        }
-        __syncthreads ();
     }
 }
 
@@ -357,8 +369,31 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx;
     a.dep = g->d_dep; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran;
     a.num_ninst = g->num_ninst; a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
+    CHECK (hipEventRecord (g_events[NUM_EVENTS - 2], g_stream));
     hipLaunchKernelGGL (dataflow_kernel, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);
     CHECK (hipGetLastError ());
+    CHECK (hipEventRecord (g_events[NUM_EVENTS - 1], g_stream));
+    return 0;
+}
+
+extern "C" int aspen_hip_profile_layers (aspen_hip_graph_t *g, uint32_t iters, float *ms_per_layer)
+{
+    if (!g || !ms_per_layer || iters == 0) return -1;
+    for (uint32_t l = 0; l < g->num_layers; l++)
+    {
+        const aspen_hip_layer_t &L = g->h_layers[l];
+        ms_per_layer[l] = 0.f;
+        if (L.type == INPUT_LAYER || L.num_ninst == 0) continue;
+        CHECK (hipEventRecord (g_events[NUM_EVENTS - 4], g_stream));
+        for (uint32_t i = 0; i < iters; i++)
+            hipLaunchKernelGGL (layer_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, g->d_layers, l);
+        CHECK (hipGetLastError ());
+        CHECK (hipEventRecord (g_events[NUM_EVENTS - 3], g_stream));
+        CHECK (hipEventSynchronize (g_events[NUM_EVENTS - 3]));
+        float ms = 0.f;
+        CHECK (hipEventElapsedTime (&ms, g_events[NUM_EVENTS - 4], g_events[NUM_EVENTS - 3]));
+        ms_per_layer[l] = ms / (float)iters;
+    }
     return 0;
 }
 

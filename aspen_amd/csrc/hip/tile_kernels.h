@@ -41,6 +41,12 @@ __device__ __forceinline__ float activate (float x, int act)
     }
 }
 
+__device__ __forceinline__ float4 act4 (float4 v, int act)
+{
+    v.x = activate (v.x, act); v.y = activate (v.y, act); v.z = activate (v.z, act); v.w = activate (v.w, act);
+    return v;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Operand loaders.  A loader fetches this thread's share of one GEMM_BK-wide K slice into registers
 // (load) and later parks it in LDS as [row][LDS_ROW] (store), so the global loads of slice i+1 fly
@@ -159,16 +165,23 @@ struct TransLoader64
 // consecutive output channels of one output column: stores are 128-byte coalesced.
 // LDS is double buffered: one barrier per K slice.
 // ---------------------------------------------------------------------------------------------
+// LDS-only barrier: waits for this wave's LDS traffic, not for global loads still in flight.
+__device__ __forceinline__ void lds_barrier ()
+{
+    asm volatile ("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 template <int BM, int BN, int WM, int WN, class ALoader, class BLoader>
 __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kiters, float *smem,
-    floatx16 (&acc)[BN / WN / 32][BM / WM / 32], int ar, int br)
+    floatx16 (&acc)[BN / WN / 32][BM / WM / 32])
 {
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     constexpr int STAGE = (BM + BN) * LDS_ROW;
+    constexpr int KK = GEMM_BK / 8;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);
-    const uint32_t frag = (lane & 31) * LDS_ROW + (lane >> 5) * 4;
-    (void)ar; (void)br;
+    const uint32_t afrag = wm0 * LDS_ROW + (lane & 31) * LDS_ROW + (lane >> 5) * 4;
+    const uint32_t bfrag = BM * LDS_ROW + wn0 * LDS_ROW + (lane & 31) * LDS_ROW + (lane >> 5) * 4;
 
     #pragma unroll
     for (int i = 0; i < TN; i++)
@@ -180,38 +193,50 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kiters,
     float4 areg[ALoader::R], breg[BLoader::R];
     al.load (0, areg); bl.load (0, breg);
     al.store (smem, areg); bl.store (smem + BM * LDS_ROW, breg);
-    __syncthreads ();
+    if (kiters > 1) { al.load (1, areg); bl.load (1, breg); }
+    lds_barrier ();
 
     for (int it = 0; it < kiters; it++)
     {
-        float *As = smem + (it & 1) * STAGE, *Bs = As + BM * LDS_ROW;
+        const float *S = smem + (it & 1) * STAGE;
+        float *Snext = smem + ((it + 1) & 1) * STAGE;
         const bool more = it + 1 < kiters;
-        if (more) { al.load (it + 1, areg); bl.load (it + 1, breg); }
+        // fragments of sub-step kk+1 are fetched from LDS while the matrix cores work on sub-step kk
+        float4 af[2][TM], bf[2][TN];
         #pragma unroll
-        for (int kk = 0; kk < GEMM_BK / 8; kk++)
+        for (int j = 0; j < TM; j++) af[0][j] = ld4 (S + afrag + j * 32 * LDS_ROW);
+        #pragma unroll
+        for (int i = 0; i < TN; i++) bf[0][i] = ld4 (S + bfrag + i * 32 * LDS_ROW);
+        #pragma unroll
+        for (int kk = 0; kk < KK; kk++)
         {
-            float4 af[TM], bf[TN];
-            #pragma unroll
-            for (int j = 0; j < TM; j++) af[j] = ld4 (As + (wm0 + j * 32) * LDS_ROW + frag + kk * 8);
-            #pragma unroll
-            for (int i = 0; i < TN; i++) bf[i] = ld4 (Bs + (wn0 + i * 32) * LDS_ROW + frag + kk * 8);
+            const int cur = kk & 1, nxt = cur ^ 1;
+            if (kk + 1 < KK)
+            {
+                #pragma unroll
+                for (int j = 0; j < TM; j++) af[nxt][j] = ld4 (S + afrag + j * 32 * LDS_ROW + (kk + 1) * 8);
+                #pragma unroll
+                for (int i = 0; i < TN; i++) bf[nxt][i] = ld4 (S + bfrag + i * 32 * LDS_ROW + (kk + 1) * 8);
+            }
+            else if (more)
+            {
+                // the next K slice (in registers since the previous iteration) goes to the other stage,
+                // overlapping with the last group of MFMAs; then its successor is requested from memory
+                al.store (Snext, areg); bl.store (Snext + BM * LDS_ROW, breg);
+                if (it + 2 < kiters) { al.load (it + 2, areg); bl.load (it + 2, breg); }
+            }
             #pragma unroll
             for (int i = 0; i < TN; i++)
                 #pragma unroll
                 for (int j = 0; j < TM; j++)
                 {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[i].x, af[j].x, acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[i].y, af[j].y, acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[i].z, af[j].z, acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[i].w, af[j].w, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[cur][i].x, af[cur][j].x, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[cur][i].y, af[cur][j].y, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[cur][i].z, af[cur][j].z, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[cur][i].w, af[cur][j].w, acc[i][j], 0, 0, 0);
                 }
         }
-        if (more)
-        {
-            float *An = smem + ((it + 1) & 1) * STAGE;
-            al.store (An, areg); bl.store (An + BM * LDS_ROW, breg);
-        }
-        __syncthreads ();
+        lds_barrier ();
     }
 }
 
@@ -234,42 +259,57 @@ __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, ui
     {
         RowLoader<BN> bl;
         bl.init (L.in0, n0, L.N - 1, L.ld0, tid);
-        gemm_core<BM, BN, WM, WN> (al, bl, kiters, smem, acc, 0, 0);
+        gemm_core<BM, BN, WM, WN> (al, bl, kiters, smem, acc);
     }
     else
     {
         ConvLoader<BN> bl;
         bl.init (L, n0, tid);
-        gemm_core<BM, BN, WM, WN> (al, bl, kiters, smem, acc, 0, 0);
+        gemm_core<BM, BN, WM, WN> (al, bl, kiters, smem, acc);
     }
     const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);
     const int act = L.act;
+    // Epilogue through LDS (free after the last K slice): the raw accumulators are parked as
+    // [column][channel]; a rolled loop then adds the bias, applies the activation and writes 128-bit
+    // pieces, so a wavefront covers whole 512-byte (BM = 128) / 256-byte (BM = 64) runs of a column.
+    // Keeping the activation out of the unrolled accumulator loops keeps the kernel's code small.
+    constexpr int TROW = BM + 8;            // (4 * TROW) % 64 == 32: the two half-waves hit disjoint banks
     #pragma unroll
     for (int j = 0; j < TM; j++)
-    {
-        const uint32_t m = m0 + wm0 + 32 * j + (lane & 31);
-        if (m >= L.M) continue;
-        const float b = L.bias ? L.bias[m] : 0.f;
         #pragma unroll
         for (int i = 0; i < TN; i++)
             #pragma unroll
             for (int v = 0; v < 16; v++)
-            {
-                const uint32_t n = n0 + ACC_N (wn0, i, v, lane);
-                if (n < L.N) L.out[(size_t)n * L.ld + m] = activate (acc[i][j][v] + b, act);
-            }
+                smem[ACC_N (wn0, i, v, lane) * TROW + wm0 + 32 * j + (lane & 31)] = acc[i][j][v];
+    __syncthreads ();
+    constexpr int C4 = BM / 4;
+    const uint32_t rows = min ((uint32_t)BN, L.N - n0);
+    const uint32_t mrem = L.M - m0;         // channels of this tile that exist (may exceed BM)
+    const uint32_t c = (tid % C4) * 4;      // WG_THREADS is a multiple of C4: a thread keeps its channels
+    if (c < mrem)
+    {
+        float4 b = make_float4 (0.f, 0.f, 0.f, 0.f);
+        if (L.bias)
+        {
+            if (c + 4 <= mrem) b = ld4 (L.bias + m0 + c);
+            else { b.x = L.bias[m0 + c]; if (c + 1 < mrem) b.y = L.bias[m0 + c + 1]; if (c + 2 < mrem) b.z = L.bias[m0 + c + 2]; }
+        }
+        for (uint32_t r = tid / C4; r < rows; r += WG_THREADS / C4)
+        {
+            float4 v = ld4 (smem + r * TROW + c);
+            v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
+            v = act4 (v, act);
+            float *o = L.out + (size_t)(n0 + r) * L.ld + m0 + c;
+            if (c + 4 <= mrem) st4 (o, v);
+            else { o[0] = v.x; if (c + 1 < mrem) o[1] = v.y; if (c + 2 < mrem) o[2] = v.z; }
+        }
     }
+    __syncthreads ();
 }
 
 // ---------------------------------------------------------------------------------------------
 // Bandwidth tiles: 128-bit accesses, a tile = tile_n whole columns.
 // ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ float4 act4 (float4 v, int act)
-{
-    v.x = activate (v.x, act); v.y = activate (v.y, act); v.z = activate (v.z, act); v.w = activate (v.w, act);
-    return v;
-}
-
 __device__ __forceinline__ void tile_residual (const aspen_hip_layer_t &L, uint32_t tn)
 {
     const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N), M4 = L.ld >> 2;
@@ -416,7 +456,7 @@ __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, ui
         floatx16 acc[TN][TM];
         RowLoader<BM> al; al.init (Kmat, k0, S - 1, L.ld1, tid);
         RowLoader<BN> bl; bl.init (Q, q0, S - 1, L.ld0, tid);
-        gemm_core<BM, BN, WM, WN> (al, bl, kiters, smem, acc, 0, 0);
+        gemm_core<BM, BN, WM, WN> (al, bl, kiters, smem, acc);
         #pragma unroll
         for (int j = 0; j < TM; j++)
         {
@@ -483,7 +523,7 @@ __device__ __forceinline__ void tile_v_attention (const aspen_hip_layer_t &L, ui
     floatx16 acc[TN][TM];
     TransLoader64 al; al.init (V, L.ld1, L.tile_m, S, tid);
     RowLoader<BN> bl; bl.init (P, q0, S - 1, L.ld0, tid);   // P's stride is a multiple of 32 with zero padding
-    gemm_core<BM, BN, WM, WN> (al, bl, (int)((S + GEMM_BK - 1) / GEMM_BK), smem, acc, 0, 0);
+    gemm_core<BM, BN, WM, WN> (al, bl, (int)((S + GEMM_BK - 1) / GEMM_BK), smem, acc);
     const uint32_t mm = wm0 + (lane & 31);
     if (mm < L.tile_m)
         #pragma unroll

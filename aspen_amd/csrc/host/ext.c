@@ -46,6 +46,12 @@ int aspen_rpool_run_stats (rpool_t *rp, uint32_t *executed, uint32_t *double_run
     return aspen_hip_dataflow_stats (rp->graph, executed, double_runs, aborted);
 }
 
+int aspen_rpool_profile_layers (rpool_t *rp, unsigned int iters, float *ms)
+{
+    if (rp == NULL || rp->graph == NULL) return -1;
+    return aspen_hip_profile_layers (rp->graph, iters, ms);
+}
+
 unsigned int aspen_rpool_num_ninst (rpool_t *rp)
 {
     unsigned int n = 0;

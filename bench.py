@@ -1,0 +1,225 @@
+#!/usr/bin/env python3
+"""Benchmark of the tiled-dataflow hot path on one MI355X.
+
+A step is one inference pass over one resident batch in the reference's own loop
+(reference main.c:116-123): rpool_reset_queue -> rpool_reset_nasm -> dse_group_run ->
+dse_wait_for_nasm_completion -> dse_group_stop.  Inputs and weights are in HBM before the timed
+region starts.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload resnet50_b32] [--mode dataflow|layers]
+"""
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3      # MI355X dense fp32 matrix peak
+PEAK_HBM_GBS = 8000.0
+
+# algorithmic GEMM-class flops per unit (2*M*N*K with the reference's K: padding taps counted, full
+# S x S attention): per image for the vision nets, per token for the transformers
+FLOP_PER_UNIT = {
+    "resnet50": 8.178369e9, "vgg16": 3.069326e10 + 2.47267e8,
+    "bert_base": 1.7459e8, "gpt2": 1.8877e8,
+}
+WORKLOADS = {
+    # name: (configs, unit, units per step, flop key per config)
+    "resnet50_b32": (["resnet50_b32"], "img/s", 32),
+    "resnet50_b1": (["resnet50_b1"], "img/s", 1),
+    "vgg16_b32": (["vgg16_b32"], "img/s", 32),
+    "co_resnet50_vgg16_b16": (["resnet50_b16", "vgg16_b16"], "img/s", 32),
+    "bert_base_b8_s128": (["bert_base_b8_s128"], "tokens/s", 8 * 128),
+    "gpt2_b4_s512": (["gpt2_b4_s512"], "tokens/s", 4 * 512),
+}
+
+
+def gemm_flops(nasm, api):
+    total = 0
+    for l in range(nasm.num_ldata):
+        i = nasm.info(l)
+        if i["type"] in (api.CONV_LAYER, api.FC_LAYER, api.MATMUL_LAYER, api.K_ATTENTION_LAYER, api.V_ATTENTION_LAYER):
+            total += i["flops"]
+    return total
+
+
+def cpu_baseline(cfgname, budget_s=20.0):
+    """Reference tile kernels (oracle/_ref, compiled from the reference's sources) timed on this host's
+    cores; falls back to the oracle port when that library is absent.  Bounded sample of the workload."""
+    from aspen_amd import models as M
+    gen, style, batch, seq, seed, kind = M.CONFIGS[cfgname]
+    threads = min(16, os.cpu_count() or 1)
+    os.environ.setdefault("OMP_NUM_THREADS", str(threads))
+    cfg = gen()
+    layers = M.parse_cfg(cfg)
+    tens = M.synth_weights(layers, seed, style)
+    x = M.synth_input(layers, seed, batch, seq, kind or "token_ids")
+    units = batch * (seq if seq else 1)
+    unit = "tokens/s" if seq else "img/s"
+    try:
+        from oracle import ref
+        if not ref.available():
+            raise OSError("oracle/_ref not built")
+        wp = tempfile.mktemp(suffix=".bin")
+        M.write_aspen_data(wp, tens)
+        net = ref.RefNet(cfg, wp, batch, seq, threads=threads)
+        os.unlink(wp)
+        net.set_input(x)
+        t0 = time.time()
+        net.forward()                         # warm-up, also gives the per-pass cost
+        one = time.time() - t0
+        iters = int(max(1, min(10, budget_s / max(one, 1e-3))))
+        sec = net.time_forward(iters)
+        net.close()
+        return {"value": units / sec, "unit": unit, "cores": threads, "kind": "reference",
+                "sample": f"{cfgname}: {iters} full passes after 1 warm-up, reference tiled_* kernels swept layer by "
+                          f"layer with {threads} OpenMP threads (tile dependency discovery skipped)",
+                "ms_per_step": sec * 1e3}
+    except (OSError, RuntimeError) as exc:
+        from oracle import cpu
+        t0 = time.time()
+        cpu.run_network(layers, tens, x, batch, seq, keep_all=False)
+        sec = time.time() - t0
+        return {"value": units / sec, "unit": unit, "cores": threads, "kind": "port",
+                "sample": f"{cfgname}: 1 full pass of the oracle port ({exc})", "ms_per_step": sec * 1e3}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="resnet50_b32", choices=list(WORKLOADS))
+    ap.add_argument("--mode", default="dataflow", choices=["dataflow", "layers"])
+    ap.add_argument("--min-ninst", type=int, default=512)
+    ap.add_argument("--workgroups", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--layer-profile", action="store_true", help="also time every layer's kernel (layer-launch mode)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
+        sys.exit(2)
+
+    from aspen_amd import api, models as M
+    L = api.lib()
+    if L.aspen_hip_init() != 0:
+        print("bench.py: no HIP device: " + L.aspen_hip_last_error().decode(), file=sys.stderr)
+        sys.exit(1)
+    dev = api.device_info()
+    cfgs, unit, units_per_step = WORKLOADS[args.workload]
+
+    pool = api.RPool()
+    dse = api.DseGroup(1, api.MODE_DATAFLOW if args.mode == "dataflow" else api.MODE_LAYERS, args.workgroups)
+    dse.set_rpool(pool)
+    nets = []
+    for name in cfgs:
+        cfg, layers, tens, x, batch, seq = M.make_config(name)
+        wp = tempfile.mktemp(suffix=".bin")
+        M.write_aspen_data(wp, tens)
+        dnn = api.Dnn(cfg, wp)
+        os.unlink(wp)
+        del tens
+        nasm = api.Nasm(dnn, batch, seq, args.min_ninst)
+        pool.add_nasm_raw_input(nasm, x)
+        nets.append((name, dnn, nasm, layers))
+    flops = sum(gemm_flops(n, api) for _, _, n, _ in nets)
+    tiles = sum(n.num_ninst for _, _, n, _ in nets)
+
+    def step():
+        pool.reset_queue()
+        for _, _, n, _ in nets:
+            pool.reset_nasm(n)
+        dse.run()
+        for _, _, n, _ in nets:
+            dse.wait(n)
+        dse.stop()
+
+    # first run happens with the freshly added input (no reset), then warm-up
+    dse.run()
+    for _, _, n, _ in nets:
+        dse.wait(n)
+    dse.stop()
+    for _ in range(args.warmup):
+        step()
+    L.aspen_hip_sync()
+    kernel_ms = []
+    ms = api.C.c_float()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+        if args.mode == "dataflow" and L.aspen_hip_event_elapsed_ms(14, 15, api.C.byref(ms)) == 0:
+            kernel_ms.append(ms.value)
+    L.aspen_hip_sync()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    value = units_per_step * args.steps / dt
+
+    out = {
+        "metric": "ResNet-50 fp32 img/s at batch 1/32 on 1 MI355X; conv-tile MFMA util vs FP32 peak",
+        "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": args.workload, "engine": args.mode, "tiles_per_step": tiles,
+                   "min_ninst_per_ldata": args.min_ninst, "device": dev["name"], "compute_units": dev["compute_units"]},
+    }
+    if args.mode == "dataflow" and kernel_ms:
+        k_ms = float(np.mean(kernel_ms))
+        ach = flops / (k_ms * 1e-3) / 1e12
+        out["roofline"] = {"bound": "mfma", "kernel": "dataflow_kernel", "achieved": ach, "peak": PEAK_FP32_MFMA_TFLOPS,
+                           "unit": "TFLOP/s", "frac": ach / PEAK_FP32_MFMA_TFLOPS, "traffic": None,
+                           "flops_per_launch": flops, "kernel_ms": k_ms}
+    else:
+        ach = flops / (ms_per_step * 1e-3) / 1e12
+        out["roofline"] = {"bound": "mfma", "kernel": "layer_kernel (all layers of one step)", "achieved": ach,
+                           "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": ach / PEAK_FP32_MFMA_TFLOPS,
+                           "traffic": None, "flops_per_launch": flops, "kernel_ms": ms_per_step}
+
+    if args.layer_profile:
+        # conv-tile MFMA utilisation and bandwidth of the elementwise tiles, one kernel per layer
+        nl = sum(n.num_ldata for _, _, n, _ in nets)
+        lms = pool.profile_layers(nl, 5)
+        per_type, base = {}, 0
+        for name, _, n, _ in nets:
+            for l in range(n.num_ldata):
+                i = n.info(l)
+                t = api.LAYER_TYPE_NAMES[i["type"]]
+                d = per_type.setdefault(t, {"ms": 0.0, "flops": 0, "bytes": 0})
+                d["ms"] += float(lms[base + l])
+                d["flops"] += i["flops"] if t in ("conv", "fc", "matmul", "attn_k", "attn_v") else 0
+                if t == "residual":
+                    d["bytes"] += 12 * i["H"] * i["W"]
+                elif t == "layernorm" or t == "softmax":
+                    d["bytes"] += 8 * i["H"] * i["W"]
+            base += n.num_ldata
+        for t, d in per_type.items():
+            if d["flops"]:
+                d["tflops"] = d["flops"] / max(d["ms"], 1e-9) / 1e9
+                d["mfma_util"] = d["tflops"] / PEAK_FP32_MFMA_TFLOPS
+            if d["bytes"]:
+                d["gbs"] = d["bytes"] / max(d["ms"], 1e-9) / 1e6
+                d["hbm_frac"] = d["gbs"] / PEAK_HBM_GBS
+        out["layer_profile"] = per_type
+        out["layer_ms"] = [round(float(v), 4) for v in lms]
+
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfgs[0])
+
+    for _, dnn, nasm, _ in nets:
+        pass
+    dse.destroy()
+    for _, dnn, nasm, _ in nets:
+        nasm.destroy()
+    pool.destroy()
+    for _, dnn, nasm, _ in nets:
+        dnn.destroy()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

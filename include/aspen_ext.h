@@ -35,6 +35,9 @@ void aspen_nasm_tile_range (nasm_t *nasm, unsigned int ninst_idx, unsigned int *
 /* counters of the last dataflow run of the pool: tiles executed, tiles executed more than once,
    abort flag (a wait on the ready queue hit its spin limit).  Returns 0 on success. */
 int aspen_rpool_run_stats (rpool_t *rpool, uint32_t *executed, uint32_t *double_runs, uint32_t *aborted);
+/* per-layer kernel time (ms) of the pool's merged graph in layer-launch mode, averaged over iters;
+   ms must hold one float per layer of every attached nasm, in attachment order */
+int aspen_rpool_profile_layers (rpool_t *rpool, unsigned int iters, float *ms);
 /* tiles in the pool's merged graph */
 unsigned int aspen_rpool_num_ninst (rpool_t *rpool);
 

@@ -110,7 +110,13 @@ int aspen_hip_idle (void);
 int aspen_hip_dataflow_stats (aspen_hip_graph_t *graph, uint32_t *executed, uint32_t *double_runs, uint32_t *abort_flag);
 
 /* ---- timing ------------------------------------------------------------------------------------- */
-/* HIP events on the library's stream: record into slot [0,16), elapsed between two recorded slots. */
+/* Average duration of each layer's kernel over `iters` back-to-back launches (HIP events around the
+   launches of one layer); ms_per_layer holds one float per layer, 0 for the input layer.  The layers
+   run in index order, so the activations are those of a real forward pass. */
+int aspen_hip_profile_layers (aspen_hip_graph_t *graph, uint32_t iters, float *ms_per_layer);
+/* HIP events on the library's stream: record into slot [0,12), elapsed between two recorded slots.
+   Slots 14 and 15 are recorded by aspen_hip_run_dataflow right before and after the persistent
+   kernel, so elapsed(14, 15) is that kernel's duration. */
 int aspen_hip_event_record (int slot);
 int aspen_hip_event_elapsed_ms (int slot_begin, int slot_end, float *ms);
 
