@@ -96,6 +96,7 @@ def lib() -> C.CDLL:
         "aspen_hip_h2d": (C.c_int, [_vp, _vp, C.c_size_t]),
         "aspen_hip_d2h": (C.c_int, [_vp, _vp, C.c_size_t]),
         "aspen_hip_sync": (C.c_int, []),
+        "aspen_hip_set_flags": (None, [C.c_uint32]),
         "aspen_hip_idle": (C.c_int, []),
         "aspen_hip_event_record": (C.c_int, [C.c_int]),
         "aspen_hip_event_elapsed_ms": (C.c_int, [C.c_int, C.c_int, _fp]),

@@ -14,6 +14,12 @@
 #include "tile_kernels.h"
 
 #define QUEUE_EMPTY 0xffffffffu
+#define ST_HEAD 0
+#define ST_TAIL 32
+#define ST_DONE 64
+#define ST_ABORT 96
+#define ST_TWICE 128
+#define ST_WORDS 160
 #define NUM_EVENTS 16
 #define DEFAULT_SPIN_LIMIT (1ull << 26)
 
@@ -25,7 +31,8 @@ struct aspen_hip_graph_t
     uint32_t *d_ninst_layer, *d_num_parents, *d_child_off, *d_child_idx, *d_roots;
     uint32_t *d_dep;        // remaining-parent counters, re-armed before every dataflow run
     uint32_t *d_queue;      // ready queue: slot t is written once, by whoever makes a tile ready
-    uint32_t *d_state;      // [0] pop tickets, [1] push cursor, [2] tiles done, [3] abort flag, [4] double-run count
+    uint32_t *d_state;      // one counter per 128-byte line: [ST_HEAD] pop tickets, [ST_TAIL] push cursor, [ST_DONE] tiles done,
+                            // [ST_ABORT] abort flag, [ST_TWICE] tiles executed more than once
     uint32_t *d_ran;        // per-tile execution count (sanity: every tile exactly once)
 };
 
@@ -34,6 +41,7 @@ static hipEvent_t g_events[NUM_EVENTS];
 static int g_inited = 0;
 static int g_num_cu = 0;
 static char g_err[512] = "";
+static uint32_t g_flags = 0;
 
 static int fail (hipError_t e, const char *what)
 {
@@ -56,7 +64,11 @@ __global__ void __launch_bounds__ (WG_THREADS, 2) layer_kernel (const aspen_hip_
     const uint32_t nt = gridDim.x, bid = blockIdx.x;
     const uint32_t xcd = bid & 7, local = bid >> 3, chunk = nt >> 3, rem = nt & 7;
     const uint32_t t = xcd * chunk + (xcd < rem ? xcd : rem) + local;
-    run_tile (L, t, smem);
+#ifdef EXP_LAYER_COH
+    run_tile<true> (L, t, smem);
+#else
+    run_tile<false> (L, t, smem);
+#endif
 }
 
 // Re-arm: counters back to the parent counts, queue emptied and seeded with the roots.
@@ -70,7 +82,7 @@ __global__ void arm_kernel (uint32_t *dep, const uint32_t *num_parents, uint32_t
         queue[i] = i < num_roots ? roots[i] : QUEUE_EMPTY;
         ran[i] = 0;
     }
-    if (i == 0) { state[0] = 0; state[1] = num_roots; state[2] = 0; state[3] = 0; state[4] = 0; }
+    if (i == 0) { state[ST_HEAD] = 0; state[ST_TAIL] = num_roots; state[ST_DONE] = 0; state[ST_ABORT] = 0; state[ST_TWICE] = 0; }
 }
 
 struct dataflow_args_t
@@ -79,61 +91,67 @@ struct dataflow_args_t
     const uint32_t *ninst_layer, *child_off, *child_idx;
     uint32_t *dep, *queue, *state, *ran;
     uint32_t num_ninst;
+    uint32_t flags;                 // ASPEN_HIP_FLAG_*
     unsigned long long spin_limit;
 };
 
+// Waits until queue slot `ticket` holds a tile and returns it; QUEUE_EMPTY when all tickets are
+// taken or the run was aborted.  The wait polls with relaxed device-scope loads (an acquire here
+// would invalidate this XCD's L2 on every poll).
+__device__ __forceinline__ uint32_t wait_for_slot (const dataflow_args_t &a, uint32_t ticket)
+{
+    if (ticket >= a.num_ninst) return QUEUE_EMPTY;
+    unsigned long long spins = 0;
+    for (;;)
+    {
+        const uint32_t id = __hip_atomic_load (&a.queue[ticket], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (id != QUEUE_EMPTY) return id;
+        ++spins;
+        if ((spins & 63) == 0 && __hip_atomic_load (&a.state[ST_ABORT], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return QUEUE_EMPTY;
+        if (spins > a.spin_limit)
+        {
+            __hip_atomic_store (&a.state[ST_ABORT], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return QUEUE_EMPTY;
+        }
+        __builtin_amdgcn_s_sleep (2);
+    }
+}
+
+// Persistent workgroup = one scheduling engine (the reference's DSE thread, src/dse.c:5-108).
+// Wavefront 1 pops: it draws the ticket for the NEXT tile before the current tile starts, so the
+// round trip of that atomic hides behind the tile, and resolves the ticket to a tile while
+// wavefront 0 publishes the finished tile (dependency countdown of its children, push of those
+// that became ready).  No cache write-back / invalidate is needed anywhere: tiles access
+// activations with device-scope coherent instructions (ActView<true>).
 __global__ void __launch_bounds__ (WG_THREADS, 2) dataflow_kernel (dataflow_args_t a)
 {
     extern __shared__ __align__ (16) float smem[];
-    __shared__ uint32_t s_tile;
+    __shared__ uint32_t s_tile[2];
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (;;)
+    const bool popper = wave == 1 && lane == 0;
+    uint32_t next_ticket = 0;
+    if (popper)
     {
-        // ---- pop: wavefront 0 takes a ticket and waits for that queue slot to be filled.  The wait
-        // polls with relaxed loads (an acquire here would invalidate this XCD's L2 on every poll);
-        // one acquire fence follows once the tile is known.
-        if (wave == 0)
-        {
-            uint32_t id = QUEUE_EMPTY;
-            if (lane == 0)
-            {
-                const uint32_t ticket = atomicAdd (&a.state[0], 1u);
-                if (ticket < a.num_ninst)
-                {
-                    unsigned long long spins = 0;
-                    for (;;)
-                    {
-                        id = __hip_atomic_load (&a.queue[ticket], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        if (id != QUEUE_EMPTY) break;
-                        if (__hip_atomic_load (&a.state[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
-                        if (++spins > a.spin_limit)
-                        {
-                            __hip_atomic_store (&a.state[3], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                            break;
-                        }
-                        __builtin_amdgcn_s_sleep (4);
-                    }
-                }
-                s_tile = id;
-            }
-            // parents' tiles were written by other XCDs: drop stale lines before anyone reads them
-            __builtin_amdgcn_fence (__ATOMIC_ACQUIRE, "agent");
-        }
+        s_tile[0] = wait_for_slot (a, atomicAdd (&a.state[ST_HEAD], 1u));
+        next_ticket = atomicAdd (&a.state[ST_HEAD], 1u);
+    }
+    for (uint32_t it = 0;; it++)
+    {
         __syncthreads ();
-        const uint32_t id = s_tile;
+        const uint32_t id = s_tile[it & 1];
         if (id == QUEUE_EMPTY) return;          // all tickets taken, or aborted
 
         const aspen_hip_layer_t &L = a.layers[a.ninst_layer[id]];
-        run_tile (L, id - L.ninst_start, smem);
+        if (!(a.flags & ASPEN_HIP_FLAG_SKIP_TILES))
+            run_tile<true> (L, id - L.ninst_start, smem);
 
-        // ---- publish: every wave waits for its own stores, wavefront 0 then writes the tile back to
-        // memory once (release) and counts down the children with relaxed atomics; whoever takes a
-        // child's counter to zero puts it into the queue.
+        // every wave waits until its (write-through, device-coherent) stores have been acknowledged
         __builtin_amdgcn_fence (__ATOMIC_RELEASE, "workgroup");
         __syncthreads ();
         if (wave == 0)
         {
-            __builtin_amdgcn_fence (__ATOMIC_RELEASE, "agent");
+            // publish: count down the children with relaxed device-scope atomics; whoever takes a
+            // child's counter to zero puts it into the ready queue
             const uint32_t c0 = a.child_off[id], c1 = a.child_off[id + 1];
             for (uint32_t c = c0 + lane; c < c1; c += 64)
             {
@@ -141,15 +159,21 @@ __global__ void __launch_bounds__ (WG_THREADS, 2) dataflow_kernel (dataflow_args
                 const uint32_t before = __hip_atomic_fetch_sub (&a.dep[child], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 if (before == 1u)
                 {
-                    const uint32_t slot = atomicAdd (&a.state[1], 1u);
+                    const uint32_t slot = atomicAdd (&a.state[ST_TAIL], 1u);
                     __hip_atomic_store (&a.queue[slot], child, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
-            if (lane == 0)
+            if (lane == 0 && (a.flags & ASPEN_HIP_FLAG_COUNT_TILES))
             {
-                if (atomicAdd (&a.ran[id], 1u) != 0) atomicAdd (&a.state[4], 1u);
-                atomicAdd (&a.state[2], 1u);
+                if (atomicAdd (&a.ran[id], 1u) != 0) atomicAdd (&a.state[ST_TWICE], 1u);
+                atomicAdd (&a.state[ST_DONE], 1u);
             }
+        }
+        else if (popper)
+        {
+            // pop: resolve the ticket drawn one tile ago, draw the one after it
+            s_tile[(it + 1) & 1] = wait_for_slot (a, next_ticket);
+            next_ticket = atomicAdd (&a.state[ST_HEAD], 1u);
         }
     }
 }
@@ -320,7 +344,7 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     g->d_dep = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
     g->d_queue = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
     g->d_ran = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
-    g->d_state = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * 16);
+    g->d_state = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * ST_WORDS);
     if (!g->d_layers || !g->d_ninst_layer || !g->d_num_parents || !g->d_child_off || !g->d_child_idx || !g->d_roots
         || !g->d_dep || !g->d_queue || !g->d_ran || !g->d_state)
     {
@@ -368,7 +392,7 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     dataflow_args_t a;
     a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx;
     a.dep = g->d_dep; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran;
-    a.num_ninst = g->num_ninst; a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
+    a.num_ninst = g->num_ninst; a.flags = g_flags; a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
     CHECK (hipEventRecord (g_events[NUM_EVENTS - 2], g_stream));
     hipLaunchKernelGGL (dataflow_kernel, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);
     CHECK (hipGetLastError ());
@@ -397,6 +421,8 @@ extern "C" int aspen_hip_profile_layers (aspen_hip_graph_t *g, uint32_t iters, f
     return 0;
 }
 
+extern "C" void aspen_hip_set_flags (uint32_t flags) { g_flags = flags; }
+
 extern "C" int aspen_hip_sync (void)
 {
     if (aspen_hip_init ()) return -1;
@@ -413,11 +439,11 @@ extern "C" int aspen_hip_idle (void)
 extern "C" int aspen_hip_dataflow_stats (aspen_hip_graph_t *g, uint32_t *executed, uint32_t *double_runs, uint32_t *abort_flag)
 {
     if (!g) return -1;
-    uint32_t st[8];
+    uint32_t st[ST_WORDS];
     if (aspen_hip_d2h (st, g->d_state, sizeof (st))) return -1;
-    if (executed) *executed = st[2];
-    if (abort_flag) *abort_flag = st[3];
-    if (double_runs) *double_runs = st[4];
+    if (executed) *executed = st[ST_DONE];
+    if (abort_flag) *abort_flag = st[ST_ABORT];
+    if (double_runs) *double_runs = st[ST_TWICE];
     return 0;
 }
 

@@ -25,6 +25,46 @@ typedef float floatx16 __attribute__ ((ext_vector_type (16)));
 __device__ __forceinline__ float4 ld4 (const float *p) { return *reinterpret_cast<const float4 *> (p); }
 __device__ __forceinline__ void st4 (float *p, float4 v) { *reinterpret_cast<float4 *> (p) = v; }
 
+// View of one activation matrix.  COH = true: every access is device-scope coherent (buffer
+// instructions with sc1: they bypass the per-CU L1 and the per-XCD L2, which are not coherent across
+// the 8 XCDs), so tiles produced and consumed inside one persistent kernel need no cache
+// write-back / invalidate between them, and the weights stay cached.  COH = false: plain cached
+// accesses for the one-launch-per-layer path, where kernel boundaries provide coherence.
+// Offsets are in floats from the start of the matrix; the descriptor bounds-checks them in hardware
+// (out-of-range loads return 0, out-of-range stores are dropped).
+typedef uint32_t u32x4 __attribute__ ((ext_vector_type (4)));
+#define CPOL_SC1 16
+template <bool COH> struct ActView
+{
+    const float *base;
+    __amdgpu_buffer_rsrc_t rsrc;
+    __device__ __forceinline__ void init (const float *p, uint32_t columns, uint32_t ld)
+    {
+        base = p;
+        if (COH) rsrc = __builtin_amdgcn_make_buffer_rsrc ((void *)p, 0, (int)(columns * ld * 4u + 256u), 0x00020000);
+    }
+    __device__ __forceinline__ float4 ld4 (uint32_t off) const
+    {
+        if (COH) return __builtin_bit_cast (float4, __builtin_amdgcn_raw_buffer_load_b128 (rsrc, (int)(off * 4u), 0, CPOL_SC1));
+        return *reinterpret_cast<const float4 *> (base + off);
+    }
+    __device__ __forceinline__ float ld1 (uint32_t off) const
+    {
+        if (COH) return __builtin_bit_cast (float, __builtin_amdgcn_raw_buffer_load_b32 (rsrc, (int)(off * 4u), 0, CPOL_SC1));
+        return base[off];
+    }
+    __device__ __forceinline__ void st4 (uint32_t off, float4 v) const
+    {
+        if (COH) __builtin_amdgcn_raw_buffer_store_b128 (__builtin_bit_cast (u32x4, v), rsrc, (int)(off * 4u), 0, CPOL_SC1);
+        else *reinterpret_cast<float4 *> (const_cast<float *> (base) + off) = v;
+    }
+    __device__ __forceinline__ void st1 (uint32_t off, float v) const
+    {
+        if (COH) __builtin_amdgcn_raw_buffer_store_b32 (__builtin_bit_cast (uint32_t, v), rsrc, (int)(off * 4u), 0, CPOL_SC1);
+        else const_cast<float *> (base)[off] = v;
+    }
+};
+
 __device__ __forceinline__ float activate (float x, int act)
 {
     switch (act)
@@ -82,19 +122,50 @@ template <int ROWS> struct RowLoader
     }
 };
 
+// Same for rows of an activation matrix (matmul / 1x1-conv operand, Q, K and probability rows).
+template <int ROWS, bool COH> struct ActRowLoader
+{
+    static constexpr int R = ROWS / 32;
+    ActView<COH> view;
+    uint32_t off[R];
+    uint32_t chunk, row0;
+    // rows first_row.. of the view (clamped to max_row), starting at float `col0` of each row
+    __device__ __forceinline__ void init (const ActView<COH> &v, uint32_t first_row, uint32_t max_row, uint32_t ld, uint32_t col0, uint32_t tid)
+    {
+        view = v; chunk = tid & 7; row0 = tid >> 3;
+        #pragma unroll
+        for (int i = 0; i < R; i++)
+        {
+            uint32_t r = first_row + row0 + 32 * i;
+            r = r < max_row ? r : max_row;
+            off[i] = r * ld + col0 + chunk * 4;
+        }
+    }
+    __device__ __forceinline__ void load (int it, float4 (&v)[R])
+    {
+        #pragma unroll
+        for (int i = 0; i < R; i++) v[i] = view.ld4 (off[i] + it * GEMM_BK);
+    }
+    __device__ __forceinline__ void store (float *lds, const float4 (&v)[R])
+    {
+        #pragma unroll
+        for (int i = 0; i < R; i++) st4 (lds + (row0 + 32 * i) * LDS_ROW + chunk * 4, v[i]);
+    }
+};
+
 // Implicit-GEMM activation operand of conv / FC: row n = output position (b, oh, ow); the K axis runs
 // over (kh, kw, ic) and is resolved through the layer's k-chunk table.  Replaces the reference's
 // pointer table + panel gather (prepare_input / load_im2col_ptr, reference src/tiled_kernels.c:3-159).
-template <int ROWS> struct ConvLoader
+template <int ROWS, bool COH> struct ConvLoader
 {
     static constexpr int R = ROWS / 32;
-    const float *in;
+    ActView<COH> in;
     const aspen_hip_ktab_t *ktab;
     int32_t base[R], ih0[R], iw0[R];
     uint32_t IH, IW, chunk, row0;
-    __device__ __forceinline__ void init (const aspen_hip_layer_t &L, uint32_t first_row, uint32_t tid)
+    __device__ __forceinline__ void init (const aspen_hip_layer_t &L, const ActView<COH> &v, uint32_t first_row, uint32_t tid)
     {
-        in = L.in0; ktab = L.ktab; IH = L.IH; IW = L.IW;
+        in = v; ktab = L.ktab; IH = L.IH; IW = L.IW;
         chunk = tid & 7; row0 = tid >> 3;
         const uint32_t ohw = L.OH * L.OW;
         #pragma unroll
@@ -115,7 +186,7 @@ template <int ROWS> struct ConvLoader
         for (int i = 0; i < R; i++)
         {
             const bool ok = (uint32_t)(ih0[i] + (int32_t)e.kh) < IH && (uint32_t)(iw0[i] + (int32_t)e.kw) < IW;
-            v[i] = ok ? ld4 (in + (ptrdiff_t)(base[i] + e.offset)) : make_float4 (0.f, 0.f, 0.f, 0.f);
+            v[i] = ok ? in.ld4 ((uint32_t)(base[i] + e.offset)) : make_float4 (0.f, 0.f, 0.f, 0.f);
         }
     }
     __device__ __forceinline__ void store (float *lds, const float4 (&v)[R])
@@ -127,25 +198,27 @@ template <int ROWS> struct ConvLoader
 
 // K-strided operand (V of attention: rows = channels, K axis = sequence position with stride ld):
 // read 64 channels x 32 positions with 128-bit loads along the channels, transpose into LDS.
-struct TransLoader64
+template <bool COH> struct TransLoader64
 {
     static constexpr int R = 2;
-    const float *ptr[2];
+    ActView<COH> view;
+    uint32_t off[2];
     uint32_t c4, s0, ld, klen;
     bool live;
-    // valid_rows: channels of this tile that exist; klen: length of the K axis (positions >= klen read as zero)
-    __device__ __forceinline__ void init (const float *base, uint32_t ld_, uint32_t valid_rows, uint32_t klen_, uint32_t tid)
+    // first: float offset of (position 0, first channel of the tile); valid_rows: channels of this tile
+    // that exist; klen: length of the K axis (positions >= klen read as zero)
+    __device__ __forceinline__ void init (const ActView<COH> &v, uint32_t first, uint32_t ld_, uint32_t valid_rows, uint32_t klen_, uint32_t tid)
     {
-        ld = ld_; klen = klen_; c4 = tid & 15; s0 = tid >> 4; live = c4 * 4 < valid_rows;
-        ptr[0] = base + (size_t)s0 * ld + c4 * 4;
-        ptr[1] = base + (size_t)(s0 + 16) * ld + c4 * 4;
+        view = v; ld = ld_; klen = klen_; c4 = tid & 15; s0 = tid >> 4; live = c4 * 4 < valid_rows;
+        off[0] = first + s0 * ld + c4 * 4;
+        off[1] = first + (s0 + 16) * ld + c4 * 4;
     }
     __device__ __forceinline__ void load (int it, float4 (&v)[2])
     {
         const float4 z = make_float4 (0.f, 0.f, 0.f, 0.f);
         const uint32_t s = it * GEMM_BK + s0;
-        v[0] = (live && s < klen) ? ld4 (ptr[0] + (size_t)it * GEMM_BK * ld) : z;
-        v[1] = (live && s + 16 < klen) ? ld4 (ptr[1] + (size_t)it * GEMM_BK * ld) : z;
+        v[0] = (live && s < klen) ? view.ld4 (off[0] + it * GEMM_BK * ld) : z;
+        v[1] = (live && s + 16 < klen) ? view.ld4 (off[1] + it * GEMM_BK * ld) : z;
     }
     __device__ __forceinline__ void store (float *lds, const float4 (&v)[2])
     {
@@ -245,26 +318,29 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kiters,
 #define ACC_N(wn0, i, v, lane) ((wn0) + 32 * (i) + 8 * ((v) >> 2) + 4 * ((lane) >> 5) + ((v) & 3))
 
 // conv / FC / matmul tile
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, bool COH>
 __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, float *smem)
 {
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t m0 = tm * BM, n0 = tn * BN;
     floatx16 acc[TN][TM];
+    ActView<COH> in, out;
+    in.init (L.in0, L.type == FC_LAYER ? L.N * L.IH * L.IW : (L.type == CONV_LAYER ? (L.N / (L.OH * L.OW)) * L.IH * L.IW : L.N), L.ld0);
+    out.init (L.out, L.N, L.ld);
     RowLoader<BM> al;
     al.init (L.weight, m0, 0xffffffffu, L.Kp, tid);
     const int kiters = (int)(L.Kp / GEMM_BK);
     if (L.direct)
     {
-        RowLoader<BN> bl;
-        bl.init (L.in0, n0, L.N - 1, L.ld0, tid);
+        ActRowLoader<BN, COH> bl;
+        bl.init (in, n0, L.N - 1, L.ld0, 0, tid);
         gemm_core<BM, BN, WM, WN> (al, bl, kiters, smem, acc);
     }
     else
     {
-        ConvLoader<BN> bl;
-        bl.init (L, n0, tid);
+        ConvLoader<BN, COH> bl;
+        bl.init (L, in, n0, tid);
         gemm_core<BM, BN, WM, WN> (al, bl, kiters, smem, acc);
     }
     const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);
@@ -299,9 +375,9 @@ __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, ui
             float4 v = ld4 (smem + r * TROW + c);
             v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
             v = act4 (v, act);
-            float *o = L.out + (size_t)(n0 + r) * L.ld + m0 + c;
-            if (c + 4 <= mrem) st4 (o, v);
-            else { o[0] = v.x; if (c + 1 < mrem) o[1] = v.y; if (c + 2 < mrem) o[2] = v.z; }
+            const uint32_t o = (n0 + r) * L.ld + m0 + c;
+            if (c + 4 <= mrem) out.st4 (o, v);
+            else { out.st1 (o, v.x); if (c + 1 < mrem) out.st1 (o + 1, v.y); if (c + 2 < mrem) out.st1 (o + 2, v.z); }
         }
     }
     __syncthreads ();
@@ -310,26 +386,30 @@ __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, ui
 // ---------------------------------------------------------------------------------------------
 // Bandwidth tiles: 128-bit accesses, a tile = tile_n whole columns.
 // ---------------------------------------------------------------------------------------------
+template <bool COH>
 __device__ __forceinline__ void tile_residual (const aspen_hip_layer_t &L, uint32_t tn)
 {
     const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N), M4 = L.ld >> 2;
     const uint32_t total = (n1 - n0) * M4;
+    ActView<COH> p0, p1, out;
+    p0.init (L.in0, L.N, L.ld0); p1.init (L.in1, L.N, L.ld1); out.init (L.out, L.N, L.ld);
     for (uint32_t i = threadIdx.x; i < total; i += WG_THREADS)
     {
-        const uint32_t c = i / M4, m = (i - c * M4) * 4;
-        const size_t n = n0 + c;
-        float4 a = ld4 (L.in0 + n * L.ld0 + m), b = ld4 (L.in1 + n * L.ld1 + m);
+        const uint32_t c = i / M4, m = (i - c * M4) * 4, n = n0 + c;
+        float4 a = p0.ld4 (n * L.ld0 + m), b = p1.ld4 (n * L.ld1 + m);
         a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
-        st4 (L.out + n * L.ld + m, act4 (a, L.act));
+        out.st4 (n * L.ld + m, act4 (a, L.act));
     }
 }
 
-template <bool IS_MAX>
+template <bool IS_MAX, bool COH>
 __device__ __forceinline__ void tile_pool (const aspen_hip_layer_t &L, uint32_t tn)
 {
     const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N), M4 = L.ld >> 2;
     const uint32_t total = (n1 - n0) * M4, ohw = L.OH * L.OW;
     const float inv = 1.0f / (float)(L.KH * L.KW);
+    ActView<COH> in, out;
+    in.init (L.in0, (L.N / ohw) * L.IH * L.IW, L.ld0); out.init (L.out, L.N, L.ld);
     for (uint32_t i = threadIdx.x; i < total; i += WG_THREADS)
     {
         const uint32_t c = i / M4, m = (i - c * M4) * 4, n = n0 + c;
@@ -343,7 +423,7 @@ __device__ __forceinline__ void tile_pool (const aspen_hip_layer_t &L, uint32_t 
             {
                 const int iw = (int)(ow * L.stride + kw) - (int)L.pad;
                 if ((uint32_t)iw >= L.IW) continue;
-                const float4 x = ld4 (L.in0 + ((size_t)(b * L.IH + ih) * L.IW + iw) * L.ld0 + m);
+                const float4 x = in.ld4 (((b * L.IH + ih) * L.IW + iw) * L.ld0 + m);
                 if (IS_MAX) { r.x = r.x >= x.x ? r.x : x.x; r.y = r.y >= x.y ? r.y : x.y; r.z = r.z >= x.z ? r.z : x.z; r.w = r.w >= x.w ? r.w : x.w; }
                 else { r.x += x.x; r.y += x.y; r.z += x.z; r.w += x.w; }
             }
@@ -352,7 +432,7 @@ __device__ __forceinline__ void tile_pool (const aspen_hip_layer_t &L, uint32_t 
         r = act4 (r, L.act);
         // keep the zero padding rows [M, ld) intact
         if (m + 4 > L.M) { if (m + 0 >= L.M) r.x = 0.f; if (m + 1 >= L.M) r.y = 0.f; if (m + 2 >= L.M) r.z = 0.f; if (m + 3 >= L.M) r.w = 0.f; }
-        st4 (L.out + (size_t)n * L.ld + m, r);
+        out.st4 (n * L.ld + m, r);
     }
 }
 
@@ -370,56 +450,60 @@ __device__ __forceinline__ float wave_max (float v)
 }
 
 // one wavefront per column: mean and E[x^2] in one pass, eps 1e-6f
+template <bool COH>
 __device__ __forceinline__ void tile_layernorm (const aspen_hip_layer_t &L, uint32_t tn)
 {
     const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N);
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, M4 = L.M >> 2;
+    ActView<COH> in, out;
+    in.init (L.in0, L.N, L.ld0); out.init (L.out, L.N, L.ld);
     for (uint32_t n = n0 + wave; n < n1; n += WG_THREADS / 64)
     {
-        const float *x = L.in0 + (size_t)n * L.ld0;
+        const uint32_t x = n * L.ld0, o = n * L.ld;
         float s = 0.f, q = 0.f;
         for (uint32_t m = lane; m < M4; m += 64)
         {
-            const float4 v = ld4 (x + m * 4);
+            const float4 v = in.ld4 (x + m * 4);
             s += v.x + v.y + v.z + v.w;
             q += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
         }
-        for (uint32_t m = M4 * 4 + lane; m < L.M; m += 64) { const float v = x[m]; s += v; q += v * v; }
+        for (uint32_t m = M4 * 4 + lane; m < L.M; m += 64) { const float v = in.ld1 (x + m); s += v; q += v * v; }
         s = wave_sum (s); q = wave_sum (q);
         const float mean = s / (float)L.M;
         float var = q / (float)L.M - mean * mean;
         const float rstd = 1.0f / sqrtf (var + 1e-6f);
-        float *o = L.out + (size_t)n * L.ld;
         for (uint32_t m = lane; m < M4; m += 64)
         {
-            const float4 v = ld4 (x + m * 4), g = ld4 (L.weight + m * 4);
+            const float4 v = in.ld4 (x + m * 4), g = ld4 (L.weight + m * 4);
             float4 r;
             r.x = (v.x - mean) * rstd * g.x; r.y = (v.y - mean) * rstd * g.y;
             r.z = (v.z - mean) * rstd * g.z; r.w = (v.w - mean) * rstd * g.w;
             if (L.bias) { const float4 b = ld4 (L.bias + m * 4); r.x += b.x; r.y += b.y; r.z += b.z; r.w += b.w; }
-            st4 (o + m * 4, r);
+            out.st4 (o + m * 4, r);
         }
         for (uint32_t m = M4 * 4 + lane; m < L.M; m += 64)
-            o[m] = (x[m] - mean) * rstd * L.weight[m] + (L.bias ? L.bias[m] : 0.f);
+            out.st1 (o + m, (in.ld1 (x + m) - mean) * rstd * L.weight[m] + (L.bias ? L.bias[m] : 0.f));
     }
 }
 
 // one wavefront per column: max-subtracted softmax over the rows
+template <bool COH>
 __device__ __forceinline__ void tile_softmax (const aspen_hip_layer_t &L, uint32_t tn)
 {
     const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N);
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    ActView<COH> in, out;
+    in.init (L.in0, L.N, L.ld0); out.init (L.out, L.N, L.ld);
     for (uint32_t n = n0 + wave; n < n1; n += WG_THREADS / 64)
     {
-        const float *x = L.in0 + (size_t)n * L.ld0;
-        float *o = L.out + (size_t)n * L.ld;
+        const uint32_t x = n * L.ld0, o = n * L.ld;
         float mx = -INFINITY;
-        for (uint32_t m = lane; m < L.M; m += 64) mx = fmaxf (mx, x[m]);
+        for (uint32_t m = lane; m < L.M; m += 64) mx = fmaxf (mx, in.ld1 (x + m));
         mx = wave_max (mx);
         float s = 0.f;
-        for (uint32_t m = lane; m < L.M; m += 64) { const float e = expf (x[m] - mx); o[m] = e; s += e; }
+        for (uint32_t m = lane; m < L.M; m += 64) s += expf (in.ld1 (x + m) - mx);
         s = wave_sum (s);
-        for (uint32_t m = lane; m < L.M; m += 64) o[m] = o[m] / s;
+        for (uint32_t m = lane; m < L.M; m += 64) out.st1 (o + m, expf (in.ld1 (x + m) - mx) / s);
     }
 }
 
@@ -430,6 +514,7 @@ __device__ __forceinline__ void tile_softmax (const aspen_hip_layer_t &L, uint32
 // sums are fused into the epilogue; a second sweep over the tile's own output divides by the sums.
 // in0 = Query matrix, in1 = Key matrix (reference cfg: parent = Query, from = Key).
 // ---------------------------------------------------------------------------------------------
+template <bool COH>
 __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, uint32_t tn, float *smem)
 {
     constexpr int BM = 128, BN = 128, WM = 2, WN = 2, TM = 2, TN = 2;
@@ -439,9 +524,9 @@ __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, ui
     const uint32_t bh = tn / qtiles, q0 = (tn - bh * qtiles) * BN;
     const uint32_t b = bh / L.heads, h = bh - b * L.heads;
     const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);
-    const float *Q = L.in0 + (size_t)b * S * L.ld0 + h * L.hd;
-    const float *Kmat = L.in1 + (size_t)b * S * L.ld1 + h * L.hd;
-    float *out = L.out + (size_t)bh * S * L.ld;          // column (b*H + h)*S + q, rows = keys
+    ActView<COH> Q, Kmat, out;
+    Q.init (L.in0, L.N / L.heads, L.ld0); Kmat.init (L.in1, L.N / L.heads, L.ld1); out.init (L.out, L.N, L.ld);
+    const uint32_t obase = bh * S * L.ld;                // column (b*H + h)*S + q, rows = keys
     const float scale = 1.0f / sqrtf ((float)L.hd);
     if (tid < BN) rowsum[tid] = 0.f;
     float part[TN][16];
@@ -454,8 +539,8 @@ __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, ui
     for (uint32_t k0 = 0; k0 < S; k0 += BM)
     {
         floatx16 acc[TN][TM];
-        RowLoader<BM> al; al.init (Kmat, k0, S - 1, L.ld1, tid);
-        RowLoader<BN> bl; bl.init (Q, q0, S - 1, L.ld0, tid);
+        ActRowLoader<BM, COH> al; al.init (Kmat, b * S + k0, b * S + S - 1, L.ld1, h * L.hd, tid);
+        ActRowLoader<BN, COH> bl; bl.init (Q, b * S + q0, b * S + S - 1, L.ld0, h * L.hd, tid);
         gemm_core<BM, BN, WM, WN> (al, bl, kiters, smem, acc);
         #pragma unroll
         for (int j = 0; j < TM; j++)
@@ -470,7 +555,7 @@ __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, ui
                     float s = acc[i][j][v];
                     if (L.masked && key > q) s = -1e10f;
                     const float e = expf (s * scale);
-                    if (key < S && q < S) { out[(size_t)q * L.ld + key] = e; part[i][v] += e; }
+                    if (key < S && q < S) { out.st1 (obase + q * L.ld + key, e); part[i][v] += e; }
                 }
         }
     }
@@ -492,17 +577,18 @@ __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, ui
         for (uint32_t i = tid; i < nq * S4; i += WG_THREADS)
         {
             const uint32_t r = i / S4, c = (i - r * S4) * 4;
-            float *p = out + (size_t)(q0 + r) * L.ld + c;
-            const float inv = rowsum[r];
-            float4 v = ld4 (p);
-            v.x /= inv; v.y /= inv; v.z /= inv; v.w /= inv;
-            st4 (p, v);
+            const uint32_t o = obase + (q0 + r) * L.ld + c;
+            const float sum = rowsum[r];
+            float4 v = out.ld4 (o);
+            v.x /= sum; v.y /= sum; v.z /= sum; v.w /= sum;
+            out.st4 (o, v);
         }
     else
         for (uint32_t i = tid; i < nq * S; i += WG_THREADS)
         {
             const uint32_t r = i / S, c = i - r * S;
-            out[(size_t)(q0 + r) * L.ld + c] /= rowsum[r];
+            const uint32_t o = obase + (q0 + r) * L.ld + c;
+            out.st1 (o, out.ld1 (o) / rowsum[r]);
         }
     __syncthreads ();
 }
@@ -510,6 +596,7 @@ __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, ui
 // V tile: one (batch, head-slice of <= 64 channels) x 128 queries:
 // out[b*S + q][h*hd + j] = sum_s P[(b*H + h)*S + q][s] * V[b*S + s][h*hd + j].
 // in0 = probabilities (K-attention output), in1 = Value matrix.
+template <bool COH>
 __device__ __forceinline__ void tile_v_attention (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, float *smem)
 {
     constexpr int BM = 64, BN = 128, WM = 2, WN = 2, TM = 1, TN = 2;
@@ -518,11 +605,12 @@ __device__ __forceinline__ void tile_v_attention (const aspen_hip_layer_t &L, ui
     const uint32_t b = tn / qtiles, q0 = (tn - b * qtiles) * BN;
     const uint32_t m0 = tm * L.tile_m, h = m0 / L.hd;
     const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);
-    const float *P = L.in0 + (size_t)(b * L.heads + h) * S * L.ld0;
-    const float *V = L.in1 + (size_t)b * S * L.ld1 + m0;
+    ActView<COH> P, V, out;
+    P.init (L.in0, L.N * L.heads, L.ld0); V.init (L.in1, L.N, L.ld1); out.init (L.out, L.N, L.ld);
+    const uint32_t prow = (b * L.heads + h) * S;
     floatx16 acc[TN][TM];
-    TransLoader64 al; al.init (V, L.ld1, L.tile_m, S, tid);
-    RowLoader<BN> bl; bl.init (P, q0, S - 1, L.ld0, tid);   // P's stride is a multiple of 32 with zero padding
+    TransLoader64<COH> al; al.init (V, b * S * L.ld1 + m0, L.ld1, L.tile_m, S, tid);
+    ActRowLoader<BN, COH> bl; bl.init (P, prow + q0, prow + S - 1, L.ld0, 0, tid);   // P's stride is a multiple of 32 with zero padding
     gemm_core<BM, BN, WM, WN> (al, bl, (int)((S + GEMM_BK - 1) / GEMM_BK), smem, acc);
     const uint32_t mm = wm0 + (lane & 31);
     if (mm < L.tile_m)
@@ -532,7 +620,7 @@ __device__ __forceinline__ void tile_v_attention (const aspen_hip_layer_t &L, ui
             for (int v = 0; v < 16; v++)
             {
                 const uint32_t q = q0 + ACC_N (wn0, i, v, lane);
-                if (q < S) L.out[(size_t)(b * S + q) * L.ld + m0 + mm] = acc[i][0][v];
+                if (q < S) out.st1 ((b * S + q) * L.ld + m0 + mm, acc[i][0][v]);
             }
 }
 
@@ -541,23 +629,24 @@ __device__ __forceinline__ void tile_v_attention (const aspen_hip_layer_t &L, ui
 // (reference src/dse.c:39-79).  `t` = tile index inside the layer, row-tile fastest
 // (reference src/apu_nasm.c:1218-1224).
 // ---------------------------------------------------------------------------------------------
+template <bool COH>
 __device__ __forceinline__ void run_tile (const aspen_hip_layer_t &L, uint32_t t, float *smem)
 {
     const uint32_t tn = t / L.tiles_m, tm = t - tn * L.tiles_m;
     switch (L.type)
     {
     case CONV_LAYER: case FC_LAYER: case MATMUL_LAYER:
-        if (L.variant == ASPEN_HIP_GEMM_128x128) tile_contraction<128, 128, 2, 2> (L, tn, tm, smem);
-        else if (L.variant == ASPEN_HIP_GEMM_64x128) tile_contraction<64, 128, 2, 2> (L, tn, tm, smem);
-        else tile_contraction<64, 64, 2, 2> (L, tn, tm, smem);
+        if (L.variant == ASPEN_HIP_GEMM_128x128) tile_contraction<128, 128, 2, 2, COH> (L, tn, tm, smem);
+        else if (L.variant == ASPEN_HIP_GEMM_64x128) tile_contraction<64, 128, 2, 2, COH> (L, tn, tm, smem);
+        else tile_contraction<64, 64, 2, 2, COH> (L, tn, tm, smem);
         break;
-    case RESIDUAL_LAYER:    tile_residual (L, tn); break;
-    case MAXPOOL_LAYER:     tile_pool<true> (L, tn); break;
-    case AVGPOOL_LAYER:     tile_pool<false> (L, tn); break;
-    case LAYERNORM_LAYER:   tile_layernorm (L, tn); break;
-    case SOFTMAX_LAYER:     tile_softmax (L, tn); break;
-    case K_ATTENTION_LAYER: tile_k_attention (L, tn, smem); break;
-    case V_ATTENTION_LAYER: tile_v_attention (L, tn, tm, smem); break;
+    case RESIDUAL_LAYER:    tile_residual<COH> (L, tn); break;
+    case MAXPOOL_LAYER:     tile_pool<true, COH> (L, tn); break;
+    case AVGPOOL_LAYER:     tile_pool<false, COH> (L, tn); break;
+    case LAYERNORM_LAYER:   tile_layernorm<COH> (L, tn); break;
+    case SOFTMAX_LAYER:     tile_softmax<COH> (L, tn); break;
+    case K_ATTENTION_LAYER: tile_k_attention<COH> (L, tn, smem); break;
+    case V_ATTENTION_LAYER: tile_v_attention<COH> (L, tn, tm, smem); break;
     default: break;
     }
 }

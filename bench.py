@@ -100,6 +100,7 @@ def main():
     ap.add_argument("--min-ninst", type=int, default=512)
     ap.add_argument("--workgroups", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--skip-tiles", action="store_true", help="scheduler-only run: dependency protocol with empty tiles")
     ap.add_argument("--layer-profile", action="store_true", help="also time every layer's kernel (layer-launch mode)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -112,6 +113,8 @@ def main():
         print("bench.py: no HIP device: " + L.aspen_hip_last_error().decode(), file=sys.stderr)
         sys.exit(1)
     dev = api.device_info()
+    if args.skip_tiles:
+        L.aspen_hip_set_flags(1)
     cfgs, unit, units_per_step = WORKLOADS[args.workload]
 
     pool = api.RPool()

@@ -103,6 +103,13 @@ int aspen_hip_run_layers (aspen_hip_graph_t *graph, uint32_t first_layer, uint32
    abort flag, all workgroups exit and aspen_hip_sync returns ASPEN_HIP_ERR_STALLED. */
 int aspen_hip_run_dataflow (aspen_hip_graph_t *graph, uint32_t workgroups, uint64_t spin_limit);
 #define ASPEN_HIP_ERR_STALLED 0x7001
+/* Debug switches for later dataflow runs.  SKIP_TILES runs the whole dependency protocol with empty
+   tiles: the scheduler-only mode of the reference (-D_SKIP_KERNELS=1, reference src/tiled_kernels.c:163). */
+#define ASPEN_HIP_FLAG_SKIP_TILES 1u
+/* COUNT_TILES keeps the per-tile execution counters that aspen_hip_dataflow_stats reports (one extra
+   pair of atomics per tile); without it `executed` and `double_runs` read 0. */
+#define ASPEN_HIP_FLAG_COUNT_TILES 2u
+void aspen_hip_set_flags (uint32_t flags);
 int aspen_hip_sync (void);
 /* 1 when everything enqueued so far has finished, 0 when still running */
 int aspen_hip_idle (void);

@@ -18,4 +18,5 @@ def gpu():
     from aspen_amd import api
     assert os.path.exists(api.LIB_PATH), "libaspen_amd.so has not been built"
     assert api.lib().aspen_hip_init() == 0, api.lib().aspen_hip_last_error().decode()
+    api.lib().aspen_hip_set_flags(2)     # count executed tiles so that run_stats() can be asserted on
     return api

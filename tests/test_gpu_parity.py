@@ -38,20 +38,23 @@ def test_micro_nets_match_reference_fixture(gpu, name, mode):
 @pytest.mark.parametrize("name", list(H.micro_cases()))
 def test_micro_nets_match_oracle(gpu, name):
     """Same nets against the CPU oracle (full tensors), dataflow engine with few workgroups so that
-    tiles of several layers are in flight together."""
+    tiles of several layers are in flight together.  The graph is re-armed and re-run with a
+    DIFFERENT input each time: a tile that read a stale (cached) copy of its parent's previous
+    output would not match the oracle of the new input."""
     from oracle import cpu
     cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()[name])
-    outs = cpu.run_network(layers, tens, x, batch, seq)
+    inputs = [x, (x * 0.5 + 0.25).astype(np.float32), (-x).astype(np.float32), x]
     net = H.GpuNet(cfg, tens, batch, seq, min_ninst=32, mode=api.MODE_DATAFLOW, workgroups=24)
     print(f"case {name} tiles {net.nasm.num_ninst}", flush=True)
     try:
-        for rep in range(3):          # re-arm and run again: results must not depend on the previous run
-            net.run(x if rep == 0 else None)
+        for rep, xin in enumerate(inputs):
+            outs = cpu.run_network(layers, tens, xin, batch, seq)
+            net.run(xin)
             st = net.rpool.run_stats()
             assert st == {"executed": net.nasm.num_ninst, "double_runs": 0, "aborted": 0}, st
-        for l in range(net.nasm.num_ldata):
-            err = H.rel_l2(net.layer(l), outs[l])
-            assert err <= H.REL_L2_TOL, f"layer {l} ({layers[l]['type']}): rel L2 {err:.3g}"
+            for l in range(net.nasm.num_ldata):
+                err = H.rel_l2(net.layer(l), outs[l])
+                assert err <= H.REL_L2_TOL, f"run {rep} layer {l} ({layers[l]['type']}): rel L2 {err:.3g}"
     finally:
         net.close()
 
