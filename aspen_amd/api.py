@@ -87,6 +87,7 @@ def lib() -> C.CDLL:
         "aspen_rpool_run_stats": (C.c_int, [_vp, _u32p, _u32p, _u32p]),
         "aspen_rpool_num_ninst": (C.c_uint, [_vp]),
         "aspen_rpool_profile_layers": (C.c_int, [_vp, C.c_uint, _fp]),
+        "aspen_rpool_dataflow_profile": (C.c_int, [_vp, C.POINTER(C.c_uint64), C.c_int]),
         # aspen_hip.h
         "aspen_hip_init": (C.c_int, []),
         "aspen_hip_last_error": (C.c_char_p, []),
@@ -234,6 +235,13 @@ class RPool:
         if lib().aspen_rpool_run_stats(self.h, C.byref(a), C.byref(b), C.byref(c)):
             raise RuntimeError("no dataflow run to report on")
         return {"executed": a.value, "double_runs": b.value, "aborted": c.value}
+
+    def dataflow_profile(self, reset: bool = True) -> dict:
+        """Summed workgroup time of dataflow runs since the last reset, in seconds (profile flag 4)."""
+        t = (C.c_uint64 * 4)()
+        if lib().aspen_rpool_dataflow_profile(self.h, t, 1 if reset else 0):
+            raise RuntimeError("no dataflow profile")
+        return {k: t[i] * 1e-8 for i, k in enumerate(["tile", "drain", "sched", "total"])}
 
     def profile_layers(self, num_layers: int, iters: int = 5) -> np.ndarray:
         """Per-layer kernel time in ms (layer-launch mode, HIP events); the pool must have run once."""

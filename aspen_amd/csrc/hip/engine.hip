@@ -34,6 +34,7 @@ struct aspen_hip_graph_t
     uint32_t *d_state;      // one counter per 128-byte line: [ST_HEAD] pop tickets, [ST_TAIL] push cursor, [ST_DONE] tiles done,
                             // [ST_ABORT] abort flag, [ST_TWICE] tiles executed more than once
     uint32_t *d_ran;        // per-tile execution count (sanity: every tile exactly once)
+    unsigned long long *d_prof;
 };
 
 static hipStream_t g_stream = nullptr;
@@ -57,18 +58,14 @@ static int fail (hipError_t e, const char *what)
 
 // Per-layer launch: workgroup -> tile with contiguous tile ranges per XCD (workgroups are dealt to
 // the 8 XCDs round-robin), so tiles that share activation rows meet in the same L2.
-__global__ void __launch_bounds__ (WG_THREADS, 2) layer_kernel (const aspen_hip_layer_t *layers, uint32_t l)
+__global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) layer_kernel (const aspen_hip_layer_t *layers, uint32_t l, uint32_t first_tile)
 {
     extern __shared__ __align__ (16) float smem[];
     const aspen_hip_layer_t &L = layers[l];
     const uint32_t nt = gridDim.x, bid = blockIdx.x;
     const uint32_t xcd = bid & 7, local = bid >> 3, chunk = nt >> 3, rem = nt & 7;
-    const uint32_t t = xcd * chunk + (xcd < rem ? xcd : rem) + local;
-#ifdef EXP_LAYER_COH
-    run_tile<true> (L, t, smem);
-#else
+    const uint32_t t = first_tile + xcd * chunk + (xcd < rem ? xcd : rem) + local;
     run_tile<false> (L, t, smem);
-#endif
 }
 
 // Re-arm: counters back to the parent counts, queue emptied and seeded with the roots.
@@ -90,10 +87,18 @@ struct dataflow_args_t
     const aspen_hip_layer_t *layers;
     const uint32_t *ninst_layer, *child_off, *child_idx;
     uint32_t *dep, *queue, *state, *ran;
+    unsigned long long *prof;       // [0] tile, [1] store drain, [2] publish / pop, [3] total: summed 100 MHz ticks of all workgroups
     uint32_t num_ninst;
     uint32_t flags;                 // ASPEN_HIP_FLAG_*
     unsigned long long spin_limit;
 };
+
+// The tile body as a real function call: the persistent loop around it then carries almost no
+// register state, and the tile code gets the whole register budget to itself.
+__device__ __noinline__ void run_tile_coherent (const aspen_hip_layer_t *L, uint32_t t, float *smem)
+{
+    run_tile<true> (*L, t, smem);
+}
 
 // Waits until queue slot `ticket` holds a tile and returns it; QUEUE_EMPTY when all tickets are
 // taken or the run was aborted.  The wait polls with relaxed device-scope loads (an acquire here
@@ -118,36 +123,44 @@ __device__ __forceinline__ uint32_t wait_for_slot (const dataflow_args_t &a, uin
 }
 
 // Persistent workgroup = one scheduling engine (the reference's DSE thread, src/dse.c:5-108).
-// Wavefront 1 pops: it draws the ticket for the NEXT tile before the current tile starts, so the
-// round trip of that atomic hides behind the tile, and resolves the ticket to a tile while
-// wavefront 0 publishes the finished tile (dependency countdown of its children, push of those
-// that became ready).  No cache write-back / invalidate is needed anywhere: tiles access
+// Wavefront 1 pops the next tile while wavefront 0 publishes the finished one (dependency countdown
+// of its children, push of those that became ready).  No cache write-back / invalidate is needed anywhere: tiles access
 // activations with device-scope coherent instructions (ActView<true>).
-__global__ void __launch_bounds__ (WG_THREADS, 2) dataflow_kernel (dataflow_args_t a)
+__global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataflow_args_t a)
 {
     extern __shared__ __align__ (16) float smem[];
     __shared__ uint32_t s_tile[2];
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const bool popper = wave == 1 && lane == 0;
     uint32_t next_ticket = 0;
-    if (popper)
-    {
-        s_tile[0] = wait_for_slot (a, atomicAdd (&a.state[ST_HEAD], 1u));
-        next_ticket = atomicAdd (&a.state[ST_HEAD], 1u);
-    }
+    const bool prof = (a.flags & ASPEN_HIP_FLAG_PROFILE) && threadIdx.x == 0;
+    unsigned long long t_tile = 0, t_drain = 0, t_sched = 0, t_begin = prof ? wall_clock64 () : 0, t0 = t_begin;
+    if (popper) s_tile[0] = wait_for_slot (a, atomicAdd (&a.state[ST_HEAD], 1u));
+    (void)next_ticket;
     for (uint32_t it = 0;; it++)
     {
         __syncthreads ();
         const uint32_t id = s_tile[it & 1];
-        if (id == QUEUE_EMPTY) return;          // all tickets taken, or aborted
+        if (prof) { const unsigned long long t = wall_clock64 (); t_sched += t - t0; t0 = t; }
+        if (id == QUEUE_EMPTY)                  // all tickets taken, or aborted
+        {
+            if (prof)
+            {
+                atomicAdd (&a.prof[0], t_tile); atomicAdd (&a.prof[1], t_drain); atomicAdd (&a.prof[2], t_sched);
+                atomicAdd (&a.prof[3], wall_clock64 () - t_begin);
+            }
+            return;
+        }
 
-        const aspen_hip_layer_t &L = a.layers[a.ninst_layer[id]];
+        const aspen_hip_layer_t *L = &a.layers[a.ninst_layer[id]];
         if (!(a.flags & ASPEN_HIP_FLAG_SKIP_TILES))
-            run_tile<true> (L, id - L.ninst_start, smem);
+            run_tile_coherent (L, id - L->ninst_start, smem);
 
+        if (prof) { const unsigned long long t = wall_clock64 (); t_tile += t - t0; t0 = t; }
         // every wave waits until its (write-through, device-coherent) stores have been acknowledged
         __builtin_amdgcn_fence (__ATOMIC_RELEASE, "workgroup");
         __syncthreads ();
+        if (prof) { const unsigned long long t = wall_clock64 (); t_drain += t - t0; t0 = t; }
         if (wave == 0)
         {
             // publish: count down the children with relaxed device-scope atomics; whoever takes a
@@ -171,9 +184,10 @@ __global__ void __launch_bounds__ (WG_THREADS, 2) dataflow_kernel (dataflow_args
         }
         else if (popper)
         {
-            // pop: resolve the ticket drawn one tile ago, draw the one after it
-            s_tile[(it + 1) & 1] = wait_for_slot (a, next_ticket);
-            next_ticket = atomicAdd (&a.state[ST_HEAD], 1u);
+            // pop: a ticket is drawn only now, when this workgroup is free.  Drawing it earlier would
+            // hide the atomic's round trip but binds a (possibly already ready) tile to a busy
+            // workgroup while idle ones wait on later slots.
+            s_tile[(it + 1) & 1] = wait_for_slot (a, atomicAdd (&a.state[ST_HEAD], 1u));
         }
     }
 }
@@ -200,6 +214,12 @@ extern "C" int aspen_hip_init (void)
 }
 
 extern "C" const char *aspen_hip_last_error (void) { return g_err; }
+
+extern "C" void aspen_hip_tile_shapes (uint32_t shapes[9])
+{
+    shapes[0] = VAR0_BM; shapes[1] = VAR0_BN; shapes[2] = VAR1_BM; shapes[3] = VAR1_BN; shapes[4] = VAR2_BM; shapes[5] = VAR2_BN;
+    shapes[6] = KATTN_BN; shapes[7] = 128; shapes[8] = WG_PER_CU;
+}
 
 extern "C" int aspen_hip_device_info (int *num_cu, int *clock_khz, size_t *mem_bytes, char *name, int name_len)
 {
@@ -279,10 +299,17 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
     if (L.type == INPUT_LAYER) return 0;
     if (!L.out || !L.in0) why = "missing buffers";
     else if (L.ld % 4 || L.ld0 % 4 || (L.in1 && L.ld1 % 4)) why = "strides must be multiples of 4 floats";
-    else if (L.tiles_m == 0 || L.tiles_n == 0 || L.num_ninst != L.tiles_m * L.tiles_n) why = "tile grid";
+    else if (L.tiles_m == 0 || L.tiles_n == 0 || L.splits == 0
+        || L.num_ninst != L.tiles_m * L.tiles_n * (L.splits > 1 ? L.splits + 1 : 1)) why = "tile grid";
+    else if (L.splits > 1 && (!L.partial || L.kiters_per_split == 0 || (uint64_t)L.splits * L.kiters_per_split * GEMM_BK < L.Kp
+        || !(L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER))) why = "split-K geometry";
+    else if ((uint64_t)L.N * L.ld * 4 * L.splits >= 0xffffff00ull) why = "matrix larger than 4 GiB";
     else if (L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER)
     {
-        const uint32_t bm = L.variant == ASPEN_HIP_GEMM_128x128 ? 128 : 64, bn = L.variant == ASPEN_HIP_GEMM_64x64 ? 64 : 128;
+        uint32_t shp[9];
+        aspen_hip_tile_shapes (shp);
+        if (L.variant < 0 || L.variant >= ASPEN_HIP_NUM_GEMM_VARIANTS) { snprintf (g_err, sizeof (g_err), "layer %u rejected: GEMM variant", idx); return -1; }
+        const uint32_t bm = shp[2 * L.variant], bn = shp[2 * L.variant + 1];
         if (!L.weight) why = "missing weight";
         else if (L.Kp == 0 || L.Kp % GEMM_BK) why = "Kp must be a positive multiple of 32";
         else if (L.tile_m != bm || L.tile_n != bn) why = "tile extent does not match the GEMM variant";
@@ -294,7 +321,7 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
     {
         if (!L.in1 || L.hd == 0 || L.hd % GEMM_BK || L.heads == 0 || L.seq == 0) why = "attention geometry";
         else if (L.ld < L.seq || L.ld % GEMM_BK) why = "probability stride must be a multiple of 32 covering seq";
-        else if (L.tile_n != 128 || L.tiles_m != 1) why = "K-attention tiles are 128 queries x all keys";
+        else if (L.tile_n != KATTN_BN || L.tiles_m != 1) why = "K-attention tile extent";
     }
     else if (L.type == V_ATTENTION_LAYER)
     {
@@ -345,6 +372,7 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     g->d_queue = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
     g->d_ran = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
     g->d_state = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * ST_WORDS);
+    g->d_prof = (unsigned long long *)aspen_hip_alloc (sizeof (unsigned long long) * 8);
     if (!g->d_layers || !g->d_ninst_layer || !g->d_num_parents || !g->d_child_off || !g->d_child_idx || !g->d_roots
         || !g->d_dep || !g->d_queue || !g->d_ran || !g->d_state)
     {
@@ -360,7 +388,7 @@ extern "C" void aspen_hip_graph_destroy (aspen_hip_graph_t *g)
     (void)hipStreamSynchronize (g_stream);
     aspen_hip_free (g->d_layers); aspen_hip_free (g->d_ninst_layer); aspen_hip_free (g->d_num_parents);
     aspen_hip_free (g->d_child_off); aspen_hip_free (g->d_child_idx); aspen_hip_free (g->d_roots);
-    aspen_hip_free (g->d_dep); aspen_hip_free (g->d_queue); aspen_hip_free (g->d_ran); aspen_hip_free (g->d_state);
+    aspen_hip_free (g->d_dep); aspen_hip_free (g->d_queue); aspen_hip_free (g->d_ran); aspen_hip_free (g->d_state); aspen_hip_free (g->d_prof);
     free (g->h_layers);
     free (g);
 }
@@ -368,6 +396,21 @@ extern "C" void aspen_hip_graph_destroy (aspen_hip_graph_t *g)
 // ------------------------------------------------------------------------------------------------
 // execution
 // ------------------------------------------------------------------------------------------------
+// One layer in launch mode; a split-K layer needs its partial tiles finished before the finishing
+// tiles start, hence two launches.
+static void launch_layer (const aspen_hip_graph_t *g, uint32_t l)
+{
+    const aspen_hip_layer_t &L = g->h_layers[l];
+    if (L.splits > 1)
+    {
+        const uint32_t T = L.tiles_m * L.tiles_n;
+        hipLaunchKernelGGL (layer_kernel, dim3 (T * L.splits), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, g->d_layers, l, 0u);
+        hipLaunchKernelGGL (layer_kernel, dim3 (T), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, g->d_layers, l, T * L.splits);
+    }
+    else
+        hipLaunchKernelGGL (layer_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, g->d_layers, l, 0u);
+}
+
 extern "C" int aspen_hip_run_layers (aspen_hip_graph_t *g, uint32_t first_layer, uint32_t last_layer)
 {
     if (!g || first_layer > last_layer || last_layer >= g->num_layers) { snprintf (g_err, sizeof (g_err), "run_layers: bad range"); return -1; }
@@ -375,7 +418,7 @@ extern "C" int aspen_hip_run_layers (aspen_hip_graph_t *g, uint32_t first_layer,
     {
         const aspen_hip_layer_t &L = g->h_layers[l];
         if (L.type == INPUT_LAYER || L.num_ninst == 0) continue;
-        hipLaunchKernelGGL (layer_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, g->d_layers, l);
+        launch_layer (g, l);
         CHECK (hipGetLastError ());
     }
     return 0;
@@ -385,13 +428,13 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
 {
     if (!g) { snprintf (g_err, sizeof (g_err), "run_dataflow: null graph"); return -1; }
     if (g->num_ninst == 0) return 0;
-    if (workgroups == 0) workgroups = 2 * (uint32_t)g_num_cu;
+    if (workgroups == 0) workgroups = WG_PER_CU * (uint32_t)g_num_cu;
     hipLaunchKernelGGL (arm_kernel, dim3 ((g->num_ninst + 255) / 256), dim3 (256), 0, g_stream,
         g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->num_ninst, g->num_roots, g->d_state);
     CHECK (hipGetLastError ());
     dataflow_args_t a;
     a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx;
-    a.dep = g->d_dep; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran;
+    a.dep = g->d_dep; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran; a.prof = g->d_prof;
     a.num_ninst = g->num_ninst; a.flags = g_flags; a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
     CHECK (hipEventRecord (g_events[NUM_EVENTS - 2], g_stream));
     hipLaunchKernelGGL (dataflow_kernel, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);
@@ -409,8 +452,7 @@ extern "C" int aspen_hip_profile_layers (aspen_hip_graph_t *g, uint32_t iters, f
         ms_per_layer[l] = 0.f;
         if (L.type == INPUT_LAYER || L.num_ninst == 0) continue;
         CHECK (hipEventRecord (g_events[NUM_EVENTS - 4], g_stream));
-        for (uint32_t i = 0; i < iters; i++)
-            hipLaunchKernelGGL (layer_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, g->d_layers, l);
+        for (uint32_t i = 0; i < iters; i++) launch_layer (g, l);
         CHECK (hipGetLastError ());
         CHECK (hipEventRecord (g_events[NUM_EVENTS - 3], g_stream));
         CHECK (hipEventSynchronize (g_events[NUM_EVENTS - 3]));
@@ -447,6 +489,16 @@ extern "C" int aspen_hip_dataflow_stats (aspen_hip_graph_t *g, uint32_t *execute
     return 0;
 }
 
+extern "C" int aspen_hip_dataflow_profile (aspen_hip_graph_t *g, uint64_t ticks[4], int reset)
+{
+    if (!g || !ticks) return -1;
+    unsigned long long h[4];
+    if (aspen_hip_d2h (h, g->d_prof, sizeof (h))) return -1;
+    for (int i = 0; i < 4; i++) ticks[i] = h[i];
+    if (reset) { CHECK (hipMemsetAsync (g->d_prof, 0, sizeof (h), g_stream)); }
+    return 0;
+}
+
 extern "C" int aspen_hip_event_record (int slot)
 {
     if (aspen_hip_init ()) return -1;
@@ -476,13 +528,13 @@ extern "C" int aspen_hip_sgemm (uint32_t M, uint32_t N, uint32_t K, const float 
     CHECK (hipMemcpy2DAsync (Ap, (size_t)K * 4, A, (size_t)lda * 4, (size_t)K * 4, M, hipMemcpyDeviceToDevice, g_stream));
     aspen_hip_layer_t L;
     memset (&L, 0, sizeof (L));
-    L.type = MATMUL_LAYER; L.act = act; L.variant = ASPEN_HIP_GEMM_64x64; L.direct = 1;
+    L.type = MATMUL_LAYER; L.act = act; L.variant = ASPEN_HIP_GEMM_SMALL; L.direct = 1;
     L.M = M; L.N = N; L.ld = ldc; L.tile_m = 64; L.tile_n = 64;
-    L.tiles_m = (M + 63) / 64; L.tiles_n = (N + 63) / 64; L.num_ninst = L.tiles_m * L.tiles_n;
+    L.tiles_m = (M + 63) / 64; L.tiles_n = (N + 63) / 64; L.num_ninst = L.tiles_m * L.tiles_n; L.splits = 1;
     L.K = K; L.Kp = K; L.ld0 = ldb; L.out = C; L.in0 = B; L.weight = Ap; L.bias = bias;
     aspen_hip_layer_t *dL = upload (&L, 1);
     if (!dL) { aspen_hip_free (Ap); return -1; }
-    hipLaunchKernelGGL (layer_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, dL, 0u);
+    hipLaunchKernelGGL (layer_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, dL, 0u, 0u);
     hipError_t e = hipGetLastError ();
     if (e == hipSuccess) e = hipStreamSynchronize (g_stream);
     aspen_hip_free (dL); aspen_hip_free (Ap);

@@ -19,7 +19,35 @@ typedef float floatx16 __attribute__ ((ext_vector_type (16)));
 #define WG_THREADS 256
 #define GEMM_BK 32            // K floats staged per iteration: one 128-byte line per operand row
 #define LDS_ROW 36            // floats per staged row: 32 + 4 padding -> conflict-free 128-bit reads
-#define GEMM_SMEM_FLOATS (2 * (128 + 128) * LDS_ROW)
+
+// Two footprints.  Default: tiles of at most 128 x 64 outputs, 32 accumulator registers per lane, one
+// LDS stage (the next K slice waits in registers) -> <= 128 VGPRs and <= 40 KB LDS per workgroup, so
+// FOUR workgroups (16 wavefronts) share a compute unit and one workgroup's load latency, epilogue
+// and scheduling gaps are covered by the other three.  ASPEN_BIG_TILES: 128 x 128 tiles, two LDS
+// stages, two workgroups per compute unit (better for very large GEMMs, worse for short ones).
+#ifdef ASPEN_BIG_TILES
+#define VAR0_BM 128
+#define VAR0_BN 128
+#define GEMM_STAGES 2
+#define WG_PER_CU 2
+#define KATTN_BN 128
+#else
+#define VAR0_BM 128
+#define VAR0_BN 64
+#define GEMM_STAGES 1
+#define WG_PER_CU 4
+#define KATTN_BN 64
+#endif
+#define VAR1_BM 64
+#define VAR1_BN 128
+#define VAR2_BM 64
+#define VAR2_BN 64
+#define CMAX(a, b) ((a) > (b) ? (a) : (b))
+#define STAGE_FLOATS(bm, bn) (GEMM_STAGES * ((bm) + (bn)) * LDS_ROW)
+#define EPI_FLOATS(bm, bn) ((bn) * ((bm) + 8))
+#define VAR_FLOATS(bm, bn) CMAX (STAGE_FLOATS (bm, bn), EPI_FLOATS (bm, bn))
+#define GEMM_SMEM_FLOATS CMAX (CMAX (VAR_FLOATS (VAR0_BM, VAR0_BN), VAR_FLOATS (VAR1_BM, VAR1_BN)), \
+                               CMAX (VAR_FLOATS (VAR2_BM, VAR2_BN), STAGE_FLOATS (128, KATTN_BN)))
 #define GEMM_SMEM_BYTES (GEMM_SMEM_FLOATS * 4)
 
 __device__ __forceinline__ float4 ld4 (const float *p) { return *reinterpret_cast<const float4 *> (p); }
@@ -236,7 +264,7 @@ template <bool COH> struct TransLoader64
 // owning (BM/WM) x (BN/WN) built from 32x32 v_mfma_f32_32x32x2_f32 blocks.  The activation row is
 // the MFMA row index and the weight row the MFMA column, so each accumulator register holds 32
 // consecutive output channels of one output column: stores are 128-byte coalesced.
-// LDS is double buffered: one barrier per K slice.
+// One or two LDS stages (GEMM_STAGES); the K slice after the staged one always waits in registers.
 // ---------------------------------------------------------------------------------------------
 // LDS-only barrier: waits for this wave's LDS traffic, not for global loads still in flight.
 __device__ __forceinline__ void lds_barrier ()
@@ -245,11 +273,11 @@ __device__ __forceinline__ void lds_barrier ()
 }
 
 template <int BM, int BN, int WM, int WN, class ALoader, class BLoader>
-__device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kiters, float *smem,
+__device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, int kiters, float *smem,
     floatx16 (&acc)[BN / WN / 32][BM / WM / 32])
 {
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-    constexpr int STAGE = (BM + BN) * LDS_ROW;
+    constexpr int STAGE = GEMM_STAGES == 2 ? (BM + BN) * LDS_ROW : 0;
     constexpr int KK = GEMM_BK / 8;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);
@@ -264,9 +292,9 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kiters,
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
     float4 areg[ALoader::R], breg[BLoader::R];
-    al.load (0, areg); bl.load (0, breg);
+    al.load (kbase, areg); bl.load (kbase, breg);
     al.store (smem, areg); bl.store (smem + BM * LDS_ROW, breg);
-    if (kiters > 1) { al.load (1, areg); bl.load (1, breg); }
+    if (kiters > 1) { al.load (kbase + 1, areg); bl.load (kbase + 1, breg); }
     lds_barrier ();
 
     for (int it = 0; it < kiters; it++)
@@ -280,9 +308,15 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kiters,
         for (int j = 0; j < TM; j++) af[0][j] = ld4 (S + afrag + j * 32 * LDS_ROW);
         #pragma unroll
         for (int i = 0; i < TN; i++) bf[0][i] = ld4 (S + bfrag + i * 32 * LDS_ROW);
+#ifdef EXP_SETPRIO
+        __builtin_amdgcn_s_setprio (EXP_SETPRIO);
+#endif
         #pragma unroll
         for (int kk = 0; kk < KK; kk++)
         {
+#ifdef EXP_IGLP
+            __builtin_amdgcn_iglp_opt (EXP_IGLP);
+#endif
             const int cur = kk & 1, nxt = cur ^ 1;
             if (kk + 1 < KK)
             {
@@ -291,12 +325,12 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kiters,
                 #pragma unroll
                 for (int i = 0; i < TN; i++) bf[nxt][i] = ld4 (S + bfrag + i * 32 * LDS_ROW + (kk + 1) * 8);
             }
-            else if (more)
+            else if (more && GEMM_STAGES == 2)
             {
                 // the next K slice (in registers since the previous iteration) goes to the other stage,
                 // overlapping with the last group of MFMAs; then its successor is requested from memory
                 al.store (Snext, areg); bl.store (Snext + BM * LDS_ROW, breg);
-                if (it + 2 < kiters) { al.load (it + 2, areg); bl.load (it + 2, breg); }
+                if (it + 2 < kiters) { al.load (kbase + it + 2, areg); bl.load (kbase + it + 2, breg); }
             }
             #pragma unroll
             for (int i = 0; i < TN; i++)
@@ -309,6 +343,17 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kiters,
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[cur][i].w, af[cur][j].w, acc[i][j], 0, 0, 0);
                 }
         }
+#ifdef EXP_SETPRIO
+        __builtin_amdgcn_s_setprio (0);
+#endif
+        if (GEMM_STAGES == 1 && more)
+        {
+            // single stage: once every wave has read its last fragments, the slice waiting in
+            // registers replaces the one in LDS and the slice after it is requested from memory
+            lds_barrier ();
+            al.store (Snext, areg); bl.store (Snext + BM * LDS_ROW, breg);
+            if (it + 2 < kiters) { al.load (kbase + it + 2, areg); bl.load (kbase + it + 2, breg); }
+        }
         lds_barrier ();
     }
 }
@@ -318,8 +363,10 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kiters,
 #define ACC_N(wn0, i, v, lane) ((wn0) + 32 * (i) + 8 * ((v) >> 2) + 4 * ((lane) >> 5) + ((v) & 3))
 
 // conv / FC / matmul tile
+// `slice` < 0: the whole K axis, bias + activation, result to the layer's matrix.  `slice` >= 0 (split-K):
+// K slices [slice*kiters_per_split, ...) only, raw sums to that slice's partial matrix.
 template <int BM, int BN, int WM, int WN, bool COH>
-__device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, float *smem)
+__device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, int slice, float *smem)
 {
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -327,24 +374,31 @@ __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, ui
     floatx16 acc[TN][TM];
     ActView<COH> in, out;
     in.init (L.in0, L.type == FC_LAYER ? L.N * L.IH * L.IW : (L.type == CONV_LAYER ? (L.N / (L.OH * L.OW)) * L.IH * L.IW : L.N), L.ld0);
-    out.init (L.out, L.N, L.ld);
+    int kbase = 0, kiters = (int)(L.Kp / GEMM_BK);
+    if (slice >= 0)
+    {
+        kbase = slice * (int)L.kiters_per_split;
+        kiters = min ((int)L.kiters_per_split, kiters - kbase);
+        out.init (L.partial + (size_t)slice * L.N * L.ld, L.N, L.ld);
+    }
+    else
+        out.init (L.out, L.N, L.ld);
     RowLoader<BM> al;
     al.init (L.weight, m0, 0xffffffffu, L.Kp, tid);
-    const int kiters = (int)(L.Kp / GEMM_BK);
     if (L.direct)
     {
         ActRowLoader<BN, COH> bl;
         bl.init (in, n0, L.N - 1, L.ld0, 0, tid);
-        gemm_core<BM, BN, WM, WN> (al, bl, kiters, smem, acc);
+        gemm_core<BM, BN, WM, WN> (al, bl, kbase, kiters, smem, acc);
     }
     else
     {
         ConvLoader<BN, COH> bl;
         bl.init (L, in, n0, tid);
-        gemm_core<BM, BN, WM, WN> (al, bl, kiters, smem, acc);
+        gemm_core<BM, BN, WM, WN> (al, bl, kbase, kiters, smem, acc);
     }
     const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);
-    const int act = L.act;
+    const int act = slice >= 0 ? NO_ACTIVATION : L.act;
     // Epilogue through LDS (free after the last K slice): the raw accumulators are parked as
     // [column][channel]; a rolled loop then adds the bias, applies the activation and writes 128-bit
     // pieces, so a wavefront covers whole 512-byte (BM = 128) / 256-byte (BM = 64) runs of a column.
@@ -365,7 +419,7 @@ __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, ui
     if (c < mrem)
     {
         float4 b = make_float4 (0.f, 0.f, 0.f, 0.f);
-        if (L.bias)
+        if (L.bias && slice < 0)
         {
             if (c + 4 <= mrem) b = ld4 (L.bias + m0 + c);
             else { b.x = L.bias[m0 + c]; if (c + 1 < mrem) b.y = L.bias[m0 + c + 1]; if (c + 2 < mrem) b.z = L.bias[m0 + c + 2]; }
@@ -381,6 +435,38 @@ __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, ui
         }
     }
     __syncthreads ();
+}
+
+// split-K finishing tile: sum of the slices + bias, activation
+template <bool COH>
+__device__ __forceinline__ void tile_splitk_finish (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm)
+{
+    const uint32_t m0 = tm * L.tile_m, n0 = tn * L.tile_n, C4 = L.tile_m >> 2;
+    const uint32_t rows = min (L.tile_n, L.N - n0), mrem = L.M - m0;
+    ActView<COH> part, out;
+    part.init (L.partial, L.N * L.splits, L.ld); out.init (L.out, L.N, L.ld);
+    for (uint32_t idx = threadIdx.x; idx < rows * C4; idx += WG_THREADS)
+    {
+        const uint32_t r = idx / C4, c = (idx - r * C4) * 4;
+        if (c >= mrem) continue;
+        float4 v = make_float4 (0.f, 0.f, 0.f, 0.f);
+        for (uint32_t s = 0; s < L.splits; s++)
+        {
+            const float4 p = part.ld4 ((s * L.N + n0 + r) * L.ld + m0 + c);
+            v.x += p.x; v.y += p.y; v.z += p.z; v.w += p.w;
+        }
+        if (L.bias)
+        {
+            v.x += L.bias[m0 + c];
+            if (c + 1 < mrem) v.y += L.bias[m0 + c + 1];
+            if (c + 2 < mrem) v.z += L.bias[m0 + c + 2];
+            if (c + 3 < mrem) v.w += L.bias[m0 + c + 3];
+        }
+        v = act4 (v, L.act);
+        const uint32_t o = (n0 + r) * L.ld + m0 + c;
+        if (c + 4 <= mrem) out.st4 (o, v);
+        else { out.st1 (o, v.x); if (c + 1 < mrem) out.st1 (o + 1, v.y); if (c + 2 < mrem) out.st1 (o + 2, v.z); }
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -509,7 +595,7 @@ __device__ __forceinline__ void tile_softmax (const aspen_hip_layer_t &L, uint32
 
 // ---------------------------------------------------------------------------------------------
 // Attention tiles.
-// K tile: one (batch, head) x 128 queries x all keys.  scores = K.Q on the matrix cores, 128 keys at
+// K tile: one (batch, head) x KATTN_BN queries x all keys.  scores = K.Q on the matrix cores, 128 keys at
 // a time; causal mask (-1e10 before the 1/sqrt(hd) scale), exp without max subtraction and the row
 // sums are fused into the epilogue; a second sweep over the tile's own output divides by the sums.
 // in0 = Query matrix, in1 = Key matrix (reference cfg: parent = Query, from = Key).
@@ -517,7 +603,7 @@ __device__ __forceinline__ void tile_softmax (const aspen_hip_layer_t &L, uint32
 template <bool COH>
 __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, uint32_t tn, float *smem)
 {
-    constexpr int BM = 128, BN = 128, WM = 2, WN = 2, TM = 2, TN = 2;
+    constexpr int BM = 128, BN = KATTN_BN, WM = 2, WN = 2, TM = BM / WM / 32, TN = BN / WN / 32;
     __shared__ float rowsum[BN];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t S = L.seq, qtiles = (S + BN - 1) / BN;
@@ -541,7 +627,7 @@ __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, ui
         floatx16 acc[TN][TM];
         ActRowLoader<BM, COH> al; al.init (Kmat, b * S + k0, b * S + S - 1, L.ld1, h * L.hd, tid);
         ActRowLoader<BN, COH> bl; bl.init (Q, b * S + q0, b * S + S - 1, L.ld0, h * L.hd, tid);
-        gemm_core<BM, BN, WM, WN> (al, bl, kiters, smem, acc);
+        gemm_core<BM, BN, WM, WN> (al, bl, 0, kiters, smem, acc);
         #pragma unroll
         for (int j = 0; j < TM; j++)
         {
@@ -611,7 +697,7 @@ __device__ __forceinline__ void tile_v_attention (const aspen_hip_layer_t &L, ui
     floatx16 acc[TN][TM];
     TransLoader64<COH> al; al.init (V, b * S * L.ld1 + m0, L.ld1, L.tile_m, S, tid);
     ActRowLoader<BN, COH> bl; bl.init (P, prow + q0, prow + S - 1, L.ld0, 0, tid);   // P's stride is a multiple of 32 with zero padding
-    gemm_core<BM, BN, WM, WN> (al, bl, (int)((S + GEMM_BK - 1) / GEMM_BK), smem, acc);
+    gemm_core<BM, BN, WM, WN> (al, bl, 0, (int)((S + GEMM_BK - 1) / GEMM_BK), smem, acc);
     const uint32_t mm = wm0 + (lane & 31);
     if (mm < L.tile_m)
         #pragma unroll
@@ -632,13 +718,27 @@ __device__ __forceinline__ void tile_v_attention (const aspen_hip_layer_t &L, ui
 template <bool COH>
 __device__ __forceinline__ void run_tile (const aspen_hip_layer_t &L, uint32_t t, float *smem)
 {
+    int slice = -1;
+    if (L.splits > 1)
+    {
+        const uint32_t T = L.tiles_m * L.tiles_n;
+        if (t >= T * L.splits)
+        {
+            t -= T * L.splits;
+            const uint32_t fn = t / L.tiles_m;
+            tile_splitk_finish<COH> (L, fn, t - fn * L.tiles_m);
+            return;
+        }
+        slice = (int)(t % L.splits);
+        t /= L.splits;
+    }
     const uint32_t tn = t / L.tiles_m, tm = t - tn * L.tiles_m;
     switch (L.type)
     {
     case CONV_LAYER: case FC_LAYER: case MATMUL_LAYER:
-        if (L.variant == ASPEN_HIP_GEMM_128x128) tile_contraction<128, 128, 2, 2, COH> (L, tn, tm, smem);
-        else if (L.variant == ASPEN_HIP_GEMM_64x128) tile_contraction<64, 128, 2, 2, COH> (L, tn, tm, smem);
-        else tile_contraction<64, 64, 2, 2, COH> (L, tn, tm, smem);
+        if (L.variant == ASPEN_HIP_GEMM_LARGE) tile_contraction<VAR0_BM, VAR0_BN, 2, 2, COH> (L, tn, tm, slice, smem);
+        else if (L.variant == ASPEN_HIP_GEMM_WIDE) tile_contraction<VAR1_BM, VAR1_BN, 2, 2, COH> (L, tn, tm, slice, smem);
+        else tile_contraction<VAR2_BM, VAR2_BN, 2, 2, COH> (L, tn, tm, slice, smem);
         break;
     case RESIDUAL_LAYER:    tile_residual<COH> (L, tn); break;
     case MAXPOOL_LAYER:     tile_pool<true, COH> (L, tn); break;

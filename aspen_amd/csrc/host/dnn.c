@@ -224,6 +224,18 @@ done:
 /* ---------------------------------------------------------------------------------------------- */
 static unsigned int round_up (unsigned int v, unsigned int to) { return (v + to - 1) / to * to; }
 
+/* padded K of the device layout / 32 (must agree with aspen_layer_to_device) */
+unsigned int aspen_layer_kiters (const aspen_layer_t *L)
+{
+    const unsigned int *p = L->params;
+    unsigned int taps, ic;
+    if (L->type == CONV_LAYER) { taps = p[WEIGHT_H] * p[WEIGHT_W]; ic = p[IN_C]; }
+    else if (L->type == FC_LAYER) { taps = p[IN_H] * p[IN_W]; ic = p[IN_C]; }
+    else if (L->type == MATMUL_LAYER) { taps = 1; ic = p[MAT_K]; }
+    else return 0;
+    return round_up (taps * round_up (ic, 4), 32) / 32;
+}
+
 /* Uploads weight / bias / k-chunk table of one layer for a parent whose column stride is parent_ld
    floats.  Idempotent; re-run after the weights changed. */
 int aspen_layer_to_device (aspen_layer_t *L, unsigned int parent_ld)

@@ -52,6 +52,12 @@ int aspen_rpool_profile_layers (rpool_t *rp, unsigned int iters, float *ms)
     return aspen_hip_profile_layers (rp->graph, iters, ms);
 }
 
+int aspen_rpool_dataflow_profile (rpool_t *rp, uint64_t ticks[4], int reset)
+{
+    if (rp == NULL || rp->graph == NULL) return -1;
+    return aspen_hip_dataflow_profile (rp->graph, ticks, reset);
+}
+
 unsigned int aspen_rpool_num_ninst (rpool_t *rp)
 {
     unsigned int n = 0;

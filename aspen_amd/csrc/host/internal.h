@@ -62,6 +62,11 @@ struct nasm_ldata_t
     unsigned int tile_dims[2];
     unsigned int tiles_w, tiles_h;
     unsigned int num_ninst, ninst_start;
+    /* split-K: a contraction layer with too few output tiles cuts its K axis into `splits` slices;
+       tile indices [0, T*splits) (T = tiles_w*tiles_h) are partial products (tile*splits + slice),
+       [T*splits, T*splits + T) the finishing tiles that sum the slices, add bias, activate */
+    unsigned int splits, kiters_per_split;
+    size_t partial_offset;                   /* floats into the arena: [splits][columns][stride] */
     int variant;
     uint64_t flops;                          /* 2*M*N*K for contraction layers, 64-bit */
 };
@@ -112,6 +117,7 @@ aspen_dnn_t *aspen_parse_cfg (const char *path);
 /* dnn.c */
 int aspen_layer_to_device (aspen_layer_t *layer, unsigned int parent_ld);
 int aspen_load_weight_file (aspen_dnn_t *dnn, const char *path);
+unsigned int aspen_layer_kiters (const aspen_layer_t *layer);   /* K slices of 32 of a contraction layer's device layout */
 /* nasm.c */
 int aspen_nasm_to_device (nasm_t *nasm);
 int aspen_nasm_fill_device_layers (nasm_t *nasm, aspen_hip_layer_t *dst, uint32_t ninst_base);

@@ -84,7 +84,7 @@ static int set_out_mat (nasm_t *nasm, nasm_ldata_t *ld)
 }
 
 /* Tile policy.  min_ninst = wanted tiles per layer (the knob of apu_create_nasm): the largest tile
-   shape that still yields that many tiles is taken, so big layers get 128 x 128 MFMA tiles and
+   shape that still yields that many tiles is taken, so big layers get the large MFMA tiles and
    small ones are cut finer to keep all compute units busy. */
 static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
 {
@@ -92,6 +92,7 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
     const unsigned int M = ld->out_mat_dims[OUT_H], N = ld->out_mat_dims[OUT_W];
     const unsigned int want = nasm->min_ninst_per_ldata;
     ld->variant = 0;
+    ld->splits = 1; ld->kiters_per_split = 0;
     if (L->type == INPUT_LAYER)
     {
         ld->tile_dims[OUT_H] = M; ld->tile_dims[OUT_W] = N; ld->tiles_h = ld->tiles_w = 0; ld->num_ninst = 0;
@@ -99,10 +100,13 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
     }
     if (is_contraction (L->type))
     {
-        static const unsigned int bm[ASPEN_HIP_NUM_GEMM_VARIANTS] = {128, 64, 64}, bn[ASPEN_HIP_NUM_GEMM_VARIANTS] = {128, 128, 64};
-        int v = M <= 64 ? ASPEN_HIP_GEMM_64x128 : ASPEN_HIP_GEMM_128x128;
-        while (v < ASPEN_HIP_GEMM_64x64 && cdiv (M, bm[v]) * cdiv (N, bn[v]) < want) v++;
-        if (N <= 64) v = ASPEN_HIP_GEMM_64x64;
+        uint32_t shp[9];
+        aspen_hip_tile_shapes (shp);
+        const unsigned int bm[ASPEN_HIP_NUM_GEMM_VARIANTS] = {shp[0], shp[2], shp[4]}, bn[ASPEN_HIP_NUM_GEMM_VARIANTS] = {shp[1], shp[3], shp[5]};
+        /* few output rows: the wide shape; otherwise the large one; either falls back to the small
+           shape when it would leave the layer with fewer tiles than wanted */
+        int v = M <= 64 ? ASPEN_HIP_GEMM_WIDE : ASPEN_HIP_GEMM_LARGE;
+        if (cdiv (M, bm[v]) * cdiv (N, bn[v]) < want || (N <= 64 && v == ASPEN_HIP_GEMM_WIDE)) v = ASPEN_HIP_GEMM_SMALL;
         ld->variant = v;
         ld->tile_dims[OUT_H] = bm[v]; ld->tile_dims[OUT_W] = bn[v];
     }
@@ -110,8 +114,10 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
     {
         const unsigned int S = nasm->tr_seq_len, hd = L->params[NUM_HIDDEN] / L->params[NUM_HEAD];
         if (hd % 32 != 0) { ERROR_PRTF ("layer %u: head size %u must be a multiple of 32\n", L->layer_idx, hd); return -1; }
-        ld->tile_dims[OUT_H] = M; ld->tile_dims[OUT_W] = 128;
-        ld->tiles_h = 1; ld->tiles_w = (N / S) * cdiv (S, 128);
+        uint32_t shp[9];
+        aspen_hip_tile_shapes (shp);
+        ld->tile_dims[OUT_H] = M; ld->tile_dims[OUT_W] = shp[6];
+        ld->tiles_h = 1; ld->tiles_w = (N / S) * cdiv (S, shp[6]);
         ld->num_ninst = ld->tiles_w;
         return 0;
     }
@@ -138,6 +144,19 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
     ld->tiles_h = cdiv (M, ld->tile_dims[OUT_H]);
     ld->tiles_w = cdiv (N, ld->tile_dims[OUT_W]);
     ld->num_ninst = ld->tiles_h * ld->tiles_w;
+    if (is_contraction (L->type))
+    {
+        /* still short of tiles with the smallest shape: cut the K axis (at least 8 slices of 32 per part) */
+        const unsigned int kiters = aspen_layer_kiters (L), T = ld->num_ninst;
+        ld->kiters_per_split = kiters;
+        if (T < want && kiters >= 16 && getenv ("ASPEN_GPU_NO_SPLITK") == NULL)
+        {
+            unsigned int s = umin (umin (cdiv (want, T), kiters / 8), 8);
+            ld->kiters_per_split = cdiv (kiters, s);
+            ld->splits = cdiv (kiters, ld->kiters_per_split);
+            if (ld->splits > 1) ld->num_ninst = T * ld->splits + T;
+        }
+    }
     return 0;
 }
 
@@ -158,6 +177,11 @@ static unsigned int col_tile_of (const nasm_ldata_t *ld, unsigned int col)
 
 static void tile_range (const nasm_ldata_t *ld, unsigned int t, unsigned int *c0, unsigned int *c1, unsigned int *r0, unsigned int *r1)
 {
+    if (ld->splits > 1)
+    {
+        const unsigned int T = ld->tiles_h * ld->tiles_w;
+        t = t < T * ld->splits ? t / ld->splits : t - T * ld->splits;
+    }
     const unsigned int tn = t / ld->tiles_h, tm = t % ld->tiles_h;      /* row tile fastest (reference src/apu_nasm.c:1218-1224) */
     const unsigned int S = seq_block (ld), tw = ld->tile_dims[OUT_W];
     if (S == 0) { *c0 = tn * tw; *c1 = umin (*c0 + tw, ld->out_mat_dims[OUT_W]); }
@@ -190,7 +214,7 @@ static void add_parents (const nasm_ldata_t *pl, unsigned int c0, unsigned int c
     const unsigned int m0 = r0 / pl->tile_dims[OUT_H], m1 = (r1 - 1) / pl->tile_dims[OUT_H];
     for (unsigned int t = t0; t <= t1; t++)
         for (unsigned int m = m0; m <= m1; m++)
-            push (out, pl->ninst_start + t * pl->tiles_h + m);
+            push (out, pl->ninst_start + (pl->splits > 1 ? pl->tiles_h * pl->tiles_w * pl->splits : 0) + t * pl->tiles_h + m);
 }
 
 /* parents of tile t of layer ld (semantics: reference src/apu_nasm.c:49-466) */
@@ -203,6 +227,12 @@ static void find_parents (const nasm_t *nasm, const nasm_ldata_t *ld, unsigned i
     unsigned int c0, c1, r0, r1;
     tile_range (ld, t, &c0, &c1, &r0, &r1);
     const unsigned int S = nasm->tr_seq_len;
+    if (ld->splits > 1 && t >= ld->tiles_h * ld->tiles_w * ld->splits)
+    {
+        const unsigned int tile = t - ld->tiles_h * ld->tiles_w * ld->splits;
+        for (unsigned int s = 0; s < ld->splits; s++) push (out, ld->ninst_start + tile * ld->splits + s);
+        return;
+    }
     switch (L->type)
     {
     case CONV_LAYER: case MAXPOOL_LAYER: case AVGPOOL_LAYER:
@@ -339,6 +369,11 @@ static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned i
         }
         ld->out_mat_offset = arena;
         arena += ((size_t)ld->out_mat_stride * ld->out_mat_dims[OUT_W] + 63) / 64 * 64;    /* 256-byte aligned matrices */
+        if (ld->splits > 1)
+        {
+            ld->partial_offset = arena;
+            arena += ((size_t)ld->splits * ld->out_mat_stride * ld->out_mat_dims[OUT_W] + 63) / 64 * 64;
+        }
         ld->ninst_start = total;
         total += ld->num_ninst;
         nasm->total_flops += ld->flops;
@@ -449,6 +484,8 @@ int aspen_nasm_fill_device_layers (nasm_t *nasm, aspen_hip_layer_t *dst, uint32_
         d->tile_m = ld->tile_dims[OUT_H]; d->tile_n = ld->tile_dims[OUT_W];
         d->tiles_m = ld->tiles_h; d->tiles_n = ld->tiles_w;
         d->ninst_start = ninst_base + ld->ninst_start; d->num_ninst = ld->num_ninst;
+        d->splits = ld->splits; d->kiters_per_split = ld->kiters_per_split;
+        d->partial = ld->splits > 1 ? nasm->d_arena + ld->partial_offset : NULL;
         d->out = nasm->d_arena + ld->out_mat_offset;
         if (ld->parent_ldata_idx[PARENT_0] >= 0)
         {

@@ -101,6 +101,7 @@ def main():
     ap.add_argument("--workgroups", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--skip-tiles", action="store_true", help="scheduler-only run: dependency protocol with empty tiles")
+    ap.add_argument("--engine-profile", action="store_true", help="report where the persistent workgroups spend their time")
     ap.add_argument("--layer-profile", action="store_true", help="also time every layer's kernel (layer-launch mode)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -113,8 +114,7 @@ def main():
         print("bench.py: no HIP device: " + L.aspen_hip_last_error().decode(), file=sys.stderr)
         sys.exit(1)
     dev = api.device_info()
-    if args.skip_tiles:
-        L.aspen_hip_set_flags(1)
+    L.aspen_hip_set_flags((1 if args.skip_tiles else 0) | (4 if args.engine_profile else 0))
     cfgs, unit, units_per_step = WORKLOADS[args.workload]
 
     pool = api.RPool()
@@ -151,6 +151,8 @@ def main():
     for _ in range(args.warmup):
         step()
     L.aspen_hip_sync()
+    if args.engine_profile and args.mode == "dataflow":
+        pool.dataflow_profile(reset=True)
     kernel_ms = []
     ms = api.C.c_float()
     t0 = time.perf_counter()
@@ -183,6 +185,10 @@ def main():
                            "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": ach / PEAK_FP32_MFMA_TFLOPS,
                            "traffic": None, "flops_per_launch": flops, "kernel_ms": ms_per_step}
 
+    if args.engine_profile and args.mode == "dataflow":
+        prof = pool.dataflow_profile()
+        out["engine_profile"] = {k: v / max(prof["total"], 1e-12) for k, v in prof.items() if k != "total"}
+        out["engine_profile"]["workgroup_seconds_per_step"] = prof["total"] / args.steps
     if args.layer_profile:
         # conv-tile MFMA utilisation and bandwidth of the elementwise tiles, one kernel per layer
         nl = sum(n.num_ldata for _, _, n, _ in nets)

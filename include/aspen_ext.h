@@ -38,6 +38,8 @@ int aspen_rpool_run_stats (rpool_t *rpool, uint32_t *executed, uint32_t *double_
 /* per-layer kernel time (ms) of the pool's merged graph in layer-launch mode, averaged over iters;
    ms must hold one float per layer of every attached nasm, in attachment order */
 int aspen_rpool_profile_layers (rpool_t *rpool, unsigned int iters, float *ms);
+/* where the workgroups of the dataflow kernel spent their time (needs ASPEN_HIP_FLAG_PROFILE) */
+int aspen_rpool_dataflow_profile (rpool_t *rpool, uint64_t ticks[4], int reset);
 /* tiles in the pool's merged graph */
 unsigned int aspen_rpool_num_ninst (rpool_t *rpool);
 

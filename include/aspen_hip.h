@@ -38,8 +38,14 @@ typedef struct aspen_hip_ktab_t
     uint16_t kh, kw;     /* tap; kh >= 0x4000 marks a chunk beyond the real K (reads as zero) */
 } aspen_hip_ktab_t;
 
-/* GEMM tile shapes (rows of the weight matrix x activation columns per workgroup). */
-enum { ASPEN_HIP_GEMM_128x128 = 0, ASPEN_HIP_GEMM_64x128 = 1, ASPEN_HIP_GEMM_64x64 = 2, ASPEN_HIP_NUM_GEMM_VARIANTS };
+/* GEMM tile shapes (rows of the weight matrix x activation columns per workgroup): LARGE = the
+   biggest shape of the build (128 x 64 by default), WIDE = 64 x 128, SMALL = 64 x 64.  The graph
+   builder asks aspen_hip_tile_shapes for the numbers instead of assuming them. */
+enum { ASPEN_HIP_GEMM_LARGE = 0, ASPEN_HIP_GEMM_WIDE = 1, ASPEN_HIP_GEMM_SMALL = 2, ASPEN_HIP_NUM_GEMM_VARIANTS };
+/* shapes[2*v] = rows, shapes[2*v+1] = columns of GEMM variant v; shapes[6] = queries per K-attention
+   tile; shapes[7] = queries per V-attention tile; shapes[8] = workgroups per compute unit the
+   kernels are built for.  Pure constants: callable without a GPU. */
+void aspen_hip_tile_shapes (uint32_t shapes[9]);
 
 /* Per-layer descriptor: everything one tile needs, so a tile is (layer, tile index).
    Replaces the fields the reference's tiled_* read through ninst->ldata->layer
@@ -59,7 +65,12 @@ typedef struct aspen_hip_layer_t
     uint32_t ld0, ld1;       /* strides of the parents */
     uint32_t IH, IW, IC, OH, OW, KH, KW, stride, pad;
     uint32_t heads, seq, hd, masked;
+    /* split-K (contraction layers): tiles [0, T*splits) with T = tiles_m*tiles_n are partial products
+       over kiters_per_split K slices each (tile*splits + slice) written to `partial`
+       ([splits][N][ld]); tiles [T*splits, T*splits + T) sum the slices, add bias, activate */
+    uint32_t splits, kiters_per_split;
     uint32_t reserved;
+    float *partial;
     float *out;
     const float *in0;        /* PARENT_0 */
     const float *in1;        /* PARENT_1 */
@@ -109,6 +120,12 @@ int aspen_hip_run_dataflow (aspen_hip_graph_t *graph, uint32_t workgroups, uint6
 /* COUNT_TILES keeps the per-tile execution counters that aspen_hip_dataflow_stats reports (one extra
    pair of atomics per tile); without it `executed` and `double_runs` read 0. */
 #define ASPEN_HIP_FLAG_COUNT_TILES 2u
+/* PROFILE makes every workgroup of the dataflow kernel accumulate where its time went. */
+#define ASPEN_HIP_FLAG_PROFILE 4u
+/* ticks (100 MHz) summed over all workgroups since the last reset: [0] inside tiles, [1] waiting for
+   the tile's stores to be acknowledged, [2] scheduling (publish, pop, waiting for a ready tile),
+   [3] total workgroup lifetime */
+int aspen_hip_dataflow_profile (aspen_hip_graph_t *graph, uint64_t ticks[4], int reset);
 void aspen_hip_set_flags (uint32_t flags);
 int aspen_hip_sync (void);
 /* 1 when everything enqueued so far has finished, 0 when still running */

@@ -68,7 +68,7 @@ def test_full_config_matches_reference_summary(gpu, name):
     reference: per layer sampled relative L2, norm and sum; identical argmax per image / token."""
     cfg, layers, tens, x, batch, seq = H.full_config(name)
     gold = np.load(os.path.join(H.GOLDEN, f"{name}.npz"))
-    net = H.GpuNet(cfg, tens, batch, seq, mode=api.MODE_DATAFLOW)
+    net = H.GpuNet(cfg, tens, batch, seq, min_ninst=1024, mode=api.MODE_DATAFLOW)
     print(f"config {name} tiles {net.nasm.num_ninst} edges {net.nasm.num_edges}", flush=True)
     try:
         net.run(x)
