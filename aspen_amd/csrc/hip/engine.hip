@@ -34,6 +34,7 @@ struct aspen_hip_graph_t
     uint32_t *d_state;      // one counter per 128-byte line: [ST_HEAD] pop tickets, [ST_TAIL] push cursor, [ST_DONE] tiles done,
                             // [ST_ABORT] abort flag, [ST_TWICE] tiles executed more than once
     uint32_t *d_ran;        // per-tile execution count (sanity: every tile exactly once)
+    uint32_t epoch;         // tag of the last run's queue entries, cycles 1..255
     unsigned long long *d_prof;
 };
 
@@ -43,6 +44,7 @@ static int g_inited = 0;
 static int g_num_cu = 0;
 static char g_err[512] = "";
 static uint32_t g_flags = 0;
+static uint32_t *g_host_abort = nullptr;    // pinned host word the persistent kernel raises when it gives up waiting
 
 static int fail (hipError_t e, const char *what)
 {
@@ -68,18 +70,31 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) layer_kernel (const as
     run_tile<false> (L, t, smem);
 }
 
-// Re-arm: counters back to the parent counts, queue emptied and seeded with the roots.
+// Re-arm: counters back to the parent counts, queue seeded with the roots.  Queue entries carry the
+// run's epoch in their top byte (entry = epoch << 24 | tile): an entry left over from an earlier
+// run never matches the current epoch, so the queue needs no clearing and a poll can never mistake
+// an old entry for a new one.  All writes are device-scope (write-through) stores, the same path
+// the persistent kernel's polls and atomics use.
+#define QUEUE_ID_BITS 24
+#define QUEUE_ID_MASK ((1u << QUEUE_ID_BITS) - 1u)
 __global__ void arm_kernel (uint32_t *dep, const uint32_t *num_parents, uint32_t *queue, uint32_t *ran,
-    const uint32_t *roots, uint32_t num_ninst, uint32_t num_roots, uint32_t *state)
+    const uint32_t *roots, uint32_t num_ninst, uint32_t num_roots, uint32_t *state, uint32_t epoch)
 {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < num_ninst)
     {
-        dep[i] = num_parents[i];
-        queue[i] = i < num_roots ? roots[i] : QUEUE_EMPTY;
-        ran[i] = 0;
+        __hip_atomic_store (&dep[i], num_parents[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (i < num_roots) __hip_atomic_store (&queue[i], (epoch << QUEUE_ID_BITS) | roots[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store (&ran[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (i == 0) { state[ST_HEAD] = 0; state[ST_TAIL] = num_roots; state[ST_DONE] = 0; state[ST_ABORT] = 0; state[ST_TWICE] = 0; }
+    if (i == 0)
+    {
+        __hip_atomic_store (&state[ST_HEAD], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store (&state[ST_TAIL], num_roots, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store (&state[ST_DONE], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store (&state[ST_ABORT], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store (&state[ST_TWICE], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 }
 
 struct dataflow_args_t
@@ -87,8 +102,10 @@ struct dataflow_args_t
     const aspen_hip_layer_t *layers;
     const uint32_t *ninst_layer, *child_off, *child_idx;
     uint32_t *dep, *queue, *state, *ran;
+    uint32_t *host_abort;
     unsigned long long *prof;       // [0] tile, [1] store drain, [2] publish / pop, [3] total: summed 100 MHz ticks of all workgroups
     uint32_t num_ninst;
+    uint32_t epoch;                 // 1..255, tag of this run's queue entries
     uint32_t flags;                 // ASPEN_HIP_FLAG_*
     unsigned long long spin_limit;
 };
@@ -109,13 +126,14 @@ __device__ __forceinline__ uint32_t wait_for_slot (const dataflow_args_t &a, uin
     unsigned long long spins = 0;
     for (;;)
     {
-        const uint32_t id = __hip_atomic_load (&a.queue[ticket], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (id != QUEUE_EMPTY) return id;
+        const uint32_t e = __hip_atomic_load (&a.queue[ticket], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((e >> QUEUE_ID_BITS) == a.epoch) return e & QUEUE_ID_MASK;
         ++spins;
         if ((spins & 63) == 0 && __hip_atomic_load (&a.state[ST_ABORT], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return QUEUE_EMPTY;
         if (spins > a.spin_limit)
         {
             __hip_atomic_store (&a.state[ST_ABORT], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store (a.host_abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
             return QUEUE_EMPTY;
         }
         __builtin_amdgcn_s_sleep (2);
@@ -157,8 +175,9 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
             run_tile_coherent (L, id - L->ninst_start, smem);
 
         if (prof) { const unsigned long long t = wall_clock64 (); t_tile += t - t0; t0 = t; }
-        // every wave waits until its (write-through, device-coherent) stores have been acknowledged
-        __builtin_amdgcn_fence (__ATOMIC_RELEASE, "workgroup");
+        // every wave waits until its (write-through, device-coherent) stores have been acknowledged.
+        // An explicit wait: a workgroup-scope fence does not have to wait for global stores.
+        asm volatile ("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads ();
         if (prof) { const unsigned long long t = wall_clock64 (); t_drain += t - t0; t0 = t; }
         if (wave == 0)
@@ -173,7 +192,7 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
                 if (before == 1u)
                 {
                     const uint32_t slot = atomicAdd (&a.state[ST_TAIL], 1u);
-                    __hip_atomic_store (&a.queue[slot], child, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store (&a.queue[slot], (a.epoch << QUEUE_ID_BITS) | child, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
             if (lane == 0 && (a.flags & ASPEN_HIP_FLAG_COUNT_TILES))
@@ -206,6 +225,8 @@ extern "C" int aspen_hip_init (void)
     CHECK (hipGetDeviceProperties (&prop, 0));
     g_num_cu = prop.multiProcessorCount;
     CHECK (hipStreamCreate (&g_stream));
+    CHECK (hipHostMalloc ((void **)&g_host_abort, 64, hipHostMallocDefault));
+    *g_host_abort = 0;
     for (int i = 0; i < NUM_EVENTS; i++) CHECK (hipEventCreate (&g_events[i]));
     CHECK (hipFuncSetAttribute ((const void *)layer_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
     CHECK (hipFuncSetAttribute ((const void *)dataflow_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
@@ -345,6 +366,7 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     const uint32_t *child_idx, uint32_t num_ninst, const uint32_t *roots, uint32_t num_roots)
 {
     if (aspen_hip_init ()) return nullptr;
+    if (num_ninst > QUEUE_ID_MASK) { snprintf (g_err, sizeof (g_err), "graph has more than %u tiles", QUEUE_ID_MASK); return nullptr; }
     for (uint32_t l = 0; l < num_layers; l++)
         if (check_layer (layers[l], l)) return nullptr;
     // host-side sanity of the dependency structure: every index in range, counts consistent
@@ -429,13 +451,14 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     if (!g) { snprintf (g_err, sizeof (g_err), "run_dataflow: null graph"); return -1; }
     if (g->num_ninst == 0) return 0;
     if (workgroups == 0) workgroups = WG_PER_CU * (uint32_t)g_num_cu;
+    g->epoch = g->epoch % 255u + 1u;
     hipLaunchKernelGGL (arm_kernel, dim3 ((g->num_ninst + 255) / 256), dim3 (256), 0, g_stream,
-        g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->num_ninst, g->num_roots, g->d_state);
+        g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->num_ninst, g->num_roots, g->d_state, g->epoch);
     CHECK (hipGetLastError ());
     dataflow_args_t a;
     a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx;
-    a.dep = g->d_dep; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran; a.prof = g->d_prof;
-    a.num_ninst = g->num_ninst; a.flags = g_flags; a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
+    a.dep = g->d_dep; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran; a.prof = g->d_prof; a.host_abort = g_host_abort;
+    a.num_ninst = g->num_ninst; a.epoch = g->epoch; a.flags = g_flags; a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
     CHECK (hipEventRecord (g_events[NUM_EVENTS - 2], g_stream));
     hipLaunchKernelGGL (dataflow_kernel, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);
     CHECK (hipGetLastError ());
@@ -469,6 +492,13 @@ extern "C" int aspen_hip_sync (void)
 {
     if (aspen_hip_init ()) return -1;
     CHECK (hipStreamSynchronize (g_stream));
+    if (*(volatile uint32_t *)g_host_abort != 0)
+    {
+        *g_host_abort = 0;
+        snprintf (g_err, sizeof (g_err), "dataflow run stalled: a wait on the ready queue exceeded its spin limit and the run was aborted");
+        fprintf (stderr, "aspen_hip: %s\n", g_err);
+        return ASPEN_HIP_ERR_STALLED;
+    }
     return 0;
 }
 

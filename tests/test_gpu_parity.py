@@ -59,6 +59,27 @@ def test_micro_nets_match_oracle(gpu, name):
         net.close()
 
 
+def test_engine_rearm_many_runs(gpu):
+    """Re-arm and re-run one graph many times: every run must execute each tile exactly once, never
+    stall, and reproduce the first run bit for bit (tiles are deterministic; only their order varies)."""
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()["gpt_mini_b2_s20"])
+    net = H.GpuNet(cfg, tens, batch, seq, min_ninst=64, mode=api.MODE_DATAFLOW)
+    print(f"tiles {net.nasm.num_ninst}", flush=True)
+    try:
+        first = None
+        for rep in range(40):
+            net.run(x if rep == 0 else None)
+            st = net.rpool.run_stats()
+            assert st == {"executed": net.nasm.num_ninst, "double_runs": 0, "aborted": 0}, (rep, st)
+            out = net.layer(net.nasm.num_ldata - 1)
+            if first is None:
+                first = out
+            else:
+                assert np.array_equal(first, out), f"run {rep} differs from run 0"
+    finally:
+        net.close()
+
+
 FULL = ["resnet50_b1", "resnet50_b32", "vgg16_b32", "bert_base_b8_s128", "gpt2_b4_s512"]
 
 
