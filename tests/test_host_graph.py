@@ -1,0 +1,257 @@
+"""Host-side logic of the C library, no GPU needed: cfg parsing, out_mat geometry, the tile grid and
+the tile dependency graph (checked against a brute-force derivation from the layer semantics), FLOP
+accounting (against the totals in the reference's shipped .nasm headers) and error behaviour."""
+import os
+
+import numpy as np
+import pytest
+
+from aspen_amd import api, models as M
+from tests import helpers as H
+
+# TOTAL_FLOPS of the reference's shipped graphs (files/resnet50/resnet50_B1.nasm:5, files/vgg16/vgg16_B1.nasm:5)
+REF_TOTAL_FLOPS = {"resnet50": 8185945088, "vgg16": 30946800640}
+
+
+def make(case, min_ninst):
+    cfg, layers, tens, x, batch, seq = H.build_case(case)
+    d = api.Dnn(cfg, None)
+    return layers, d, api.Nasm(d, batch, seq, min_ninst), batch, seq
+
+
+def test_total_flops_match_reference_headers():
+    for gen, key in ((M.resnet50_cfg, "resnet50"), (M.vgg16_cfg, "vgg16")):
+        d = api.Dnn(gen(), None)
+        n = api.Nasm(d, 1, 0, 64)
+        assert n.total_flops == REF_TOTAL_FLOPS[key]
+        n.destroy(); d.destroy()
+    # 64-bit accounting: batch 32 is exactly 32x batch 1 (the reference's 32-bit sum overflows here)
+    d = api.Dnn(M.resnet50_cfg(), None)
+    n = api.Nasm(d, 32, 0, 64)
+    assert n.total_flops == 32 * REF_TOTAL_FLOPS["resnet50"] == 261950242816
+    n.destroy(); d.destroy()
+
+
+def test_out_mat_geometry_matches_cfg():
+    """rows = channels (or S for K-attention), columns = batch x positions; stride >= rows, multiple of 4."""
+    for name, case in H.micro_cases().items():
+        layers, d, n, batch, seq = make(case, 64)
+        assert n.num_ldata == len(layers)
+        for l, L in enumerate(layers):
+            i = n.info(l)
+            assert api.LAYER_TYPE_NAMES[i["type"]] == L["type"], (name, l)
+            if L["type"] == "attn_k":
+                assert (i["H"], i["W"]) == (seq, batch * L["n_head"] * seq)
+            elif seq:
+                assert (i["H"], i["W"]) == (L["C"], batch * seq)
+            else:
+                assert (i["H"], i["W"]) == (L["C"], batch * L["H"] * L["W"])
+            assert i["stride"] >= i["H"] and i["stride"] % 4 == 0
+        n.destroy(); d.destroy()
+
+
+def needed_regions(L, layers, c0, c1, r0, r1, batch, seq):
+    """Brute force from the layer semantics: for output columns [c0,c1) x rows [r0,r1) of layer L the
+    list of (parent layer, set of parent columns, row0, row1) it reads.  row1 None = all rows."""
+    t = L["type"]
+    p0, p1 = L["p0"], L["p1"]
+    cols = range(c0, c1)
+    if t in ("conv", "maxpool", "avgpool"):
+        OH, OW, IH, IW, k, s, p = L["H"], L["W"], L["inH"], L["inW"], L["size"], L["stride"], L["pad"]
+        need = set()
+        for c in cols:
+            b, oh, ow = c // (OH * OW), (c // OW) % OH, c % OW
+            for kh in range(k):
+                for kw in range(k):
+                    ih, iw = oh * s - p + kh, ow * s - p + kw
+                    if 0 <= ih < IH and 0 <= iw < IW:
+                        need.add((b * IH + ih) * IW + iw)
+        return [(p0, need, 0, None)] if t == "conv" else [(p0, need, r0, r1)]
+    if t == "fc":
+        hw = L["inH"] * L["inW"]
+        return [(p0, {b * hw + j for b in cols for j in range(hw)}, 0, None)]
+    if t == "residual":
+        return [(p0, set(cols), r0, r1), (p1, set(cols), r0, r1)]
+    if t in ("matmul", "layernorm", "softmax"):
+        return [(p0, set(cols), 0, None)]
+    if t == "attn_k":       # column = (b, head, query); rows = keys
+        Hn, hd = L["n_head"], L["n_embd"] // L["n_head"]
+        out = []
+        for c in cols:
+            b, h, q = c // (Hn * seq), (c // seq) % Hn, c % seq
+            out.append((p0, {b * seq + q}, h * hd, (h + 1) * hd))
+            out.append((p1, {b * seq + q}, h * hd, (h + 1) * hd))
+            # one parent holds the queries (only token q needed), the other the keys (every token of b);
+            # which is which is the cfg's business: require the union, accept it on both
+            out.append((p0, set(), 0, 0))
+        keys = {(c // (Hn * seq)) for c in cols}
+        heads = {((c // seq) % Hn) for c in cols}
+        for b in keys:
+            for h in heads:
+                out.append(("either", {b * seq + s for s in range(seq)}, h * hd, (h + 1) * hd))
+        return out
+    if t == "attn_v":       # column = token (b, s); rows = h*hd + d;  p0 = probabilities, p1 = values
+        Hn, hd = L["n_head"], L["n_embd"] // L["n_head"]
+        out = []
+        for h in range(r0 // hd, (r1 - 1) // hd + 1):
+            out.append((p0, {(c // seq) * Hn * seq + h * seq + c % seq for c in cols}, 0, None))
+        for b in {c // seq for c in cols}:
+            out.append((p1, {b * seq + s for s in range(seq)}, r0, r1))
+        return out
+    raise ValueError(t)
+
+
+@pytest.mark.parametrize("name,min_ninst", [("custom_b3", 16), ("resnet_mini_b2", 64), ("resnet_mini_b2", 1024),
+                                            ("vgg_mini_b5", 32), ("bert_mini_b2_s24", 16), ("gpt_mini_b2_s20", 256)])
+def test_tile_graph_against_brute_force(name, min_ninst):
+    layers, d, n, batch, seq = make(H.micro_cases()[name], min_ninst)
+    tl, npar, off, idx = n.graph()
+    T = n.num_ninst
+    infos = [n.info(l) for l in range(n.num_ldata)]
+    # ---- tiles partition every out_mat; split-K layers have splits*T partial tiles + T finishing tiles
+    owner, partial_of = [], {}
+    for l, i in enumerate(infos):
+        own = -np.ones((i["W"], i["H"]), dtype=np.int64)
+        tiles = [t for t in range(i["ninst_start"], i["ninst_start"] + i["num_ninst"])]
+        assert all(tl[t] == l for t in tiles)
+        ranges = {}
+        for t in tiles:
+            ranges.setdefault(n.tile_range(t), []).append(t)
+        for (c0, c1, r0, r1), ts in ranges.items():
+            assert 0 <= c0 < c1 <= i["W"] and 0 <= r0 < r1 <= i["H"]
+            assert (own[c0:c1, r0:r1] == -1).all(), (name, l, "tiles overlap")
+            own[c0:c1, r0:r1] = max(ts)            # the finishing tile has the highest index
+            if len(ts) > 1:
+                partial_of[max(ts)] = sorted(ts)[:-1]
+        if i["num_ninst"]:
+            assert (own >= 0).all(), (name, l, "tiles leave a gap")
+        owner.append(own)
+    # ---- parents from the CSR children lists
+    parents = [set() for _ in range(T)]
+    for t in range(T):
+        for c in idx[off[t]:off[t + 1]]:
+            assert tl[c] > tl[t] or (tl[c] == tl[t] and c > t)      # edges point forward
+            assert t not in parents[c]                               # no duplicate edges
+            parents[c].add(t)
+    assert [len(p) for p in parents] == list(npar)
+    # ---- every tile's parents = owners of every element it reads
+    finals = {f for f in partial_of}
+    partials = {p: f for f, ps in partial_of.items() for p in ps}
+    for t in range(T):
+        l = int(tl[t])
+        L = layers[l]
+        if t in finals:
+            assert parents[t] == set(partial_of[t]), (name, l, t)
+            continue
+        c0, c1, r0, r1 = n.tile_range(t)
+        need = set()
+        for (p, cols, ra, rb) in needed_regions(L, layers, c0, c1, r0, r1, batch, seq):
+            for pp in ([L["p0"], L["p1"]] if p == "either" else [p]):
+                if pp is None or not cols or infos[pp]["num_ninst"] == 0:
+                    continue
+                rb_ = infos[pp]["H"] if rb is None else rb
+                own = owner[pp][sorted(cols)][:, ra:rb_]
+                need |= {int(v) for v in np.unique(own)}
+        if L["type"] == "attn_k":
+            assert need <= parents[t], (name, l, t)                 # safe: everything read is awaited
+            both = set()
+            for pp in (L["p0"], L["p1"]):                            # and nothing beyond the two heads' columns
+                hd = L["n_embd"] // L["n_head"]
+                bs = {c // (L["n_head"] * seq) for c in range(c0, c1)}
+                hs = {(c // seq) % L["n_head"] for c in range(c0, c1)}
+                for b in bs:
+                    for h in hs:
+                        both |= {int(v) for v in np.unique(owner[pp][b * seq:(b + 1) * seq, h * hd:(h + 1) * hd])}
+            assert parents[t] <= both, (name, l, t)
+        elif L["type"] in ("conv", "maxpool", "avgpool"):
+            # the library may await the contiguous hull of the window's input columns (a superset for
+            # strided windows): everything read is awaited, nothing outside the hull is
+            assert need <= parents[t], (name, l, t)
+            pp = L["p0"]
+            if infos[pp]["num_ninst"]:
+                cols = set().union(*[c for (_, c, _, _) in needed_regions(L, layers, c0, c1, r0, r1, batch, seq)])
+                rr = (0, infos[pp]["H"]) if L["type"] == "conv" else (r0, r1)
+                hull = {int(v) for v in np.unique(owner[pp][min(cols):max(cols) + 1, rr[0]:rr[1]])}
+                assert parents[t] <= hull, (name, l, t)
+        else:
+            assert parents[t] == need, (name, l, t, L["type"], sorted(parents[t]), sorted(need))
+    # ---- executing by the counters runs every tile exactly once (what the device engine does)
+    cnt = npar.copy().astype(np.int64)
+    ready = [t for t in range(T) if cnt[t] == 0]
+    ran = 0
+    while ready:
+        t = ready.pop()
+        ran += 1
+        for c in idx[off[t]:off[t + 1]]:
+            cnt[c] -= 1
+            if cnt[c] == 0:
+                ready.append(int(c))
+    assert ran == T and (cnt == 0).all()
+    n.destroy(); d.destroy()
+
+
+def test_min_ninst_raises_tile_count():
+    case = H.micro_cases()["resnet_mini_b2"]
+    counts = []
+    for m in (1, 64, 512):
+        layers, d, n, _, _ = make(case, m)
+        counts.append(n.num_ninst)
+        n.destroy(); d.destroy()
+    assert counts[0] <= counts[1] <= counts[2] and counts[0] < counts[2]
+
+
+def test_error_paths(tmp_path, capfd):
+    L = api.lib()
+    assert not L.apu_create_dnn(b"/nonexistent/file.cfg", None)
+    bad = tmp_path / "bad.cfg"
+    bad.write_text("[net]\nheight=8\nwidth=8\nchannels=3\n[bogus_layer]\nfoo=1\n")
+    h = L.apu_create_dnn(str(bad).encode(), None)                    # unknown sections are reported and skipped,
+    assert h                                                         # as the reference's parser does (src/darknet_parser.c:447)
+    assert "Unsupported section type" in capfd.readouterr().err
+    L.apu_destroy_dnn(h)
+    good = tmp_path / "good.cfg"
+    good.write_text(M.custom_cifar_cfg())
+    # a missing or malformed weight file is reported and the dnn stays without weights, as in the
+    # reference (src/apu.c apu_load_dnn_data_from_file prints and returns)
+    h = L.apu_create_dnn(str(good).encode(), b"/nonexistent/weights.bin")
+    assert h and "not found" in capfd.readouterr().err
+    L.apu_destroy_dnn(h)
+    garbage = tmp_path / "w.bin"
+    garbage.write_bytes(b"not an aspen data file" * 10)
+    h = L.apu_create_dnn(str(good).encode(), str(garbage).encode())
+    assert h and capfd.readouterr().err != ""
+    L.apu_destroy_dnn(h)
+    d = api.Dnn(M.custom_cifar_cfg(), None)
+    assert not L.apu_create_nasm(d.h, 0, 1)                          # min_ninst_per_ldata must be >= 1
+    h = L.apu_create_nasm(d.h, 64, 0)                                # batch 0 means batch 1
+    a = (api.C.c_uint * 12)()
+    L.aspen_nasm_ldata_info(h, 0, a)
+    assert a[3] == 32 * 32
+    L.apu_destroy_nasm(h)
+    assert not L.apu_create_nasm(None, 64, 1)
+    t = api.Dnn(M.bert_cfg(1, 128, 2, 256), None)
+    assert not L.apu_create_transformer_nasm(t.h, 64, 1, 0)          # transformer without a sequence length
+    n = api.Nasm(d, 2, 0, 16)
+    L.apu_destroy_dnn(d.h)                                           # refused while a nasm refers to it
+    assert n.info(1)["H"] > 0
+    n.destroy(); d.destroy(); t.destroy()
+    capfd.readouterr()
+
+
+def test_weight_file_round_trip(tmp_path, capfd):
+    """ASPEN_DATA written by the model tools loads; a file missing a tensor is rejected."""
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()["custom_b3"])
+    wp = str(tmp_path / "w.bin")
+    M.write_aspen_data(wp, tens)
+    d = api.Dnn(cfg, wp)
+    d.destroy()
+    capfd.readouterr()
+    # a tensor whose element count does not fit its layer is reported
+    broken = [(i, k, (a[:-1] if (i, k) == (tens[0][0], tens[0][1]) else a)) for (i, k, a) in tens]
+    M.write_aspen_data(wp, [(i, k, np.ascontiguousarray(a).reshape(-1)) for (i, k, a) in broken])
+    cfgp = tmp_path / "c.cfg"
+    cfgp.write_text(cfg)
+    h = api.lib().apu_create_dnn(str(cfgp).encode(), wp.encode())
+    assert capfd.readouterr().err != ""
+    if h:
+        api.lib().apu_destroy_dnn(h)
