@@ -96,6 +96,8 @@ def lib() -> C.CDLL:
         "aspen_hip_free": (None, [_vp]),
         "aspen_hip_h2d": (C.c_int, [_vp, _vp, C.c_size_t]),
         "aspen_hip_d2h": (C.c_int, [_vp, _vp, C.c_size_t]),
+        "aspen_hip_copy": (C.c_int, [_vp, _vp, C.c_size_t]),
+        "aspen_hip_zero": (C.c_int, [_vp, C.c_size_t]),
         "aspen_hip_sync": (C.c_int, []),
         "aspen_hip_set_flags": (None, [C.c_uint32]),
         "aspen_hip_idle": (C.c_int, []),

@@ -110,12 +110,7 @@ struct dataflow_args_t
     unsigned long long spin_limit;
 };
 
-// The tile body as a real function call: the persistent loop around it then carries almost no
-// register state, and the tile code gets the whole register budget to itself.
-__device__ __noinline__ void run_tile_coherent (const aspen_hip_layer_t *L, uint32_t t, float *smem)
-{
-    run_tile<true> (*L, t, smem);
-}
+#define QUEUE_EMPTY_TILE QUEUE_EMPTY
 
 // Waits until queue slot `ticket` holds a tile and returns it; QUEUE_EMPTY when all tickets are
 // taken or the run was aborted.  The wait polls with relaxed device-scope loads (an acquire here
@@ -140,74 +135,107 @@ __device__ __forceinline__ uint32_t wait_for_slot (const dataflow_args_t &a, uin
     }
 }
 
-// Persistent workgroup = one scheduling engine (the reference's DSE thread, src/dse.c:5-108).
-// Wavefront 1 pops the next tile while wavefront 0 publishes the finished one (dependency countdown
-// of its children, push of those that became ready).  No cache write-back / invalidate is needed anywhere: tiles access
-// activations with device-scope coherent instructions (ActView<true>).
-__global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataflow_args_t a)
+// Workgroup-local scheduler state.  It lives in LDS so that nothing of it occupies registers while a
+// tile runs: the tile code is inlined into the persistent loop and owns the whole register budget.
+struct sched_lds_t
 {
-    extern __shared__ __align__ (16) float smem[];
-    __shared__ uint32_t s_tile[2];
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const bool popper = wave == 1 && lane == 0;
-    uint32_t next_ticket = 0;
-    const bool prof = (a.flags & ASPEN_HIP_FLAG_PROFILE) && threadIdx.x == 0;
-    unsigned long long t_tile = 0, t_drain = 0, t_sched = 0, t_begin = prof ? wall_clock64 () : 0, t0 = t_begin;
-    if (popper) s_tile[0] = wait_for_slot (a, atomicAdd (&a.state[ST_HEAD], 1u));
-    (void)next_ticket;
-    for (uint32_t it = 0;; it++)
+    dataflow_args_t a;
+    uint32_t tile;                       // tile to run next (QUEUE_EMPTY: leave)
+    unsigned long long t0, ticks[3];     // profiling: last time stamp; tile / drain / scheduling ticks
+};
+__shared__ sched_lds_t s_sched;
+
+__device__ __forceinline__ void prof_lap (int which)
+{
+    if ((s_sched.a.flags & ASPEN_HIP_FLAG_PROFILE) && threadIdx.x == 0)
     {
-        __syncthreads ();
-        const uint32_t id = s_tile[it & 1];
-        if (prof) { const unsigned long long t = wall_clock64 (); t_sched += t - t0; t0 = t; }
-        if (id == QUEUE_EMPTY)                  // all tickets taken, or aborted
-        {
-            if (prof)
-            {
-                atomicAdd (&a.prof[0], t_tile); atomicAdd (&a.prof[1], t_drain); atomicAdd (&a.prof[2], t_sched);
-                atomicAdd (&a.prof[3], wall_clock64 () - t_begin);
-            }
-            return;
-        }
+        const unsigned long long t = wall_clock64 ();
+        s_sched.ticks[which] += t - s_sched.t0; s_sched.t0 = t;
+    }
+}
 
-        const aspen_hip_layer_t *L = &a.layers[a.ninst_layer[id]];
-        if (!(a.flags & ASPEN_HIP_FLAG_SKIP_TILES))
-            run_tile_coherent (L, id - L->ninst_start, smem);
-
-        if (prof) { const unsigned long long t = wall_clock64 (); t_tile += t - t0; t0 = t; }
+// One scheduling step of a workgroup, as a real function call (it needs few registers, all of them
+// caller-saved, so the call costs no register traffic): wavefront 0 publishes the finished tile
+// (dependency countdown of its children, push of those that became ready) while wavefront 1 pops the
+// next one.  done == QUEUE_EMPTY: nothing to publish (first step).  Returns the tile to run next.
+// The reference's counterpart is dse_schedule / update_children (src/dse.c:20-108, :363-401).
+__device__ __noinline__ uint32_t schedule_step (uint32_t done)
+{
+    const dataflow_args_t &a = s_sched.a;
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (done != QUEUE_EMPTY)
+    {
+        prof_lap (0);
         // every wave waits until its (write-through, device-coherent) stores have been acknowledged.
         // An explicit wait: a workgroup-scope fence does not have to wait for global stores.
         asm volatile ("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads ();
-        if (prof) { const unsigned long long t = wall_clock64 (); t_drain += t - t0; t0 = t; }
-        if (wave == 0)
+        prof_lap (1);
+    }
+    if (wave == 0 && done != QUEUE_EMPTY)
+    {
+        // publish: count down the children with relaxed device-scope atomics; whoever takes a
+        // child's counter to zero puts it into the ready queue
+        const uint32_t c0 = a.child_off[done], c1 = a.child_off[done + 1];
+        for (uint32_t c = c0 + lane; c < c1; c += 64)
         {
-            // publish: count down the children with relaxed device-scope atomics; whoever takes a
-            // child's counter to zero puts it into the ready queue
-            const uint32_t c0 = a.child_off[id], c1 = a.child_off[id + 1];
-            for (uint32_t c = c0 + lane; c < c1; c += 64)
+            const uint32_t child = a.child_idx[c];
+            const uint32_t before = __hip_atomic_fetch_sub (&a.dep[child], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (before == 1u)
             {
-                const uint32_t child = a.child_idx[c];
-                const uint32_t before = __hip_atomic_fetch_sub (&a.dep[child], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (before == 1u)
-                {
-                    const uint32_t slot = atomicAdd (&a.state[ST_TAIL], 1u);
-                    __hip_atomic_store (&a.queue[slot], (a.epoch << QUEUE_ID_BITS) | child, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
-            }
-            if (lane == 0 && (a.flags & ASPEN_HIP_FLAG_COUNT_TILES))
-            {
-                if (atomicAdd (&a.ran[id], 1u) != 0) atomicAdd (&a.state[ST_TWICE], 1u);
-                atomicAdd (&a.state[ST_DONE], 1u);
+                const uint32_t slot = atomicAdd (&a.state[ST_TAIL], 1u);
+                __hip_atomic_store (&a.queue[slot], (a.epoch << QUEUE_ID_BITS) | child, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
-        else if (popper)
+        if (lane == 0 && (a.flags & ASPEN_HIP_FLAG_COUNT_TILES))
         {
-            // pop: a ticket is drawn only now, when this workgroup is free.  Drawing it earlier would
-            // hide the atomic's round trip but binds a (possibly already ready) tile to a busy
-            // workgroup while idle ones wait on later slots.
-            s_tile[(it + 1) & 1] = wait_for_slot (a, atomicAdd (&a.state[ST_HEAD], 1u));
+            if (atomicAdd (&a.ran[done], 1u) != 0) atomicAdd (&a.state[ST_TWICE], 1u);
+            atomicAdd (&a.state[ST_DONE], 1u);
         }
+    }
+    else if (wave == 1 && lane == 0)
+    {
+        // pop: a ticket is drawn only now, when this workgroup is free.  Drawing it earlier would
+        // hide the atomic's round trip but binds a (possibly already ready) tile to a busy
+        // workgroup while idle ones wait on later slots.
+        s_sched.tile = wait_for_slot (a, atomicAdd (&a.state[ST_HEAD], 1u));
+    }
+    __syncthreads ();
+    const uint32_t next = s_sched.tile;
+    prof_lap (2);
+    return next;
+}
+
+// Persistent workgroup = one scheduling engine (the reference's DSE thread, src/dse.c:5-108).
+// No cache write-back / invalidate is needed anywhere: tiles access activations with device-scope
+// coherent instructions (ActView<true>).
+__global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataflow_args_t args)
+{
+    extern __shared__ __align__ (16) float smem[];
+    if (threadIdx.x == 0)
+    {
+        s_sched.a = args;
+        s_sched.t0 = wall_clock64 ();
+        s_sched.ticks[0] = s_sched.ticks[1] = s_sched.ticks[2] = 0;
+    }
+    __syncthreads ();
+    const unsigned long long t_begin = wall_clock64 ();
+    uint32_t id = QUEUE_EMPTY;
+    for (;;)
+    {
+        id = __builtin_amdgcn_readfirstlane (schedule_step (id));
+        if (id == QUEUE_EMPTY) break;           // all tickets taken, or aborted
+        if (!(s_sched.a.flags & ASPEN_HIP_FLAG_SKIP_TILES))
+        {
+            const aspen_hip_layer_t *L = &s_sched.a.layers[s_sched.a.ninst_layer[id]];
+            run_tile<true> (*L, id - L->ninst_start, smem);
+        }
+    }
+    if ((s_sched.a.flags & ASPEN_HIP_FLAG_PROFILE) && threadIdx.x == 0)
+    {
+        unsigned long long *prof = s_sched.a.prof;
+        atomicAdd (&prof[0], s_sched.ticks[0]); atomicAdd (&prof[1], s_sched.ticks[1]); atomicAdd (&prof[2], s_sched.ticks[2]);
+        atomicAdd (&prof[3], wall_clock64 () - t_begin);
     }
 }
 
@@ -301,6 +329,27 @@ extern "C" int aspen_hip_zero (void *dst, size_t bytes)
 {
     if (aspen_hip_init ()) return -1;
     CHECK (hipMemsetAsync (dst, 0, bytes, g_stream));
+    return 0;
+}
+
+// plain streaming copy, 16 bytes per lane per step; also the yardstick the HBM byte counters of a
+// profiler are calibrated with (its traffic is known: `bytes` read + `bytes` written)
+__global__ void __launch_bounds__ (WG_THREADS) copy_kernel (const float4 *__restrict__ src, float4 *__restrict__ dst, size_t n4)
+{
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += step) dst[i] = src[i];
+}
+extern "C" int aspen_hip_copy (void *dst, const void *src, size_t bytes)
+{
+    if (aspen_hip_init ()) return -1;
+    if (bytes % 16 || ((uintptr_t)dst | (uintptr_t)src) % 16)
+    { snprintf (g_err, sizeof (g_err), "copy: size and addresses must be multiples of 16 bytes"); return -1; }
+    if (bytes == 0) return 0;
+    const size_t n4 = bytes / 16;
+    const size_t want = (n4 + WG_THREADS - 1) / WG_THREADS;
+    const unsigned grid = (unsigned)(want < (size_t)g_num_cu * 16 ? want : (size_t)g_num_cu * 16);
+    hipLaunchKernelGGL (copy_kernel, dim3 (grid), dim3 (WG_THREADS), 0, g_stream, (const float4 *)src, (float4 *)dst, n4);
+    CHECK (hipGetLastError ());
     return 0;
 }
 

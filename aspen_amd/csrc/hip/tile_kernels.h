@@ -93,19 +93,32 @@ template <bool COH> struct ActView
     }
 };
 
-__device__ __forceinline__ float activate (float x, int act)
+// The transcendental activations follow the reference's C expressions, which evaluate in double
+// (reference src/tiled_kernels.c naive_activate).  They are rare and carry many double-precision
+// constants, so they live in a real function: inlined, their constants would be set up in front of
+// the persistent loop and occupy registers during every tile.
+__device__ __noinline__ float activate_transcendental (float x, int act)
 {
     switch (act)
     {
-    case RELU:          return x > 0 ? x : 0;
-    case LEAKY_RELU:    return x > 0 ? x : (float)(0.1 * (double)x);
     case ELU:           return x > 0 ? x : (float)(0.1 * (exp ((double)x) - 1));
     case SELU:          return x > 0 ? (float)(1.0507 * (double)x) : (float)(1.0507 * 1.67326 * (exp ((double)x) - 1));
     case SIGMOID:       return (float)(1 / (1 + exp (-(double)x)));
     case TANH:          return (float)tanh ((double)x);
+    default:            return x;
+    }
+}
+
+__device__ __forceinline__ float activate (float x, int act)
+{
+    switch (act)
+    {
+    case NO_ACTIVATION: case LINEAR: return x;
+    case RELU:          return x > 0 ? x : 0;
+    case LEAKY_RELU:    return x > 0 ? x : (float)(0.1 * (double)x);
     case GELU:          return (float)(0.5 * (double)x * (double)(1 + erff (x * 0.7071067811865475f)));
     case GELU_ACCURATE: return (float)(0.5 * (double)x * (double)(1 + tanhf (0.7978845608028654f * (float)((double)x + 0.044715 * (double)x * (double)x * (double)x))));
-    default:            return x;
+    default:            return activate_transcendental (x, act);
     }
 }
 
@@ -267,6 +280,16 @@ template <bool COH> struct TransLoader64
 // One or two LDS stages (GEMM_STAGES); the K slice after the staged one always waits in registers.
 // ---------------------------------------------------------------------------------------------
 // LDS-only barrier: waits for this wave's LDS traffic, not for global loads still in flight.
+// The thread index as a value the optimiser cannot move out of an enclosing persistent loop: the
+// per-lane address arithmetic of every tile kind is loop-invariant there, would be hoisted in front of
+// the loop and then be kept alive (spilled to scratch) across all tiles.
+__device__ __forceinline__ uint32_t tile_thread ()
+{
+    uint32_t t = threadIdx.x;
+    asm volatile ("" : "+v"(t));
+    return t & (WG_THREADS - 1);
+}
+
 __device__ __forceinline__ void lds_barrier ()
 {
     asm volatile ("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -279,7 +302,7 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     constexpr int STAGE = GEMM_STAGES == 2 ? (BM + BN) * LDS_ROW : 0;
     constexpr int KK = GEMM_BK / 8;
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
     const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);
     const uint32_t afrag = wm0 * LDS_ROW + (lane & 31) * LDS_ROW + (lane >> 5) * 4;
     const uint32_t bfrag = BM * LDS_ROW + wn0 * LDS_ROW + (lane & 31) * LDS_ROW + (lane >> 5) * 4;
@@ -308,15 +331,9 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
         for (int j = 0; j < TM; j++) af[0][j] = ld4 (S + afrag + j * 32 * LDS_ROW);
         #pragma unroll
         for (int i = 0; i < TN; i++) bf[0][i] = ld4 (S + bfrag + i * 32 * LDS_ROW);
-#ifdef EXP_SETPRIO
-        __builtin_amdgcn_s_setprio (EXP_SETPRIO);
-#endif
         #pragma unroll
         for (int kk = 0; kk < KK; kk++)
         {
-#ifdef EXP_IGLP
-            __builtin_amdgcn_iglp_opt (EXP_IGLP);
-#endif
             const int cur = kk & 1, nxt = cur ^ 1;
             if (kk + 1 < KK)
             {
@@ -343,9 +360,6 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[cur][i].w, af[cur][j].w, acc[i][j], 0, 0, 0);
                 }
         }
-#ifdef EXP_SETPRIO
-        __builtin_amdgcn_s_setprio (0);
-#endif
         if (GEMM_STAGES == 1 && more)
         {
             // single stage: once every wave has read its last fragments, the slice waiting in
@@ -369,7 +383,7 @@ template <int BM, int BN, int WM, int WN, bool COH>
 __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, int slice, float *smem)
 {
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
     const uint32_t m0 = tm * BM, n0 = tn * BN;
     floatx16 acc[TN][TM];
     ActView<COH> in, out;
@@ -445,7 +459,7 @@ __device__ __forceinline__ void tile_splitk_finish (const aspen_hip_layer_t &L, 
     const uint32_t rows = min (L.tile_n, L.N - n0), mrem = L.M - m0;
     ActView<COH> part, out;
     part.init (L.partial, L.N * L.splits, L.ld); out.init (L.out, L.N, L.ld);
-    for (uint32_t idx = threadIdx.x; idx < rows * C4; idx += WG_THREADS)
+    for (uint32_t idx = tile_thread (); idx < rows * C4; idx += WG_THREADS)
     {
         const uint32_t r = idx / C4, c = (idx - r * C4) * 4;
         if (c >= mrem) continue;
@@ -479,7 +493,7 @@ __device__ __forceinline__ void tile_residual (const aspen_hip_layer_t &L, uint3
     const uint32_t total = (n1 - n0) * M4;
     ActView<COH> p0, p1, out;
     p0.init (L.in0, L.N, L.ld0); p1.init (L.in1, L.N, L.ld1); out.init (L.out, L.N, L.ld);
-    for (uint32_t i = threadIdx.x; i < total; i += WG_THREADS)
+    for (uint32_t i = tile_thread (); i < total; i += WG_THREADS)
     {
         const uint32_t c = i / M4, m = (i - c * M4) * 4, n = n0 + c;
         float4 a = p0.ld4 (n * L.ld0 + m), b = p1.ld4 (n * L.ld1 + m);
@@ -496,7 +510,7 @@ __device__ __forceinline__ void tile_pool (const aspen_hip_layer_t &L, uint32_t 
     const float inv = 1.0f / (float)(L.KH * L.KW);
     ActView<COH> in, out;
     in.init (L.in0, (L.N / ohw) * L.IH * L.IW, L.ld0); out.init (L.out, L.N, L.ld);
-    for (uint32_t i = threadIdx.x; i < total; i += WG_THREADS)
+    for (uint32_t i = tile_thread (); i < total; i += WG_THREADS)
     {
         const uint32_t c = i / M4, m = (i - c * M4) * 4, n = n0 + c;
         const uint32_t b = n / ohw, rem = n - b * ohw, oh = rem / L.OW, ow = rem - oh * L.OW;
@@ -540,7 +554,7 @@ template <bool COH>
 __device__ __forceinline__ void tile_layernorm (const aspen_hip_layer_t &L, uint32_t tn)
 {
     const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N);
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, M4 = L.M >> 2;
+    const uint32_t lane = tile_thread () & 63, wave = tile_thread () >> 6, M4 = L.M >> 2;
     ActView<COH> in, out;
     in.init (L.in0, L.N, L.ld0); out.init (L.out, L.N, L.ld);
     for (uint32_t n = n0 + wave; n < n1; n += WG_THREADS / 64)
@@ -577,7 +591,7 @@ template <bool COH>
 __device__ __forceinline__ void tile_softmax (const aspen_hip_layer_t &L, uint32_t tn)
 {
     const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N);
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t lane = tile_thread () & 63, wave = tile_thread () >> 6;
     ActView<COH> in, out;
     in.init (L.in0, L.N, L.ld0); out.init (L.out, L.N, L.ld);
     for (uint32_t n = n0 + wave; n < n1; n += WG_THREADS / 64)
@@ -605,7 +619,7 @@ __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, ui
 {
     constexpr int BM = 128, BN = KATTN_BN, WM = 2, WN = 2, TM = BM / WM / 32, TN = BN / WN / 32;
     __shared__ float rowsum[BN];
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
     const uint32_t S = L.seq, qtiles = (S + BN - 1) / BN;
     const uint32_t bh = tn / qtiles, q0 = (tn - bh * qtiles) * BN;
     const uint32_t b = bh / L.heads, h = bh - b * L.heads;
@@ -686,7 +700,7 @@ template <bool COH>
 __device__ __forceinline__ void tile_v_attention (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, float *smem)
 {
     constexpr int BM = 64, BN = 128, WM = 2, WN = 2, TM = 1, TN = 2;
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
     const uint32_t S = L.seq, qtiles = (S + BN - 1) / BN;
     const uint32_t b = tn / qtiles, q0 = (tn - b * qtiles) * BN;
     const uint32_t m0 = tm * L.tile_m, h = m0 / L.hd;
@@ -715,9 +729,28 @@ __device__ __forceinline__ void tile_v_attention (const aspen_hip_layer_t &L, ui
 // (reference src/dse.c:39-79).  `t` = tile index inside the layer, row-tile fastest
 // (reference src/apu_nasm.c:1218-1224).
 // ---------------------------------------------------------------------------------------------
-template <bool COH>
-__device__ __forceinline__ void run_tile (const aspen_hip_layer_t &L, uint32_t t, float *smem)
+// A wave-uniform copy of a layer descriptor in scalar registers.  The descriptor sits in memory the
+// kernel also writes, so the compiler reads it with vector loads; without this copy every value
+// derived from it counts as per-lane data: buffer descriptors get rebuilt in a per-lane "waterfall"
+// loop around each access and all tile-level control flow runs on the vector unit.
+__device__ __forceinline__ aspen_hip_layer_t uniform_layer (const aspen_hip_layer_t &Lg)
 {
+    constexpr int W = sizeof (aspen_hip_layer_t) / 4;
+    static_assert (sizeof (aspen_hip_layer_t) % 4 == 0, "descriptor is a whole number of dwords");
+    uint32_t w[W];
+    __builtin_memcpy (w, &Lg, sizeof (aspen_hip_layer_t));
+    #pragma unroll
+    for (int i = 0; i < W; i++) w[i] = __builtin_amdgcn_readfirstlane (w[i]);
+    aspen_hip_layer_t L;
+    __builtin_memcpy (&L, w, sizeof (aspen_hip_layer_t));
+    return L;
+}
+
+template <bool COH>
+__device__ __forceinline__ void run_tile (const aspen_hip_layer_t &Lg, uint32_t t, float *smem)
+{
+    const aspen_hip_layer_t L = uniform_layer (Lg);
+    t = __builtin_amdgcn_readfirstlane (t);
     int slice = -1;
     if (L.splits > 1)
     {

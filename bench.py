@@ -103,6 +103,9 @@ def main():
     ap.add_argument("--skip-tiles", action="store_true", help="scheduler-only run: dependency protocol with empty tiles")
     ap.add_argument("--engine-profile", action="store_true", help="report where the persistent workgroups spend their time")
     ap.add_argument("--layer-profile", action="store_true", help="also time every layer's kernel (layer-launch mode)")
+    ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
+                    help="instead of a workload: run the library's streaming copy kernel over MIB MiB (--steps launches); "
+                         "under a profiler this calibrates the HBM byte counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
@@ -114,6 +117,22 @@ def main():
         print("bench.py: no HIP device: " + L.aspen_hip_last_error().decode(), file=sys.stderr)
         sys.exit(1)
     dev = api.device_info()
+    if args.copy_probe:
+        nbytes = args.copy_probe << 20
+        src, dst = L.aspen_hip_alloc(nbytes), L.aspen_hip_alloc(nbytes)
+        for _ in range(args.warmup):
+            L.aspen_hip_copy(dst, src, nbytes)
+        L.aspen_hip_event_record(0)
+        for _ in range(args.steps):
+            L.aspen_hip_copy(dst, src, nbytes)
+        L.aspen_hip_event_record(1)
+        L.aspen_hip_sync()
+        ms = api.C.c_float()
+        L.aspen_hip_event_elapsed_ms(0, 1, api.C.byref(ms))
+        print(json.dumps({"copy_probe_bytes_read": nbytes, "copy_probe_bytes_written": nbytes, "launches": args.steps,
+                          "ms_per_launch": ms.value / args.steps,
+                          "GB_per_s": 2 * nbytes * args.steps / (ms.value * 1e-3) / 1e9}))
+        return
     L.aspen_hip_set_flags((1 if args.skip_tiles else 0) | (4 if args.engine_profile else 0))
     cfgs, unit, units_per_step = WORKLOADS[args.workload]
 

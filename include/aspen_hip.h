@@ -94,6 +94,10 @@ int aspen_hip_d2h (void *dst, const void *src, size_t bytes);
 int aspen_hip_h2d_2d (void *dst, size_t dpitch, const void *src, size_t spitch, size_t width, size_t rows);
 int aspen_hip_d2h_2d (void *dst, size_t dpitch, const void *src, size_t spitch, size_t width, size_t rows);
 int aspen_hip_zero (void *dst, size_t bytes);
+/* device-to-device copy by a plain streaming kernel on the library's stream (asynchronous); size and
+   addresses multiples of 16 bytes.  Its memory traffic is exactly 2 x bytes, which makes it the
+   calibration point for a profiler's HBM byte counters. */
+int aspen_hip_copy (void *dst, const void *src, size_t bytes);
 
 /* ---- graph ----------------------------------------------------------------------------------- */
 /* Uploads a tile graph.  ninst_layer[i] = layer of tile i; num_parents[i] = its dependency count;

@@ -133,3 +133,46 @@ def test_co_inference_resnet50_vgg16_b16(gpu):
             net.dnn.destroy()
         dse.destroy()
         pool.destroy()
+
+
+# ---- the flat seam on its own ---------------------------------------------------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K,act", [(64, 64, 32, 0), (100, 37, 96, 4), (8, 300, 64, 0), (257, 129, 160, 8)])
+def test_sgemm_seam_matches_oracle(gpu, M, N, K, act):
+    """aspen_hip_sgemm (C-ABI, device pointers) against the oracle's packed micro-kernel."""
+    from oracle import cpu
+    L = api.lib()
+    rng = np.random.default_rng(M * 1000 + N)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = rng.standard_normal((N, K)).astype(np.float32)
+    bias = rng.standard_normal(M).astype(np.float32)
+    ldc = (M + 3) // 4 * 4
+    want = cpu.activate(cpu.sgemm_packed(cpu.pack_weight(A), B, M, np.tile(bias, (N, 1))), act)
+    dA, dB, dC, db = (L.aspen_hip_alloc(x) for x in (A.nbytes, B.nbytes, N * ldc * 4, bias.nbytes))
+    assert dA and dB and dC and db
+    for d, h in ((dA, A), (dB, B), (db, bias)):
+        assert L.aspen_hip_h2d(d, h.ctypes.data, h.nbytes) == 0
+    assert L.aspen_hip_sgemm(M, N, K, dA, K, dB, K, dC, ldc, db, act) == 0, L.aspen_hip_last_error()
+    got = np.zeros((N, ldc), np.float32)
+    assert L.aspen_hip_d2h(got.ctypes.data, dC, got.nbytes) == 0
+    assert H.rel_l2(got[:, :M], want) <= H.REL_L2_TOL
+    assert (got[:, M:] == 0).all()                      # padding rows are never written
+    # argument checks fail with a message instead of launching
+    assert L.aspen_hip_sgemm(M, N, K + 1, dA, K, dB, K, dC, ldc, db, act) != 0
+    assert b"multiple" in L.aspen_hip_last_error()
+    for d in (dA, dB, dC, db):
+        L.aspen_hip_free(d)
+
+
+@pytest.mark.gpu
+def test_copy_kernel(gpu):
+    L = api.lib()
+    x = np.arange(1 << 20, dtype=np.float32)
+    a, b = L.aspen_hip_alloc(x.nbytes), L.aspen_hip_alloc(x.nbytes)
+    assert L.aspen_hip_h2d(a, x.ctypes.data, x.nbytes) == 0
+    assert L.aspen_hip_copy(b, a, x.nbytes) == 0 and L.aspen_hip_sync() == 0
+    y = np.zeros_like(x)
+    assert L.aspen_hip_d2h(y.ctypes.data, b, y.nbytes) == 0
+    assert np.array_equal(x, y)
+    assert L.aspen_hip_copy(b, a, 24) != 0
+    L.aspen_hip_free(a); L.aspen_hip_free(b)
