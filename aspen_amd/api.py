@@ -88,6 +88,7 @@ def lib() -> C.CDLL:
         "aspen_rpool_num_ninst": (C.c_uint, [_vp]),
         "aspen_rpool_profile_layers": (C.c_int, [_vp, C.c_uint, _fp]),
         "aspen_rpool_dataflow_profile": (C.c_int, [_vp, C.POINTER(C.c_uint64), C.c_int]),
+        "aspen_rpool_dataflow_trace": (C.c_int, [_vp, _vp]),
         # aspen_hip.h
         "aspen_hip_init": (C.c_int, []),
         "aspen_hip_last_error": (C.c_char_p, []),
@@ -240,10 +241,18 @@ class RPool:
 
     def dataflow_profile(self, reset: bool = True) -> dict:
         """Summed workgroup time of dataflow runs since the last reset, in seconds (profile flag 4)."""
-        t = (C.c_uint64 * 4)()
+        t = (C.c_uint64 * 8)()
         if lib().aspen_rpool_dataflow_profile(self.h, t, 1 if reset else 0):
             raise RuntimeError("no dataflow profile")
-        return {k: t[i] * 1e-8 for i, k in enumerate(["tile", "drain", "sched", "total"])}
+        return {k: t[i] * 1e-8 for i, k in enumerate(["tile", "drain", "sched", "total", "publish", "ticket", "slot_wait"])}
+
+    def dataflow_trace(self) -> np.ndarray:
+        """[tiles][2] start / end stamps (100 MHz ticks) of the last run made with the trace flag (8)."""
+        n = lib().aspen_rpool_num_ninst(self.h)
+        t = np.zeros((n, 2), dtype=np.uint64)
+        if lib().aspen_rpool_dataflow_trace(self.h, t.ctypes.data):
+            raise RuntimeError("no dataflow trace: " + lib().aspen_hip_last_error().decode())
+        return t
 
     def profile_layers(self, num_layers: int, iters: int = 5) -> np.ndarray:
         """Per-layer kernel time in ms (layer-launch mode, HIP events); the pool must have run once."""

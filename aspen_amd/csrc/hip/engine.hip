@@ -36,6 +36,8 @@ struct aspen_hip_graph_t
     uint32_t *d_ran;        // per-tile execution count (sanity: every tile exactly once)
     uint32_t epoch;         // tag of the last run's queue entries, cycles 1..255
     unsigned long long *d_prof;
+    int cached_loads;       // 1: no cache line of an activation is shared by two producer tiles
+    unsigned long long *d_trace;    // [2*tile] start, [2*tile+1] end time stamps (allocated on first traced run)
 };
 
 static hipStream_t g_stream = nullptr;
@@ -67,7 +69,7 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) layer_kernel (const as
     const uint32_t nt = gridDim.x, bid = blockIdx.x;
     const uint32_t xcd = bid & 7, local = bid >> 3, chunk = nt >> 3, rem = nt & 7;
     const uint32_t t = first_tile + xcd * chunk + (xcd < rem ? xcd : rem) + local;
-    run_tile<false> (L, t, smem);
+    run_tile<0> (L, t, smem);
 }
 
 // Re-arm: counters back to the parent counts, queue seeded with the roots.  Queue entries carry the
@@ -103,7 +105,8 @@ struct dataflow_args_t
     const uint32_t *ninst_layer, *child_off, *child_idx;
     uint32_t *dep, *queue, *state, *ran;
     uint32_t *host_abort;
-    unsigned long long *prof;       // [0] tile, [1] store drain, [2] publish / pop, [3] total: summed 100 MHz ticks of all workgroups
+    unsigned long long *trace;      // per-tile start / end time stamps when ASPEN_HIP_FLAG_TRACE is set
+    unsigned long long *prof;       // 8 counters of summed 100 MHz ticks, see aspen_hip_dataflow_profile
     uint32_t num_ninst;
     uint32_t epoch;                 // 1..255, tag of this run's queue entries
     uint32_t flags;                 // ASPEN_HIP_FLAG_*
@@ -141,7 +144,7 @@ struct sched_lds_t
 {
     dataflow_args_t a;
     uint32_t tile;                       // tile to run next (QUEUE_EMPTY: leave)
-    unsigned long long t0, ticks[3];     // profiling: last time stamp; tile / drain / scheduling ticks
+    unsigned long long t0, ticks[6];     // profiling: last time stamp; tile / drain / scheduling / publish / ticket / slot-wait ticks
 };
 __shared__ sched_lds_t s_sched;
 
@@ -171,9 +174,12 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done)
         asm volatile ("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads ();
         prof_lap (1);
+        if ((a.flags & ASPEN_HIP_FLAG_TRACE) && threadIdx.x == 0) a.trace[2 * (size_t)done + 1] = wall_clock64 ();
     }
+    const bool prof = (a.flags & ASPEN_HIP_FLAG_PROFILE) && lane == 0;
     if (wave == 0 && done != QUEUE_EMPTY)
     {
+        const unsigned long long tp = prof ? wall_clock64 () : 0;
         // publish: count down the children with relaxed device-scope atomics; whoever takes a
         // child's counter to zero puts it into the ready queue
         const uint32_t c0 = a.child_off[done], c1 = a.child_off[done + 1];
@@ -192,13 +198,18 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done)
             if (atomicAdd (&a.ran[done], 1u) != 0) atomicAdd (&a.state[ST_TWICE], 1u);
             atomicAdd (&a.state[ST_DONE], 1u);
         }
+        if (prof) { asm volatile ("s_waitcnt vmcnt(0)" ::: "memory"); s_sched.ticks[3] += wall_clock64 () - tp; }
     }
     else if (wave == 1 && lane == 0)
     {
         // pop: a ticket is drawn only now, when this workgroup is free.  Drawing it earlier would
         // hide the atomic's round trip but binds a (possibly already ready) tile to a busy
         // workgroup while idle ones wait on later slots.
-        s_sched.tile = wait_for_slot (a, atomicAdd (&a.state[ST_HEAD], 1u));
+        const unsigned long long t1 = prof ? wall_clock64 () : 0;
+        const uint32_t ticket = atomicAdd (&a.state[ST_HEAD], 1u);
+        const unsigned long long t2 = prof ? wall_clock64 () : 0;
+        s_sched.tile = wait_for_slot (a, ticket);
+        if (prof) { s_sched.ticks[4] += t2 - t1; s_sched.ticks[5] += wall_clock64 () - t2; }
     }
     __syncthreads ();
     const uint32_t next = s_sched.tile;
@@ -207,8 +218,10 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done)
 }
 
 // Persistent workgroup = one scheduling engine (the reference's DSE thread, src/dse.c:5-108).
-// No cache write-back / invalidate is needed anywhere: tiles access activations with device-scope
-// coherent instructions (ActView<true>).
+// No cache write-back / invalidate is needed anywhere: tiles store activations with device-scope
+// write-through instructions and load them either coherently (COH = 1) or, when the host has checked
+// that no cache line is shared between producer tiles, through the caches (COH = 2); see ActView.
+template <int COH>
 __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataflow_args_t args)
 {
     extern __shared__ __align__ (16) float smem[];
@@ -216,7 +229,7 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
     {
         s_sched.a = args;
         s_sched.t0 = wall_clock64 ();
-        s_sched.ticks[0] = s_sched.ticks[1] = s_sched.ticks[2] = 0;
+        for (int i = 0; i < 6; i++) s_sched.ticks[i] = 0;
     }
     __syncthreads ();
     const unsigned long long t_begin = wall_clock64 ();
@@ -225,10 +238,11 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
     {
         id = __builtin_amdgcn_readfirstlane (schedule_step (id));
         if (id == QUEUE_EMPTY) break;           // all tickets taken, or aborted
+        if ((s_sched.a.flags & ASPEN_HIP_FLAG_TRACE) && threadIdx.x == 0) s_sched.a.trace[2 * (size_t)id] = wall_clock64 ();
         if (!(s_sched.a.flags & ASPEN_HIP_FLAG_SKIP_TILES))
         {
             const aspen_hip_layer_t *L = &s_sched.a.layers[s_sched.a.ninst_layer[id]];
-            run_tile<true> (*L, id - L->ninst_start, smem);
+            run_tile<COH> (*L, id - L->ninst_start, smem);
         }
     }
     if ((s_sched.a.flags & ASPEN_HIP_FLAG_PROFILE) && threadIdx.x == 0)
@@ -236,6 +250,7 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
         unsigned long long *prof = s_sched.a.prof;
         atomicAdd (&prof[0], s_sched.ticks[0]); atomicAdd (&prof[1], s_sched.ticks[1]); atomicAdd (&prof[2], s_sched.ticks[2]);
         atomicAdd (&prof[3], wall_clock64 () - t_begin);
+        atomicAdd (&prof[4], s_sched.ticks[3]); atomicAdd (&prof[5], s_sched.ticks[4]); atomicAdd (&prof[6], s_sched.ticks[5]);
     }
 }
 
@@ -257,7 +272,8 @@ extern "C" int aspen_hip_init (void)
     *g_host_abort = 0;
     for (int i = 0; i < NUM_EVENTS; i++) CHECK (hipEventCreate (&g_events[i]));
     CHECK (hipFuncSetAttribute ((const void *)layer_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
-    CHECK (hipFuncSetAttribute ((const void *)dataflow_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
+    CHECK (hipFuncSetAttribute ((const void *)dataflow_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
+    CHECK (hipFuncSetAttribute ((const void *)dataflow_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
     g_inited = 1;
     return 0;
 }
@@ -399,8 +415,14 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
         else if (L.tile_n != 128 || L.tile_m > 64 || L.hd % L.tile_m) why = "V-attention tiles are 128 queries x <=64 channels of one head";
         else if (L.ld0 % GEMM_BK || L.ld0 < L.seq) why = "probability stride must be a multiple of 32 covering seq";
     }
-    else if (L.type == RESIDUAL_LAYER) { if (!L.in1) why = "missing second parent"; }
-    else if (L.type == LAYERNORM_LAYER) { if (!L.weight) why = "missing gamma"; }
+    else if (L.type == MAXPOOL_LAYER || L.type == AVGPOOL_LAYER)
+    {
+        if (L.tiles_m > 1 && (L.tile_m % 4 || (uint64_t)L.tiles_m * L.tile_m < L.M || (uint64_t)(L.tiles_m - 1) * L.tile_m >= L.M)) why = "pool row tiles";
+        else if ((uint64_t)L.tiles_n * L.tile_n < L.N) why = "tile grid does not cover the matrix";
+    }
+    else if (L.type == RESIDUAL_LAYER) { if (!L.in1 || L.tiles_m != 1) why = "missing second parent, or row tiles"; }
+    else if (L.type == LAYERNORM_LAYER) { if (!L.weight || L.tiles_m != 1) why = "missing gamma, or row tiles"; }
+    else if (L.type == SOFTMAX_LAYER) { if (L.tiles_m != 1) why = "row tiles"; }
     if (why)
     {
         snprintf (g_err, sizeof (g_err), "layer %u rejected: %s", idx, why);
@@ -408,6 +430,25 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
         return -1;
     }
     return 0;
+}
+
+// True when every activation some tile reads is laid out so that a 128-byte cache line belongs to
+// exactly one producer tile: matrix start and column stride are multiples of 128 bytes, and a tile
+// spans either all rows or a multiple of 32 rows.  Then activation loads may go through the caches
+// inside the persistent kernel (see ActView, mode 2).
+static bool lines_have_one_producer (const aspen_hip_layer_t *layers, uint32_t num_layers)
+{
+    for (uint32_t l = 0; l < num_layers; l++)
+    {
+        const aspen_hip_layer_t &P = layers[l];
+        if (P.type == INPUT_LAYER || P.num_ninst == 0) continue;      // written by the host before the launch
+        bool is_read = false;
+        for (uint32_t c = 0; c < num_layers && !is_read; c++) is_read = layers[c].in0 == P.out || layers[c].in1 == P.out;
+        const bool aligned = (uintptr_t)P.out % 128 == 0 && ((size_t)P.ld * 4) % 128 == 0 && (P.tiles_m == 1 || (P.tile_m * 4) % 128 == 0);
+        if (is_read && !aligned) return false;
+        if (P.splits > 1 && ((uintptr_t)P.partial % 128 != 0 || !aligned)) return false;
+    }
+    return true;
 }
 
 extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *layers, uint32_t num_layers,
@@ -430,6 +471,7 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
         if (!ok) { snprintf (g_err, sizeof (g_err), "inconsistent dependency arrays"); fprintf (stderr, "aspen_hip: %s\n", g_err); return nullptr; }
     }
     aspen_hip_graph_t *g = (aspen_hip_graph_t *)calloc (1, sizeof (aspen_hip_graph_t));
+    g->cached_loads = lines_have_one_producer (layers, num_layers) && getenv ("ASPEN_GPU_COHERENT_LOADS") == nullptr;
     g->num_layers = num_layers; g->num_ninst = num_ninst; g->num_roots = num_roots; g->num_edges = num_edges;
     g->h_layers = (aspen_hip_layer_t *)malloc (sizeof (aspen_hip_layer_t) * num_layers);
     memcpy (g->h_layers, layers, sizeof (aspen_hip_layer_t) * num_layers);
@@ -459,7 +501,7 @@ extern "C" void aspen_hip_graph_destroy (aspen_hip_graph_t *g)
     (void)hipStreamSynchronize (g_stream);
     aspen_hip_free (g->d_layers); aspen_hip_free (g->d_ninst_layer); aspen_hip_free (g->d_num_parents);
     aspen_hip_free (g->d_child_off); aspen_hip_free (g->d_child_idx); aspen_hip_free (g->d_roots);
-    aspen_hip_free (g->d_dep); aspen_hip_free (g->d_queue); aspen_hip_free (g->d_ran); aspen_hip_free (g->d_state); aspen_hip_free (g->d_prof);
+    aspen_hip_free (g->d_dep); aspen_hip_free (g->d_queue); aspen_hip_free (g->d_ran); aspen_hip_free (g->d_state); aspen_hip_free (g->d_prof); aspen_hip_free (g->d_trace);
     free (g->h_layers);
     free (g);
 }
@@ -507,9 +549,16 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     dataflow_args_t a;
     a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx;
     a.dep = g->d_dep; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran; a.prof = g->d_prof; a.host_abort = g_host_abort;
+    if ((g_flags & ASPEN_HIP_FLAG_TRACE) && !g->d_trace)
+    {
+        g->d_trace = (unsigned long long *)aspen_hip_alloc (sizeof (unsigned long long) * 2 * (size_t)g->num_ninst);
+        if (!g->d_trace) return -1;
+    }
+    a.trace = g->d_trace;
     a.num_ninst = g->num_ninst; a.epoch = g->epoch; a.flags = g_flags; a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
     CHECK (hipEventRecord (g_events[NUM_EVENTS - 2], g_stream));
-    hipLaunchKernelGGL (dataflow_kernel, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);
+    if (g->cached_loads) hipLaunchKernelGGL (dataflow_kernel<2>, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);
+    else hipLaunchKernelGGL (dataflow_kernel<1>, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);
     CHECK (hipGetLastError ());
     CHECK (hipEventRecord (g_events[NUM_EVENTS - 1], g_stream));
     return 0;
@@ -568,14 +617,21 @@ extern "C" int aspen_hip_dataflow_stats (aspen_hip_graph_t *g, uint32_t *execute
     return 0;
 }
 
-extern "C" int aspen_hip_dataflow_profile (aspen_hip_graph_t *g, uint64_t ticks[4], int reset)
+extern "C" int aspen_hip_dataflow_profile (aspen_hip_graph_t *g, uint64_t ticks[8], int reset)
 {
     if (!g || !ticks) return -1;
-    unsigned long long h[4];
+    unsigned long long h[8];
     if (aspen_hip_d2h (h, g->d_prof, sizeof (h))) return -1;
-    for (int i = 0; i < 4; i++) ticks[i] = h[i];
+    for (int i = 0; i < 8; i++) ticks[i] = h[i];
     if (reset) { CHECK (hipMemsetAsync (g->d_prof, 0, sizeof (h), g_stream)); }
     return 0;
+}
+
+extern "C" int aspen_hip_dataflow_trace (aspen_hip_graph_t *g, uint64_t *start_end, uint32_t num_ninst)
+{
+    if (!g || !start_end || !g->d_trace || num_ninst != g->num_ninst)
+    { snprintf (g_err, sizeof (g_err), "dataflow_trace: no traced run, or wrong tile count"); return -1; }
+    return aspen_hip_d2h (start_end, g->d_trace, sizeof (uint64_t) * 2 * (size_t)num_ninst);
 }
 
 extern "C" int aspen_hip_event_record (int slot)

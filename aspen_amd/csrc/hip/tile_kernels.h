@@ -53,16 +53,22 @@ typedef float floatx16 __attribute__ ((ext_vector_type (16)));
 __device__ __forceinline__ float4 ld4 (const float *p) { return *reinterpret_cast<const float4 *> (p); }
 __device__ __forceinline__ void st4 (float *p, float4 v) { *reinterpret_cast<float4 *> (p) = v; }
 
-// View of one activation matrix.  COH = true: every access is device-scope coherent (buffer
-// instructions with sc1: they bypass the per-CU L1 and the per-XCD L2, which are not coherent across
-// the 8 XCDs), so tiles produced and consumed inside one persistent kernel need no cache
-// write-back / invalidate between them, and the weights stay cached.  COH = false: plain cached
-// accesses for the one-launch-per-layer path, where kernel boundaries provide coherence.
+// View of one activation matrix.  COH selects how it is accessed:
+//   0  plain cached loads and stores: the one-launch-per-layer path, where kernel boundaries provide
+//      coherence.
+//   1  every access is device-scope coherent (buffer instructions with sc1): loads bypass the per-CU
+//      L1 and the per-XCD L2 (which are not coherent across the 8 XCDs), stores write through, so
+//      tiles produced and consumed inside one persistent kernel need no cache write-back /
+//      invalidate between them, and the weights stay cached.
+//   2  stores write through (sc1), loads are cached.  Correct when no cache line of an activation is
+//      shared by two producer tiles (the host checks strides and tile heights): a line is first
+//      fetched after its only producer has finished, every element is written once per launch, and
+//      the caches start a launch invalidated, so a cached line can never be stale.
 // Offsets are in floats from the start of the matrix; the descriptor bounds-checks them in hardware
 // (out-of-range loads return 0, out-of-range stores are dropped).
 typedef uint32_t u32x4 __attribute__ ((ext_vector_type (4)));
 #define CPOL_SC1 16
-template <bool COH> struct ActView
+template <int COH> struct ActView
 {
     const float *base;
     __amdgpu_buffer_rsrc_t rsrc;
@@ -73,12 +79,12 @@ template <bool COH> struct ActView
     }
     __device__ __forceinline__ float4 ld4 (uint32_t off) const
     {
-        if (COH) return __builtin_bit_cast (float4, __builtin_amdgcn_raw_buffer_load_b128 (rsrc, (int)(off * 4u), 0, CPOL_SC1));
+        if (COH) return __builtin_bit_cast (float4, __builtin_amdgcn_raw_buffer_load_b128 (rsrc, (int)(off * 4u), 0, COH == 1 ? CPOL_SC1 : 0));
         return *reinterpret_cast<const float4 *> (base + off);
     }
     __device__ __forceinline__ float ld1 (uint32_t off) const
     {
-        if (COH) return __builtin_bit_cast (float, __builtin_amdgcn_raw_buffer_load_b32 (rsrc, (int)(off * 4u), 0, CPOL_SC1));
+        if (COH) return __builtin_bit_cast (float, __builtin_amdgcn_raw_buffer_load_b32 (rsrc, (int)(off * 4u), 0, COH == 1 ? CPOL_SC1 : 0));
         return base[off];
     }
     __device__ __forceinline__ void st4 (uint32_t off, float4 v) const
@@ -164,7 +170,7 @@ template <int ROWS> struct RowLoader
 };
 
 // Same for rows of an activation matrix (matmul / 1x1-conv operand, Q, K and probability rows).
-template <int ROWS, bool COH> struct ActRowLoader
+template <int ROWS, int COH> struct ActRowLoader
 {
     static constexpr int R = ROWS / 32;
     ActView<COH> view;
@@ -197,7 +203,7 @@ template <int ROWS, bool COH> struct ActRowLoader
 // Implicit-GEMM activation operand of conv / FC: row n = output position (b, oh, ow); the K axis runs
 // over (kh, kw, ic) and is resolved through the layer's k-chunk table.  Replaces the reference's
 // pointer table + panel gather (prepare_input / load_im2col_ptr, reference src/tiled_kernels.c:3-159).
-template <int ROWS, bool COH> struct ConvLoader
+template <int ROWS, int COH> struct ConvLoader
 {
     static constexpr int R = ROWS / 32;
     ActView<COH> in;
@@ -239,7 +245,7 @@ template <int ROWS, bool COH> struct ConvLoader
 
 // K-strided operand (V of attention: rows = channels, K axis = sequence position with stride ld):
 // read 64 channels x 32 positions with 128-bit loads along the channels, transpose into LDS.
-template <bool COH> struct TransLoader64
+template <int COH> struct TransLoader64
 {
     static constexpr int R = 2;
     ActView<COH> view;
@@ -379,7 +385,7 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
 // conv / FC / matmul tile
 // `slice` < 0: the whole K axis, bias + activation, result to the layer's matrix.  `slice` >= 0 (split-K):
 // K slices [slice*kiters_per_split, ...) only, raw sums to that slice's partial matrix.
-template <int BM, int BN, int WM, int WN, bool COH>
+template <int BM, int BN, int WM, int WN, int COH>
 __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, int slice, float *smem)
 {
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
@@ -452,7 +458,7 @@ __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, ui
 }
 
 // split-K finishing tile: sum of the slices + bias, activation
-template <bool COH>
+template <int COH>
 __device__ __forceinline__ void tile_splitk_finish (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm)
 {
     const uint32_t m0 = tm * L.tile_m, n0 = tn * L.tile_n, C4 = L.tile_m >> 2;
@@ -486,7 +492,7 @@ __device__ __forceinline__ void tile_splitk_finish (const aspen_hip_layer_t &L, 
 // ---------------------------------------------------------------------------------------------
 // Bandwidth tiles: 128-bit accesses, a tile = tile_n whole columns.
 // ---------------------------------------------------------------------------------------------
-template <bool COH>
+template <int COH>
 __device__ __forceinline__ void tile_residual (const aspen_hip_layer_t &L, uint32_t tn)
 {
     const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N), M4 = L.ld >> 2;
@@ -502,17 +508,19 @@ __device__ __forceinline__ void tile_residual (const aspen_hip_layer_t &L, uint3
     }
 }
 
-template <bool IS_MAX, bool COH>
-__device__ __forceinline__ void tile_pool (const aspen_hip_layer_t &L, uint32_t tn)
+template <bool IS_MAX, int COH>
+__device__ __forceinline__ void tile_pool (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm)
 {
-    const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N), M4 = L.ld >> 2;
+    // rows [r0, r1) of the tile; the last row tile also covers the padding rows up to the stride
+    const uint32_t r0 = tm * L.tile_m, r1 = tm + 1 == L.tiles_m ? L.ld : r0 + L.tile_m;
+    const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N), M4 = (r1 - r0) >> 2;
     const uint32_t total = (n1 - n0) * M4, ohw = L.OH * L.OW;
     const float inv = 1.0f / (float)(L.KH * L.KW);
     ActView<COH> in, out;
     in.init (L.in0, (L.N / ohw) * L.IH * L.IW, L.ld0); out.init (L.out, L.N, L.ld);
     for (uint32_t i = tile_thread (); i < total; i += WG_THREADS)
     {
-        const uint32_t c = i / M4, m = (i - c * M4) * 4, n = n0 + c;
+        const uint32_t c = i / M4, m = r0 + (i - c * M4) * 4, n = n0 + c;
         const uint32_t b = n / ohw, rem = n - b * ohw, oh = rem / L.OW, ow = rem - oh * L.OW;
         float4 r = IS_MAX ? make_float4 (-INFINITY, -INFINITY, -INFINITY, -INFINITY) : make_float4 (0.f, 0.f, 0.f, 0.f);
         for (uint32_t kh = 0; kh < L.KH; kh++)
@@ -550,7 +558,7 @@ __device__ __forceinline__ float wave_max (float v)
 }
 
 // one wavefront per column: mean and E[x^2] in one pass, eps 1e-6f
-template <bool COH>
+template <int COH>
 __device__ __forceinline__ void tile_layernorm (const aspen_hip_layer_t &L, uint32_t tn)
 {
     const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N);
@@ -587,7 +595,7 @@ __device__ __forceinline__ void tile_layernorm (const aspen_hip_layer_t &L, uint
 }
 
 // one wavefront per column: max-subtracted softmax over the rows
-template <bool COH>
+template <int COH>
 __device__ __forceinline__ void tile_softmax (const aspen_hip_layer_t &L, uint32_t tn)
 {
     const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N);
@@ -614,7 +622,7 @@ __device__ __forceinline__ void tile_softmax (const aspen_hip_layer_t &L, uint32
 // sums are fused into the epilogue; a second sweep over the tile's own output divides by the sums.
 // in0 = Query matrix, in1 = Key matrix (reference cfg: parent = Query, from = Key).
 // ---------------------------------------------------------------------------------------------
-template <bool COH>
+template <int COH>
 __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, uint32_t tn, float *smem)
 {
     constexpr int BM = 128, BN = KATTN_BN, WM = 2, WN = 2, TM = BM / WM / 32, TN = BN / WN / 32;
@@ -696,7 +704,7 @@ __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, ui
 // V tile: one (batch, head-slice of <= 64 channels) x 128 queries:
 // out[b*S + q][h*hd + j] = sum_s P[(b*H + h)*S + q][s] * V[b*S + s][h*hd + j].
 // in0 = probabilities (K-attention output), in1 = Value matrix.
-template <bool COH>
+template <int COH>
 __device__ __forceinline__ void tile_v_attention (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, float *smem)
 {
     constexpr int BM = 64, BN = 128, WM = 2, WN = 2, TM = 1, TN = 2;
@@ -746,7 +754,7 @@ __device__ __forceinline__ aspen_hip_layer_t uniform_layer (const aspen_hip_laye
     return L;
 }
 
-template <bool COH>
+template <int COH>
 __device__ __forceinline__ void run_tile (const aspen_hip_layer_t &Lg, uint32_t t, float *smem)
 {
     const aspen_hip_layer_t L = uniform_layer (Lg);
@@ -774,8 +782,8 @@ __device__ __forceinline__ void run_tile (const aspen_hip_layer_t &Lg, uint32_t 
         else tile_contraction<VAR2_BM, VAR2_BN, 2, 2, COH> (L, tn, tm, slice, smem);
         break;
     case RESIDUAL_LAYER:    tile_residual<COH> (L, tn); break;
-    case MAXPOOL_LAYER:     tile_pool<true, COH> (L, tn); break;
-    case AVGPOOL_LAYER:     tile_pool<false, COH> (L, tn); break;
+    case MAXPOOL_LAYER:     tile_pool<true, COH> (L, tn, tm); break;
+    case AVGPOOL_LAYER:     tile_pool<false, COH> (L, tn, tm); break;
     case LAYERNORM_LAYER:   tile_layernorm<COH> (L, tn); break;
     case SOFTMAX_LAYER:     tile_softmax<COH> (L, tn); break;
     case K_ATTENTION_LAYER: tile_k_attention<COH> (L, tn, smem); break;

@@ -2,6 +2,7 @@
 #include "internal.h"
 #include "aspen_ext.h"
 
+unsigned int aspen_rpool_num_ninst (rpool_t *rp);
 void aspen_nasm_tile_range_internal (const nasm_ldata_t *ld, unsigned int t, unsigned int *r);
 
 void aspen_dse_group_set_mode (dse_group_t *g, int mode) { if (g) g->mode = mode ? 1 : 0; }
@@ -52,10 +53,16 @@ int aspen_rpool_profile_layers (rpool_t *rp, unsigned int iters, float *ms)
     return aspen_hip_profile_layers (rp->graph, iters, ms);
 }
 
-int aspen_rpool_dataflow_profile (rpool_t *rp, uint64_t ticks[4], int reset)
+int aspen_rpool_dataflow_profile (rpool_t *rp, uint64_t ticks[8], int reset)
 {
     if (rp == NULL || rp->graph == NULL) return -1;
     return aspen_hip_dataflow_profile (rp->graph, ticks, reset);
+}
+
+int aspen_rpool_dataflow_trace (rpool_t *rp, uint64_t *start_end)
+{
+    if (rp == NULL || rp->graph == NULL) return -1;
+    return aspen_hip_dataflow_trace (rp->graph, start_end, aspen_rpool_num_ninst (rp));
 }
 
 unsigned int aspen_rpool_num_ninst (rpool_t *rp)

@@ -140,6 +140,14 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
         while (tn > 4 && cdiv (N, tn) < want) tn /= 2;
         while (tn < 1024 && (uint64_t)tn * ld->out_mat_stride < 16384 && cdiv (N, tn * 2) >= 2 * want) tn *= 2;
         ld->tile_dims[OUT_H] = M; ld->tile_dims[OUT_W] = tn;
+        /* pooling layers with few output positions (global average pooling) are cut along the
+           channels as well, in multiples of 32 rows */
+        if ((L->type == MAXPOOL_LAYER || L->type == AVGPOOL_LAYER) && cdiv (N, tn) < want && M >= 64)
+        {
+            unsigned int tm = 256;
+            while (tm > 32 && cdiv (N, tn) * cdiv (M, tm) < want) tm /= 2;
+            if (tm < M) ld->tile_dims[OUT_H] = tm;
+        }
     }
     ld->tiles_h = cdiv (M, ld->tile_dims[OUT_H]);
     ld->tiles_w = cdiv (N, ld->tile_dims[OUT_W]);

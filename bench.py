@@ -102,6 +102,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--skip-tiles", action="store_true", help="scheduler-only run: dependency protocol with empty tiles")
     ap.add_argument("--engine-profile", action="store_true", help="report where the persistent workgroups spend their time")
+    ap.add_argument("--trace", default="", metavar="NPZ", help="write per-tile start/end stamps of the last timed step (dataflow mode)")
     ap.add_argument("--layer-profile", action="store_true", help="also time every layer's kernel (layer-launch mode)")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
                     help="instead of a workload: run the library's streaming copy kernel over MIB MiB (--steps launches); "
@@ -133,7 +134,7 @@ def main():
                           "ms_per_launch": ms.value / args.steps,
                           "GB_per_s": 2 * nbytes * args.steps / (ms.value * 1e-3) / 1e9}))
         return
-    L.aspen_hip_set_flags((1 if args.skip_tiles else 0) | (4 if args.engine_profile else 0))
+    L.aspen_hip_set_flags((1 if args.skip_tiles else 0) | (4 if args.engine_profile else 0) | (8 if args.trace else 0))
     cfgs, unit, units_per_step = WORKLOADS[args.workload]
 
     pool = api.RPool()
@@ -208,6 +209,14 @@ def main():
         prof = pool.dataflow_profile()
         out["engine_profile"] = {k: v / max(prof["total"], 1e-12) for k, v in prof.items() if k != "total"}
         out["engine_profile"]["workgroup_seconds_per_step"] = prof["total"] / args.steps
+    if args.trace and args.mode == "dataflow":
+        stamps = pool.dataflow_trace()
+        tile_layer, base = [], 0
+        for _, _, n, _ in nets:
+            tile_layer.append(n.graph()[0].astype(np.int64) + base)
+            base += n.num_ldata
+        types = [n.info(l)["type"] for _, _, n, _ in nets for l in range(n.num_ldata)]
+        np.savez(args.trace, stamps=stamps, tile_layer=np.concatenate(tile_layer), layer_type=np.array(types))
     if args.layer_profile:
         # conv-tile MFMA utilisation and bandwidth of the elementwise tiles, one kernel per layer
         nl = sum(n.num_ldata for _, _, n, _ in nets)

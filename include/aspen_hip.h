@@ -127,9 +127,16 @@ int aspen_hip_run_dataflow (aspen_hip_graph_t *graph, uint32_t workgroups, uint6
 /* PROFILE makes every workgroup of the dataflow kernel accumulate where its time went. */
 #define ASPEN_HIP_FLAG_PROFILE 4u
 /* ticks (100 MHz) summed over all workgroups since the last reset: [0] inside tiles, [1] waiting for
-   the tile's stores to be acknowledged, [2] scheduling (publish, pop, waiting for a ready tile),
-   [3] total workgroup lifetime */
-int aspen_hip_dataflow_profile (aspen_hip_graph_t *graph, uint64_t ticks[4], int reset);
+   the tile's stores to be acknowledged, [2] scheduling step (publish, pop, waiting for a ready tile),
+   [3] total workgroup lifetime; detail of [2]: [4] publishing wavefront (countdown of the children,
+   pushes), [5] popping wavefront drawing its ticket, [6] popping wavefront waiting for its queue slot
+   to be filled; [7] unused */
+int aspen_hip_dataflow_profile (aspen_hip_graph_t *graph, uint64_t ticks[8], int reset);
+/* TRACE makes the dataflow kernel stamp every tile's start and end (100 MHz device clock);
+   aspen_hip_dataflow_trace copies the stamps of the last traced run: start_end[2*i], [2*i+1] for tile i
+   of the graph's num_ninst tiles. */
+#define ASPEN_HIP_FLAG_TRACE 8u
+int aspen_hip_dataflow_trace (aspen_hip_graph_t *graph, uint64_t *start_end, uint32_t num_ninst);
 void aspen_hip_set_flags (uint32_t flags);
 int aspen_hip_sync (void);
 /* 1 when everything enqueued so far has finished, 0 when still running */
