@@ -445,8 +445,14 @@ static bool lines_have_one_producer (const aspen_hip_layer_t *layers, uint32_t n
         bool is_read = false;
         for (uint32_t c = 0; c < num_layers && !is_read; c++) is_read = layers[c].in0 == P.out || layers[c].in1 == P.out;
         const bool aligned = (uintptr_t)P.out % 128 == 0 && ((size_t)P.ld * 4) % 128 == 0 && (P.tiles_m == 1 || (P.tile_m * 4) % 128 == 0);
-        if (is_read && !aligned) return false;
-        if (P.splits > 1 && ((uintptr_t)P.partial % 128 != 0 || !aligned)) return false;
+        const bool ok = !(is_read && !aligned) && !(P.splits > 1 && ((uintptr_t)P.partial % 128 != 0 || !aligned));
+        if (!ok)
+        {
+            if (getenv ("ASPEN_GPU_VERBOSE"))
+                fprintf (stderr, "aspen_hip: layer %u (type %d, ld %u, tile_m %u, tiles_m %u) shares cache lines between tiles: coherent loads\n",
+                    l, P.type, P.ld, P.tile_m, P.tiles_m);
+            return false;
+        }
     }
     return true;
 }

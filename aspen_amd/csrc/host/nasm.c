@@ -77,9 +77,12 @@ static int set_out_mat (nasm_t *nasm, nasm_ldata_t *ld)
         return -1;
     }
     ld->flops = flop_per_out * ld->out_mat_dims[OUT_H] * ld->out_mat_dims[OUT_W];
-    ld->out_mat_stride = aspen_ld_for_rows (ld->out_mat_dims[OUT_H]);
-    if (L->type == K_ATTENTION_LAYER)
-        ld->out_mat_stride = cdiv (S, 32) * 32;     /* the V tile streams it 32 keys at a time */
+    /* the input keeps the tight 16-byte column alignment (3-channel images would otherwise be read
+       8x); every matrix produced on the device gets 128-byte columns, so that no cache line is shared
+       between two columns (and hence between two producer tiles), which lets consumers read it
+       through the caches.  K-attention needs the multiple of 32 anyway: the V tile streams the
+       probabilities 32 keys at a time. */
+    ld->out_mat_stride = L->type == INPUT_LAYER ? aspen_ld_for_rows (ld->out_mat_dims[OUT_H]) : cdiv (ld->out_mat_dims[OUT_H], 32) * 32;
     return 0;
 }
 

@@ -97,7 +97,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="resnet50_b32", choices=list(WORKLOADS))
     ap.add_argument("--mode", default="dataflow", choices=["dataflow", "layers"])
-    ap.add_argument("--min-ninst", type=int, default=512)
+    ap.add_argument("--min-ninst", type=int, default=1536)
     ap.add_argument("--workgroups", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--skip-tiles", action="store_true", help="scheduler-only run: dependency protocol with empty tiles")
