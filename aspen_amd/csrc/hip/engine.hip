@@ -294,7 +294,12 @@ extern "C" int aspen_hip_device_info (int *num_cu, int *clock_khz, size_t *mem_b
     if (num_cu) *num_cu = prop.multiProcessorCount;
     if (clock_khz) *clock_khz = prop.clockRate;
     if (mem_bytes) *mem_bytes = prop.totalGlobalMem;
-    if (name && name_len > 0) { strncpy (name, prop.name, name_len - 1); name[name_len - 1] = 0; }
+    if (name && name_len > 0)
+    {
+        // some driver stacks leave the marketing name empty: fall back to the architecture name
+        strncpy (name, prop.name[0] ? prop.name : prop.gcnArchName, name_len - 1);
+        name[name_len - 1] = 0;
+    }
     return 0;
 }
 

@@ -22,6 +22,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3      # MI355X dense fp32 matrix peak
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the persistent kernel, measured with rocprofv3 FETCH_SIZE / WRITE_SIZE passes
+# calibrated on the library's copy kernel (summary: profiles/dataflow_kernel_resnet50_b32_hbm_traffic.txt);
+# valid for the default configuration of that workload only
+MEASURED_TRAFFIC_BYTES = {("resnet50_b32", "dataflow", 1536): 11.57e9}
 
 # algorithmic GEMM-class flops per unit (2*M*N*K with the reference's K: padding taps counted, full
 # S x S attention): per image for the vision nets, per token for the transformers
@@ -197,13 +201,35 @@ def main():
         k_ms = float(np.mean(kernel_ms))
         ach = flops / (k_ms * 1e-3) / 1e12
         out["roofline"] = {"bound": "mfma", "kernel": "dataflow_kernel", "achieved": ach, "peak": PEAK_FP32_MFMA_TFLOPS,
-                           "unit": "TFLOP/s", "frac": ach / PEAK_FP32_MFMA_TFLOPS, "traffic": None,
+                           "unit": "TFLOP/s", "frac": ach / PEAK_FP32_MFMA_TFLOPS,
+                           "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, args.mode, args.min_ninst)),
                            "flops_per_launch": flops, "kernel_ms": k_ms}
     else:
         ach = flops / (ms_per_step * 1e-3) / 1e12
         out["roofline"] = {"bound": "mfma", "kernel": "layer_kernel (all layers of one step)", "achieved": ach,
                            "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": ach / PEAK_FP32_MFMA_TFLOPS,
                            "traffic": None, "flops_per_launch": flops, "kernel_ms": ms_per_step}
+
+    # the same step with the host boundary inside: input upload before, logits download after
+    # (PCIe-inclusive rate; reported beside `value`, never as `value`)
+    if not args.skip_tiles:
+        xs = [M.make_config(name)[3] for name in cfgs]
+        t0 = time.perf_counter()
+        io_steps = max(1, min(5, args.steps))
+        for _ in range(io_steps):
+            pool.reset_queue()
+            for (_, _, n, _), x in zip(nets, xs):
+                pool.reset_nasm(n)
+                pool.add_nasm_raw_input(n, x)
+            dse.run()
+            for _, _, n, _ in nets:
+                dse.wait(n)
+            dse.stop()
+            for _, _, n, _ in nets:
+                n.result()
+        dt_io = (time.perf_counter() - t0) / io_steps
+        out["host_io_inclusive"] = {"value": units_per_step / dt_io, "unit": unit, "ms_per_step": dt_io * 1e3, "steps": io_steps,
+                                    "note": "input copied from pageable host memory and final layer copied back every step"}
 
     if args.engine_profile and args.mode == "dataflow":
         prof = pool.dataflow_profile()
