@@ -348,10 +348,13 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
                 #pragma unroll
                 for (int i = 0; i < TN; i++) bf[nxt][i] = ld4 (S + bfrag + i * 32 * LDS_ROW + (kk + 1) * 8);
             }
-            else if (more && GEMM_STAGES == 2)
+            else if (more)
             {
-                // the next K slice (in registers since the previous iteration) goes to the other stage,
-                // overlapping with the last group of MFMAs; then its successor is requested from memory
+                // the next K slice (in registers since the previous iteration) goes to LDS while the
+                // matrix cores work on the last sub-step; then its successor is requested from memory.
+                // Single stage: every wave has fetched its last fragments of the current slice by now,
+                // so after a barrier the slice can be overwritten in place.
+                if (GEMM_STAGES == 1) lds_barrier ();
                 al.store (Snext, areg); bl.store (Snext + BM * LDS_ROW, breg);
                 if (it + 2 < kiters) { al.load (kbase + it + 2, areg); bl.load (kbase + it + 2, breg); }
             }
@@ -365,14 +368,6 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[cur][i].z, af[cur][j].z, acc[i][j], 0, 0, 0);
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[cur][i].w, af[cur][j].w, acc[i][j], 0, 0, 0);
                 }
-        }
-        if (GEMM_STAGES == 1 && more)
-        {
-            // single stage: once every wave has read its last fragments, the slice waiting in
-            // registers replaces the one in LDS and the slice after it is requested from memory
-            lds_barrier ();
-            al.store (Snext, areg); bl.store (Snext + BM * LDS_ROW, breg);
-            if (it + 2 < kiters) { al.load (kbase + it + 2, areg); bl.load (kbase + it + 2, breg); }
         }
         lds_barrier ();
     }
