@@ -20,30 +20,21 @@ typedef float floatx16 __attribute__ ((ext_vector_type (16)));
 #define GEMM_BK 32            // K floats staged per iteration: one 128-byte line per operand row
 #define LDS_ROW 36            // floats per staged row: 32 + 4 padding -> conflict-free 128-bit reads
 
-// Two footprints.  Default: tiles of at most 128 x 64 outputs, 32 accumulator registers per lane, one
-// LDS stage (the next K slice waits in registers) -> <= 128 VGPRs and <= 40 KB LDS per workgroup, so
-// FOUR workgroups (16 wavefronts) share a compute unit and one workgroup's load latency, epilogue
-// and scheduling gaps are covered by the other three.  ASPEN_BIG_TILES: 128 x 128 tiles, two LDS
-// stages, two workgroups per compute unit (better for very large GEMMs, worse for short ones).
-#ifdef ASPEN_BIG_TILES
-#define VAR0_BM 128
-#define VAR0_BN 128
-#define GEMM_STAGES 2
-#define WG_PER_CU 2
-#define KATTN_BN 128
-#else
+// Tiles of at most 128 x 64 outputs, 32 accumulator registers per lane, one LDS stage (the next K
+// slice waits in registers) -> <= 128 VGPRs and <= 40 KB LDS per workgroup, so FOUR workgroups (16
+// wavefronts) share a compute unit and one workgroup's load latency, epilogue and scheduling gaps are
+// covered by the other three.  (128 x 128 tiles with two LDS stages and two workgroups per compute
+// unit were measured too: better for very large GEMMs only, worse for every network here.)
 #define VAR0_BM 128
 #define VAR0_BN 64
-#define GEMM_STAGES 1
 #define WG_PER_CU 4
 #define KATTN_BN 64
-#endif
 #define VAR1_BM 64
 #define VAR1_BN 128
 #define VAR2_BM 64
 #define VAR2_BN 64
 #define CMAX(a, b) ((a) > (b) ? (a) : (b))
-#define STAGE_FLOATS(bm, bn) (GEMM_STAGES * ((bm) + (bn)) * LDS_ROW)
+#define STAGE_FLOATS(bm, bn) (((bm) + (bn)) * LDS_ROW)
 #define EPI_FLOATS(bm, bn) ((bn) * ((bm) + 8))
 #define VAR_FLOATS(bm, bn) CMAX (STAGE_FLOATS (bm, bn), EPI_FLOATS (bm, bn))
 #define GEMM_SMEM_FLOATS CMAX (CMAX (VAR_FLOATS (VAR0_BM, VAR0_BN), VAR_FLOATS (VAR1_BM, VAR1_BN)), \
@@ -283,7 +274,7 @@ template <int COH> struct TransLoader64
 // owning (BM/WM) x (BN/WN) built from 32x32 v_mfma_f32_32x32x2_f32 blocks.  The activation row is
 // the MFMA row index and the weight row the MFMA column, so each accumulator register holds 32
 // consecutive output channels of one output column: stores are 128-byte coalesced.
-// One or two LDS stages (GEMM_STAGES); the K slice after the staged one always waits in registers.
+// One LDS stage; the K slice after the staged one waits in registers.
 // ---------------------------------------------------------------------------------------------
 // LDS-only barrier: waits for this wave's LDS traffic, not for global loads still in flight.
 // The thread index as a value the optimiser cannot move out of an enclosing persistent loop: the
@@ -301,17 +292,22 @@ __device__ __forceinline__ void lds_barrier ()
     asm volatile ("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+// Instruction-group hints for the machine scheduler (masks of __builtin_amdgcn_sched_group_barrier)
+#define SG_MFMA 0x008
+#define SG_VMEM_READ 0x020
+#define SG_DS_READ 0x100
+#define SG_DS_WRITE 0x200
+
 template <int BM, int BN, int WM, int WN, class ALoader, class BLoader>
 __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, int kiters, float *smem,
     floatx16 (&acc)[BN / WN / 32][BM / WM / 32])
 {
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-    constexpr int STAGE = GEMM_STAGES == 2 ? (BM + BN) * LDS_ROW : 0;
     constexpr int KK = GEMM_BK / 8;
     const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
     const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);
-    const uint32_t afrag = wm0 * LDS_ROW + (lane & 31) * LDS_ROW + (lane >> 5) * 4;
-    const uint32_t bfrag = BM * LDS_ROW + wn0 * LDS_ROW + (lane & 31) * LDS_ROW + (lane >> 5) * 4;
+    const float *afrag = smem + wm0 * LDS_ROW + (lane & 31) * LDS_ROW + (lane >> 5) * 4;
+    const float *bfrag = smem + BM * LDS_ROW + wn0 * LDS_ROW + (lane & 31) * LDS_ROW + (lane >> 5) * 4;
 
     #pragma unroll
     for (int i = 0; i < TN; i++)
@@ -320,57 +316,90 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
             #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
+    // fragments of sub-step s (8 K values: lanes 0-31 take the first four, lanes 32-63 the last four)
+    float4 af[2][TM], bf[2][TN];
+    auto read_frags = [&] (int buf, int sub)
+    {
+        #pragma unroll
+        for (int j = 0; j < TM; j++) af[buf][j] = ld4 (afrag + j * 32 * LDS_ROW + sub * 8);
+        #pragma unroll
+        for (int i = 0; i < TN; i++) bf[buf][i] = ld4 (bfrag + i * 32 * LDS_ROW + sub * 8);
+    };
+    // half = 0: K components x, y of the fragments; half = 1: z, w
+    auto mfma_half = [&] (int buf, int half)
+    {
+        #pragma unroll
+        for (int i = 0; i < TN; i++)
+            #pragma unroll
+            for (int j = 0; j < TM; j++)
+            {
+                if (half == 0)
+                {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[buf][i].x, af[buf][j].x, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[buf][i].y, af[buf][j].y, acc[i][j], 0, 0, 0);
+                }
+                else
+                {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[buf][i].z, af[buf][j].z, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[buf][i].w, af[buf][j].w, acc[i][j], 0, 0, 0);
+                }
+            }
+    };
+
     float4 areg[ALoader::R], breg[BLoader::R];
     al.load (kbase, areg); bl.load (kbase, breg);
     al.store (smem, areg); bl.store (smem + BM * LDS_ROW, breg);
     if (kiters > 1) { al.load (kbase + 1, areg); bl.load (kbase + 1, breg); }
     lds_barrier ();
+    read_frags (0, 0);
 
-    for (int it = 0; it < kiters; it++)
+    // One K slice per iteration, single LDS stage, software-pipelined by hand:
+    //   sub-steps 0 .. KK-2: the fragments of sub-step s+1 are fetched between the two halves of the
+    //   MFMAs of sub-step s, so they have arrived even if the compiler waits for ALL LDS traffic before s+1;
+    //   last sub-step: once every wave holds its last fragments (barrier), the next slice (waiting in
+    //   registers) overwrites the stage and the slice after it is requested from memory, all under
+    //   the first half of the sub-step's MFMAs; after the second barrier the first fragments of the new
+    //   slice are fetched under the second half.
+    // The scheduling-group hints pin that order; left alone, the compiler fetches each fragment right
+    // before its use and the LDS latency shows.
+    for (int it = 0; it + 1 < kiters; it++)
     {
-        const float *S = smem + (it & 1) * STAGE;
-        float *Snext = smem + ((it + 1) & 1) * STAGE;
-        const bool more = it + 1 < kiters;
-        // fragments of sub-step kk+1 are fetched from LDS while the matrix cores work on sub-step kk
-        float4 af[2][TM], bf[2][TN];
         #pragma unroll
-        for (int j = 0; j < TM; j++) af[0][j] = ld4 (S + afrag + j * 32 * LDS_ROW);
-        #pragma unroll
-        for (int i = 0; i < TN; i++) bf[0][i] = ld4 (S + bfrag + i * 32 * LDS_ROW);
-        #pragma unroll
-        for (int kk = 0; kk < KK; kk++)
+        for (int kk = 0; kk + 1 < KK; kk++)
         {
-            const int cur = kk & 1, nxt = cur ^ 1;
-            if (kk + 1 < KK)
-            {
-                #pragma unroll
-                for (int j = 0; j < TM; j++) af[nxt][j] = ld4 (S + afrag + j * 32 * LDS_ROW + (kk + 1) * 8);
-                #pragma unroll
-                for (int i = 0; i < TN; i++) bf[nxt][i] = ld4 (S + bfrag + i * 32 * LDS_ROW + (kk + 1) * 8);
-            }
-            else if (more)
-            {
-                // the next K slice (in registers since the previous iteration) goes to LDS while the
-                // matrix cores work on the last sub-step; then its successor is requested from memory.
-                // Single stage: every wave has fetched its last fragments of the current slice by now,
-                // so after a barrier the slice can be overwritten in place.
-                if (GEMM_STAGES == 1) lds_barrier ();
-                al.store (Snext, areg); bl.store (Snext + BM * LDS_ROW, breg);
-                if (it + 2 < kiters) { al.load (kbase + it + 2, areg); bl.load (kbase + it + 2, breg); }
-            }
-            #pragma unroll
-            for (int i = 0; i < TN; i++)
-                #pragma unroll
-                for (int j = 0; j < TM; j++)
-                {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[cur][i].x, af[cur][j].x, acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[cur][i].y, af[cur][j].y, acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[cur][i].z, af[cur][j].z, acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32 (bf[cur][i].w, af[cur][j].w, acc[i][j], 0, 0, 0);
-                }
+            mfma_half (kk & 1, 0);
+            read_frags ((kk + 1) & 1, kk + 1);
+            mfma_half (kk & 1, 1);
+            __builtin_amdgcn_sched_group_barrier (SG_MFMA, 2 * TM * TN, 0);
+            __builtin_amdgcn_sched_group_barrier (SG_DS_READ, TM + TN, 0);
+            __builtin_amdgcn_sched_group_barrier (SG_MFMA, 2 * TM * TN, 0);
         }
+        __builtin_amdgcn_sched_barrier (0);
         lds_barrier ();
+        __builtin_amdgcn_sched_barrier (0);
+        al.store (smem, areg); bl.store (smem + BM * LDS_ROW, breg);
+        if (it + 2 < kiters) { al.load (kbase + it + 2, areg); bl.load (kbase + it + 2, breg); }
+        mfma_half ((KK - 1) & 1, 0);
+        __builtin_amdgcn_sched_barrier (0);
+        lds_barrier ();
+        __builtin_amdgcn_sched_barrier (0);
+        read_frags (0, 0);
+        mfma_half ((KK - 1) & 1, 1);
+        __builtin_amdgcn_sched_group_barrier (SG_DS_READ, TM + TN, 0);
+        __builtin_amdgcn_sched_group_barrier (SG_MFMA, 2 * TM * TN, 0);
     }
+    // last slice: nothing left to stage
+    #pragma unroll
+    for (int kk = 0; kk < KK; kk++)
+    {
+        mfma_half (kk & 1, 0);
+        if (kk + 1 < KK) read_frags ((kk + 1) & 1, kk + 1);
+        mfma_half (kk & 1, 1);
+        __builtin_amdgcn_sched_group_barrier (SG_MFMA, 2 * TM * TN, 0);
+        if (kk + 1 < KK) __builtin_amdgcn_sched_group_barrier (SG_DS_READ, TM + TN, 0);
+        __builtin_amdgcn_sched_group_barrier (SG_MFMA, 2 * TM * TN, 0);
+    }
+    lds_barrier ();          // the caller reuses the stage (epilogue)
 }
 
 // Accumulator register v of MFMA block (i, j) holds output (row n, channel m):
