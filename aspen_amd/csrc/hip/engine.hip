@@ -14,6 +14,7 @@
 #include "tile_kernels.h"
 
 #define QUEUE_EMPTY 0xffffffffu
+typedef unsigned long long qentry_t;      // ready-queue entry / child-record entry, see arm_kernel
 #define ST_HEAD 0
 #define ST_TAIL 32
 #define ST_DONE 64
@@ -30,7 +31,8 @@ struct aspen_hip_graph_t
     aspen_hip_layer_t *d_layers;
     uint32_t *d_ninst_layer, *d_num_parents, *d_child_off, *d_child_idx, *d_roots;
     uint32_t *d_dep;        // remaining-parent counters, re-armed before every dataflow run
-    uint32_t *d_queue;      // ready queue: slot t is written once, by whoever makes a tile ready
+    qentry_t *d_queue;      // ready queue: slot t is written once, by whoever makes a tile ready
+    qentry_t *d_child_rec;  // per tile: child count + its first CHILD_REC-1 children with their layers
     uint32_t *d_state;      // one counter per 128-byte line: [ST_HEAD] pop tickets, [ST_TAIL] push cursor, [ST_DONE] tiles done,
                             // [ST_ABORT] abort flag, [ST_TWICE] tiles executed more than once
     uint32_t *d_ran;        // per-tile execution count (sanity: every tile exactly once)
@@ -72,21 +74,27 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) layer_kernel (const as
     run_tile<0> (L, t, smem);
 }
 
-// Re-arm: counters back to the parent counts, queue seeded with the roots.  Queue entries carry the
-// run's epoch in their top byte (entry = epoch << 24 | tile): an entry left over from an earlier
-// run never matches the current epoch, so the queue needs no clearing and a poll can never mistake
-// an old entry for a new one.  All writes are device-scope (write-through) stores, the same path
-// the persistent kernel's polls and atomics use.
+// Re-arm: counters back to the parent counts, queue seeded with the roots.  A queue entry is 64 bits:
+// tile [31:0], layer [47:32], the run's epoch [63:56].  An entry left over from an earlier run never
+// matches the current epoch, so the queue needs no clearing and a poll can never mistake an old
+// entry for a new one; carrying the layer saves the consumer a dependent lookup.  All writes are
+// device-scope (write-through) stores, the same path the persistent kernel's polls and atomics use.
 #define QUEUE_ID_BITS 24
 #define QUEUE_ID_MASK ((1u << QUEUE_ID_BITS) - 1u)
-__global__ void arm_kernel (uint32_t *dep, const uint32_t *num_parents, uint32_t *queue, uint32_t *ran,
-    const uint32_t *roots, uint32_t num_ninst, uint32_t num_roots, uint32_t *state, uint32_t epoch)
+#define MAX_GRAPH_LAYERS 65535u
+__device__ __forceinline__ qentry_t make_entry (uint32_t epoch, uint32_t layer, uint32_t tile)
+{
+    return ((qentry_t)epoch << 56) | ((qentry_t)layer << 32) | tile;
+}
+__global__ void arm_kernel (uint32_t *dep, const uint32_t *num_parents, qentry_t *queue, uint32_t *ran,
+    const uint32_t *roots, const uint32_t *ninst_layer, uint32_t num_ninst, uint32_t num_roots, uint32_t *state, uint32_t epoch)
 {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < num_ninst)
     {
         __hip_atomic_store (&dep[i], num_parents[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (i < num_roots) __hip_atomic_store (&queue[i], (epoch << QUEUE_ID_BITS) | roots[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (i < num_roots)
+            __hip_atomic_store (&queue[i], make_entry (epoch, ninst_layer[roots[i]], roots[i]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store (&ran[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (i == 0)
@@ -103,7 +111,9 @@ struct dataflow_args_t
 {
     const aspen_hip_layer_t *layers;
     const uint32_t *ninst_layer, *child_off, *child_idx;
-    uint32_t *dep, *queue, *state, *ran;
+    const qentry_t *child_rec;      // [num_ninst][CHILD_REC]: [0] = number of children, then the first CHILD_REC-1 as (layer << 32 | tile)
+    qentry_t *queue;
+    uint32_t *dep, *state, *ran;
     uint32_t *host_abort;
     unsigned long long *trace;      // per-tile start / end time stamps when ASPEN_HIP_FLAG_TRACE is set
     unsigned long long *prof;       // 8 counters of summed 100 MHz ticks, see aspen_hip_dataflow_profile
@@ -113,26 +123,27 @@ struct dataflow_args_t
     unsigned long long spin_limit;
 };
 
-#define QUEUE_EMPTY_TILE QUEUE_EMPTY
+#define CHILD_REC 64     // entries per child record: one per lane of the publishing wavefront
+#define QENTRY_EMPTY (~(qentry_t)0)
 
-// Waits until queue slot `ticket` holds a tile and returns it; QUEUE_EMPTY when all tickets are
-// taken or the run was aborted.  The wait polls with relaxed device-scope loads (an acquire here
-// would invalidate this XCD's L2 on every poll).
-__device__ __forceinline__ uint32_t wait_for_slot (const dataflow_args_t &a, uint32_t ticket)
+// Waits until queue slot `ticket` holds a tile of this run and returns the entry; QENTRY_EMPTY when all
+// tickets are taken or the run was aborted.  The wait polls with relaxed device-scope loads (an
+// acquire here would invalidate this XCD's L2 on every poll).
+__device__ __forceinline__ qentry_t wait_for_slot (const dataflow_args_t &a, uint32_t ticket)
 {
-    if (ticket >= a.num_ninst) return QUEUE_EMPTY;
+    if (ticket >= a.num_ninst) return QENTRY_EMPTY;
     unsigned long long spins = 0;
     for (;;)
     {
-        const uint32_t e = __hip_atomic_load (&a.queue[ticket], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if ((e >> QUEUE_ID_BITS) == a.epoch) return e & QUEUE_ID_MASK;
+        const qentry_t e = __hip_atomic_load (&a.queue[ticket], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((uint32_t)(e >> 56) == a.epoch) return e;
         ++spins;
-        if ((spins & 63) == 0 && __hip_atomic_load (&a.state[ST_ABORT], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return QUEUE_EMPTY;
+        if ((spins & 63) == 0 && __hip_atomic_load (&a.state[ST_ABORT], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return QENTRY_EMPTY;
         if (spins > a.spin_limit)
         {
             __hip_atomic_store (&a.state[ST_ABORT], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store (a.host_abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-            return QUEUE_EMPTY;
+            return QENTRY_EMPTY;
         }
         __builtin_amdgcn_s_sleep (2);
     }
@@ -143,7 +154,7 @@ __device__ __forceinline__ uint32_t wait_for_slot (const dataflow_args_t &a, uin
 struct sched_lds_t
 {
     dataflow_args_t a;
-    uint32_t tile;                       // tile to run next (QUEUE_EMPTY: leave)
+    uint32_t tile, layer;                // tile to run next (QUEUE_EMPTY: leave) and its layer
     unsigned long long t0, ticks[6];     // profiling: last time stamp; tile / drain / scheduling / publish / ticket / slot-wait ticks
 };
 __shared__ sched_lds_t s_sched;
@@ -157,12 +168,25 @@ __device__ __forceinline__ void prof_lap (int which)
     }
 }
 
+// Counts down one child; whoever takes its counter to zero puts it into the ready queue.
+__device__ __forceinline__ void release_child (const dataflow_args_t &a, uint32_t child, uint32_t layer)
+{
+    const uint32_t before = __hip_atomic_fetch_sub (&a.dep[child], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (before == 1u)
+    {
+        const uint32_t slot = atomicAdd (&a.state[ST_TAIL], 1u);
+        __hip_atomic_store (&a.queue[slot], make_entry (a.epoch, layer, child), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
 // One scheduling step of a workgroup, as a real function call (it needs few registers, all of them
 // caller-saved, so the call costs no register traffic): wavefront 0 publishes the finished tile
 // (dependency countdown of its children, push of those that became ready) while wavefront 1 pops the
-// next one.  done == QUEUE_EMPTY: nothing to publish (first step).  Returns the tile to run next.
+// next one.  done == QUEUE_EMPTY: nothing to publish (first step).  `rec` is this lane's entry of the
+// finished tile's child record, fetched by wavefront 0 before the tile ran, so publishing starts
+// with the atomics right away.  Returns the tile to run next; its layer is left in s_sched.layer.
 // The reference's counterpart is dse_schedule / update_children (src/dse.c:20-108, :363-401).
-__device__ __noinline__ uint32_t schedule_step (uint32_t done)
+__device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
 {
     const dataflow_args_t &a = s_sched.a;
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -180,17 +204,17 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done)
     if (wave == 0 && done != QUEUE_EMPTY)
     {
         const unsigned long long tp = prof ? wall_clock64 () : 0;
-        // publish: count down the children with relaxed device-scope atomics; whoever takes a
-        // child's counter to zero puts it into the ready queue
-        const uint32_t c0 = a.child_off[done], c1 = a.child_off[done + 1];
-        for (uint32_t c = c0 + lane; c < c1; c += 64)
+        // publish: relaxed device-scope atomics on the children's counters, one child per lane
+        const uint32_t count = (uint32_t)__shfl (rec, 0, 64);
+        if (lane >= 1 && lane <= count) release_child (a, (uint32_t)rec, (uint32_t)(rec >> 32));
+        if (count > CHILD_REC - 1)
         {
-            const uint32_t child = a.child_idx[c];
-            const uint32_t before = __hip_atomic_fetch_sub (&a.dep[child], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (before == 1u)
+            // more children than the record holds: the rest comes from the CSR lists
+            const uint32_t c0 = a.child_off[done] + (CHILD_REC - 1), c1 = a.child_off[done + 1];
+            for (uint32_t c = c0 + lane; c < c1; c += 64)
             {
-                const uint32_t slot = atomicAdd (&a.state[ST_TAIL], 1u);
-                __hip_atomic_store (&a.queue[slot], (a.epoch << QUEUE_ID_BITS) | child, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const uint32_t child = a.child_idx[c];
+                release_child (a, child, a.ninst_layer[child]);
             }
         }
         if (lane == 0 && (a.flags & ASPEN_HIP_FLAG_COUNT_TILES))
@@ -208,7 +232,9 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done)
         const unsigned long long t1 = prof ? wall_clock64 () : 0;
         const uint32_t ticket = atomicAdd (&a.state[ST_HEAD], 1u);
         const unsigned long long t2 = prof ? wall_clock64 () : 0;
-        s_sched.tile = wait_for_slot (a, ticket);
+        const qentry_t e = wait_for_slot (a, ticket);
+        s_sched.tile = e == QENTRY_EMPTY ? QUEUE_EMPTY : (uint32_t)e;
+        s_sched.layer = (uint32_t)(e >> 32) & 0xffffu;
         if (prof) { s_sched.ticks[4] += t2 - t1; s_sched.ticks[5] += wall_clock64 () - t2; }
     }
     __syncthreads ();
@@ -234,14 +260,17 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
     __syncthreads ();
     const unsigned long long t_begin = wall_clock64 ();
     uint32_t id = QUEUE_EMPTY;
+    qentry_t rec = 0;
     for (;;)
     {
-        id = __builtin_amdgcn_readfirstlane (schedule_step (id));
+        id = __builtin_amdgcn_readfirstlane (schedule_step (id, rec));
         if (id == QUEUE_EMPTY) break;           // all tickets taken, or aborted
+        // wavefront 0 requests this tile's child record now; it arrives while the tile runs
+        if (threadIdx.x < CHILD_REC) rec = s_sched.a.child_rec[(size_t)id * CHILD_REC + threadIdx.x];
         if ((s_sched.a.flags & ASPEN_HIP_FLAG_TRACE) && threadIdx.x == 0) s_sched.a.trace[2 * (size_t)id] = wall_clock64 ();
         if (!(s_sched.a.flags & ASPEN_HIP_FLAG_SKIP_TILES))
         {
-            const aspen_hip_layer_t *L = &s_sched.a.layers[s_sched.a.ninst_layer[id]];
+            const aspen_hip_layer_t *L = &s_sched.a.layers[__builtin_amdgcn_readfirstlane (s_sched.layer)];
             run_tile<COH> (*L, id - L->ninst_start, smem);
         }
     }
@@ -468,6 +497,7 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
 {
     if (aspen_hip_init ()) return nullptr;
     if (num_ninst > QUEUE_ID_MASK) { snprintf (g_err, sizeof (g_err), "graph has more than %u tiles", QUEUE_ID_MASK); return nullptr; }
+    if (num_layers > MAX_GRAPH_LAYERS) { snprintf (g_err, sizeof (g_err), "graph has more than %u layers", MAX_GRAPH_LAYERS); return nullptr; }
     for (uint32_t l = 0; l < num_layers; l++)
         if (check_layer (layers[l], l)) return nullptr;
     // host-side sanity of the dependency structure: every index in range, counts consistent
@@ -493,12 +523,25 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     g->d_child_idx = upload (child_idx, num_edges);
     g->d_roots = upload (roots, num_roots);
     g->d_dep = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
-    g->d_queue = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
+    g->d_queue = (qentry_t *)aspen_hip_alloc (sizeof (qentry_t) * (num_ninst + 1));
+    {
+        // child records: what the publishing wavefront fetches with one 64-lane load
+        qentry_t *rec = (qentry_t *)calloc ((size_t)(num_ninst ? num_ninst : 1) * CHILD_REC, sizeof (qentry_t));
+        for (uint32_t t = 0; t < num_ninst; t++)
+        {
+            const uint32_t c0 = child_off[t], n = child_off[t + 1] - c0;
+            rec[(size_t)t * CHILD_REC] = n;
+            for (uint32_t c = 0; c < n && c < CHILD_REC - 1; c++)
+                rec[(size_t)t * CHILD_REC + 1 + c] = ((qentry_t)ninst_layer[child_idx[c0 + c]] << 32) | child_idx[c0 + c];
+        }
+        g->d_child_rec = upload (rec, (size_t)num_ninst * CHILD_REC);
+        free (rec);
+    }
     g->d_ran = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
     g->d_state = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * ST_WORDS);
     g->d_prof = (unsigned long long *)aspen_hip_alloc (sizeof (unsigned long long) * 8);
     if (!g->d_layers || !g->d_ninst_layer || !g->d_num_parents || !g->d_child_off || !g->d_child_idx || !g->d_roots
-        || !g->d_dep || !g->d_queue || !g->d_ran || !g->d_state)
+        || !g->d_dep || !g->d_queue || !g->d_ran || !g->d_state || !g->d_child_rec)
     {
         aspen_hip_graph_destroy (g);
         return nullptr;
@@ -512,7 +555,7 @@ extern "C" void aspen_hip_graph_destroy (aspen_hip_graph_t *g)
     (void)hipStreamSynchronize (g_stream);
     aspen_hip_free (g->d_layers); aspen_hip_free (g->d_ninst_layer); aspen_hip_free (g->d_num_parents);
     aspen_hip_free (g->d_child_off); aspen_hip_free (g->d_child_idx); aspen_hip_free (g->d_roots);
-    aspen_hip_free (g->d_dep); aspen_hip_free (g->d_queue); aspen_hip_free (g->d_ran); aspen_hip_free (g->d_state); aspen_hip_free (g->d_prof); aspen_hip_free (g->d_trace);
+    aspen_hip_free (g->d_child_rec); aspen_hip_free (g->d_dep); aspen_hip_free (g->d_queue); aspen_hip_free (g->d_ran); aspen_hip_free (g->d_state); aspen_hip_free (g->d_prof); aspen_hip_free (g->d_trace);
     free (g->h_layers);
     free (g);
 }
@@ -555,10 +598,10 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     if (workgroups == 0) workgroups = WG_PER_CU * (uint32_t)g_num_cu;
     g->epoch = g->epoch % 255u + 1u;
     hipLaunchKernelGGL (arm_kernel, dim3 ((g->num_ninst + 255) / 256), dim3 (256), 0, g_stream,
-        g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->num_ninst, g->num_roots, g->d_state, g->epoch);
+        g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->d_ninst_layer, g->num_ninst, g->num_roots, g->d_state, g->epoch);
     CHECK (hipGetLastError ());
     dataflow_args_t a;
-    a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx;
+    a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx; a.child_rec = g->d_child_rec;
     a.dep = g->d_dep; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran; a.prof = g->d_prof; a.host_abort = g_host_abort;
     if ((g_flags & ASPEN_HIP_FLAG_TRACE) && !g->d_trace)
     {
