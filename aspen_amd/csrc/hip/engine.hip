@@ -416,7 +416,7 @@ template <class T> static T *upload (const T *src, size_t n)
 static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
 {
     const char *why = nullptr;
-    if (L.type == INPUT_LAYER) return 0;
+    if (L.type == INPUT_LAYER || L.num_ninst == 0) return 0;     // no tiles: written by the host, or by another layer's epilogue
     if (!L.out || !L.in0) why = "missing buffers";
     else if (L.ld % 4 || L.ld0 % 4 || (L.in1 && L.ld1 % 4)) why = "strides must be multiples of 4 floats";
     else if (L.tiles_m == 0 || L.tiles_n == 0 || L.splits == 0
@@ -435,6 +435,7 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
         else if (L.tile_m != bm || L.tile_n != bn) why = "tile extent does not match the GEMM variant";
         else if ((uint64_t)L.tiles_m * bm < L.M || (uint64_t)L.tiles_n * bn < L.N) why = "tile grid does not cover the matrix";
         else if (!L.direct && !L.ktab) why = "missing k-chunk table";
+        else if (L.fuse_out && (!L.fuse_in || L.fuse_ld_in % 4 || L.fuse_ld_in < L.M)) why = "fused shortcut operand";
         else if (L.direct && (L.ld0 < L.Kp)) why = "direct operand shorter than Kp";
     }
     else if (L.type == K_ATTENTION_LAYER)
@@ -477,9 +478,10 @@ static bool lines_have_one_producer (const aspen_hip_layer_t *layers, uint32_t n
         const aspen_hip_layer_t &P = layers[l];
         if (P.type == INPUT_LAYER || P.num_ninst == 0) continue;      // written by the host before the launch
         bool is_read = false;
-        for (uint32_t c = 0; c < num_layers && !is_read; c++) is_read = layers[c].in0 == P.out || layers[c].in1 == P.out;
+        for (uint32_t c = 0; c < num_layers && !is_read; c++) is_read = layers[c].in0 == P.out || layers[c].in1 == P.out || layers[c].fuse_in == P.out;
         const bool aligned = (uintptr_t)P.out % 128 == 0 && ((size_t)P.ld * 4) % 128 == 0 && (P.tiles_m == 1 || (P.tile_m * 4) % 128 == 0);
-        const bool ok = !(is_read && !aligned) && !(P.splits > 1 && ((uintptr_t)P.partial % 128 != 0 || !aligned));
+        const bool ok = !(is_read && !aligned) && !(P.splits > 1 && ((uintptr_t)P.partial % 128 != 0 || !aligned))
+            && !(P.fuse_out && ((uintptr_t)P.fuse_out % 128 != 0 || !aligned));
         if (!ok)
         {
             if (getenv ("ASPEN_GPU_VERBOSE"))

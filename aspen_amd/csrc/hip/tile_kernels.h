@@ -406,6 +406,28 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
 //   n = wn0 + 32 i + 8 (v / 4) + 4 (lane / 32) + v % 4,   m = wm0 + 32 j + lane % 32
 #define ACC_N(wn0, i, v, lane) ((wn0) + 32 * (i) + 8 * ((v) >> 2) + 4 * ((lane) >> 5) + ((v) & 3))
 
+// Shortcut fused into a contraction epilogue: fuse_out = fuse_act (v + fuse_in) for the (up to) four
+// channels m .. m+3 of column n; `left` = channels of the matrix from m on.  Same arithmetic, in the same
+// order, as a residual tile reading the stored v would do.
+template <int COH>
+__device__ __forceinline__ void fused_shortcut (const aspen_hip_layer_t &L, const ActView<COH> &fin, const ActView<COH> &fout,
+    float4 v, uint32_t n, uint32_t m, uint32_t left)
+{
+    const uint32_t oi = n * L.fuse_ld_in + m, oo = n * L.ld + m;
+    if (left >= 4)
+    {
+        const float4 s = fin.ld4 (oi);
+        v.x += s.x; v.y += s.y; v.z += s.z; v.w += s.w;
+        fout.st4 (oo, act4 (v, L.fuse_act));
+    }
+    else
+    {
+        fout.st1 (oo, activate (v.x + fin.ld1 (oi), L.fuse_act));
+        if (left > 1) fout.st1 (oo + 1, activate (v.y + fin.ld1 (oi + 1), L.fuse_act));
+        if (left > 2) fout.st1 (oo + 2, activate (v.z + fin.ld1 (oi + 2), L.fuse_act));
+    }
+}
+
 // conv / FC / matmul tile
 // `slice` < 0: the whole K axis, bias + activation, result to the layer's matrix.  `slice` >= 0 (split-K):
 // K slices [slice*kiters_per_split, ...) only, raw sums to that slice's partial matrix.
@@ -468,6 +490,9 @@ __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, ui
             if (c + 4 <= mrem) b = ld4 (L.bias + m0 + c);
             else { b.x = L.bias[m0 + c]; if (c + 1 < mrem) b.y = L.bias[m0 + c + 1]; if (c + 2 < mrem) b.z = L.bias[m0 + c + 2]; }
         }
+        const bool fuse = L.fuse_out != nullptr && slice < 0;
+        ActView<COH> fin, fout;
+        if (fuse) { fin.init (L.fuse_in, L.N, L.fuse_ld_in); fout.init (L.fuse_out, L.N, L.ld); }
         for (uint32_t r = tid / C4; r < rows; r += WG_THREADS / C4)
         {
             float4 v = ld4 (smem + r * TROW + c);
@@ -476,6 +501,7 @@ __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, ui
             const uint32_t o = (n0 + r) * L.ld + m0 + c;
             if (c + 4 <= mrem) out.st4 (o, v);
             else { out.st1 (o, v.x); if (c + 1 < mrem) out.st1 (o + 1, v.y); if (c + 2 < mrem) out.st1 (o + 2, v.z); }
+            if (fuse) fused_shortcut<COH> (L, fin, fout, v, n0 + r, m0 + c, mrem - c);
         }
     }
     __syncthreads ();
@@ -487,8 +513,10 @@ __device__ __forceinline__ void tile_splitk_finish (const aspen_hip_layer_t &L, 
 {
     const uint32_t m0 = tm * L.tile_m, n0 = tn * L.tile_n, C4 = L.tile_m >> 2;
     const uint32_t rows = min (L.tile_n, L.N - n0), mrem = L.M - m0;
-    ActView<COH> part, out;
+    ActView<COH> part, out, fin, fout;
     part.init (L.partial, L.N * L.splits, L.ld); out.init (L.out, L.N, L.ld);
+    const bool fuse = L.fuse_out != nullptr;
+    if (fuse) { fin.init (L.fuse_in, L.N, L.fuse_ld_in); fout.init (L.fuse_out, L.N, L.ld); }
     for (uint32_t idx = tile_thread (); idx < rows * C4; idx += WG_THREADS)
     {
         const uint32_t r = idx / C4, c = (idx - r * C4) * 4;
@@ -510,6 +538,7 @@ __device__ __forceinline__ void tile_splitk_finish (const aspen_hip_layer_t &L, 
         const uint32_t o = (n0 + r) * L.ld + m0 + c;
         if (c + 4 <= mrem) out.st4 (o, v);
         else { out.st1 (o, v.x); if (c + 1 < mrem) out.st1 (o + 1, v.y); if (c + 2 < mrem) out.st1 (o + 2, v.z); }
+        if (fuse) fused_shortcut<COH> (L, fin, fout, v, n0 + r, m0 + c, mrem - c);
     }
 }
 

@@ -68,6 +68,11 @@ struct nasm_ldata_t
     unsigned int splits, kiters_per_split;
     size_t partial_offset;                   /* floats into the arena: [splits][columns][stride] */
     int variant;
+    /* shortcut fusion: a residual layer whose first parent is a contraction layer that feeds nothing
+       else is computed in that layer's epilogue (the contraction tile writes its own matrix AND the
+       residual's); the residual then owns no tiles.  -1 = not fused */
+    int fused_residual;                      /* contraction layer: index of the residual it also produces */
+    int fused_into;                          /* residual layer: index of the contraction layer producing it */
     uint64_t flops;                          /* 2*M*N*K for contraction layers, 64-bit */
 };
 

@@ -219,6 +219,7 @@ static void push (u32vec *a, uint32_t x)
 /* all tiles of `pl` that overlap columns [c0, c1) x rows [r0, r1) become parents */
 static void add_parents (const nasm_ldata_t *pl, unsigned int c0, unsigned int c1, unsigned int r0, unsigned int r1, u32vec *out)
 {
+    if (pl->fused_into >= 0) pl = &pl->nasm->ldata_arr[pl->fused_into];   /* a fused shortcut is written by its contraction layer's tiles */
     if (pl->num_ninst == 0 || c1 <= c0 || r1 <= r0) return;   /* the input layer is complete from the start */
     c1 = umin (c1, pl->out_mat_dims[OUT_W]); r1 = umin (r1, pl->out_mat_dims[OUT_H]);
     const unsigned int t0 = col_tile_of (pl, c0), t1 = col_tile_of (pl, c1 - 1);
@@ -238,6 +239,13 @@ static void find_parents (const nasm_t *nasm, const nasm_ldata_t *ld, unsigned i
     unsigned int c0, c1, r0, r1;
     tile_range (ld, t, &c0, &c1, &r0, &r1);
     const unsigned int S = nasm->tr_seq_len;
+    /* the tile that runs the epilogue of a layer with a fused shortcut also reads the shortcut's other operand */
+    const int epilogue_tile = ld->splits == 1 || t >= ld->tiles_h * ld->tiles_w * ld->splits;
+    if (ld->fused_residual >= 0 && epilogue_tile)
+    {
+        const nasm_ldata_t *res = &nasm->ldata_arr[ld->fused_residual];
+        add_parents (&nasm->ldata_arr[res->parent_ldata_idx[PARENT_1]], c0, c1, r0, r1, out);
+    }
     if (ld->splits > 1 && t >= ld->tiles_h * ld->tiles_w * ld->splits)
     {
         const unsigned int tile = t - ld->tiles_h * ld->tiles_w * ld->splits;
@@ -351,6 +359,33 @@ static int build_graph (nasm_t *nasm)
     return 0;
 }
 
+/* Shortcut fusion.  out = act (p0 + p1) (reference tiled_residual, src/tiled_kernels.c:613-638) is a
+   pure bandwidth layer and one more dependency level.  When p0 is a contraction layer that feeds only
+   this shortcut, its tiles compute the shortcut in their epilogue: they still write p0's own matrix
+   (every layer's output stays readable), read p1 at the same positions and write the shortcut's
+   matrix too.  The shortcut layer keeps its matrix and loses its tiles. */
+static void fuse_shortcuts (nasm_t *nasm)
+{
+    for (unsigned int r = 0; r < nasm->num_ldata; r++)
+    {
+        nasm_ldata_t *res = &nasm->ldata_arr[r];
+        if (res->layer->type != RESIDUAL_LAYER) continue;
+        const int i0 = res->parent_ldata_idx[PARENT_0], i1 = res->parent_ldata_idx[PARENT_1];
+        if (i0 < 0 || i1 < 0 || i1 >= i0) continue;
+        nasm_ldata_t *prod = &nasm->ldata_arr[i0];
+        if (!is_contraction (prod->layer->type) || prod->fused_residual >= 0) continue;
+        if (prod->out_mat_stride != res->out_mat_stride) continue;
+        unsigned int consumers = 0;
+        for (unsigned int l = 0; l < nasm->num_ldata; l++)
+            for (int k = PARENT_0; k <= PARENT_1; k++)
+                consumers += nasm->ldata_arr[l].parent_ldata_idx[k] == i0;
+        if (consumers != 1) continue;
+        prod->fused_residual = (int)r;
+        res->fused_into = i0;
+        res->num_ninst = 0; res->tiles_h = res->tiles_w = 0;
+    }
+}
+
 static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned int batch, unsigned int seq)
 {
     if (dnn == NULL) { ERROR_PRTF ("apu_create_nasm: dnn is NULL\n"); return NULL; }
@@ -368,6 +403,7 @@ static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned i
     {
         nasm_ldata_t *ld = &nasm->ldata_arr[l];
         ld->nasm = nasm; ld->layer = &dnn->layers[l];
+        ld->fused_residual = ld->fused_into = -1;
         for (int k = 0; k < NUM_PARENT_ELEMENTS; k++) ld->parent_ldata_idx[k] = ld->layer->parent_idx[k];
         if (set_out_mat (nasm, ld) || set_tiles (nasm, ld)) { bad = 1; break; }
         for (int k = PARENT_0; k <= PARENT_1; k++)
@@ -378,6 +414,11 @@ static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned i
             if (ld->layer->type == RESIDUAL_LAYER && (pl->out_mat_dims[OUT_H] != ld->out_mat_dims[OUT_H] || pl->out_mat_dims[OUT_W] != ld->out_mat_dims[OUT_W]))
             { ERROR_PRTF ("layer %u: shortcut parents differ in shape\n", l); bad = 1; }
         }
+    }
+    if (!bad && getenv ("ASPEN_GPU_NO_FUSE") == NULL) fuse_shortcuts (nasm);
+    for (unsigned int l = 0; l < nasm->num_ldata && !bad; l++)
+    {
+        nasm_ldata_t *ld = &nasm->ldata_arr[l];
         ld->out_mat_offset = arena;
         arena += ((size_t)ld->out_mat_stride * ld->out_mat_dims[OUT_W] + 63) / 64 * 64;    /* 256-byte aligned matrices */
         if (ld->splits > 1)
@@ -520,6 +561,14 @@ int aspen_nasm_fill_device_layers (nasm_t *nasm, aspen_hip_layer_t *dst, uint32_
                 || (L->type == CONV_LAYER && p[WEIGHT_H] == 1 && p[WEIGHT_W] == 1 && p[STRIDE] == 1 && p[PADDING] == 0)
                 || (L->type == FC_LAYER && p[IN_H] == 1 && p[IN_W] == 1);
             d->direct = pointwise && (d->IC % 32 == 0) && d->ld0 >= d->Kp;
+        }
+        if (ld->fused_residual >= 0)
+        {
+            const nasm_ldata_t *res = &nasm->ldata_arr[ld->fused_residual];
+            const nasm_ldata_t *other = &nasm->ldata_arr[res->parent_ldata_idx[PARENT_1]];
+            d->fuse_out = nasm->d_arena + res->out_mat_offset;
+            d->fuse_in = nasm->d_arena + other->out_mat_offset; d->fuse_ld_in = other->out_mat_stride;
+            d->fuse_act = res->layer->activation;
         }
         if (L->type == K_ATTENTION_LAYER || L->type == V_ATTENTION_LAYER)
         {

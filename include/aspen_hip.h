@@ -77,6 +77,14 @@ typedef struct aspen_hip_layer_t
     const float *weight;     /* [roundup(M,128)][Kp] row-major, zero padded; layernorm: gamma[M] */
     const float *bias;       /* [M] or NULL */
     const aspen_hip_ktab_t *ktab; /* Kp/4 entries, NULL when direct */
+    /* fused shortcut (contraction layers; reference tiled_residual, src/tiled_kernels.c:613-638, run in
+       the epilogue): besides out = act(...) the tile also writes
+       fuse_out = fuse_act (out + fuse_in) at the same rows / columns; fuse_out has stride ld.
+       fuse_out == NULL: no fusion.  The residual layer itself then has num_ninst == 0. */
+    float *fuse_out;
+    const float *fuse_in;
+    uint32_t fuse_ld_in;
+    int32_t fuse_act;
 } aspen_hip_layer_t;
 
 typedef struct aspen_hip_graph_t aspen_hip_graph_t;

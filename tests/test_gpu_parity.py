@@ -35,17 +35,21 @@ def test_micro_nets_match_reference_fixture(gpu, name, mode):
         net.close()
 
 
-@pytest.mark.parametrize("loads", ["cached", "coherent"])
+@pytest.mark.parametrize("loads", ["cached", "coherent", "unfused"])
 @pytest.mark.parametrize("name", list(H.micro_cases()))
 def test_micro_nets_match_oracle(gpu, name, loads, monkeypatch):
     """Same nets against the CPU oracle (full tensors), dataflow engine with few workgroups so that
     tiles of several layers are in flight together.  The graph is re-armed and re-run with a
     DIFFERENT input each time: a tile that read a stale (cached) copy of its parent's previous
     output would not match the oracle of the new input.  Both load policies of the persistent kernel
-    run: activations through the caches (the default when the layout allows it) and device-coherent."""
+    run: activations through the caches (the default when the layout allows it) and device-coherent;
+    a third variant keeps the shortcut layers as tiles of their own instead of fusing them into the
+    producing contraction tile."""
     from oracle import cpu
     if loads == "coherent":
         monkeypatch.setenv("ASPEN_GPU_COHERENT_LOADS", "1")      # read when the device graph is built (first run)
+    if loads == "unfused":
+        monkeypatch.setenv("ASPEN_GPU_NO_FUSE", "1")             # shortcuts as tiles of their own (read when the nasm is built)
     cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()[name])
     inputs = [x, (x * 0.5 + 0.25).astype(np.float32), (-x).astype(np.float32), x]
     net = H.GpuNet(cfg, tens, batch, seq, min_ninst=32, mode=api.MODE_DATAFLOW, workgroups=24)

@@ -101,13 +101,26 @@ def needed_regions(L, layers, c0, c1, r0, r1, batch, seq):
     raise ValueError(t)
 
 
+@pytest.mark.parametrize("fuse", [True, False], ids=["fused", "unfused"])
 @pytest.mark.parametrize("name,min_ninst", [("custom_b3", 16), ("resnet_mini_b2", 64), ("resnet_mini_b2", 1024),
                                             ("vgg_mini_b5", 32), ("bert_mini_b2_s24", 16), ("gpt_mini_b2_s20", 256)])
-def test_tile_graph_against_brute_force(name, min_ninst):
+def test_tile_graph_against_brute_force(name, min_ninst, fuse, monkeypatch):
+    if not fuse:
+        monkeypatch.setenv("ASPEN_GPU_NO_FUSE", "1")
     layers, d, n, batch, seq = make(H.micro_cases()[name], min_ninst)
     tl, npar, off, idx = n.graph()
     T = n.num_ninst
     infos = [n.info(l) for l in range(n.num_ldata)]
+    fused_res = {i["fused_into"]: l for l, i in enumerate(infos) if i["fused_into"] >= 0}     # producer -> shortcut layer
+    if fuse and any(L["type"] == "residual" for L in layers):
+        assert fused_res, "shortcuts after a contraction layer should be fused"
+    if not fuse:
+        assert not fused_res
+    for prod, res in fused_res.items():
+        assert infos[res]["num_ninst"] == 0 and infos[prod]["fused_residual"] == res
+        assert layers[res]["type"] == "residual" and layers[res]["p0"] == prod and layers[prod]["type"] in ("conv", "fc", "matmul")
+        # the producer feeds nothing but the shortcut
+        assert [l for l, L in enumerate(layers) if prod in (L["p0"], L["p1"])] == [res]
     # ---- tiles partition every out_mat; split-K layers have splits*T partial tiles + T finishing tiles
     owner, partial_of = [], {}
     for l, i in enumerate(infos):
@@ -125,6 +138,9 @@ def test_tile_graph_against_brute_force(name, min_ninst):
                 partial_of[max(ts)] = sorted(ts)[:-1]
         if i["num_ninst"]:
             assert (own >= 0).all(), (name, l, "tiles leave a gap")
+        if i["fused_into"] >= 0:
+            own = owner[i["fused_into"]]            # written by the producer's tiles (same geometry)
+            assert own.shape == (i["W"], i["H"])
         owner.append(own)
     # ---- parents from the CSR children lists
     parents = [set() for _ in range(T)]
@@ -140,14 +156,21 @@ def test_tile_graph_against_brute_force(name, min_ninst):
     for t in range(T):
         l = int(tl[t])
         L = layers[l]
-        if t in finals:
-            assert parents[t] == set(partial_of[t]), (name, l, t)
-            continue
         c0, c1, r0, r1 = n.tile_range(t)
-        need = set()
+        produced = lambda pp: infos[pp]["num_ninst"] > 0 or infos[pp]["fused_into"] >= 0
+        # the tile that runs a fused epilogue also reads the shortcut's other operand
+        shortcut_need = set()
+        if l in fused_res and (t in finals or t not in partials):
+            other = layers[fused_res[l]]["p1"]
+            if produced(other):
+                shortcut_need = {int(v) for v in np.unique(owner[other][c0:c1, r0:r1])}
+        if t in finals:
+            assert parents[t] == set(partial_of[t]) | shortcut_need, (name, l, t)
+            continue
+        need = set(shortcut_need)
         for (p, cols, ra, rb) in needed_regions(L, layers, c0, c1, r0, r1, batch, seq):
             for pp in ([L["p0"], L["p1"]] if p == "either" else [p]):
-                if pp is None or not cols or infos[pp]["num_ninst"] == 0:
+                if pp is None or not cols or not produced(pp):
                     continue
                 rb_ = infos[pp]["H"] if rb is None else rb
                 own = owner[pp][sorted(cols)][:, ra:rb_]
@@ -168,11 +191,11 @@ def test_tile_graph_against_brute_force(name, min_ninst):
             # strided windows): everything read is awaited, nothing outside the hull is
             assert need <= parents[t], (name, l, t)
             pp = L["p0"]
-            if infos[pp]["num_ninst"]:
+            if produced(pp):
                 cols = set().union(*[c for (_, c, _, _) in needed_regions(L, layers, c0, c1, r0, r1, batch, seq)])
                 rr = (0, infos[pp]["H"]) if L["type"] == "conv" else (r0, r1)
                 hull = {int(v) for v in np.unique(owner[pp][min(cols):max(cols) + 1, rr[0]:rr[1]])}
-                assert parents[t] <= hull, (name, l, t)
+                assert parents[t] <= hull | shortcut_need, (name, l, t)
         else:
             assert parents[t] == need, (name, l, t, L["type"], sorted(parents[t]), sorted(need))
     # ---- executing by the counters runs every tile exactly once (what the device engine does)
@@ -224,7 +247,7 @@ def test_error_paths(tmp_path, capfd):
     d = api.Dnn(M.custom_cifar_cfg(), None)
     assert not L.apu_create_nasm(d.h, 0, 1)                          # min_ninst_per_ldata must be >= 1
     h = L.apu_create_nasm(d.h, 64, 0)                                # batch 0 means batch 1
-    a = (api.C.c_uint * 12)()
+    a = (api.C.c_uint * 16)()
     L.aspen_nasm_ldata_info(h, 0, a)
     assert a[3] == 32 * 32
     L.apu_destroy_nasm(h)
