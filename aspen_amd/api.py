@@ -53,6 +53,9 @@ def lib() -> C.CDLL:
         "apu_destroy_nasm": (None, [_vp]),
         "apu_reset_nasm": (None, [_vp]),
         "apu_load_nasm_from_file": (_vp, [C.c_char_p, _vp]),
+        "apu_save_nasm_to_file": (None, [_vp, C.c_char_p]),
+        "apu_save_dnn_to_file": (None, [_vp, C.c_char_p]),
+        "apu_load_dnn_from_file": (_vp, [C.c_char_p]),
         "rpool_init": (_vp, []),
         "rpool_destroy": (None, [_vp]),
         "rpool_add_nasm_raw_input": (None, [_vp, _vp, _vp]),
@@ -159,9 +162,14 @@ class Dnn:
 class Nasm:
     """``nasm_t`` -- ``apu_create_nasm`` / ``apu_create_transformer_nasm`` / ``apu_destroy_nasm``."""
 
-    def __init__(self, dnn: Dnn, batch: int, seq: int = 0, min_ninst: int = 512):
+    def __init__(self, dnn: Dnn, batch: int, seq: int = 0, min_ninst: int = 512, generate_iters: Optional[int] = None):
+        """``generate_iters`` not None: ``apu_generate_nasm`` / ``apu_generate_transformer_nasm`` (the tile count
+        is chosen by timing that many candidates beyond the default on the GPU) instead of ``min_ninst``."""
         self.dnn = dnn
-        if seq:
+        if generate_iters is not None:
+            self.h = (lib().apu_generate_transformer_nasm(dnn.h, batch, seq, generate_iters) if seq
+                      else lib().apu_generate_nasm(dnn.h, batch, generate_iters))
+        elif seq:
             self.h = lib().apu_create_transformer_nasm(dnn.h, min_ninst, batch, seq)
         else:
             self.h = lib().apu_create_nasm(dnn.h, min_ninst, batch)

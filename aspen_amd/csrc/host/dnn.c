@@ -44,6 +44,15 @@ static void create_layer_tensors (aspen_layer_t *L, uint64_t *rng)
     fill_uniform (&L->bias, rng, 0.3f);
 }
 
+/* tensors of a layer whose parameters are known, zero filled (the .aspen reader fills them) */
+void aspen_create_layer_tensors (aspen_layer_t *L)
+{
+    uint64_t rng = 1;
+    create_layer_tensors (L, &rng);
+    if (L->weight.data) memset (L->weight.data, 0, L->weight.num_elements * sizeof (float));
+    if (L->bias.data) memset (L->bias.data, 0, L->bias.num_elements * sizeof (float));
+}
+
 aspen_dnn_t *apu_create_dnn (char *input_path, char *data_path)
 {
     if (input_path == NULL) { ERROR_PRTF ("apu_create_dnn: input_path is NULL\n"); return NULL; }
@@ -288,14 +297,4 @@ int aspen_layer_to_device (aspen_layer_t *L, unsigned int parent_ld)
     return rc;
 }
 
-void apu_save_dnn_to_file (aspen_dnn_t *dnn, char *filename)
-{
-    (void)dnn;
-    ERROR_PRTF ("apu_save_dnn_to_file (%s): the .aspen container is not implemented in this build.\n", filename ? filename : "NULL");
-}
 
-aspen_dnn_t *apu_load_dnn_from_file (char *filename)
-{
-    ERROR_PRTF ("apu_load_dnn_from_file (%s): the .aspen container is not implemented in this build.\n", filename ? filename : "NULL");
-    return NULL;
-}

@@ -448,18 +448,72 @@ nasm_t *apu_create_transformer_nasm (aspen_dnn_t *dnn, unsigned int min_ninst_pe
     return create_nasm (dnn, min_ninst_per_ldata, batch_size, seq_num);
 }
 
-/* The reference searches min_ninst by timing 50-iteration runs (reference src/apu_nasm.c:601-639);
-   this build uses a fixed policy: six tiles per compute unit, i.e. 1.5 x the number of resident workgroups (best for all five benchmark configurations). */
+/* ---- auto-tuner --------------------------------------------------------------------------------
+   The reference searches the tile count by timing 50-iteration runs of candidate graphs on its DSE
+   threads (reference src/apu_nasm.c:578-679: test_nasm_time_sec, apu_generate_nasm).  Same idea on the
+   GPU: candidate values of min_ninst_per_ldata are built and timed on the dataflow engine (zero input,
+   2 warm-up + 10 timed inferences each), the fastest wins.  num_iter = how many candidates beyond the
+   default are tried, in the order below (nearest to the default first); 0 = take the default without
+   timing.  Without a GPU the default is returned as well. */
 #define DEFAULT_MIN_NINST 1536
+#include <time.h>
+static const unsigned int tuner_candidates[] = {DEFAULT_MIN_NINST, 1024, 2048, 768, 3072, 512, 256};
+
+static double test_nasm_time_sec (nasm_t *nasm, unsigned int iters)
+{
+    rpool_t *rpool = rpool_init ();
+    dse_group_t *dse = dse_group_init (1);
+    dse_group_set_rpool (dse, rpool);
+    rpool_add_nasm (rpool, nasm, NULL);
+    struct timespec t0, t1;
+    double sec = -1.0;
+    for (unsigned int i = 0; i < 2 + iters; i++)
+    {
+        if (i == 2) { aspen_hip_sync (); clock_gettime (CLOCK_MONOTONIC, &t0); }
+        dse_group_run (dse);
+        dse_wait_for_nasm_completion (nasm);
+        dse_group_stop (dse);
+        rpool_reset_queue (rpool);
+        rpool_reset_nasm (rpool, nasm);
+    }
+    if (aspen_hip_sync () == 0)
+    {
+        clock_gettime (CLOCK_MONOTONIC, &t1);
+        sec = ((double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec)) / (double)iters;
+    }
+    dse_group_destroy (dse);
+    rpool_destroy (rpool);
+    return sec;
+}
+
+static nasm_t *generate_nasm (aspen_dnn_t *dnn, unsigned int batch, unsigned int seq, unsigned int num_iter)
+{
+    const unsigned int ncand = sizeof (tuner_candidates) / sizeof (tuner_candidates[0]);
+    if (num_iter == 0 || aspen_hip_init () != 0) return create_nasm (dnn, DEFAULT_MIN_NINST, batch, seq);
+    unsigned int best = DEFAULT_MIN_NINST;
+    double best_time = -1.0;
+    for (unsigned int c = 0; c < ncand && c <= num_iter; c++)
+    {
+        nasm_t *cand = create_nasm (dnn, tuner_candidates[c], batch, seq);
+        if (cand == NULL) return NULL;
+        const double t = test_nasm_time_sec (cand, 10);
+        printf ("APU: min_ninst_per_ldata %u: %u tiles, %f sec per inference\n", tuner_candidates[c], cand->num_ninst, t);
+        fflush (stdout);
+        apu_destroy_nasm (cand);
+        if (t > 0 && (best_time < 0 || t < best_time)) { best_time = t; best = tuner_candidates[c]; }
+    }
+    printf ("APU: NASM with min_ninst_per_ldata %u, time = %f sec selected.\n", best, best_time);
+    fflush (stdout);
+    return create_nasm (dnn, best, batch, seq);
+}
+
 nasm_t *apu_generate_nasm (aspen_dnn_t *dnn, unsigned int batch_size, unsigned int num_iter)
 {
-    (void)num_iter;
-    return create_nasm (dnn, DEFAULT_MIN_NINST, batch_size, 0);
+    return generate_nasm (dnn, batch_size, 0, num_iter);
 }
 nasm_t *apu_generate_transformer_nasm (aspen_dnn_t *dnn, unsigned int batch_size, unsigned int seq_num, unsigned int num_iter)
 {
-    (void)num_iter;
-    return create_nasm (dnn, DEFAULT_MIN_NINST, batch_size, seq_num);
+    return generate_nasm (dnn, batch_size, seq_num, num_iter);
 }
 
 void apu_destroy_nasm (nasm_t *nasm)
@@ -491,18 +545,7 @@ void apu_reset_nasm (nasm_t *nasm)
     nasm->armed = 1;
 }
 
-nasm_t *apu_load_nasm_from_file (char *filename, aspen_dnn_t *dnn)
-{
-    (void)dnn;
-    ERROR_PRTF ("apu_load_nasm_from_file (%s): .nasm files describe the reference's CPU tile grid and are not read by this build; use apu_create_nasm.\n", filename ? filename : "NULL");
-    return NULL;
-}
 
-void apu_save_nasm_to_file (nasm_t *nasm, char *filename)
-{
-    (void)nasm;
-    ERROR_PRTF ("apu_save_nasm_to_file (%s): not implemented in this build.\n", filename ? filename : "NULL");
-}
 
 /* ---- device ------------------------------------------------------------------------------------ */
 int aspen_nasm_to_device (nasm_t *nasm)

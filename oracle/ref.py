@@ -48,6 +48,8 @@ def lib():
         L.refglue_layer_weight.restype = C.c_long
         L.refglue_result.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int, _fp, C.c_long]
         L.refglue_result.restype = C.c_long
+        L.refglue_save_dnn.argtypes = [C.c_void_p, C.c_char_p]
+        L.refglue_save_nasm.argtypes = [C.c_void_p, C.c_uint, C.c_uint, C.c_uint, C.c_char_p]
         L.refglue_close.argtypes = [C.c_void_p]
         _lib = L
     return _lib
@@ -88,6 +90,14 @@ class RefNet:
         out = np.empty((i["W"], i["H"]), dtype=np.float32)
         lib().refglue_layer_copy(self.h, l, out.ctypes.data_as(_fp))
         return out
+
+    def save_dnn(self, path: str):
+        """The reference's apu_save_dnn_to_file."""
+        lib().refglue_save_dnn(self.h, path.encode())
+
+    def save_nasm(self, path: str, batch: int, seq: int, min_ninst: int) -> int:
+        """apu_create_nasm (full dependency search) + apu_save_nasm_to_file; returns the tile count."""
+        return lib().refglue_save_nasm(self.h, batch, seq, min_ninst, path.encode())
 
     def weight(self, l: int, tensor_type: int) -> np.ndarray:
         n = lib().refglue_layer_weight(self.h, l, tensor_type, None, 0)

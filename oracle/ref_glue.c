@@ -174,6 +174,26 @@ long refglue_result (void *h, int l, int *order, int num_order, float *dst, long
     return sz;
 }
 
+/* the reference's own container writers, for fixtures: the model as a .aspen file, and a .nasm file of
+   a graph built with the reference's full tile-dependency search */
+void refglue_save_dnn (void *h, char *path)
+{
+    apu_save_dnn_to_file (((refglue_t*)h)->dnn, path);
+}
+
+int refglue_save_nasm (void *h, unsigned int batch, unsigned int seq, unsigned int min_ninst_per_ldata, char *path)
+{
+    refglue_t *g = h;
+    nasm_t *nasm = seq ? apu_create_transformer_nasm (g->dnn, min_ninst_per_ldata, batch, seq)
+                       : apu_create_nasm (g->dnn, min_ninst_per_ldata, batch);
+    if (nasm == NULL)
+        return -1;
+    apu_save_nasm_to_file (nasm, path);
+    int n = nasm->num_ninst;
+    apu_destroy_nasm (nasm);
+    return n;
+}
+
 void refglue_close (void *h)
 {
     refglue_t *g = h;

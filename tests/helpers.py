@@ -118,3 +118,22 @@ def check_against_summary(net, gold, layers, label):
     final = net.layer(n - 1)
     assert (final.argmax(axis=1) == gold["argmax"]).all(), f"{label}: argmax differs"
     return worst
+
+
+def tiny_cfg():
+    """A few-kilobyte network for file-format fixtures: odd channel counts exercise the padding of the
+    reference's 8-row weight interleave (the layer in front of the FC layer has 64 channels:
+    the reference requires the FC parent's column stride to equal its channel count)."""
+    return ("[net]\nheight=8\nwidth=8\nchannels=3\n\n"
+            "[convolutional]\nfilters=5\nsize=3\nstride=1\npad=1\nactivation=relu\n\n"
+            "[maxpool]\nsize=2\nstride=2\n\n"
+            "[convolutional]\nfilters=64\nsize=1\nstride=1\npad=0\nactivation=leaky\n\n"
+            "[connected]\noutput=10\nactivation=linear\n\n")
+
+
+def tiny_case():
+    cfg = tiny_cfg()
+    layers = M.parse_cfg(cfg)
+    tens = M.synth_weights(layers, 77, "he")
+    x = M.synth_input(layers, 77, 2, 0, "embeddings")
+    return cfg, layers, tens, x, 2, 0

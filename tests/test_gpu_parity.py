@@ -184,3 +184,46 @@ def test_copy_kernel(gpu):
     assert np.array_equal(x, y)
     assert L.aspen_hip_copy(b, a, 24) != 0
     L.aspen_hip_free(a); L.aspen_hip_free(b)
+
+
+@pytest.mark.gpu
+def test_generate_nasm_times_candidates(gpu, capfd):
+    """apu_generate_nasm (reference src/apu_nasm.c:601-639) on the GPU: candidates are timed, the chosen
+    graph runs and matches the oracle."""
+    from oracle import cpu
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()["resnet_mini_b2"])
+    wp = os.path.join(os.environ.get("TMPDIR", "/tmp"), "gen_nasm_w.bin")
+    M.write_aspen_data(wp, tens)
+    dnn = api.Dnn(cfg, wp)
+    os.unlink(wp)
+    nasm = api.Nasm(dnn, batch, seq, generate_iters=2)
+    out = capfd.readouterr().out
+    assert out.count("sec per inference") == 3 and "selected" in out
+    pool, dse = api.RPool(), api.DseGroup(1, api.MODE_DATAFLOW)
+    dse.set_rpool(pool)
+    pool.add_nasm_raw_input(nasm, x)
+    dse.run(); dse.wait(nasm); dse.stop()
+    outs = cpu.run_network(layers, tens, x, batch, seq)
+    for l in range(nasm.num_ldata):
+        assert H.rel_l2(nasm.layer_output(l), outs[l]) <= H.REL_L2_TOL, l
+    dse.destroy(); pool.destroy(); nasm.destroy(); dnn.destroy()
+
+
+@pytest.mark.gpu
+def test_model_loaded_from_reference_aspen_file_runs(gpu):
+    """A .aspen file written by the compiled reference (tests/golden/tiny_ref.aspen), loaded through
+    apu_load_dnn_from_file, must compute what the oracle computes from the original weights."""
+    from oracle import cpu
+    cfg, layers, tens, x, batch, seq = H.tiny_case()
+    h = api.lib().apu_load_dnn_from_file(os.path.join(H.GOLDEN, "tiny_ref.aspen").encode())
+    assert h
+    dnn = api.Dnn.__new__(api.Dnn); dnn.h = h
+    nasm = api.Nasm(dnn, batch, seq, 8)
+    pool, dse = api.RPool(), api.DseGroup(1, api.MODE_DATAFLOW)
+    dse.set_rpool(pool)
+    pool.add_nasm_raw_input(nasm, x)
+    dse.run(); dse.wait(nasm); dse.stop()
+    outs = cpu.run_network(layers, tens, x, batch, seq)
+    for l in range(nasm.num_ldata):
+        assert H.rel_l2(nasm.layer_output(l), outs[l]) <= H.REL_L2_TOL, l
+    dse.destroy(); pool.destroy(); nasm.destroy(); dnn.destroy()

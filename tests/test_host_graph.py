@@ -278,3 +278,17 @@ def test_weight_file_round_trip(tmp_path, capfd):
     assert capfd.readouterr().err != ""
     if h:
         api.lib().apu_destroy_dnn(h)
+
+
+def test_generate_nasm_without_gpu_takes_the_default(capfd):
+    """apu_generate_nasm times candidates on the GPU; with num_iter 0 (and on a machine without a GPU) it
+    returns the default tile policy."""
+    d = api.Dnn(M.custom_cifar_cfg(), None)
+    g = api.Nasm(d, 2, 0, generate_iters=0)
+    ref = api.Nasm(d, 2, 0, 1536)
+    assert g.num_ninst == ref.num_ninst and g.num_edges == ref.num_edges
+    if not api.gpu_available():
+        g2 = api.Nasm(d, 2, 0, generate_iters=3)
+        assert g2.num_ninst == ref.num_ninst
+        g2.destroy()
+    g.destroy(); ref.destroy(); d.destroy()
