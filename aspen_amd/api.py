@@ -182,10 +182,10 @@ class Nasm:
         self.total_flops = lib().aspen_nasm_total_flops(self.h)
 
     def info(self, l: int) -> dict:
-        a = (C.c_uint * 16)()
+        a = (C.c_uint * 20)()
         lib().aspen_nasm_ldata_info(self.h, l, a)
         keys = ["type", "act", "H", "W", "stride", "num_ninst", "tile_H", "tile_W", "p0", "p1", "ninst_start", "variant",
-                "fused_into", "fused_residual", "splits", "tiles_H"]
+                "fused_into", "fused_residual", "splits", "tiles_H", "kiters_per_split"]
         d = dict(zip(keys, [int(v) for v in a]))
         for k in ("fused_into", "fused_residual"):
             d[k] = -1 if d[k] == 0xffffffff else d[k]

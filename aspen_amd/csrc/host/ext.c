@@ -23,7 +23,8 @@ void aspen_nasm_ldata_info (nasm_t *n, unsigned int l, unsigned int *info)
     info[8] = (unsigned int)ld->parent_ldata_idx[PARENT_0]; info[9] = (unsigned int)ld->parent_ldata_idx[PARENT_1];
     info[10] = ld->ninst_start; info[11] = (unsigned int)ld->variant;
     info[12] = (unsigned int)ld->fused_into; info[13] = (unsigned int)ld->fused_residual;
-    info[14] = ld->splits; info[15] = ld->tiles_h;
+    info[14] = ld->splits; info[15] = ld->tiles_h; info[16] = ld->kiters_per_split;
+    info[17] = info[18] = info[19] = 0;
 }
 
 void aspen_nasm_graph (nasm_t *n, const uint32_t **ninst_ldata, const uint32_t **num_parents,

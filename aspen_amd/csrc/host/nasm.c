@@ -140,7 +140,7 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
            line up) and halve until there are enough tiles */
         unsigned int tn = 128;
         if (L->type == SOFTMAX_LAYER || L->type == LAYERNORM_LAYER) tn = 32;
-        while (tn > 4 && cdiv (N, tn) < want) tn /= 2;
+        while (tn > 4 && cdiv (N, tn) < want) tn /= 2;      /* small tiles finish sooner: measured better than fewer edges */
         while (tn < 1024 && (uint64_t)tn * ld->out_mat_stride < 16384 && cdiv (N, tn * 2) >= 2 * want) tn *= 2;
         ld->tile_dims[OUT_H] = M; ld->tile_dims[OUT_W] = tn;
         /* pooling layers with few output positions (global average pooling) are cut along the
@@ -162,7 +162,9 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
         ld->kiters_per_split = kiters;
         if (T < want && kiters >= 16 && getenv ("ASPEN_GPU_NO_SPLITK") == NULL)
         {
-            unsigned int s = umin (umin (cdiv (want, T), kiters / 8), 8);
+            const char *e1 = getenv ("ASPEN_GPU_MAX_SPLITS"), *e2 = getenv ("ASPEN_GPU_MIN_KITERS");
+            const unsigned int max_splits = e1 ? (unsigned int)atoi (e1) : 8, min_kiters = e2 ? (unsigned int)atoi (e2) : 8;
+            unsigned int s = umin (umin (cdiv (want, T), kiters / umax (min_kiters, 1)), umax (max_splits, 1));
             ld->kiters_per_split = cdiv (kiters, s);
             ld->splits = cdiv (kiters, ld->kiters_per_split);
             if (ld->splits > 1) ld->num_ninst = T * ld->splits + T;
@@ -252,12 +254,23 @@ static void find_parents (const nasm_t *nasm, const nasm_ldata_t *ld, unsigned i
         for (unsigned int s = 0; s < ld->splits; s++) push (out, ld->ninst_start + tile * ld->splits + s);
         return;
     }
+    /* A split-K partial tile of a pointwise layer (matmul, 1x1 convolution: the K index IS the parent's
+       row index) reads only the parent rows of its K slice, so it waits only for the parent tiles
+       holding those rows: fewer edges, and it can start before the rest of the parent is done. */
+    unsigned int k_row0 = 0, k_row1 = p0 ? p0->out_mat_dims[OUT_H] : 0;
+    if (ld->splits > 1 && !epilogue_tile
+        && (L->type == MATMUL_LAYER || (L->type == CONV_LAYER && p[WEIGHT_H] == 1 && p[WEIGHT_W] == 1)))
+    {
+        const unsigned int slice = t % ld->splits;
+        k_row0 = umin (slice * ld->kiters_per_split * 32, k_row1);
+        k_row1 = umin ((slice + 1) * ld->kiters_per_split * 32, k_row1);
+    }
     switch (L->type)
     {
     case CONV_LAYER: case MAXPOOL_LAYER: case AVGPOOL_LAYER:
     {
         const unsigned int ohw = p[OUT_H] * p[OUT_W], ihw = p[IN_H] * p[IN_W];
-        const unsigned int pr0 = L->type == CONV_LAYER ? 0 : r0, pr1 = L->type == CONV_LAYER ? p0->out_mat_dims[OUT_H] : r1;
+        const unsigned int pr0 = L->type == CONV_LAYER ? k_row0 : r0, pr1 = L->type == CONV_LAYER ? k_row1 : r1;
         for (unsigned int b = c0 / ohw; b <= (c1 - 1) / ohw; b++)
         {
             const unsigned int first = umax (c0, b * ohw) - b * ohw, last = umin (c1, (b + 1) * ohw) - 1 - b * ohw;
@@ -284,7 +297,10 @@ static void find_parents (const nasm_t *nasm, const nasm_ldata_t *ld, unsigned i
         add_parents (p0, c0 * ihw, c1 * ihw, 0, p0->out_mat_dims[OUT_H], out);
         break;
     }
-    case MATMUL_LAYER: case LAYERNORM_LAYER: case SOFTMAX_LAYER:
+    case MATMUL_LAYER:
+        add_parents (p0, c0, c1, k_row0, k_row1, out);
+        break;
+    case LAYERNORM_LAYER: case SOFTMAX_LAYER:
         add_parents (p0, c0, c1, 0, p0->out_mat_dims[OUT_H], out);
         break;
     case RESIDUAL_LAYER:

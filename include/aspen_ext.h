@@ -22,11 +22,11 @@ unsigned int aspen_nasm_num_ldata (nasm_t *nasm);
 unsigned int aspen_nasm_num_ninst (nasm_t *nasm);
 unsigned int aspen_nasm_num_edges (nasm_t *nasm);
 uint64_t aspen_nasm_total_flops (nasm_t *nasm);
-/* info[0..15] = type, activation, rows, columns, stride, num_ninst, tile_rows, tile_columns,
+/* info[0..19] = type, activation, rows, columns, stride, num_ninst, tile_rows, tile_columns,
    parent0, parent1 (0xffffffff = none), first tile index, GEMM variant,
    [12] shortcut layers: index of the contraction layer whose tiles produce this layer (0xffffffff = own tiles),
    [13] contraction layers: index of the shortcut layer fused into the epilogue (0xffffffff = none),
-   [14] split-K slices, [15] row tiles */
+   [14] split-K slices, [15] row tiles, [16] K slices of 32 per split-K part, [17..19] reserved (0) */
 void aspen_nasm_ldata_info (nasm_t *nasm, unsigned int ldata_idx, unsigned int *info);
 uint64_t aspen_nasm_ldata_flops (nasm_t *nasm, unsigned int ldata_idx);
 /* dependency graph in CSR form; pointers stay valid until the nasm is destroyed */

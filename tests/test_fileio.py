@@ -115,7 +115,7 @@ def test_nasm_file_from_the_reference_loads(tmp_path, capfd):
     assert "another tile grid" in capfd.readouterr().out
     ref_hdr = dict(l.split(":", 1) for l in open(REF_NASM).read().split("NASM_NINSTS:")[0].strip().split("\n")[1:])
     assert L.aspen_nasm_total_flops(h) == int(ref_hdr["TOTAL_FLOPS"])
-    a = (api.C.c_uint * 16)()
+    a = (api.C.c_uint * 20)()
     L.aspen_nasm_ldata_info(h, 0, a)
     assert a[3] == int(ref_hdr["NUM_BATCH"]) * 8 * 8
     L.apu_destroy_nasm(h)

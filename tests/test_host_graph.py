@@ -168,7 +168,15 @@ def test_tile_graph_against_brute_force(name, min_ninst, fuse, monkeypatch):
             assert parents[t] == set(partial_of[t]) | shortcut_need, (name, l, t)
             continue
         need = set(shortcut_need)
-        for (p, cols, ra, rb) in needed_regions(L, layers, c0, c1, r0, r1, batch, seq):
+        regions = needed_regions(L, layers, c0, c1, r0, r1, batch, seq)
+        pointwise = L["type"] == "matmul" or (L["type"] == "conv" and L["size"] == 1)
+        if t in partials and pointwise:
+            # a partial tile of a pointwise layer reads only the parent rows (= K indices) of its K slice
+            slice_ = (t - infos[l]["ninst_start"]) % infos[l]["splits"]
+            k0 = slice_ * infos[l]["kiters_per_split"] * 32
+            k1 = min(k0 + infos[l]["kiters_per_split"] * 32, infos[L["p0"]]["H"])
+            regions = [(p, cols, k0, k1) for (p, cols, _, _) in regions]
+        for (p, cols, ra, rb) in regions:
             for pp in ([L["p0"], L["p1"]] if p == "either" else [p]):
                 if pp is None or not cols or not produced(pp):
                     continue
@@ -192,8 +200,10 @@ def test_tile_graph_against_brute_force(name, min_ninst, fuse, monkeypatch):
             assert need <= parents[t], (name, l, t)
             pp = L["p0"]
             if produced(pp):
-                cols = set().union(*[c for (_, c, _, _) in needed_regions(L, layers, c0, c1, r0, r1, batch, seq)])
+                cols = set().union(*[c for (_, c, _, _) in regions])
                 rr = (0, infos[pp]["H"]) if L["type"] == "conv" else (r0, r1)
+                if t in partials and pointwise:
+                    rr = (k0, k1)
                 hull = {int(v) for v in np.unique(owner[pp][min(cols):max(cols) + 1, rr[0]:rr[1]])}
                 assert parents[t] <= hull | shortcut_need, (name, l, t)
         else:
@@ -247,7 +257,7 @@ def test_error_paths(tmp_path, capfd):
     d = api.Dnn(M.custom_cifar_cfg(), None)
     assert not L.apu_create_nasm(d.h, 0, 1)                          # min_ninst_per_ldata must be >= 1
     h = L.apu_create_nasm(d.h, 64, 0)                                # batch 0 means batch 1
-    a = (api.C.c_uint * 16)()
+    a = (api.C.c_uint * 20)()
     L.aspen_nasm_ldata_info(h, 0, a)
     assert a[3] == 32 * 32
     L.apu_destroy_nasm(h)
