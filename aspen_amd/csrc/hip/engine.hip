@@ -455,6 +455,16 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
         if (L.tiles_m > 1 && (L.tile_m % 4 || (uint64_t)L.tiles_m * L.tile_m < L.M || (uint64_t)(L.tiles_m - 1) * L.tile_m >= L.M)) why = "pool row tiles";
         else if ((uint64_t)L.tiles_n * L.tile_n < L.N) why = "tile grid does not cover the matrix";
     }
+    else if (L.type == YOLO_LAYER)
+    {
+        if (!L.weight || L.M < 5 || L.IC % L.M || L.IC / L.M > 3 || L.tiles_m != 1 || L.ld0 < L.IC) why = "yolo geometry";
+        else if (L.N % (L.IH * L.IW * (L.IC / L.M))) why = "yolo columns";
+    }
+    else if (L.type == APPEND_LAYER)
+    {
+        if (!L.in1 || L.stride == 0 || L.OH % L.stride || L.OW % L.stride || L.IC >= L.M || L.tiles_m != 1
+            || L.ld0 < L.IC || L.ld1 < L.M - L.IC || L.N % (L.OH * L.OW)) why = "append geometry";
+    }
     else if (L.type == RESIDUAL_LAYER) { if (!L.in1 || L.tiles_m != 1) why = "missing second parent, or row tiles"; }
     else if (L.type == LAYERNORM_LAYER) { if (!L.weight || L.tiles_m != 1) why = "missing gamma, or row tiles"; }
     else if (L.type == SOFTMAX_LAYER) { if (L.tiles_m != 1) why = "row tiles"; }

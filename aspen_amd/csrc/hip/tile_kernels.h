@@ -597,6 +597,51 @@ __device__ __forceinline__ void tile_pool (const aspen_hip_layer_t &L, uint32_t 
     }
 }
 
+// YOLO box decode (reference tiled_yolo, src/tiled_kernels.c:675-708).  Output column = (batch, anchor,
+// cell); rows = classes + 5 read from channels [anchor * M, anchor * M + M) of input column (batch, cell).
+// L.weight holds the three anchor boxes (w0, h0, w1, h1, w2, h2).
+template <int COH>
+__device__ __forceinline__ void tile_yolo (const aspen_hip_layer_t &L, uint32_t tn)
+{
+    const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N);
+    const uint32_t cells = L.IH * L.IW, A = L.IC / L.M, total = (n1 - n0) * L.M;
+    ActView<COH> in, out;
+    in.init (L.in0, (L.N / (cells * A)) * cells, L.ld0); out.init (L.out, L.N, L.ld);
+    for (uint32_t i = tile_thread (); i < total; i += WG_THREADS)
+    {
+        const uint32_t c = i / L.M, j = i - c * L.M, n = n0 + c;
+        const uint32_t seg = n / cells, b = seg / A, a = seg - b * A, cell = n - seg * cells;
+        const uint32_t h = cell / L.IW, w = cell - h * L.IW;
+        const float x = in.ld1 ((b * cells + cell) * L.ld0 + a * L.M + j);
+        float r;
+        if (j == 0) r = (1.0f / (1.0f + expf (-x)) + (float)w) * (float)L.stride;
+        else if (j == 1) r = (1.0f / (1.0f + expf (-x)) + (float)h) * (float)L.stride;
+        else if (j == 2) r = expf (x) * L.weight[2 * a];
+        else if (j == 3) r = expf (x) * L.weight[2 * a + 1];
+        else r = 1.0f / (1.0f + expf (-x));
+        out.st1 (n * L.ld + j, r);
+    }
+}
+
+// Nearest-neighbour upsampling of the first parent by `stride`, concatenated along the channels with
+// the second parent (reference tiled_append, src/tiled_kernels.c:710-741).  IC = channels of the first parent.
+template <int COH>
+__device__ __forceinline__ void tile_append (const aspen_hip_layer_t &L, uint32_t tn)
+{
+    const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N), total = (n1 - n0) * L.M;
+    const uint32_t ohw = L.OH * L.OW, iw = L.OW / L.stride, ih = L.OH / L.stride;
+    ActView<COH> p0, p1, out;
+    p0.init (L.in0, (L.N / ohw) * ih * iw, L.ld0); p1.init (L.in1, L.N, L.ld1); out.init (L.out, L.N, L.ld);
+    for (uint32_t i = tile_thread (); i < total; i += WG_THREADS)
+    {
+        const uint32_t c = i / L.M, m = i - c * L.M, n = n0 + c;
+        const uint32_t b = n / ohw, rem = n - b * ohw, oh = rem / L.OW, ow = rem - oh * L.OW;
+        const float v = m < L.IC ? p0.ld1 (((b * ih + oh / L.stride) * iw + ow / L.stride) * L.ld0 + m)
+                                 : p1.ld1 (n * L.ld1 + (m - L.IC));
+        out.st1 (n * L.ld + m, v);
+    }
+}
+
 __device__ __forceinline__ float wave_sum (float v)
 {
     #pragma unroll
@@ -837,6 +882,8 @@ __device__ __forceinline__ void run_tile (const aspen_hip_layer_t &Lg, uint32_t 
     case RESIDUAL_LAYER:    tile_residual<COH> (L, tn); break;
     case MAXPOOL_LAYER:     tile_pool<true, COH> (L, tn, tm); break;
     case AVGPOOL_LAYER:     tile_pool<false, COH> (L, tn, tm); break;
+    case YOLO_LAYER:        tile_yolo<COH> (L, tn); break;
+    case APPEND_LAYER:      tile_append<COH> (L, tn); break;
     case LAYERNORM_LAYER:   tile_layernorm<COH> (L, tn); break;
     case SOFTMAX_LAYER:     tile_softmax<COH> (L, tn); break;
     case K_ATTENTION_LAYER: tile_k_attention<COH> (L, tn, smem); break;

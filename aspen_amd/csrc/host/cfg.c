@@ -100,6 +100,40 @@ static int conv_out (unsigned int in, unsigned int pad, unsigned int dil, unsign
     return (int)(in + 2 * pad - dil * (k - 1) - 1) / (int)stride + 1;
 }
 
+/* number list "a, b,  c" -> up to max values; returns the count */
+static int parse_numbers (const char *str, float *dst, int max)
+{
+    int n = 0;
+    while (str && *str && n < max)
+    {
+        char *end;
+        const float v = strtof (str, &end);
+        if (end == str) break;
+        dst[n++] = v;
+        str = end;
+        while (*str == ',' || isspace ((unsigned char)*str)) str++;
+    }
+    return n;
+}
+
+/* [yolo]: rows = classes + 5; the layer's three anchor boxes are picked from `anchors` by `mask`
+   (reference src/darknet_parser.c:487-545) */
+static int parse_yolo (const section_t *s, aspen_layer_t *L)
+{
+    float mask[16], anchors[64];
+    const int nm = parse_numbers (opt_str (s, "mask"), mask, 16), na = parse_numbers (opt_str (s, "anchors"), anchors, 64);
+    if (nm < 3) { ERROR_PRTF ("YOLO layer has no mask.\n"); return -1; }
+    if (na < 2) { ERROR_PRTF ("YOLO layer has no anchors.\n"); return -1; }
+    L->params[OUT_C] = (unsigned int)opt_int (s, "classes", 0) + 5;
+    for (int i = 0; i < 3; i++)
+    {
+        const int m = (int)mask[i];
+        if (m < 0 || 2 * m + 1 >= na) { ERROR_PRTF ("YOLO layer: mask %d has no anchor.\n", m); return -1; }
+        L->anchors[2 * i] = anchors[2 * m]; L->anchors[2 * i + 1] = anchors[2 * m + 1];
+    }
+    return 0;
+}
+
 /* in/out geometry of one layer from its parent (reference src/input_parser.c:35-127) */
 static int set_inout (aspen_dnn_t *dnn, aspen_layer_t *L)
 {
@@ -142,6 +176,22 @@ static int set_inout (aspen_dnn_t *dnn, aspen_layer_t *L)
     case LAYERNORM_LAYER: case V_ATTENTION_LAYER:
         if (L->type == V_ATTENTION_LAYER && (L->parent_idx[PARENT_1] < 0 || p[NUM_HEAD] == 0)) { ERROR_PRTF ("layer %u: attention_v needs from= and n_head=\n", L->layer_idx); return -1; }
         return 0;
+    case YOLO_LAYER:
+        if (p[STRIDE] == 0) p[STRIDE] = 1;
+        if (p[OUT_C] < 5 || p[IN_C] % p[OUT_C] != 0 || p[IN_C] / p[OUT_C] > 3)
+        { ERROR_PRTF ("layer %u: yolo needs (classes + 5) x (at most 3 anchors) input channels, got %u for %u rows\n", L->layer_idx, p[IN_C], p[OUT_C]); return -1; }
+        p[OUT_H] = 1; p[OUT_W] = p[IN_H] * p[IN_W] * (p[IN_C] / p[OUT_C]);
+        return 0;
+    case APPEND_LAYER:
+    {
+        if (L->parent_idx[PARENT_1] < 0) { ERROR_PRTF ("layer %u: append without from=\n", L->layer_idx); return -1; }
+        if (p[STRIDE] == 0) p[STRIDE] = 1;
+        const aspen_layer_t *Q = &dnn->layers[L->parent_idx[PARENT_1]];
+        p[OUT_C] = p[IN_C] + Q->params[OUT_C]; p[OUT_H] = p[IN_H] * p[STRIDE]; p[OUT_W] = p[IN_W] * p[STRIDE];
+        if (Q->params[OUT_H] != p[OUT_H] || Q->params[OUT_W] != p[OUT_W])
+        { ERROR_PRTF ("layer %u: append: the second parent is %ux%u, the upsampled first parent %ux%u\n", L->layer_idx, Q->params[OUT_H], Q->params[OUT_W], p[OUT_H], p[OUT_W]); return -1; }
+        return 0;
+    }
     case K_ATTENTION_LAYER:
         if (L->parent_idx[PARENT_1] < 0 || p[NUM_HEAD] == 0 || p[NUM_HIDDEN] == 0) { ERROR_PRTF ("layer %u: attention_k needs from=, n_head= and n_embd=\n", L->layer_idx); return -1; }
         p[MAT_K] = p[NUM_HIDDEN] / p[NUM_HEAD];
@@ -198,8 +248,7 @@ aspen_dnn_t *aspen_parse_cfg (const char *path)
                 { ERROR_PRTF ("layer %d: parent offset points outside the preceding layers\n", i); bad = 1; }
         }
         else if (i != 0) { ERROR_PRTF ("layer %d: only the first section may be [net]\n", i); bad = 1; }
-        if (L->type == YOLO_LAYER || L->type == APPEND_LAYER)
-        { ERROR_PRTF ("layer %d: %s layers are not supported by this build\n", i, s->name); bad = 1; }
+        if (L->type == YOLO_LAYER && parse_yolo (s, L)) bad = 1;
         if (!bad && set_inout (dnn, L)) bad = 1;
     }
     free (secs);

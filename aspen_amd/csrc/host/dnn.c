@@ -249,6 +249,12 @@ unsigned int aspen_layer_kiters (const aspen_layer_t *L)
    floats.  Idempotent; re-run after the weights changed. */
 int aspen_layer_to_device (aspen_layer_t *L, unsigned int parent_ld)
 {
+    if (L->type == YOLO_LAYER)
+    {
+        /* the anchor boxes travel in the weight slot of the device descriptor */
+        if (L->d_weight == NULL && (L->d_weight = aspen_hip_alloc (8 * sizeof (float))) == NULL) return -1;
+        return aspen_hip_h2d (L->d_weight, L->anchors, 6 * sizeof (float));
+    }
     if (L->weight.data == NULL) return 0;
     if (L->d_weight != NULL && L->dev_in_ld == parent_ld) return 0;
     invalidate_device (L);

@@ -110,6 +110,12 @@ void apu_save_dnn_to_file (aspen_dnn_t *dnn, char *filename)
                 dims[rows] = L->gemm_m;
                 write_tensor (fp, j, &rows, 1, dims, j == BIAS_TENSOR ? L->bias.data : L->weight.data, L->gemm_m);
             }
+            else if (L->type == YOLO_LAYER && j == ANCHOR_TENSOR)
+            {
+                const LAYER_PARAMS rows = OUT_C;        /* as the reference creates it: one dimension of 6 (src/darknet_parser.c:536-541) */
+                dims[OUT_C] = 6;
+                write_tensor (fp, j, &rows, 1, dims, L->anchors, 6);
+            }
             else
                 fprintf (fp, "\t\t%d -1\n", j);
         }
@@ -163,6 +169,12 @@ static int place_tensor (aspen_layer_t *L, int slot, const int *order, int num_d
         aspen_tensor_t *t = slot == BIAS_TENSOR ? &L->bias : &L->weight;
         if (t->data == NULL || n < L->gemm_m) return -1;
         memcpy (t->data, data, L->gemm_m * sizeof (float));
+        return 0;
+    }
+    if (slot == ANCHOR_TENSOR && L->type == YOLO_LAYER)
+    {
+        if (n < 6) return -1;
+        memcpy (L->anchors, data, 6 * sizeof (float));
         return 0;
     }
     return 0;    /* tensors this build has no use for (anchors, BN statistics already folded) are skipped */

@@ -36,6 +36,7 @@ struct aspen_layer_t
        matmul (the reference's K order, src/apu.c:16,25,34, without its 8-row interleave) */
     aspen_tensor_t weight, bias;
     unsigned int gemm_m, gemm_k;              /* rows / contraction length of `weight` */
+    float anchors[6];                         /* YOLO layers: (width, height) of the layer's three anchor boxes */
     /* device copies, created on first use */
     float *d_weight, *d_bias;
     aspen_hip_ktab_t *d_ktab;

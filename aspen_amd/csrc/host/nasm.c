@@ -45,7 +45,7 @@ static int set_out_mat (nasm_t *nasm, nasm_ldata_t *ld)
         flop_per_out = (uint64_t)p[WEIGHT_H] * p[WEIGHT_W];
         ld->out_mat_dims[OUT_H] = p[OUT_C]; ld->out_mat_dims[OUT_W] = p[OUT_H] * p[OUT_W] * B;
         break;
-    case INPUT_LAYER: case RESIDUAL_LAYER:
+    case INPUT_LAYER: case RESIDUAL_LAYER: case YOLO_LAYER: case APPEND_LAYER:
         if (S != 0) { ld->out_mat_dims[OUT_H] = p[MAT_M]; ld->out_mat_dims[OUT_W] = S * B; }
         else { ld->out_mat_dims[OUT_H] = p[OUT_C]; ld->out_mat_dims[OUT_W] = p[OUT_H] * p[OUT_W] * B; }
         break;
@@ -307,6 +307,36 @@ static void find_parents (const nasm_t *nasm, const nasm_ldata_t *ld, unsigned i
         add_parents (p0, c0, c1, r0, r1, out);
         add_parents (p1, c0, c1, r0, r1, out);
         break;
+    case YOLO_LAYER:
+    {
+        /* output column = (batch, anchor, cell); it reads rows [anchor*R, anchor*R + R) of parent
+           column (batch, cell) (reference src/tiled_kernels.c:686-697) */
+        const unsigned int cells = p[IN_H] * p[IN_W], R = p[OUT_C], A = p[IN_C] / R;
+        for (unsigned int c = c0; c < c1; )
+        {
+            const unsigned int seg = c / cells, b = seg / A, a = seg % A, cell0 = c % cells;
+            const unsigned int end = umin (c1, (seg + 1) * cells), cell1 = cell0 + (end - c);
+            add_parents (p0, b * cells + cell0, b * cells + cell1, a * R, (a + 1) * R, out);
+            c = end;
+        }
+        break;
+    }
+    case APPEND_LAYER:
+    {
+        /* rows [0, IN_C): first parent, upsampled by `stride`; rows [IN_C, OUT_C): second parent at
+           the output resolution (reference src/tiled_kernels.c:710-741) */
+        const unsigned int ohw = p[OUT_H] * p[OUT_W], ihw = p[IN_H] * p[IN_W], st = p[STRIDE];
+        add_parents (p1, c0, c1, 0, p1->out_mat_dims[OUT_H], out);
+        for (unsigned int b = c0 / ohw; b <= (c1 - 1) / ohw; b++)
+        {
+            const unsigned int first = umax (c0, b * ohw) - b * ohw, last = umin (c1, (b + 1) * ohw) - 1 - b * ohw;
+            const unsigned int ih0 = first / p[OUT_W] / st, ih1 = last / p[OUT_W] / st;
+            unsigned int iw0 = 0, iw1 = p[IN_W] - 1;
+            if (first / p[OUT_W] == last / p[OUT_W]) { iw0 = first % p[OUT_W] / st; iw1 = last % p[OUT_W] / st; }
+            add_parents (p0, b * ihw + ih0 * p[IN_W] + iw0, b * ihw + ih1 * p[IN_W] + iw1 + 1, 0, p0->out_mat_dims[OUT_H], out);
+        }
+        break;
+    }
     case K_ATTENTION_LAYER:
     {
         const unsigned int H = p[NUM_HEAD], hd = p[NUM_HIDDEN] / H;

@@ -280,7 +280,42 @@ void dse_group_run_until_nasm_completion (dse_group_t *dse_group, nasm_t *nasm)
 /* ---- results ------------------------------------------------------------------------------------ */
 /* Layer output as a dense tensor in the caller's dimension order (reference get_ldata_output,
    src/apu.c:227-297): stride padding stripped, native order (batch, positions..., channels) permuted. */
+static ssize_t get_ldata_output (nasm_t *nasm, unsigned int ldata_idx, LAYER_PARAMS *order, void **out_ptr);
+
+/* For a YOLO layer the reference returns ALL detection heads of the network, concatenated per image
+   in layer order (reference src/dse.c:472-513); so does this function when a dimension order is given.
+   order == NULL (an extension) always returns the one layer's own matrix as [columns][rows]. */
 ssize_t dse_get_ldata_result (nasm_t *nasm, unsigned int ldata_idx, LAYER_PARAMS *order, void **out_ptr)
+{
+    if (nasm == NULL || ldata_idx >= nasm->num_ldata) { ERROR_PRTF ("Error in get_ldata_output: ldata is NULL.\n"); return -1; }
+    if (order == NULL || nasm->ldata_arr[ldata_idx].layer->type != YOLO_LAYER) return get_ldata_output (nasm, ldata_idx, order, out_ptr);
+    if (out_ptr == NULL) { ERROR_PRTF ("Error in get_ldata_output: out_ptr is NULL.\n"); return -1; }
+    void *parts[64];
+    ssize_t bytes[64], total = 0;
+    int n = 0;
+    for (unsigned int l = 0; l < nasm->num_ldata && n < 64; l++)
+    {
+        if (nasm->ldata_arr[l].layer->type != YOLO_LAYER) continue;
+        bytes[n] = get_ldata_output (nasm, l, order, &parts[n]);
+        if (bytes[n] < 0) { for (int i = 0; i < n; i++) free (parts[i]); return -1; }
+        total += bytes[n++];
+    }
+    char *outp = calloc (total ? (size_t)total : 1, 1);
+    size_t off = 0;
+    const size_t B = nasm->batch_size;
+    for (size_t b = 0; b < B; b++)
+        for (int i = 0; i < n; i++)
+        {
+            const size_t per = (size_t)bytes[i] / B;
+            memcpy (outp + off, (char *)parts[i] + per * b, per);
+            off += per;
+        }
+    for (int i = 0; i < n; i++) free (parts[i]);
+    *out_ptr = outp;
+    return total;
+}
+
+static ssize_t get_ldata_output (nasm_t *nasm, unsigned int ldata_idx, LAYER_PARAMS *order, void **out_ptr)
 {
     if (nasm == NULL || ldata_idx >= nasm->num_ldata) { ERROR_PRTF ("Error in get_ldata_output: ldata is NULL.\n"); return -1; }
     if (out_ptr == NULL) { ERROR_PRTF ("Error in get_ldata_output: out_ptr is NULL.\n"); return -1; }

@@ -115,6 +115,24 @@ def gpt2_cfg(n_layer=12, n_embd=768, n_head=12, ffn=3072) -> str:
     return s
 
 
+def yolo_mini_cfg(size=32, classes=3) -> str:
+    """A two-scale detector in the style of the reference's YOLO-v3 cfg (files/yolov3/yolov3_aspen.cfg):
+    leaky convolutions, a detection head, a branch that is upsampled and appended to an earlier
+    feature map, a second head."""
+    rows = 3 * (classes + 5)
+    anchors = "10,13,  16,30,  33,23,  30,61,  62,45,  59,119,  116,90,  156,198,  373,326"
+    s = f"[net]\nheight={size}\nwidth={size}\nchannels=3\n\n"
+    s += _conv(16, 3, 1, 1, "leaky") + _conv(32, 3, 2, 1, "leaky")          # 1, 2: size/2
+    s += _conv(64, 3, 2, 1, "leaky") + _conv(32, 1, 1, 0, "leaky")          # 3, 4: size/4
+    s += _conv(rows, 1, 1, 0, "linear")                                     # 5
+    s += f"[yolo]\nmask = 6,7,8\nstride = 4\nanchors = {anchors}\nclasses={classes}\nnum=9\n\n"   # 6
+    s += "[convolutional]\nparent=-3\nfilters=16\nsize=1\nstride=1\npad=0\nactivation=leaky\n\n"  # 7 (from 4)
+    s += "[append]\nstride=2\nparent=-1\nfrom=-6\n\n"                    # 8: upsample 7, concat with 2
+    s += _conv(32, 3, 1, 1, "leaky") + _conv(rows, 1, 1, 0, "linear")       # 9, 10
+    s += f"[yolo]\nmask = 3,4,5\nstride = 2\nanchors = {anchors}\nclasses={classes}\nnum=9\n\n"   # 11
+    return s
+
+
 def custom_cifar_cfg() -> str:
     """The small CIFAR-10 net of the reference's third example (conv5/pool/conv3/pool/3 FC)."""
     s = "[net]\nheight=32\nwidth=32\nchannels=3\n\n"
@@ -134,7 +152,7 @@ _TYPES = {
     "[shortcut]": "residual", "[max]": "maxpool", "[maxpool]": "maxpool", "[avg]": "avgpool",
     "[avgpool]": "avgpool", "[conn]": "fc", "[connected]": "fc", "[soft]": "softmax",
     "[softmax]": "softmax", "[matmul]": "matmul", "[attention_k]": "attn_k",
-    "[attention_v]": "attn_v", "[layernorm]": "layernorm",
+    "[attention_v]": "attn_v", "[layernorm]": "layernorm", "[yolo]": "yolo", "[append]": "append",
 }
 
 
@@ -183,6 +201,17 @@ def parse_cfg(text: str) -> List[Dict]:
             L["C"] = P["C"]
             L["H"] = (P["H"] + 2 * L["pad"] - (L["size"] - 1) - 1) // L["stride"] + 1
             L["W"] = (P["W"] + 2 * L["pad"] - (L["size"] - 1) - 1) // L["stride"] + 1
+        elif t == "yolo":
+            # rows = classes + 5; one output column per (anchor, cell); the layer's three anchors are
+            # picked from the anchor list by `mask` (reference src/darknet_parser.c:487-545)
+            L["C"] = gi("classes") + 5
+            L["H"], L["W"] = 1, P["H"] * P["W"] * (P["C"] // L["C"])
+            mask = [int(v) for v in o["mask"].split(",")]
+            anch = [float(v) for v in o["anchors"].split(",")]
+            L["anchors"] = np.array([anch[2 * m + k] for m in mask[:3] for k in (0, 1)], dtype=np.float32)
+        elif t == "append":
+            Q = layers[L["p1"]]
+            L["C"], L["H"], L["W"] = P["C"] + Q["C"], P["H"] * L["stride"], P["W"] * L["stride"]
         elif t == "fc":
             L["C"], L["H"], L["W"] = gi("output") or gi("filters"), 1, 1
         elif t == "softmax":

@@ -273,6 +273,44 @@ void oracle_residual (const float *p0, unsigned int ld0, const float *p1, unsign
     }
 }
 
+/* YOLO box decode (reference src/tiled_kernels.c:675-708).  Output column = (batch, anchor a, h, w),
+   rows = classes + 5; reads channel a * rows + j of input column (batch, h, w):
+   x, y = (sigmoid + cell index) * stride; w, h = exp * anchor size; the rest = sigmoid. */
+void oracle_yolo (const float *in, unsigned int ldin, float *out, unsigned int ldout, const float *anchors,
+    unsigned int B, unsigned int IH, unsigned int IW, unsigned int IC, unsigned int rows, unsigned int stride)
+{
+    const unsigned int A = IC / rows;
+    for (unsigned int n = 0; n < B * IH * IW * A; n++)
+    {
+        const unsigned int b = n / (IH * IW * A), rem = n % (IH * IW * A), a = rem / (IH * IW), hw = rem % (IH * IW);
+        const unsigned int h = hw / IW, w = hw % IW;
+        const float *x = in + (size_t)((b * IH + h) * IW + w) * ldin + a * rows;
+        float *o = out + (size_t)n * ldout;
+        o[0] = (1.0f / (1.0f + expf (-x[0])) + w) * stride;
+        o[1] = (1.0f / (1.0f + expf (-x[1])) + h) * stride;
+        o[2] = expf (x[2]) * anchors[2 * a];
+        o[3] = expf (x[3]) * anchors[2 * a + 1];
+        for (unsigned int j = 4; j < rows; j++) o[j] = 1.0f / (1.0f + expf (-x[j]));
+    }
+}
+
+/* nearest-neighbour upsampling of p0 by `stride`, concatenated along the channels with p1 at the
+   output resolution (reference src/tiled_kernels.c:710-741) */
+void oracle_append (const float *p0, unsigned int ld0, const float *p1, unsigned int ld1, float *out, unsigned int ldout,
+    unsigned int B, unsigned int OH, unsigned int OW, unsigned int C0, unsigned int C1, unsigned int stride)
+{
+    const unsigned int IW = OW / stride, IH = OH / stride;
+    for (unsigned int n = 0; n < B * OH * OW; n++)
+    {
+        const unsigned int b = n / (OH * OW), oh = (n / OW) % OH, ow = n % OW;
+        const float *a = p0 + (size_t)((b * IH + oh / stride) * IW + ow / stride) * ld0;
+        const float *c = p1 + (size_t)n * ld1;
+        float *o = out + (size_t)n * ldout;
+        memcpy (o, a, C0 * sizeof (float));
+        memcpy (o + C0, c, C1 * sizeof (float));
+    }
+}
+
 /* max-subtracted softmax over rows of each column (reference src/tiled_kernels.c:640-673) */
 void oracle_softmax (const float *in, unsigned int ldin, float *out, unsigned int ldout, unsigned int M, unsigned int N)
 {

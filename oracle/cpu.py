@@ -122,6 +122,22 @@ def residual(a, b, act):
     return out
 
 
+def yolo(x, anchors, B, IH, IW, rows, stride):
+    IC = x.shape[1]
+    A = IC // rows
+    out = np.empty((B * IH * IW * A, rows), dtype=np.float32)
+    anchors = np.ascontiguousarray(anchors, dtype=np.float32)
+    lib().oracle_yolo(_p(x), _u(IC), _p(out), _u(rows), _p(anchors), _u(B), _u(IH), _u(IW), _u(IC), _u(rows), _u(stride))
+    return out
+
+
+def append(a, b, B, OH, OW, stride):
+    C0, C1 = a.shape[1], b.shape[1]
+    out = np.empty((B * OH * OW, C0 + C1), dtype=np.float32)
+    lib().oracle_append(_p(a), _u(C0), _p(b), _u(C1), _p(out), _u(C0 + C1), _u(B), _u(OH), _u(OW), _u(C0), _u(C1), _u(stride))
+    return out
+
+
 def softmax(x):
     N, M = x.shape
     out = np.empty((N, M), dtype=np.float32)
@@ -180,6 +196,10 @@ def run_network(layers: List[Dict], tensors, x_dense: np.ndarray, batch: int, se
             o = conv2d(p0, w, b, batch, L["inH"], L["inW"], L["stride"], L["pad"], act)
         elif t in ("maxpool", "avgpool"):
             o = pool(t, p0, batch, L["inH"], L["inW"], L["inC"], L["size"], L["stride"], L["pad"], act)
+        elif t == "yolo":
+            o = yolo(p0, L["anchors"], batch, L["inH"], L["inW"], L["C"], L["stride"])
+        elif t == "append":
+            o = append(p0, p1, batch, L["H"], L["W"], L["stride"])
         elif t == "fc":
             o = fc(p0, w, b, batch, act)
         elif t == "residual":

@@ -30,6 +30,7 @@ MICRO = {
     "vgg_mini_b5": (M.vgg16_cfg(32, 32, 10, (8, "M", 16, "M", 64, 64, "M"), (128,)), "he", 5, 0, 9, None),
     "bert_mini_b2_s24": (M.bert_cfg(2, 128, 2, 256), "gpt", 2, 24, 10, "embeddings"),
     "gpt_mini_b2_s20": (M.gpt2_cfg(2, 128, 2, 256), "gpt", 2, 20, 11, "token_ids"),
+    "yolo_mini_b2": (M.yolo_mini_cfg(), "he", 2, 0, 12, None),
 }
 
 

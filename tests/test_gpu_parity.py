@@ -227,3 +227,20 @@ def test_model_loaded_from_reference_aspen_file_runs(gpu):
     for l in range(nasm.num_ldata):
         assert H.rel_l2(nasm.layer_output(l), outs[l]) <= H.REL_L2_TOL, l
     dse.destroy(); pool.destroy(); nasm.destroy(); dnn.destroy()
+
+
+@pytest.mark.gpu
+def test_yolo_result_gathers_all_heads(gpu):
+    """dse_get_ldata_result on a YOLO layer with a dimension order returns every detection head of the
+    network, concatenated per image in layer order (reference src/dse.c:472-513)."""
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()["yolo_mini_b2"])
+    net = H.GpuNet(cfg, tens, batch, seq, min_ninst=16)
+    net.run(x)
+    try:
+        heads = [l for l, L in enumerate(layers) if L["type"] == "yolo"]
+        mats = [net.layer(l) for l in heads]                         # [batch * boxes][rows] each
+        got = net.nasm.layer_output(heads[-1], order=[api.BATCH, api.OUT_H, api.OUT_W, api.OUT_C])
+        want = np.concatenate([m.reshape(batch, -1)[b] for b in range(batch) for m in mats])
+        assert got.shape == want.shape and np.array_equal(got, want)
+    finally:
+        net.close()

@@ -72,6 +72,23 @@ def needed_regions(L, layers, c0, c1, r0, r1, batch, seq):
         return [(p0, {b * hw + j for b in cols for j in range(hw)}, 0, None)]
     if t == "residual":
         return [(p0, set(cols), r0, r1), (p1, set(cols), r0, r1)]
+    if t == "yolo":         # column = (batch, anchor, cell): rows [anchor*R, anchor*R + R) of parent column (batch, cell)
+        cells, R = L["inH"] * L["inW"], L["C"]
+        A = L["inC"] // R
+        out = []
+        for c in cols:
+            seg, cell = divmod(c, cells)
+            b, a = divmod(seg, A)
+            out.append((p0, {b * cells + cell}, a * R, (a + 1) * R))
+        return out
+    if t == "append":       # first parent upsampled by stride (all its rows), second parent at the same column
+        OH, OW, st = L["H"], L["W"], L["stride"]
+        IH, IW = OH // st, OW // st
+        up = set()
+        for c in cols:
+            b, oh, ow = c // (OH * OW), (c // OW) % OH, c % OW
+            up.add((b * IH + oh // st) * IW + ow // st)
+        return [(p0, up, 0, None), (p1, set(cols), 0, None)]
     if t in ("matmul", "layernorm", "softmax"):
         return [(p0, set(cols), 0, None)]
     if t == "attn_k":       # column = (b, head, query); rows = keys
@@ -103,7 +120,8 @@ def needed_regions(L, layers, c0, c1, r0, r1, batch, seq):
 
 @pytest.mark.parametrize("fuse", [True, False], ids=["fused", "unfused"])
 @pytest.mark.parametrize("name,min_ninst", [("custom_b3", 16), ("resnet_mini_b2", 64), ("resnet_mini_b2", 1024),
-                                            ("vgg_mini_b5", 32), ("bert_mini_b2_s24", 16), ("gpt_mini_b2_s20", 256)])
+                                            ("vgg_mini_b5", 32), ("bert_mini_b2_s24", 16), ("gpt_mini_b2_s20", 256),
+                                            ("yolo_mini_b2", 16), ("yolo_mini_b2", 512)])
 def test_tile_graph_against_brute_force(name, min_ninst, fuse, monkeypatch):
     if not fuse:
         monkeypatch.setenv("ASPEN_GPU_NO_FUSE", "1")
@@ -194,6 +212,13 @@ def test_tile_graph_against_brute_force(name, min_ninst, fuse, monkeypatch):
                     for h in hs:
                         both |= {int(v) for v in np.unique(owner[pp][b * seq:(b + 1) * seq, h * hd:(h + 1) * hd])}
             assert parents[t] <= both, (name, l, t)
+        elif L["type"] == "append":
+            # second parent exact; first parent: everything read is awaited, nothing outside the hull of its columns
+            assert need <= parents[t], (name, l, t)
+            up = regions[0][1]
+            hull = {int(v) for v in np.unique(owner[L["p0"]][min(up):max(up) + 1, :])} if produced(L["p0"]) else set()
+            exact = {int(v) for v in np.unique(owner[L["p1"]][c0:c1, :])} if produced(L["p1"]) else set()
+            assert parents[t] <= hull | exact, (name, l, t)
         elif L["type"] in ("conv", "maxpool", "avgpool"):
             # the library may await the contiguous hull of the window's input columns (a superset for
             # strided windows): everything read is awaited, nothing outside the hull is

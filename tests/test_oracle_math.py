@@ -160,3 +160,27 @@ def test_attention_matches_textbook(masked):
     o = cpu.v_attention(p, v, B, H, S)
     want_o = (want_p @ vt).permute(0, 2, 1, 3).reshape(B * S, E)
     assert np.allclose(o, want_o.numpy(), rtol=1e-4, atol=1e-6)
+
+
+# ---- detection layers ------------------------------------------------------------------------------
+def test_yolo_and_append_match_torch():
+    B, IH, IW, R, A, stride = 2, 3, 4, 7, 3, 8
+    x = rnd(B, A * R, IH, IW)
+    anchors = np.array([10, 13, 16, 30, 33, 23], dtype=np.float32)
+    got = cpu.yolo(nhwc(x), anchors, B, IH, IW, R, stride)           # [(b, a, h, w)][R]
+    t = torch.from_numpy(x).reshape(B, A, R, IH, IW)
+    gx = torch.arange(IW).float().view(1, 1, 1, IW)
+    gy = torch.arange(IH).float().view(1, 1, IH, 1)
+    want = torch.empty_like(t)
+    want[:, :, 0] = (torch.sigmoid(t[:, :, 0]) + gx) * stride
+    want[:, :, 1] = (torch.sigmoid(t[:, :, 1]) + gy) * stride
+    want[:, :, 2] = torch.exp(t[:, :, 2]) * torch.tensor(anchors[0::2]).view(1, A, 1, 1)
+    want[:, :, 3] = torch.exp(t[:, :, 3]) * torch.tensor(anchors[1::2]).view(1, A, 1, 1)
+    want[:, :, 4:] = torch.sigmoid(t[:, :, 4:])
+    want = want.permute(0, 1, 3, 4, 2).reshape(B * A * IH * IW, R)
+    assert np.allclose(got, want.numpy(), rtol=1e-5, atol=1e-6)
+    # append = nearest upsampling of the first operand, channel concatenation with the second
+    a, b = rnd(B, 5, 3, 2), rnd(B, 4, 6, 4)
+    got = cpu.append(nhwc(a), nhwc(b), B, 6, 4, 2)
+    want = torch.cat([F.interpolate(torch.from_numpy(a), scale_factor=2, mode="nearest"), torch.from_numpy(b)], dim=1)
+    assert np.array_equal(to_nchw(got, B, 6, 4), want.numpy())
