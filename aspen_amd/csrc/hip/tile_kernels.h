@@ -493,16 +493,54 @@ __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, ui
         const bool fuse = L.fuse_out != nullptr && slice < 0;
         ActView<COH> fin, fout;
         if (fuse) { fin.init (L.fuse_in, L.N, L.fuse_ld_in); fout.init (L.fuse_out, L.N, L.ld); }
-        for (uint32_t r = tid / C4; r < rows; r += WG_THREADS / C4)
+        constexpr uint32_t STEP = WG_THREADS / C4, U = 4;
+        if (c + 4 <= mrem)
         {
-            float4 v = ld4 (smem + r * TROW + c);
-            v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
-            v = act4 (v, act);
-            const uint32_t o = (n0 + r) * L.ld + m0 + c;
-            if (c + 4 <= mrem) out.st4 (o, v);
-            else { out.st1 (o, v.x); if (c + 1 < mrem) out.st1 (o + 1, v.y); if (c + 2 < mrem) out.st1 (o + 2, v.z); }
-            if (fuse) fused_shortcut<COH> (L, fin, fout, v, n0 + r, m0 + c, mrem - c);
+            // whole float4 of channels: rows are handled U at a time, all LDS reads and shortcut loads of a
+            // group issued before the first use, so their latencies overlap instead of adding up
+            for (uint32_t r0 = tid / C4; r0 < rows; r0 += U * STEP)
+            {
+                float4 v[U], s[U];
+                #pragma unroll
+                for (uint32_t u = 0; u < U; u++)
+                {
+                    const uint32_t r = r0 + u * STEP;
+                    if (r < rows)
+                    {
+                        v[u] = ld4 (smem + r * TROW + c);
+                        if (fuse) s[u] = fin.ld4 ((n0 + r) * L.fuse_ld_in + m0 + c);
+                    }
+                }
+                #pragma unroll
+                for (uint32_t u = 0; u < U; u++)
+                {
+                    const uint32_t r = r0 + u * STEP;
+                    if (r < rows)
+                    {
+                        float4 y = v[u];
+                        y.x += b.x; y.y += b.y; y.z += b.z; y.w += b.w;
+                        y = act4 (y, act);
+                        const uint32_t o = (n0 + r) * L.ld + m0 + c;
+                        out.st4 (o, y);
+                        if (fuse)
+                        {
+                            y.x += s[u].x; y.y += s[u].y; y.z += s[u].z; y.w += s[u].w;
+                            fout.st4 (o, act4 (y, L.fuse_act));
+                        }
+                    }
+                }
+            }
         }
+        else
+            for (uint32_t r = tid / C4; r < rows; r += STEP)      // last, partial group of channels
+            {
+                float4 v = ld4 (smem + r * TROW + c);
+                v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
+                v = act4 (v, act);
+                const uint32_t o = (n0 + r) * L.ld + m0 + c;
+                out.st1 (o, v.x); if (c + 1 < mrem) out.st1 (o + 1, v.y); if (c + 2 < mrem) out.st1 (o + 2, v.z);
+                if (fuse) fused_shortcut<COH> (L, fin, fout, v, n0 + r, m0 + c, mrem - c);
+            }
     }
     __syncthreads ();
 }
