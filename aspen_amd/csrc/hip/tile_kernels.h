@@ -493,11 +493,12 @@ __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, ui
         const bool fuse = L.fuse_out != nullptr && slice < 0;
         ActView<COH> fin, fout;
         if (fuse) { fin.init (L.fuse_in, L.N, L.fuse_ld_in); fout.init (L.fuse_out, L.N, L.ld); }
-        constexpr uint32_t STEP = WG_THREADS / C4, U = 4;
+        constexpr uint32_t STEP = WG_THREADS / C4, U = 4;      // 4 rows at a time: all 8 of the larger tiles measured slower (code size, registers)
         if (c + 4 <= mrem)
         {
             // whole float4 of channels: rows are handled U at a time, all LDS reads and shortcut loads of a
-            // group issued before the first use, so their latencies overlap instead of adding up
+            // group issued before its first store.  Loads and stores share one in-order counter, so a
+            // shortcut load issued after a (write-through) store waits for that store's acknowledgement.
             for (uint32_t r0 = tid / C4; r0 < rows; r0 += U * STEP)
             {
                 float4 v[U], s[U];
