@@ -46,6 +46,7 @@ static hipStream_t g_stream = nullptr;
 static hipEvent_t g_events[NUM_EVENTS];
 static int g_inited = 0;
 static int g_num_cu = 0;
+static int g_resident_wg = WG_PER_CU;     // workgroups of the dataflow kernel that fit one compute unit
 static char g_err[512] = "";
 static uint32_t g_flags = 0;
 static uint32_t *g_host_abort = nullptr;    // pinned host word the persistent kernel raises when it gives up waiting
@@ -149,12 +150,19 @@ __device__ __forceinline__ qentry_t wait_for_slot (const dataflow_args_t &a, uin
     }
 }
 
+#define DESC_CACHE 4
+static_assert (sizeof (aspen_hip_layer_t) % 4 == 0 && sizeof (aspen_hip_layer_t) / 4 <= 64, "one descriptor dword per lane of a wavefront");
+
 // Workgroup-local scheduler state.  It lives in LDS so that nothing of it occupies registers while a
 // tile runs: the tile code is inlined into the persistent loop and owns the whole register budget.
 struct sched_lds_t
 {
     dataflow_args_t a;
     uint32_t tile, layer;                // tile to run next (QUEUE_EMPTY: leave) and its layer
+    // the descriptors of the last few layers this workgroup worked on: consecutive tiles mostly belong
+    // to the same two or three layers, so most tiles find theirs here instead of fetching it from memory
+    uint32_t desc_slot, desc_next, desc_id[DESC_CACHE];
+    aspen_hip_layer_t desc[DESC_CACHE];
     unsigned long long t0, ticks[6];     // profiling: last time stamp; tile / drain / scheduling / publish / ticket / slot-wait ticks
 };
 __shared__ sched_lds_t s_sched;
@@ -224,18 +232,38 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
         }
         if (prof) { asm volatile ("s_waitcnt vmcnt(0)" ::: "memory"); s_sched.ticks[3] += wall_clock64 () - tp; }
     }
-    else if (wave == 1 && lane == 0)
+    else if (wave == 1)
     {
-        // pop: a ticket is drawn only now, when this workgroup is free.  Drawing it earlier would
-        // hide the atomic's round trip but binds a (possibly already ready) tile to a busy
-        // workgroup while idle ones wait on later slots.
-        const unsigned long long t1 = prof ? wall_clock64 () : 0;
-        const uint32_t ticket = atomicAdd (&a.state[ST_HEAD], 1u);
-        const unsigned long long t2 = prof ? wall_clock64 () : 0;
-        const qentry_t e = wait_for_slot (a, ticket);
-        s_sched.tile = e == QENTRY_EMPTY ? QUEUE_EMPTY : (uint32_t)e;
-        s_sched.layer = (uint32_t)(e >> 32) & 0xffffu;
-        if (prof) { s_sched.ticks[4] += t2 - t1; s_sched.ticks[5] += wall_clock64 () - t2; }
+        if (lane == 0)
+        {
+            // pop: a ticket is drawn only now, when this workgroup is free.  Drawing it earlier would
+            // hide the atomic's round trip but binds a (possibly already ready) tile to a busy
+            // workgroup while idle ones wait on later slots.
+            const unsigned long long t1 = prof ? wall_clock64 () : 0;
+            const uint32_t ticket = atomicAdd (&a.state[ST_HEAD], 1u);
+            const unsigned long long t2 = prof ? wall_clock64 () : 0;
+            const qentry_t e = wait_for_slot (a, ticket);
+            s_sched.tile = e == QENTRY_EMPTY ? QUEUE_EMPTY : (uint32_t)e;
+            s_sched.layer = (uint32_t)(e >> 32) & 0xffffu;
+            if (prof) { s_sched.ticks[4] += t2 - t1; s_sched.ticks[5] += wall_clock64 () - t2; }
+        }
+        // the popping wavefront also makes sure the tile's layer descriptor is in the LDS cache
+        // (same wavefront, program order: lane 0's LDS writes above are visible to all lanes here)
+        const uint32_t tile = __builtin_amdgcn_readfirstlane (s_sched.tile), layer = __builtin_amdgcn_readfirstlane (s_sched.layer);
+        if (tile != QUEUE_EMPTY)
+        {
+            uint32_t slot = DESC_CACHE;
+            for (uint32_t i = 0; i < DESC_CACHE; i++) if (s_sched.desc_id[i] == layer) slot = i;
+            slot = __builtin_amdgcn_readfirstlane (slot);
+            if (slot == DESC_CACHE)
+            {
+                slot = __builtin_amdgcn_readfirstlane (s_sched.desc_next);
+                if (lane < sizeof (aspen_hip_layer_t) / 4)
+                    reinterpret_cast<uint32_t *> (&s_sched.desc[slot])[lane] = reinterpret_cast<const uint32_t *> (&a.layers[layer])[lane];
+                if (lane == 0) { s_sched.desc_id[slot] = layer; s_sched.desc_next = (slot + 1) % DESC_CACHE; }
+            }
+            if (lane == 0) s_sched.desc_slot = slot;
+        }
     }
     __syncthreads ();
     const uint32_t next = s_sched.tile;
@@ -256,6 +284,8 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
         s_sched.a = args;
         s_sched.t0 = wall_clock64 ();
         for (int i = 0; i < 6; i++) s_sched.ticks[i] = 0;
+        s_sched.desc_next = 0;
+        for (int i = 0; i < DESC_CACHE; i++) s_sched.desc_id[i] = 0xffffffffu;
     }
     __syncthreads ();
     const unsigned long long t_begin = wall_clock64 ();
@@ -270,7 +300,7 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
         if ((s_sched.a.flags & ASPEN_HIP_FLAG_TRACE) && threadIdx.x == 0) s_sched.a.trace[2 * (size_t)id] = wall_clock64 ();
         if (!(s_sched.a.flags & ASPEN_HIP_FLAG_SKIP_TILES))
         {
-            const aspen_hip_layer_t *L = &s_sched.a.layers[__builtin_amdgcn_readfirstlane (s_sched.layer)];
+            const aspen_hip_layer_t *L = &s_sched.desc[__builtin_amdgcn_readfirstlane (s_sched.desc_slot)];
             run_tile<COH> (*L, id - L->ninst_start, smem);
         }
     }
@@ -303,6 +333,13 @@ extern "C" int aspen_hip_init (void)
     CHECK (hipFuncSetAttribute ((const void *)layer_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
     CHECK (hipFuncSetAttribute ((const void *)dataflow_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
     CHECK (hipFuncSetAttribute ((const void *)dataflow_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
+    // how many persistent workgroups really fit a compute unit (registers, LDS): the default grid
+    int occ1 = 0, occ2 = 0;
+    CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&occ1, dataflow_kernel<1>, WG_THREADS, GEMM_SMEM_BYTES));
+    CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&occ2, dataflow_kernel<2>, WG_THREADS, GEMM_SMEM_BYTES));
+    g_resident_wg = occ1 < occ2 ? occ1 : occ2;
+    if (g_resident_wg < 1) g_resident_wg = 1;
+    if (getenv ("ASPEN_GPU_VERBOSE")) fprintf (stderr, "aspen_hip: %d resident dataflow workgroups per compute unit (built for %d)\n", g_resident_wg, WG_PER_CU);
     g_inited = 1;
     return 0;
 }
@@ -607,7 +644,7 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
 {
     if (!g) { snprintf (g_err, sizeof (g_err), "run_dataflow: null graph"); return -1; }
     if (g->num_ninst == 0) return 0;
-    if (workgroups == 0) workgroups = WG_PER_CU * (uint32_t)g_num_cu;
+    if (workgroups == 0) workgroups = (uint32_t)g_resident_wg * (uint32_t)g_num_cu;
     g->epoch = g->epoch % 255u + 1u;
     hipLaunchKernelGGL (arm_kernel, dim3 ((g->num_ninst + 255) / 256), dim3 (256), 0, g_stream,
         g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->d_ninst_layer, g->num_ninst, g->num_roots, g->d_state, g->epoch);
