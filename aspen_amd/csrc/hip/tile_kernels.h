@@ -90,11 +90,12 @@ template <int COH> struct ActView
     }
 };
 
-// The transcendental activations follow the reference's C expressions, which evaluate in double
-// (reference src/tiled_kernels.c naive_activate).  They are rare and carry many double-precision
-// constants, so they live in a real function: inlined, their constants would be set up in front of
-// the persistent loop and occupy registers during every tile.
-__device__ __noinline__ float activate_transcendental (float x, int act)
+// Activations other than the three cheap ones follow the reference's C expressions, which evaluate
+// in double or call libm (reference src/naive_kernels.c:11-57).  Their code is large (erff, tanhf, exp,
+// double-precision constants), so they live in ONE real function: inlined into every epilogue copy they
+// multiplied the kernel's code far beyond the instruction cache, and their constants were set up in
+// front of the persistent loop and occupied registers during every tile.
+__device__ __noinline__ float activate_slow (float x, int act)
 {
     switch (act)
     {
@@ -102,6 +103,8 @@ __device__ __noinline__ float activate_transcendental (float x, int act)
     case SELU:          return x > 0 ? (float)(1.0507 * (double)x) : (float)(1.0507 * 1.67326 * (exp ((double)x) - 1));
     case SIGMOID:       return (float)(1 / (1 + exp (-(double)x)));
     case TANH:          return (float)tanh ((double)x);
+    case GELU:          return (float)(0.5 * (double)x * (double)(1 + erff (x * 0.7071067811865475f)));
+    case GELU_ACCURATE: return (float)(0.5 * (double)x * (double)(1 + tanhf (0.7978845608028654f * (float)((double)x + 0.044715 * (double)x * (double)x * (double)x))));
     default:            return x;
     }
 }
@@ -113,9 +116,7 @@ __device__ __forceinline__ float activate (float x, int act)
     case NO_ACTIVATION: case LINEAR: return x;
     case RELU:          return x > 0 ? x : 0;
     case LEAKY_RELU:    return x > 0 ? x : (float)(0.1 * (double)x);
-    case GELU:          return (float)(0.5 * (double)x * (double)(1 + erff (x * 0.7071067811865475f)));
-    case GELU_ACCURATE: return (float)(0.5 * (double)x * (double)(1 + tanhf (0.7978845608028654f * (float)((double)x + 0.044715 * (double)x * (double)x * (double)x))));
-    default:            return activate_transcendental (x, act);
+    default:            return activate_slow (x, act);
     }
 }
 
