@@ -432,24 +432,23 @@ __device__ __forceinline__ void fused_shortcut (const aspen_hip_layer_t &L, cons
 // conv / FC / matmul tile
 // `slice` < 0: the whole K axis, bias + activation, result to the layer's matrix.  `slice` >= 0 (split-K):
 // K slices [slice*kiters_per_split, ...) only, raw sums to that slice's partial matrix.
+// This part (operand loaders, K loop, accumulators parked in LDS) exists once per tile shape; the
+// epilogue that follows it is shared by all shapes, which keeps the kernel's code small.
 template <int BM, int BN, int WM, int WN, int COH>
-__device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, int slice, float *smem)
+__device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, int slice, float *smem)
 {
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
     const uint32_t m0 = tm * BM, n0 = tn * BN;
     floatx16 acc[TN][TM];
-    ActView<COH> in, out;
+    ActView<COH> in;
     in.init (L.in0, L.type == FC_LAYER ? L.N * L.IH * L.IW : (L.type == CONV_LAYER ? (L.N / (L.OH * L.OW)) * L.IH * L.IW : L.N), L.ld0);
     int kbase = 0, kiters = (int)(L.Kp / GEMM_BK);
     if (slice >= 0)
     {
         kbase = slice * (int)L.kiters_per_split;
         kiters = min ((int)L.kiters_per_split, kiters - kbase);
-        out.init (L.partial + (size_t)slice * L.N * L.ld, L.N, L.ld);
     }
-    else
-        out.init (L.out, L.N, L.ld);
     RowLoader<BM> al;
     al.init (L.weight, m0, 0xffffffffu, L.Kp, tid);
     if (L.direct)
@@ -465,11 +464,8 @@ __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, ui
         gemm_core<BM, BN, WM, WN> (al, bl, kbase, kiters, smem, acc);
     }
     const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);
-    const int act = slice >= 0 ? NO_ACTIVATION : L.act;
     // Epilogue through LDS (free after the last K slice): the raw accumulators are parked as
-    // [column][channel]; a rolled loop then adds the bias, applies the activation and writes 128-bit
-    // pieces, so a wavefront covers whole 512-byte (BM = 128) / 256-byte (BM = 64) runs of a column.
-    // Keeping the activation out of the unrolled accumulator loops keeps the kernel's code small.
+    // [column][channel] for contraction_epilogue.
     constexpr int TROW = BM + 8;            // (4 * TROW) % 64 == 32: the two half-waves hit disjoint banks
     #pragma unroll
     for (int j = 0; j < TM; j++)
@@ -479,10 +475,25 @@ __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, ui
             for (int v = 0; v < 16; v++)
                 smem[ACC_N (wn0, i, v, lane) * TROW + wm0 + 32 * j + (lane & 31)] = acc[i][j][v];
     __syncthreads ();
-    constexpr int C4 = BM / 4;
-    const uint32_t rows = min ((uint32_t)BN, L.N - n0);
+}
+
+// Second part of a contraction tile of BM = 4 << c4_log2 channels by BN columns, accumulators parked in
+// LDS as [column][BM + 8]: a rolled loop adds the bias, applies the activation and writes 128-bit pieces,
+// so a wavefront covers whole 512-byte (BM = 128) / 256-byte (BM = 64) runs of a column.
+template <int COH>
+__device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, int slice, float *smem,
+    uint32_t c4_log2, uint32_t BN)
+{
+    const uint32_t tid = tile_thread ();
+    const uint32_t C4 = 1u << c4_log2, BM = 4u << c4_log2, TROW = BM + 8;
+    const uint32_t m0 = tm * BM, n0 = tn * BN;
+    const int act = slice >= 0 ? NO_ACTIVATION : L.act;
+    ActView<COH> out;
+    if (slice >= 0) out.init (L.partial + (size_t)slice * L.N * L.ld, L.N, L.ld);
+    else out.init (L.out, L.N, L.ld);
+    const uint32_t rows = min (BN, L.N - n0);
     const uint32_t mrem = L.M - m0;         // channels of this tile that exist (may exceed BM)
-    const uint32_t c = (tid % C4) * 4;      // WG_THREADS is a multiple of C4: a thread keeps its channels
+    const uint32_t c = (tid & (C4 - 1)) * 4;      // WG_THREADS is a multiple of C4: a thread keeps its channels
     if (c < mrem)
     {
         float4 b = make_float4 (0.f, 0.f, 0.f, 0.f);
@@ -494,13 +505,14 @@ __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, ui
         const bool fuse = L.fuse_out != nullptr && slice < 0;
         ActView<COH> fin, fout;
         if (fuse) { fin.init (L.fuse_in, L.N, L.fuse_ld_in); fout.init (L.fuse_out, L.N, L.ld); }
-        constexpr uint32_t STEP = WG_THREADS / C4, U = 4;      // 4 rows at a time: all 8 of the larger tiles measured slower (code size, registers)
+        const uint32_t STEP = WG_THREADS >> c4_log2;
+        constexpr uint32_t U = 4;                              // 4 rows at a time: all 8 of the larger tiles measured slower (code size, registers)
         if (c + 4 <= mrem)
         {
             // whole float4 of channels: rows are handled U at a time, all LDS reads and shortcut loads of a
             // group issued before its first store.  Loads and stores share one in-order counter, so a
             // shortcut load issued after a (write-through) store waits for that store's acknowledgement.
-            for (uint32_t r0 = tid / C4; r0 < rows; r0 += U * STEP)
+            for (uint32_t r0 = tid >> c4_log2; r0 < rows; r0 += U * STEP)
             {
                 float4 v[U], s[U];
                 #pragma unroll
@@ -534,7 +546,7 @@ __device__ __forceinline__ void tile_contraction (const aspen_hip_layer_t &L, ui
             }
         }
         else
-            for (uint32_t r = tid / C4; r < rows; r += STEP)      // last, partial group of channels
+            for (uint32_t r = tid >> c4_log2; r < rows; r += STEP)      // last, partial group of channels
             {
                 float4 v = ld4 (smem + r * TROW + c);
                 v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
@@ -915,10 +927,15 @@ __device__ __forceinline__ void run_tile (const aspen_hip_layer_t &Lg, uint32_t 
     switch (L.type)
     {
     case CONV_LAYER: case FC_LAYER: case MATMUL_LAYER:
-        if (L.variant == ASPEN_HIP_GEMM_LARGE) tile_contraction<VAR0_BM, VAR0_BN, 2, 2, COH> (L, tn, tm, slice, smem);
-        else if (L.variant == ASPEN_HIP_GEMM_WIDE) tile_contraction<VAR1_BM, VAR1_BN, 2, 2, COH> (L, tn, tm, slice, smem);
-        else tile_contraction<VAR2_BM, VAR2_BN, 2, 2, COH> (L, tn, tm, slice, smem);
+    {
+        uint32_t c4_log2, bn;
+        if (L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, COH> (L, tn, tm, slice, smem); c4_log2 = 5; bn = VAR0_BN; }
+        else if (L.variant == ASPEN_HIP_GEMM_WIDE) { contraction_mainloop<VAR1_BM, VAR1_BN, 2, 2, COH> (L, tn, tm, slice, smem); c4_log2 = 4; bn = VAR1_BN; }
+        else { contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, COH> (L, tn, tm, slice, smem); c4_log2 = 4; bn = VAR2_BN; }
+        static_assert (VAR0_BM == 128 && VAR1_BM == 64 && VAR2_BM == 64, "c4_log2 above");
+        contraction_epilogue<COH> (L, tn, tm, slice, smem, c4_log2, bn);
         break;
+    }
     case RESIDUAL_LAYER:    tile_residual<COH> (L, tn); break;
     case MAXPOOL_LAYER:     tile_pool<true, COH> (L, tn, tm); break;
     case AVGPOOL_LAYER:     tile_pool<false, COH> (L, tn, tm); break;
