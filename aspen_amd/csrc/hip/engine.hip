@@ -38,6 +38,7 @@ struct aspen_hip_graph_t
     uint32_t *d_ran;        // per-tile execution count (sanity: every tile exactly once)
     uint32_t epoch;         // tag of the last run's queue entries, cycles 1..255
     unsigned long long *d_prof;
+    uint32_t default_workgroups;    // grid of a dataflow run when the caller names none, see graph_parallelism
     int cached_loads;       // 1: no cache line of an activation is shared by two producer tiles
     unsigned long long *d_trace;    // [2*tile] start, [2*tile+1] end time stamps (allocated on first traced run)
 };
@@ -87,15 +88,28 @@ __device__ __forceinline__ qentry_t make_entry (uint32_t epoch, uint32_t layer, 
 {
     return ((qentry_t)epoch << 56) | ((qentry_t)layer << 32) | tile;
 }
+// Ticket t lives in queue entry (t % QUEUE_LANES) * row + t / QUEUE_LANES, row >= QUEUE_MIN_ROW entries:
+// the workgroups that wait hold consecutive tickets and each polls its entry, so neighbouring tickets
+// are placed at least 4 KiB apart and the polls spread over all memory channels instead of
+// hammering the one or two that would hold a dense array's next few lines.
+#define QUEUE_LANES 1024u
+#define QUEUE_MIN_ROW 512u
+__device__ __forceinline__ size_t queue_slot (uint32_t ticket, uint32_t row) { return (size_t)(ticket % QUEUE_LANES) * row + ticket / QUEUE_LANES; }
+static uint32_t queue_row (uint32_t num_ninst)
+{
+    const uint32_t r = (num_ninst + QUEUE_LANES) / QUEUE_LANES;
+    return r < QUEUE_MIN_ROW ? QUEUE_MIN_ROW : r;
+}
+
 __global__ void arm_kernel (uint32_t *dep, const uint32_t *num_parents, qentry_t *queue, uint32_t *ran,
-    const uint32_t *roots, const uint32_t *ninst_layer, uint32_t num_ninst, uint32_t num_roots, uint32_t *state, uint32_t epoch)
+    const uint32_t *roots, const uint32_t *ninst_layer, uint32_t num_ninst, uint32_t num_roots, uint32_t *state, uint32_t epoch, uint32_t qrow)
 {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < num_ninst)
     {
         __hip_atomic_store (&dep[i], num_parents[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (i < num_roots)
-            __hip_atomic_store (&queue[i], make_entry (epoch, ninst_layer[roots[i]], roots[i]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store (&queue[queue_slot (i, qrow)], make_entry (epoch, ninst_layer[roots[i]], roots[i]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store (&ran[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (i == 0)
@@ -121,6 +135,7 @@ struct dataflow_args_t
     uint32_t num_ninst;
     uint32_t epoch;                 // 1..255, tag of this run's queue entries
     uint32_t flags;                 // ASPEN_HIP_FLAG_*
+    uint32_t queue_row;             // see queue_slot
     unsigned long long spin_limit;
 };
 
@@ -136,7 +151,7 @@ __device__ __forceinline__ qentry_t wait_for_slot (const dataflow_args_t &a, uin
     unsigned long long spins = 0;
     for (;;)
     {
-        const qentry_t e = __hip_atomic_load (&a.queue[ticket], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const qentry_t e = __hip_atomic_load (&a.queue[queue_slot (ticket, a.queue_row)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if ((uint32_t)(e >> 56) == a.epoch) return e;
         ++spins;
         if ((spins & 63) == 0 && __hip_atomic_load (&a.state[ST_ABORT], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return QENTRY_EMPTY;
@@ -183,7 +198,7 @@ __device__ __forceinline__ void release_child (const dataflow_args_t &a, uint32_
     if (before == 1u)
     {
         const uint32_t slot = atomicAdd (&a.state[ST_TAIL], 1u);
-        __hip_atomic_store (&a.queue[slot], make_entry (a.epoch, layer, child), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store (&a.queue[queue_slot (slot, a.queue_row)], make_entry (a.epoch, layer, child), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 
@@ -540,6 +555,42 @@ static bool lines_have_one_producer (const aspen_hip_layer_t *layers, uint32_t n
     return true;
 }
 
+// Average parallelism of the tile graph = total tile cost / cost of the longest dependency chain, with a
+// crude cost per tile (K slices of a contraction tile plus a constant for fetching and storing).  Workgroups
+// beyond it only wait, and those that wait next to a working one on the same compute unit are the ones
+// that get the next tile as likely as those on an idle unit: tiles then share a matrix pipeline while
+// other units sit idle, which stretches exactly the chains that bound a run with little parallelism.
+static double graph_parallelism (const aspen_hip_layer_t *layers, const uint32_t *ninst_layer, const uint32_t *child_off,
+    const uint32_t *child_idx, uint32_t num_ninst)
+{
+    if (num_ninst == 0) return 0.0;
+    float *dist = (float *)calloc (num_ninst, sizeof (float));
+    double total = 0.0, longest = 0.0;
+    bool ordered = true;
+    for (uint32_t t = 0; t < num_ninst && ordered; t++)
+    {
+        const aspen_hip_layer_t &L = layers[ninst_layer[t]];
+        float cost = 4.f;
+        if (L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER)
+        {
+            if (L.splits > 1) cost = t - L.ninst_start < L.tiles_m * L.tiles_n * L.splits ? 8.f + (float)L.kiters_per_split : 4.f;
+            else cost = 8.f + (float)(L.Kp / GEMM_BK);
+        }
+        else if (L.type == K_ATTENTION_LAYER || L.type == V_ATTENTION_LAYER) cost = 16.f;
+        dist[t] += cost;
+        total += cost;
+        if (dist[t] > longest) longest = dist[t];
+        for (uint32_t e = child_off[t]; e < child_off[t + 1]; e++)
+        {
+            const uint32_t c = child_idx[e];
+            if (c <= t) { ordered = false; break; }       // not listed parents-first: no estimate
+            if (dist[c] < dist[t]) dist[c] = dist[t];
+        }
+    }
+    free (dist);
+    return ordered && longest > 0.0 ? total / longest : 1e30;
+}
+
 extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *layers, uint32_t num_layers,
     const uint32_t *ninst_layer, const uint32_t *num_parents, const uint32_t *child_off,
     const uint32_t *child_idx, uint32_t num_ninst, const uint32_t *roots, uint32_t num_roots)
@@ -563,6 +614,18 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     aspen_hip_graph_t *g = (aspen_hip_graph_t *)calloc (1, sizeof (aspen_hip_graph_t));
     g->cached_loads = lines_have_one_producer (layers, num_layers) && getenv ("ASPEN_GPU_COHERENT_LOADS") == nullptr;
     g->num_layers = num_layers; g->num_ninst = num_ninst; g->num_roots = num_roots; g->num_edges = num_edges;
+    {
+        // default grid: a whole number of workgroups per compute unit, no more than the graph can keep busy
+        const double par = graph_parallelism (layers, ninst_layer, child_off, child_idx, num_ninst);
+        uint32_t per_cu = (uint32_t)g_resident_wg;
+        // measured on 256 compute units (ResNet-50 batch 1 / 32, VGG-16, BERT, GPT-2): one more workgroup per
+        // unit pays once the average parallelism grows by another two tiles per unit
+        if (par < 2.0 * g_num_cu * g_resident_wg) per_cu = (uint32_t)(par / (2.0 * g_num_cu)) + 1;
+        if (per_cu > (uint32_t)g_resident_wg) per_cu = (uint32_t)g_resident_wg;
+        g->default_workgroups = per_cu * (uint32_t)g_num_cu;
+        if (getenv ("ASPEN_GPU_VERBOSE"))
+            fprintf (stderr, "aspen_hip: %u tiles, average parallelism %.0f: %u workgroups by default\n", num_ninst, par, g->default_workgroups);
+    }
     g->h_layers = (aspen_hip_layer_t *)malloc (sizeof (aspen_hip_layer_t) * num_layers);
     memcpy (g->h_layers, layers, sizeof (aspen_hip_layer_t) * num_layers);
     g->d_layers = upload (layers, num_layers);
@@ -572,7 +635,7 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     g->d_child_idx = upload (child_idx, num_edges);
     g->d_roots = upload (roots, num_roots);
     g->d_dep = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
-    g->d_queue = (qentry_t *)aspen_hip_alloc (sizeof (qentry_t) * (num_ninst + 1));
+    g->d_queue = (qentry_t *)aspen_hip_alloc (sizeof (qentry_t) * (size_t)QUEUE_LANES * queue_row (num_ninst));
     {
         // child records: what the publishing wavefront fetches with one 64-lane load
         qentry_t *rec = (qentry_t *)calloc ((size_t)(num_ninst ? num_ninst : 1) * CHILD_REC, sizeof (qentry_t));
@@ -644,10 +707,10 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
 {
     if (!g) { snprintf (g_err, sizeof (g_err), "run_dataflow: null graph"); return -1; }
     if (g->num_ninst == 0) return 0;
-    if (workgroups == 0) workgroups = (uint32_t)g_resident_wg * (uint32_t)g_num_cu;
+    if (workgroups == 0) workgroups = g->default_workgroups;
     g->epoch = g->epoch % 255u + 1u;
     hipLaunchKernelGGL (arm_kernel, dim3 ((g->num_ninst + 255) / 256), dim3 (256), 0, g_stream,
-        g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->d_ninst_layer, g->num_ninst, g->num_roots, g->d_state, g->epoch);
+        g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->d_ninst_layer, g->num_ninst, g->num_roots, g->d_state, g->epoch, queue_row (g->num_ninst));
     CHECK (hipGetLastError ());
     dataflow_args_t a;
     a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx; a.child_rec = g->d_child_rec;
@@ -658,7 +721,7 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
         if (!g->d_trace) return -1;
     }
     a.trace = g->d_trace;
-    a.num_ninst = g->num_ninst; a.epoch = g->epoch; a.flags = g_flags; a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
+    a.num_ninst = g->num_ninst; a.epoch = g->epoch; a.flags = g_flags; a.queue_row = queue_row (g->num_ninst); a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
     CHECK (hipEventRecord (g_events[NUM_EVENTS - 2], g_stream));
     if (g->cached_loads) hipLaunchKernelGGL (dataflow_kernel<2>, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);
     else hipLaunchKernelGGL (dataflow_kernel<1>, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);
