@@ -503,7 +503,9 @@ nasm_t *apu_create_transformer_nasm (aspen_dnn_t *dnn, unsigned int min_ninst_pe
    timing.  Without a GPU the default is returned as well. */
 #define DEFAULT_MIN_NINST 1536
 #include <time.h>
-static const unsigned int tuner_candidates[] = {DEFAULT_MIN_NINST, 1024, 2048, 768, 3072, 512, 256};
+/* large batches of vision nets like 1024-2048; transformers with a few hundred columns and batch 1 like
+   few, large tiles (128-384) on one workgroup per compute unit */
+static const unsigned int tuner_candidates[] = {DEFAULT_MIN_NINST, 384, 128, 768, 1024, 2048, 256, 512, 3072};
 
 static double test_nasm_time_sec (nasm_t *nasm, unsigned int iters)
 {

@@ -138,3 +138,44 @@ def tiny_case():
     tens = M.synth_weights(layers, 77, "he")
     x = M.synth_input(layers, 77, 2, 0, "embeddings")
     return cfg, layers, tens, x, 2, 0
+
+
+def export_example_model():
+    """A small PyTorch network with batch-norm after its convolutions, its cfg, and the state-dict
+    entries of its tensor-owning layers in cfg order (for aspen_amd.export.export_weights)."""
+    import torch
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv1 = torch.nn.Conv2d(3, 8, 3, padding=1, bias=False)
+            self.bn1 = torch.nn.BatchNorm2d(8)
+            self.conv2 = torch.nn.Conv2d(8, 16, 3, stride=2, padding=1, bias=True)
+            self.bn2 = torch.nn.BatchNorm2d(16)
+            self.conv3 = torch.nn.Conv2d(16, 64, 1, bias=True)
+            self.fc1 = torch.nn.Linear(64 * 4 * 4, 32)
+            self.fc2 = torch.nn.Linear(32, 10)
+
+        def forward(self, x):
+            x = torch.relu(self.bn1(self.conv1(x)))
+            x = torch.nn.functional.max_pool2d(x, 2, 2)
+            x = torch.nn.functional.leaky_relu(self.bn2(self.conv2(x)), 0.1)
+            x = torch.relu(self.conv3(x))
+            x = torch.relu(self.fc1(torch.flatten(x, 1)))
+            return self.fc2(x)
+
+    torch.manual_seed(5)
+    net = Net()
+    for bn in (net.bn1, net.bn2):
+        bn.running_mean.uniform_(-0.5, 0.5); bn.running_var.uniform_(0.5, 2.0)
+        bn.weight.data.uniform_(0.5, 1.5); bn.bias.data.uniform_(-0.5, 0.5)
+    net.eval()
+    cfg = ("[net]\nheight=16\nwidth=16\nchannels=3\n\n"
+           "[convolutional]\nfilters=8\nsize=3\nstride=1\npad=1\nactivation=relu\n\n"
+           "[maxpool]\nsize=2\nstride=2\n\n"
+           "[convolutional]\nfilters=16\nsize=3\nstride=2\npad=1\nactivation=leaky\n\n"
+           "[convolutional]\nfilters=64\nsize=1\nstride=1\npad=0\nactivation=relu\n\n"
+           "[connected]\noutput=32\nactivation=relu\n\n"
+           "[connected]\noutput=10\nactivation=linear\n\n")
+    entries = [("conv1", "bn1"), ("conv2", "bn2"), "conv3", "fc1", "fc2"]
+    return net, cfg, entries

@@ -244,3 +244,28 @@ def test_yolo_result_gathers_all_heads(gpu):
         assert got.shape == want.shape and np.array_equal(got, want)
     finally:
         net.close()
+
+
+@pytest.mark.gpu
+def test_exported_pytorch_model_runs_like_pytorch(gpu, tmp_path):
+    """Migration path of the reference's custom example (examples/3. custom_example): a PyTorch model
+    exported by aspen_amd.export (batch-norm folded), its images written as the raw NCHW file that
+    rpool_add_nasm reads, run on the GPU: logits within 1e-4 of PyTorch's, same argmax."""
+    import torch
+    from aspen_amd import export
+    net, cfg, entries = H.export_example_model()
+    wp, ip = str(tmp_path / "w.bin"), str(tmp_path / "in.bin")
+    export.export_weights(wp, cfg, net.state_dict(), entries)
+    x = torch.rand(5, 3, 16, 16)
+    export.write_input_file(ip, x.numpy())
+    want = net(x).detach().numpy()
+    dnn = api.Dnn(cfg, wp)
+    nasm = api.Nasm(dnn, 5, 0, 64)
+    pool, dse = api.RPool(), api.DseGroup(1, api.MODE_DATAFLOW)
+    dse.set_rpool(pool)
+    api.lib().rpool_add_nasm(pool.h, nasm.h, ip.encode())
+    dse.run(); dse.wait(nasm); dse.stop()
+    got = nasm.result().reshape(5, -1)
+    assert H.rel_l2(got, want) <= H.REL_L2_TOL
+    assert (got.argmax(1) == want.argmax(1)).all()
+    dse.destroy(); pool.destroy(); nasm.destroy(); dnn.destroy()
