@@ -133,6 +133,37 @@ def yolo_mini_cfg(size=32, classes=3) -> str:
     return s
 
 
+def yolov3_cfg(size=416, classes=80) -> str:
+    """YOLO-v3: Darknet-53 backbone (1, 2, 8, 8, 4 residual blocks after the five stride-2 convolutions),
+    three detection heads at strides 32 / 16 / 8; the two finer heads take a 1x1-reduced branch of the
+    previous head, upsampled and appended to the backbone map of their scale.  Same section sequence as
+    the reference's files/yolov3/yolov3_aspen.cfg ([append] instead of darknet's route + upsample)."""
+    rows = 3 * (classes + 5)
+    anchors = "10,13,  16,30,  33,23,  30,61,  62,45,  59,119,  116,90,  156,198,  373,326"
+    s = f"[net]\nheight={size}\nwidth={size}\nchannels=3\n\n"
+    s += _conv(32, 3, 1, 1, "leaky")
+    n = 1                                   # sections so far after [net] = index of the next layer
+    scale_end = {}                          # filters -> index of the last backbone layer at that width
+    for f, blocks in ((64, 1), (128, 2), (256, 8), (512, 8), (1024, 4)):
+        s += _conv(f, 3, 2, 1, "leaky"); n += 1
+        for _ in range(blocks):
+            s += _conv(f // 2, 1, 1, 0, "leaky") + _conv(f, 3, 1, 1, "leaky")
+            s += "[shortcut]\nfrom=-3\nactivation=linear\n\n"
+            n += 3
+        scale_end[f] = n - 1
+    for head, (f, mask, stride) in enumerate(((512, "6,7,8", 32), (256, "3,4,5", 16), (128, "0,1,2", 8))):
+        if head > 0:
+            # branch from the fifth convolution of the previous head (4 sections back), reduced,
+            # upsampled twice and appended to the backbone map that has this head's resolution
+            s += _conv(f, 1, 1, 0, "leaky", parent=-4); n += 1
+            s += f"[append]\nstride=2\nparent=-1\nfrom={scale_end[2 * f] - n}\n\n"; n += 1
+        for _ in range(3):
+            s += _conv(f, 1, 1, 0, "leaky") + _conv(2 * f, 3, 1, 1, "leaky"); n += 2
+        s += _conv(rows, 1, 1, 0, "linear"); n += 1
+        s += f"[yolo]\nmask = {mask}\nstride = {stride}\nanchors = {anchors}\nclasses={classes}\nnum=9\n\n"; n += 1
+    return s
+
+
 def custom_cifar_cfg() -> str:
     """The small CIFAR-10 net of the reference's third example (conv5/pool/conv3/pool/3 FC)."""
     s = "[net]\nheight=32\nwidth=32\nchannels=3\n\n"
@@ -272,6 +303,7 @@ Tensor = Tuple[int, str, np.ndarray]  # (1-based weighted-layer index, "WEIGHT"/
 
 def synth_weights(layers: List[Dict], seed: int, style: str) -> List[Tensor]:
     """style "he": conv/FC ~ N(0, 2/fan_in), bias ~ N(0, 0.01^2) (stands in for folded BN);
+    style "yolo": the same with two damped kinds of convolution, see below;
     style "gpt": matmul W,b ~ N(0, 0.02^2), layernorm w = 1 + N(0, 0.02^2), b ~ N(0, 0.02^2)."""
     out: List[Tensor] = []
     widx = 0
@@ -296,8 +328,15 @@ def synth_weights(layers: List[Dict], seed: int, style: str) -> List[Tensor]:
         if t == "layernorm":
             w = normal(seed, tid, shp, 0.02, 1.0)
             b = normal(seed, tid + 1, shp, 0.02)
-        elif style == "he":
-            w = normal(seed, tid, shp, math.sqrt(2.0 / fan))
+        elif style in ("he", "yolo"):
+            gain = 1.0
+            if style == "yolo":
+                # 23 unnormalised residual additions would double the variance 23 times and the box decode
+                # exponentiates its input: damp the branch that closes a residual block and the
+                # convolution that feeds a detection layer
+                nxt = layers[L["idx"] + 1]["type"] if L["idx"] + 1 < len(layers) else None
+                gain = 0.3 if nxt == "residual" else (0.1 if nxt == "yolo" else 1.0)
+            w = normal(seed, tid, shp, gain * math.sqrt(2.0 / fan))
             b = normal(seed, tid + 1, (shp[0],), 0.01)
         elif style == "gpt":
             w = normal(seed, tid, shp, 0.02)
@@ -331,6 +370,8 @@ CONFIGS = {
     "vgg16_b32": (vgg16_cfg, "he", 32, 0, 202, None),
     "resnet50_b16": (resnet50_cfg, "he", 16, 0, 101, None),
     "vgg16_b16": (vgg16_cfg, "he", 16, 0, 202, None),
+    "yolov3_b1": (yolov3_cfg, "yolo", 1, 0, 505, None),
+    "yolov3_b8": (yolov3_cfg, "yolo", 8, 0, 505, None),
     "bert_base_b8_s128": (bert_cfg, "gpt", 8, 128, 303, "embeddings"),
     "gpt2_b4_s512": (gpt2_cfg, "gpt", 4, 512, 404, "token_ids"),
 }

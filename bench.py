@@ -44,6 +44,8 @@ WORKLOADS = {
     "co_resnet50_vgg16_b16": (["resnet50_b16", "vgg16_b16"], "img/s", 32, 1536),
     "bert_base_b8_s128": (["bert_base_b8_s128"], "tokens/s", 8 * 128, 128),
     "gpt2_b4_s512": (["gpt2_b4_s512"], "tokens/s", 4 * 512, 384),
+    "yolov3_b1": (["yolov3_b1"], "img/s", 1, 512),
+    "yolov3_b8": (["yolov3_b8"], "img/s", 8, 1536),
 }
 
 

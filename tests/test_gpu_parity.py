@@ -88,7 +88,7 @@ def test_engine_rearm_many_runs(gpu):
         net.close()
 
 
-FULL = ["resnet50_b1", "resnet50_b32", "vgg16_b32", "bert_base_b8_s128", "gpt2_b4_s512"]
+FULL = ["resnet50_b1", "resnet50_b32", "vgg16_b32", "bert_base_b8_s128", "gpt2_b4_s512", "yolov3_b1"]
 
 
 @pytest.mark.parametrize("name", FULL)
