@@ -36,6 +36,7 @@ struct aspen_hip_graph_t
     uint32_t *d_state;      // one counter per 128-byte line: [ST_HEAD] pop tickets, [ST_TAIL] push cursor, [ST_DONE] tiles done,
                             // [ST_ABORT] abort flag, [ST_TWICE] tiles executed more than once
     uint32_t *d_ran;        // per-tile execution count (sanity: every tile exactly once)
+    uint32_t *d_arrivals;   // split-K arrival counters, see run_tile
     uint32_t epoch;         // tag of the last run's queue entries, cycles 1..255
     unsigned long long *d_prof;
     uint32_t default_workgroups;    // grid of a dataflow run when the caller names none, see graph_parallelism
@@ -66,14 +67,14 @@ static int fail (hipError_t e, const char *what)
 
 // Per-layer launch: workgroup -> tile with contiguous tile ranges per XCD (workgroups are dealt to
 // the 8 XCDs round-robin), so tiles that share activation rows meet in the same L2.
-__global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) layer_kernel (const aspen_hip_layer_t *layers, uint32_t l, uint32_t first_tile)
+__global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) layer_kernel (const aspen_hip_layer_t *layers, uint32_t l, uint32_t first_tile, uint32_t *arrivals)
 {
     extern __shared__ __align__ (16) float smem[];
     const aspen_hip_layer_t &L = layers[l];
     const uint32_t nt = gridDim.x, bid = blockIdx.x;
     const uint32_t xcd = bid & 7, local = bid >> 3, chunk = nt >> 3, rem = nt & 7;
     const uint32_t t = first_tile + xcd * chunk + (xcd < rem ? xcd : rem) + local;
-    run_tile<0> (L, t, smem);
+    run_tile<0> (L, t, smem, [=] () { return arrivals; });
 }
 
 // Re-arm: counters back to the parent counts, queue seeded with the roots.  A queue entry is 64 bits:
@@ -102,7 +103,8 @@ static uint32_t queue_row (uint32_t num_ninst)
 }
 
 __global__ void arm_kernel (uint32_t *dep, const uint32_t *num_parents, qentry_t *queue, uint32_t *ran,
-    const uint32_t *roots, const uint32_t *ninst_layer, uint32_t num_ninst, uint32_t num_roots, uint32_t *state, uint32_t epoch, uint32_t qrow)
+    const uint32_t *roots, const uint32_t *ninst_layer, uint32_t num_ninst, uint32_t num_roots, uint32_t *state, uint32_t epoch, uint32_t qrow,
+    uint32_t *arrivals)
 {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < num_ninst)
@@ -111,6 +113,7 @@ __global__ void arm_kernel (uint32_t *dep, const uint32_t *num_parents, qentry_t
         if (i < num_roots)
             __hip_atomic_store (&queue[queue_slot (i, qrow)], make_entry (epoch, ninst_layer[roots[i]], roots[i]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store (&ran[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store (&arrivals[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (i == 0)
     {
@@ -129,6 +132,7 @@ struct dataflow_args_t
     const qentry_t *child_rec;      // [num_ninst][CHILD_REC]: [0] = number of children, then the first CHILD_REC-1 as (layer << 32 | tile)
     qentry_t *queue;
     uint32_t *dep, *state, *ran;
+    uint32_t *arrivals;             // per split-K group (at its first tile's index): slices that have finished, see run_tile
     uint32_t *host_abort;
     unsigned long long *trace;      // per-tile start / end time stamps when ASPEN_HIP_FLAG_TRACE is set
     unsigned long long *prof;       // 8 counters of summed 100 MHz ticks, see aspen_hip_dataflow_profile
@@ -174,6 +178,7 @@ struct sched_lds_t
 {
     dataflow_args_t a;
     uint32_t tile, layer;                // tile to run next (QUEUE_EMPTY: leave) and its layer
+    uint32_t complete;                   // 0: the tile just run was a split-K slice that did not finish its group
     // the descriptors of the last few layers this workgroup worked on: consecutive tiles mostly belong
     // to the same two or three layers, so most tiles find theirs here instead of fetching it from memory
     uint32_t desc_slot, desc_next, desc_id[DESC_CACHE];
@@ -228,7 +233,8 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
     {
         const unsigned long long tp = prof ? wall_clock64 () : 0;
         // publish: relaxed device-scope atomics on the children's counters, one child per lane
-        const uint32_t count = (uint32_t)__shfl (rec, 0, 64);
+        // a split-K slice that was not the last of its group leaves the children to the one that is
+        const uint32_t count = s_sched.complete ? (uint32_t)__shfl (rec, 0, 64) : 0u;
         if (lane >= 1 && lane <= count) release_child (a, (uint32_t)rec, (uint32_t)(rec >> 32));
         if (count > CHILD_REC - 1)
         {
@@ -313,11 +319,17 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
         // wavefront 0 requests this tile's child record now; it arrives while the tile runs
         if (threadIdx.x < CHILD_REC) rec = s_sched.a.child_rec[(size_t)id * CHILD_REC + threadIdx.x];
         if ((s_sched.a.flags & ASPEN_HIP_FLAG_TRACE) && threadIdx.x == 0) s_sched.a.trace[2 * (size_t)id] = wall_clock64 ();
+        const aspen_hip_layer_t *L = &s_sched.desc[__builtin_amdgcn_readfirstlane (s_sched.desc_slot)];
+        bool complete;
         if (!(s_sched.a.flags & ASPEN_HIP_FLAG_SKIP_TILES))
+            complete = run_tile<COH> (*L, id - L->ninst_start, smem, [] () { return s_sched.a.arrivals; });
+        else
         {
-            const aspen_hip_layer_t *L = &s_sched.desc[__builtin_amdgcn_readfirstlane (s_sched.desc_slot)];
-            run_tile<COH> (*L, id - L->ninst_start, smem);
+            // scheduler-only run: the split-K groups still elect the member that releases the children
+            const uint32_t splits = __builtin_amdgcn_readfirstlane (L->splits), t = id - __builtin_amdgcn_readfirstlane (L->ninst_start);
+            complete = splits <= 1 || splitk_arrived_last (&s_sched.a.arrivals[id - t % splits], splits, smem);
         }
+        if (threadIdx.x == 0) s_sched.complete = complete;      // read by schedule_step behind its barrier
     }
     if ((s_sched.a.flags & ASPEN_HIP_FLAG_PROFILE) && threadIdx.x == 0)
     {
@@ -472,7 +484,7 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
     if (!L.out || !L.in0) why = "missing buffers";
     else if (L.ld % 4 || L.ld0 % 4 || (L.in1 && L.ld1 % 4)) why = "strides must be multiples of 4 floats";
     else if (L.tiles_m == 0 || L.tiles_n == 0 || L.splits == 0
-        || L.num_ninst != L.tiles_m * L.tiles_n * (L.splits > 1 ? L.splits + 1 : 1)) why = "tile grid";
+        || L.num_ninst != L.tiles_m * L.tiles_n * L.splits) why = "tile grid";
     else if (L.splits > 1 && (!L.partial || L.kiters_per_split == 0 || (uint64_t)L.splits * L.kiters_per_split * GEMM_BK < L.Kp
         || !(L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER))) why = "split-K geometry";
     else if ((uint64_t)L.N * L.ld * 4 * L.splits >= 0xffffff00ull) why = "matrix larger than 4 GiB";
@@ -573,8 +585,7 @@ static double graph_parallelism (const aspen_hip_layer_t *layers, const uint32_t
         float cost = 4.f;
         if (L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER)
         {
-            if (L.splits > 1) cost = t - L.ninst_start < L.tiles_m * L.tiles_n * L.splits ? 8.f + (float)L.kiters_per_split : 4.f;
-            else cost = 8.f + (float)(L.Kp / GEMM_BK);
+            cost = 8.f + (float)(L.splits > 1 ? L.kiters_per_split : L.Kp / GEMM_BK);
         }
         else if (L.type == K_ATTENTION_LAYER || L.type == V_ATTENTION_LAYER) cost = 16.f;
         dist[t] += cost;
@@ -605,7 +616,20 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     {
         uint32_t *seen = (uint32_t *)calloc (num_ninst ? num_ninst : 1, sizeof (uint32_t));
         bool ok = true;
-        for (uint32_t e = 0; e < num_edges && ok; e++) { if (child_idx[e] >= num_ninst) ok = false; else seen[child_idx[e]]++; }
+        // the members of a split-K group carry the same child list and count as one parent
+        for (uint32_t t = 0; t < num_ninst && ok; t++)
+        {
+            if (ninst_layer[t] >= num_layers) { ok = false; break; }
+            const aspen_hip_layer_t &L = layers[ninst_layer[t]];
+            const uint32_t slice = L.splits > 1 ? (t - L.ninst_start) % L.splits : 0;
+            if (slice != 0 && child_off[t + 1] - child_off[t] != child_off[t - slice + 1] - child_off[t - slice]) ok = false;
+            for (uint32_t e = child_off[t]; e < child_off[t + 1] && ok; e++)
+            {
+                if (child_idx[e] >= num_ninst) ok = false;
+                else if (slice != 0) { if (child_idx[e] != child_idx[child_off[t - slice] + (e - child_off[t])]) ok = false; }
+                else seen[child_idx[e]]++;
+            }
+        }
         for (uint32_t i = 0; i < num_ninst && ok; i++) if (seen[i] != num_parents[i] || ninst_layer[i] >= num_layers) ok = false;
         for (uint32_t r = 0; r < num_roots && ok; r++) if (roots[r] >= num_ninst || num_parents[roots[r]] != 0) ok = false;
         free (seen);
@@ -651,9 +675,10 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     }
     g->d_ran = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
     g->d_state = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * ST_WORDS);
+    g->d_arrivals = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
     g->d_prof = (unsigned long long *)aspen_hip_alloc (sizeof (unsigned long long) * 8);
     if (!g->d_layers || !g->d_ninst_layer || !g->d_num_parents || !g->d_child_off || !g->d_child_idx || !g->d_roots
-        || !g->d_dep || !g->d_queue || !g->d_ran || !g->d_state || !g->d_child_rec)
+        || !g->d_dep || !g->d_queue || !g->d_ran || !g->d_state || !g->d_child_rec || !g->d_arrivals)
     {
         aspen_hip_graph_destroy (g);
         return nullptr;
@@ -667,7 +692,7 @@ extern "C" void aspen_hip_graph_destroy (aspen_hip_graph_t *g)
     (void)hipStreamSynchronize (g_stream);
     aspen_hip_free (g->d_layers); aspen_hip_free (g->d_ninst_layer); aspen_hip_free (g->d_num_parents);
     aspen_hip_free (g->d_child_off); aspen_hip_free (g->d_child_idx); aspen_hip_free (g->d_roots);
-    aspen_hip_free (g->d_child_rec); aspen_hip_free (g->d_dep); aspen_hip_free (g->d_queue); aspen_hip_free (g->d_ran); aspen_hip_free (g->d_state); aspen_hip_free (g->d_prof); aspen_hip_free (g->d_trace);
+    aspen_hip_free (g->d_child_rec); aspen_hip_free (g->d_dep); aspen_hip_free (g->d_queue); aspen_hip_free (g->d_ran); aspen_hip_free (g->d_arrivals); aspen_hip_free (g->d_state); aspen_hip_free (g->d_prof); aspen_hip_free (g->d_trace);
     free (g->h_layers);
     free (g);
 }
@@ -675,19 +700,12 @@ extern "C" void aspen_hip_graph_destroy (aspen_hip_graph_t *g)
 // ------------------------------------------------------------------------------------------------
 // execution
 // ------------------------------------------------------------------------------------------------
-// One layer in launch mode; a split-K layer needs its partial tiles finished before the finishing
-// tiles start, hence two launches.
+// One layer in launch mode (split-K needs no second launch: the slice of a group that finishes last
+// adds the group's partial sums up).
 static void launch_layer (const aspen_hip_graph_t *g, uint32_t l)
 {
     const aspen_hip_layer_t &L = g->h_layers[l];
-    if (L.splits > 1)
-    {
-        const uint32_t T = L.tiles_m * L.tiles_n;
-        hipLaunchKernelGGL (layer_kernel, dim3 (T * L.splits), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, g->d_layers, l, 0u);
-        hipLaunchKernelGGL (layer_kernel, dim3 (T), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, g->d_layers, l, T * L.splits);
-    }
-    else
-        hipLaunchKernelGGL (layer_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, g->d_layers, l, 0u);
+    hipLaunchKernelGGL (layer_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, g->d_layers, l, 0u, g->d_arrivals);
 }
 
 extern "C" int aspen_hip_run_layers (aspen_hip_graph_t *g, uint32_t first_layer, uint32_t last_layer)
@@ -710,11 +728,11 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     if (workgroups == 0) workgroups = g->default_workgroups;
     g->epoch = g->epoch % 255u + 1u;
     hipLaunchKernelGGL (arm_kernel, dim3 ((g->num_ninst + 255) / 256), dim3 (256), 0, g_stream,
-        g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->d_ninst_layer, g->num_ninst, g->num_roots, g->d_state, g->epoch, queue_row (g->num_ninst));
+        g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->d_ninst_layer, g->num_ninst, g->num_roots, g->d_state, g->epoch, queue_row (g->num_ninst), g->d_arrivals);
     CHECK (hipGetLastError ());
     dataflow_args_t a;
     a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx; a.child_rec = g->d_child_rec;
-    a.dep = g->d_dep; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran; a.prof = g->d_prof; a.host_abort = g_host_abort;
+    a.dep = g->d_dep; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran; a.arrivals = g->d_arrivals; a.prof = g->d_prof; a.host_abort = g_host_abort;
     if ((g_flags & ASPEN_HIP_FLAG_TRACE) && !g->d_trace)
     {
         g->d_trace = (unsigned long long *)aspen_hip_alloc (sizeof (unsigned long long) * 2 * (size_t)g->num_ninst);
@@ -835,7 +853,7 @@ extern "C" int aspen_hip_sgemm (uint32_t M, uint32_t N, uint32_t K, const float 
     L.K = K; L.Kp = K; L.ld0 = ldb; L.out = C; L.in0 = B; L.weight = Ap; L.bias = bias;
     aspen_hip_layer_t *dL = upload (&L, 1);
     if (!dL) { aspen_hip_free (Ap); return -1; }
-    hipLaunchKernelGGL (layer_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, dL, 0u, 0u);
+    hipLaunchKernelGGL (layer_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, dL, 0u, 0u, (uint32_t *)nullptr);      // no split-K: the arrival counters are not touched
     hipError_t e = hipGetLastError ();
     if (e == hipSuccess) e = hipStreamSynchronize (g_stream);
     aspen_hip_free (dL); aspen_hip_free (Ap);

@@ -559,7 +559,7 @@ __device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L
     __syncthreads ();
 }
 
-// split-K finishing tile: sum of the slices + bias, activation
+// split-K, run by the slice that finishes last: sum of the slices (in slice order, whoever runs it) + bias, activation
 template <int COH>
 __device__ __forceinline__ void tile_splitk_finish (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm)
 {
@@ -904,23 +904,38 @@ __device__ __forceinline__ aspen_hip_layer_t uniform_layer (const aspen_hip_laye
     return L;
 }
 
-template <int COH>
-__device__ __forceinline__ void run_tile (const aspen_hip_layer_t &Lg, uint32_t t, float *smem)
+// Counts this workgroup's arrival in its split-K group; true for the last of the `splits` members.  The
+// group's (write-through) stores must have been acknowledged before an arrival is counted: the last
+// one reads them.  The counter only ever grows by `splits` per run, so it needs no reset between runs.
+__device__ __forceinline__ bool splitk_arrived_last (uint32_t *counter, uint32_t splits, float *smem)
+{
+    asm volatile ("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads ();
+    uint32_t *flag = reinterpret_cast<uint32_t *> (smem);
+    if (tile_thread () == 0)
+        *flag = __hip_atomic_fetch_add (counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads ();
+    const uint32_t before = __builtin_amdgcn_readfirstlane (*flag);
+    __syncthreads ();                       // the flag's word is LDS the next tile reuses
+    return before % splits == splits - 1;
+}
+
+// Runs tile t of the layer.  `arrivals ()` yields the graph's array of zero-initialised counters, one per
+// tile (used at the index of a split-K group's first tile); it is a callable so that the pointer is
+// fetched where it is needed instead of occupying registers while the tile runs.  Returns false for
+// a split-K partial tile that was not the last of its group to finish: the output tile is not
+// complete yet and nothing may be released.
+template <int COH, class Arrivals>
+__device__ __forceinline__ bool run_tile (const aspen_hip_layer_t &Lg, uint32_t t, float *smem, Arrivals arrivals)
 {
     const aspen_hip_layer_t L = uniform_layer (Lg);
     t = __builtin_amdgcn_readfirstlane (t);
     int slice = -1;
+    uint32_t group = 0;
     if (L.splits > 1)
     {
-        const uint32_t T = L.tiles_m * L.tiles_n;
-        if (t >= T * L.splits)
-        {
-            t -= T * L.splits;
-            const uint32_t fn = t / L.tiles_m;
-            tile_splitk_finish<COH> (L, fn, t - fn * L.tiles_m);
-            return;
-        }
         slice = (int)(t % L.splits);
+        group = L.ninst_start + t - (uint32_t)slice;
         t /= L.splits;
     }
     const uint32_t tn = t / L.tiles_m, tm = t - tn * L.tiles_m;
@@ -934,6 +949,12 @@ __device__ __forceinline__ void run_tile (const aspen_hip_layer_t &Lg, uint32_t 
         else { contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, COH> (L, tn, tm, slice, smem); c4_log2 = 4; bn = VAR2_BN; }
         static_assert (VAR0_BM == 128 && VAR1_BM == 64 && VAR2_BM == 64, "c4_log2 above");
         contraction_epilogue<COH> (L, tn, tm, slice, smem, c4_log2, bn);
+        if (slice >= 0)
+        {
+            // split-K: every slice has written its partial sums; whoever arrives last adds them up
+            if (!splitk_arrived_last (arrivals () + group, L.splits, smem)) return false;
+            tile_splitk_finish<COH> (L, tn, tm);
+        }
         break;
     }
     case RESIDUAL_LAYER:    tile_residual<COH> (L, tn); break;
@@ -947,4 +968,5 @@ __device__ __forceinline__ void run_tile (const aspen_hip_layer_t &Lg, uint32_t 
     case V_ATTENTION_LAYER: tile_v_attention<COH> (L, tn, tm, smem); break;
     default: break;
     }
+    return true;
 }

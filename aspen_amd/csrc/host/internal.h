@@ -64,8 +64,8 @@ struct nasm_ldata_t
     unsigned int tiles_w, tiles_h;
     unsigned int num_ninst, ninst_start;
     /* split-K: a contraction layer with too few output tiles cuts its K axis into `splits` slices;
-       tile indices [0, T*splits) (T = tiles_w*tiles_h) are partial products (tile*splits + slice),
-       [T*splits, T*splits + T) the finishing tiles that sum the slices, add bias, activate */
+       the T*splits tiles (T = tiles_w*tiles_h; index tile*splits + slice) each write one partial product,
+       and the one of a group that finishes last sums the slices, adds the bias and activates */
     unsigned int splits, kiters_per_split;
     size_t partial_offset;                   /* floats into the arena: [splits][columns][stride] */
     int variant;

@@ -167,7 +167,7 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
             unsigned int s = umin (umin (cdiv (want, T), kiters / umax (min_kiters, 1)), umax (max_splits, 1));
             ld->kiters_per_split = cdiv (kiters, s);
             ld->splits = cdiv (kiters, ld->kiters_per_split);
-            if (ld->splits > 1) ld->num_ninst = T * ld->splits + T;
+            if (ld->splits > 1) ld->num_ninst = T * ld->splits;
         }
     }
     return 0;
@@ -190,11 +190,7 @@ static unsigned int col_tile_of (const nasm_ldata_t *ld, unsigned int col)
 
 static void tile_range (const nasm_ldata_t *ld, unsigned int t, unsigned int *c0, unsigned int *c1, unsigned int *r0, unsigned int *r1)
 {
-    if (ld->splits > 1)
-    {
-        const unsigned int T = ld->tiles_h * ld->tiles_w;
-        t = t < T * ld->splits ? t / ld->splits : t - T * ld->splits;
-    }
+    if (ld->splits > 1) t /= ld->splits;
     const unsigned int tn = t / ld->tiles_h, tm = t % ld->tiles_h;      /* row tile fastest (reference src/apu_nasm.c:1218-1224) */
     const unsigned int S = seq_block (ld), tw = ld->tile_dims[OUT_W];
     if (S == 0) { *c0 = tn * tw; *c1 = umin (*c0 + tw, ld->out_mat_dims[OUT_W]); }
@@ -228,7 +224,7 @@ static void add_parents (const nasm_ldata_t *pl, unsigned int c0, unsigned int c
     const unsigned int m0 = r0 / pl->tile_dims[OUT_H], m1 = (r1 - 1) / pl->tile_dims[OUT_H];
     for (unsigned int t = t0; t <= t1; t++)
         for (unsigned int m = m0; m <= m1; m++)
-            push (out, pl->ninst_start + (pl->splits > 1 ? pl->tiles_h * pl->tiles_w * pl->splits : 0) + t * pl->tiles_h + m);
+            push (out, pl->ninst_start + (t * pl->tiles_h + m) * pl->splits);   /* split layer: slice 0 stands for the group */
 }
 
 /* parents of tile t of layer ld (semantics: reference src/apu_nasm.c:49-466) */
@@ -241,24 +237,18 @@ static void find_parents (const nasm_t *nasm, const nasm_ldata_t *ld, unsigned i
     unsigned int c0, c1, r0, r1;
     tile_range (ld, t, &c0, &c1, &r0, &r1);
     const unsigned int S = nasm->tr_seq_len;
-    /* the tile that runs the epilogue of a layer with a fused shortcut also reads the shortcut's other operand */
-    const int epilogue_tile = ld->splits == 1 || t >= ld->tiles_h * ld->tiles_w * ld->splits;
-    if (ld->fused_residual >= 0 && epilogue_tile)
+    /* the tile that runs the epilogue of a layer with a fused shortcut also reads the shortcut's other
+       operand; in a split layer that is whichever slice finishes last, so all of them wait for it */
+    if (ld->fused_residual >= 0)
     {
         const nasm_ldata_t *res = &nasm->ldata_arr[ld->fused_residual];
         add_parents (&nasm->ldata_arr[res->parent_ldata_idx[PARENT_1]], c0, c1, r0, r1, out);
-    }
-    if (ld->splits > 1 && t >= ld->tiles_h * ld->tiles_w * ld->splits)
-    {
-        const unsigned int tile = t - ld->tiles_h * ld->tiles_w * ld->splits;
-        for (unsigned int s = 0; s < ld->splits; s++) push (out, ld->ninst_start + tile * ld->splits + s);
-        return;
     }
     /* A split-K partial tile of a pointwise layer (matmul, 1x1 convolution: the K index IS the parent's
        row index) reads only the parent rows of its K slice, so it waits only for the parent tiles
        holding those rows: fewer edges, and it can start before the rest of the parent is done. */
     unsigned int k_row0 = 0, k_row1 = p0 ? p0->out_mat_dims[OUT_H] : 0;
-    if (ld->splits > 1 && !epilogue_tile
+    if (ld->splits > 1
         && (L->type == MATMUL_LAYER || (L->type == CONV_LAYER && p[WEIGHT_H] == 1 && p[WEIGHT_W] == 1)))
     {
         const unsigned int slice = t % ld->splits;
@@ -386,9 +376,16 @@ static int build_graph (nasm_t *nasm)
                 if (tmp.v[i] == prev) continue;         /* the two parents of a shortcut may be the same tile */
                 prev = tmp.v[i];
                 if (prev >= id) { ERROR_PRTF ("tile %u depends on a later tile %u\n", id, prev); return -1; }
-                push (&edges_parent, prev); push (&edges_child, id);
+                /* A parent in a split layer stands for its group of `splits` partial tiles: the member
+                   that finishes last completes the output and releases the children, so every member
+                   carries the child list and the child counts the group once. */
+                const unsigned int members = nasm->ldata_arr[nasm->ninst_ldata[prev]].splits;
+                for (unsigned int s = 0; s < members; s++)
+                {
+                    push (&edges_parent, prev + s); push (&edges_child, id);
+                    nasm->child_off[prev + s + 1]++;
+                }
                 nasm->num_parents[id]++;
-                nasm->child_off[prev + 1]++;
             }
         }
     }

@@ -65,9 +65,11 @@ typedef struct aspen_hip_layer_t
     uint32_t ld0, ld1;       /* strides of the parents */
     uint32_t IH, IW, IC, OH, OW, KH, KW, stride, pad;
     uint32_t heads, seq, hd, masked;
-    /* split-K (contraction layers): tiles [0, T*splits) with T = tiles_m*tiles_n are partial products
-       over kiters_per_split K slices each (tile*splits + slice) written to `partial`
-       ([splits][N][ld]); tiles [T*splits, T*splits + T) sum the slices, add bias, activate */
+    /* split-K (contraction layers): the layer has T*splits tiles, T = tiles_m*tiles_n; tile
+       (tile*splits + slice) computes the partial products over kiters_per_split K slices and writes
+       them to `partial` ([splits][N][ld]).  The `splits` tiles of one output tile form a group: the
+       member that finishes last (an arrival counter decides) sums the slices in slice order, adds
+       the bias, activates and writes the output; only it releases the group's children */
     uint32_t splits, kiters_per_split;
     uint32_t reserved;
     float *partial;
@@ -110,7 +112,9 @@ int aspen_hip_copy (void *dst, const void *src, size_t bytes);
 /* ---- graph ----------------------------------------------------------------------------------- */
 /* Uploads a tile graph.  ninst_layer[i] = layer of tile i; num_parents[i] = its dependency count;
    children of tile i are child_idx[child_off[i] .. child_off[i+1]).  roots = tiles with no parent
-   left once the input layer counts as complete.  (reference: ninst_t, include/nasm.h:50-66) */
+   left once the input layer counts as complete.  The members of a split-K group (see
+   aspen_hip_layer_t.splits) all carry the same child list, and a child counts the whole group as
+   ONE parent: whichever member finishes last releases it.  (reference: ninst_t, include/nasm.h:50-66) */
 aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *layers, uint32_t num_layers,
     const uint32_t *ninst_layer, const uint32_t *num_parents, const uint32_t *child_off,
     const uint32_t *child_idx, uint32_t num_ninst, const uint32_t *roots, uint32_t num_roots);

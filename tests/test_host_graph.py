@@ -139,8 +139,9 @@ def test_tile_graph_against_brute_force(name, min_ninst, fuse, monkeypatch):
         assert layers[res]["type"] == "residual" and layers[res]["p0"] == prod and layers[prod]["type"] in ("conv", "fc", "matmul")
         # the producer feeds nothing but the shortcut
         assert [l for l, L in enumerate(layers) if prod in (L["p0"], L["p1"])] == [res]
-    # ---- tiles partition every out_mat; split-K layers have splits*T partial tiles + T finishing tiles
-    owner, partial_of = [], {}
+    # ---- tiles partition every out_mat; in a split-K layer the `splits` partial tiles of an output tile
+    #      form a group (same range): its first member stands for the group as a parent
+    owner, group_of = [], {}
     for l, i in enumerate(infos):
         own = -np.ones((i["W"], i["H"]), dtype=np.int64)
         tiles = [t for t in range(i["ninst_start"], i["ninst_start"] + i["num_ninst"])]
@@ -151,9 +152,12 @@ def test_tile_graph_against_brute_force(name, min_ninst, fuse, monkeypatch):
         for (c0, c1, r0, r1), ts in ranges.items():
             assert 0 <= c0 < c1 <= i["W"] and 0 <= r0 < r1 <= i["H"]
             assert (own[c0:c1, r0:r1] == -1).all(), (name, l, "tiles overlap")
-            own[c0:c1, r0:r1] = max(ts)            # the finishing tile has the highest index
+            own[c0:c1, r0:r1] = min(ts)            # the group's first member owns the region
+            assert len(ts) == i["splits"] and sorted(ts) == list(range(min(ts), min(ts) + len(ts)))
             if len(ts) > 1:
-                partial_of[max(ts)] = sorted(ts)[:-1]
+                assert (min(ts) - i["ninst_start"]) % i["splits"] == 0
+                for t in ts:
+                    group_of[t] = min(ts)
         if i["num_ninst"]:
             assert (own >= 0).all(), (name, l, "tiles leave a gap")
         if i["fused_into"] >= 0:
@@ -163,14 +167,18 @@ def test_tile_graph_against_brute_force(name, min_ninst, fuse, monkeypatch):
     # ---- parents from the CSR children lists
     parents = [set() for _ in range(T)]
     for t in range(T):
+        rep = group_of.get(t, t)
+        if rep != t:
+            # every member of a group carries the group's child list; the child counts the group once
+            assert list(idx[off[t]:off[t + 1]]) == list(idx[off[rep]:off[rep + 1]])
+            continue
         for c in idx[off[t]:off[t + 1]]:
-            assert tl[c] > tl[t] or (tl[c] == tl[t] and c > t)      # edges point forward
+            assert tl[c] > tl[t]                                     # edges point forward
             assert t not in parents[c]                               # no duplicate edges
             parents[c].add(t)
     assert [len(p) for p in parents] == list(npar)
     # ---- every tile's parents = owners of every element it reads
-    finals = {f for f in partial_of}
-    partials = {p: f for f, ps in partial_of.items() for p in ps}
+    partials = group_of
     for t in range(T):
         l = int(tl[t])
         L = layers[l]
@@ -178,13 +186,10 @@ def test_tile_graph_against_brute_force(name, min_ninst, fuse, monkeypatch):
         produced = lambda pp: infos[pp]["num_ninst"] > 0 or infos[pp]["fused_into"] >= 0
         # the tile that runs a fused epilogue also reads the shortcut's other operand
         shortcut_need = set()
-        if l in fused_res and (t in finals or t not in partials):
+        if l in fused_res:            # any member of a split-K group may be the one that runs the epilogue
             other = layers[fused_res[l]]["p1"]
             if produced(other):
                 shortcut_need = {int(v) for v in np.unique(owner[other][c0:c1, r0:r1])}
-        if t in finals:
-            assert parents[t] == set(partial_of[t]) | shortcut_need, (name, l, t)
-            continue
         need = set(shortcut_need)
         regions = needed_regions(L, layers, c0, c1, r0, r1, batch, seq)
         pointwise = L["type"] == "matmul" or (L["type"] == "conv" and L["size"] == 1)
@@ -233,15 +238,22 @@ def test_tile_graph_against_brute_force(name, min_ninst, fuse, monkeypatch):
                 assert parents[t] <= hull | shortcut_need, (name, l, t)
         else:
             assert parents[t] == need, (name, l, t, L["type"], sorted(parents[t]), sorted(need))
-    # ---- executing by the counters runs every tile exactly once (what the device engine does)
+    # ---- executing by the counters runs every tile exactly once (what the device engine does: the
+    #      member of a split-K group that arrives last releases the group's children)
     cnt = npar.copy().astype(np.int64)
     ready = [t for t in range(T) if cnt[t] == 0]
-    ran = 0
+    ran, arrived = 0, {}
     while ready:
         t = ready.pop()
         ran += 1
+        if t in group_of:
+            g = group_of[t]
+            arrived[g] = arrived.get(g, 0) + 1
+            if arrived[g] < infos[int(tl[t])]["splits"]:
+                continue
         for c in idx[off[t]:off[t + 1]]:
             cnt[c] -= 1
+            assert cnt[c] >= 0
             if cnt[c] == 0:
                 ready.append(int(c))
     assert ran == T and (cnt == 0).all()
