@@ -503,6 +503,7 @@ __device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L
             else { b.x = L.bias[m0 + c]; if (c + 1 < mrem) b.y = L.bias[m0 + c + 1]; if (c + 2 < mrem) b.z = L.bias[m0 + c + 2]; }
         }
         const bool fuse = L.fuse_out != nullptr && slice < 0;
+        const bool keep = !(fuse && L.fuse_discard);        // the pre-shortcut sums are stored unless the host has no use for them
         ActView<COH> fin, fout;
         if (fuse) { fin.init (L.fuse_in, L.N, L.fuse_ld_in); fout.init (L.fuse_out, L.N, L.ld); }
         const uint32_t STEP = WG_THREADS >> c4_log2;
@@ -535,7 +536,7 @@ __device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L
                         y.x += b.x; y.y += b.y; y.z += b.z; y.w += b.w;
                         y = act4 (y, act);
                         const uint32_t o = (n0 + r) * L.ld + m0 + c;
-                        out.st4 (o, y);
+                        if (keep) out.st4 (o, y);
                         if (fuse)
                         {
                             y.x += s[u].x; y.y += s[u].y; y.z += s[u].z; y.w += s[u].w;
@@ -552,7 +553,7 @@ __device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L
                 v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
                 v = act4 (v, act);
                 const uint32_t o = (n0 + r) * L.ld + m0 + c;
-                out.st1 (o, v.x); if (c + 1 < mrem) out.st1 (o + 1, v.y); if (c + 2 < mrem) out.st1 (o + 2, v.z);
+                if (keep) { out.st1 (o, v.x); if (c + 1 < mrem) out.st1 (o + 1, v.y); if (c + 2 < mrem) out.st1 (o + 2, v.z); }
                 if (fuse) fused_shortcut<COH> (L, fin, fout, v, n0 + r, m0 + c, mrem - c);
             }
     }
@@ -567,7 +568,7 @@ __device__ __forceinline__ void tile_splitk_finish (const aspen_hip_layer_t &L, 
     const uint32_t rows = min (L.tile_n, L.N - n0), mrem = L.M - m0;
     ActView<COH> part, out, fin, fout;
     part.init (L.partial, L.N * L.splits, L.ld); out.init (L.out, L.N, L.ld);
-    const bool fuse = L.fuse_out != nullptr;
+    const bool fuse = L.fuse_out != nullptr, keep = !(fuse && L.fuse_discard);
     if (fuse) { fin.init (L.fuse_in, L.N, L.fuse_ld_in); fout.init (L.fuse_out, L.N, L.ld); }
     for (uint32_t idx = tile_thread (); idx < rows * C4; idx += WG_THREADS)
     {
@@ -588,7 +589,8 @@ __device__ __forceinline__ void tile_splitk_finish (const aspen_hip_layer_t &L, 
         }
         v = act4 (v, L.act);
         const uint32_t o = (n0 + r) * L.ld + m0 + c;
-        if (c + 4 <= mrem) out.st4 (o, v);
+        if (!keep) { }
+        else if (c + 4 <= mrem) out.st4 (o, v);
         else { out.st1 (o, v.x); if (c + 1 < mrem) out.st1 (o + 1, v.y); if (c + 2 < mrem) out.st1 (o + 2, v.z); }
         if (fuse) fused_shortcut<COH> (L, fin, fout, v, n0 + r, m0 + c, mrem - c);
     }

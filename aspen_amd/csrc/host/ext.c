@@ -7,6 +7,18 @@ void aspen_nasm_tile_range_internal (const nasm_ldata_t *ld, unsigned int t, uns
 
 void aspen_dse_group_set_mode (dse_group_t *g, int mode) { if (g) g->mode = mode ? 1 : 0; }
 void aspen_dse_group_set_workgroups (dse_group_t *g, unsigned int w) { if (g) g->workgroups = w; }
+
+static int keep_layer_outputs = -1;          /* -1: not set yet, take the environment's word */
+void aspen_keep_layer_outputs (int keep) { keep_layer_outputs = keep ? 1 : 0; }
+int aspen_keep_layer_outputs_enabled (void)
+{
+    if (keep_layer_outputs < 0)
+    {
+        const char *e = getenv ("ASPEN_GPU_KEEP_LAYER_OUTPUTS");
+        keep_layer_outputs = e != NULL && atoi (e) != 0;
+    }
+    return keep_layer_outputs;
+}
 unsigned int aspen_nasm_num_ldata (nasm_t *n) { return n ? n->num_ldata : 0; }
 unsigned int aspen_nasm_num_ninst (nasm_t *n) { return n ? n->num_ninst : 0; }
 unsigned int aspen_nasm_num_edges (nasm_t *n) { return n ? n->num_edges : 0; }

@@ -63,6 +63,7 @@ struct nasm_ldata_t
     unsigned int tile_dims[2];
     unsigned int tiles_w, tiles_h;
     unsigned int num_ninst, ninst_start;
+    int out_discarded;                       /* fused producer whose own (pre-shortcut) matrix is not written */
     /* split-K: a contraction layer with too few output tiles cuts its K axis into `splits` slices;
        the T*splits tiles (T = tiles_w*tiles_h; index tile*splits + slice) each write one partial product,
        and the one of a group that finishes last sums the slices, adds the bias and activates */
@@ -128,5 +129,7 @@ unsigned int aspen_layer_kiters (const aspen_layer_t *layer);   /* K slices of 3
 int aspen_nasm_to_device (nasm_t *nasm);
 int aspen_nasm_fill_device_layers (nasm_t *nasm, aspen_hip_layer_t *dst, uint32_t ninst_base);
 unsigned int aspen_ld_for_rows (unsigned int rows);
+
+int aspen_keep_layer_outputs_enabled (void);   /* ext.c: see aspen_keep_layer_outputs */
 
 #endif

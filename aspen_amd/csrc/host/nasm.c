@@ -425,6 +425,9 @@ static void fuse_shortcuts (nasm_t *nasm)
         if (consumers != 1) continue;
         prod->fused_residual = (int)r;
         res->fused_into = i0;
+        /* nothing on the device reads the producer's own matrix any more; like the reference, which
+           frees a layer's matrix once its children are done (src/dse.c:84-92), it is not kept unless asked */
+        prod->out_discarded = !aspen_keep_layer_outputs_enabled ();
         res->num_ninst = 0; res->tiles_h = res->tiles_w = 0;
     }
 }
@@ -447,6 +450,7 @@ static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned i
         nasm_ldata_t *ld = &nasm->ldata_arr[l];
         ld->nasm = nasm; ld->layer = &dnn->layers[l];
         ld->fused_residual = ld->fused_into = -1;
+        ld->out_discarded = 0;
         for (int k = 0; k < NUM_PARENT_ELEMENTS; k++) ld->parent_ldata_idx[k] = ld->layer->parent_idx[k];
         if (set_out_mat (nasm, ld) || set_tiles (nasm, ld)) { bad = 1; break; }
         for (int k = PARENT_0; k <= PARENT_1; k++)
@@ -657,6 +661,7 @@ int aspen_nasm_fill_device_layers (nasm_t *nasm, aspen_hip_layer_t *dst, uint32_
             d->fuse_out = nasm->d_arena + res->out_mat_offset;
             d->fuse_in = nasm->d_arena + other->out_mat_offset; d->fuse_ld_in = other->out_mat_stride;
             d->fuse_act = res->layer->activation;
+            d->fuse_discard = ld->out_discarded;
         }
         if (L->type == K_ATTENTION_LAYER || L->type == V_ATTENTION_LAYER)
         {

@@ -323,6 +323,12 @@ static ssize_t get_ldata_output (nasm_t *nasm, unsigned int ldata_idx, LAYER_PAR
     if (nasm->completed == 2) finish (nasm->rpool);
     const nasm_ldata_t *ld = &nasm->ldata_arr[ldata_idx];
     const aspen_layer_t *L = ld->layer;
+    if (ld->out_discarded)
+    {
+        ERROR_PRTF ("Error in get_ldata_output: layer %u feeds only the shortcut computed in its own epilogue and its matrix was not kept "
+                    "(aspen_keep_layer_outputs (1) before creating the nasm keeps it).\n", ldata_idx);
+        return -1;
+    }
     const size_t H = ld->out_mat_dims[OUT_H], W = ld->out_mat_dims[OUT_W];
     float *dense = malloc (H * W * sizeof (float));
     if (dense == NULL) return -1;

@@ -18,6 +18,13 @@ void aspen_dse_group_set_mode (dse_group_t *dse_group, int mode);
 /* persistent workgroups of the dataflow kernel; 0 = two per compute unit */
 void aspen_dse_group_set_workgroups (dse_group_t *dse_group, unsigned int workgroups);
 
+/* Graphs created AFTER this call keep (1) or do not keep (0, the default) the matrix of a contraction
+   layer whose shortcut is computed in its own epilogue.  Nothing on the device reads that matrix, and
+   the reference frees a layer's matrix as soon as its children are done (src/dse.c:84-92), so by
+   default it is not written; dse_get_ldata_result on such a layer then reports an error.  The
+   environment variable ASPEN_GPU_KEEP_LAYER_OUTPUTS=1 sets the initial value. */
+void aspen_keep_layer_outputs (int keep);
+
 unsigned int aspen_nasm_num_ldata (nasm_t *nasm);
 unsigned int aspen_nasm_num_ninst (nasm_t *nasm);
 unsigned int aspen_nasm_num_edges (nasm_t *nasm);

@@ -71,7 +71,7 @@ typedef struct aspen_hip_layer_t
        member that finishes last (an arrival counter decides) sums the slices in slice order, adds
        the bias, activates and writes the output; only it releases the group's children */
     uint32_t splits, kiters_per_split;
-    uint32_t reserved;
+    uint32_t fuse_discard;   /* 1 (only with fuse_out): the layer's own, pre-shortcut matrix `out` is not written */
     float *partial;
     float *out;
     const float *in0;        /* PARENT_0 */

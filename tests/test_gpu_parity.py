@@ -269,3 +269,33 @@ def test_exported_pytorch_model_runs_like_pytorch(gpu, tmp_path):
     assert H.rel_l2(got, want) <= H.REL_L2_TOL
     assert (got.argmax(1) == want.argmax(1)).all()
     dse.destroy(); pool.destroy(); nasm.destroy(); dnn.destroy()
+
+
+@pytest.mark.gpu
+def test_default_discards_outputs_only_a_fused_shortcut_reads(gpu):
+    """Default setting (what bench.py times): a contraction layer whose shortcut runs in its own epilogue does
+    not write its pre-shortcut matrix.  Every other layer still matches the compiled reference's fixture,
+    and asking for the discarded one is an error, not stale data."""
+    name = "resnet_mini_b2"
+    case = H.micro_cases()[name]
+    cfg, layers, tens, x, batch, seq = H.build_case(case)
+    gold = np.load(os.path.join(H.GOLDEN, f"micro_{name}.npz"))
+    api.lib().aspen_keep_layer_outputs(0)
+    try:
+        for min_ninst in (64, 1024):          # without and with split-K
+            net = H.GpuNet(cfg, tens, batch, seq, min_ninst=min_ninst)
+            try:
+                net.run(x)
+                infos = [net.nasm.info(l) for l in range(net.nasm.num_ldata)]
+                dropped = [l for l, i in enumerate(infos) if i["fused_residual"] >= 0]
+                assert dropped
+                for l in range(net.nasm.num_ldata):
+                    if l in dropped:
+                        with pytest.raises(RuntimeError):
+                            net.layer(l)
+                    else:
+                        assert H.rel_l2(net.layer(l), gold[f"layer{l}"]) <= H.REL_L2_TOL, l
+            finally:
+                net.close()
+    finally:
+        api.lib().aspen_keep_layer_outputs(1)
