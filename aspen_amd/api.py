@@ -27,7 +27,7 @@ LAYER_TYPE_NAMES = ["none", "input", "conv", "fc", "residual", "batchnorm", "yol
                     "maxpool", "avgpool", "route", "softmax", "matmul", "layernorm", "attn_k", "attn_v"]
 (NO_ACTIVATION, SIGMOID, LINEAR, TANH, RELU, LEAKY_RELU, ELU, SELU, GELU, GELU_ACCURATE) = range(10)
 
-MODE_LAYERS, MODE_DATAFLOW = 0, 1
+MODE_LAYERS, MODE_DATAFLOW, MODE_AUTO = 0, 1, 2
 
 _vp = C.c_void_p
 _fp = C.POINTER(C.c_float)
@@ -78,6 +78,7 @@ def lib() -> C.CDLL:
         "print_rpool_info": (None, [_vp]),
         # aspen_ext.h
         "aspen_dse_group_set_mode": (None, [_vp, C.c_int]),
+        "aspen_dse_group_last_mode": (C.c_int, [_vp]),
         "aspen_dse_group_set_workgroups": (None, [_vp, C.c_uint]),
         "aspen_keep_layer_outputs": (None, [C.c_int]),
         "aspen_nasm_num_ldata": (C.c_uint, [_vp]),
@@ -289,6 +290,10 @@ class DseGroup:
 
     def set_mode(self, mode: int):
         lib().aspen_dse_group_set_mode(self.h, mode)
+
+    def last_mode(self) -> int:
+        """The engine the last run() used: MODE_LAYERS or MODE_DATAFLOW (-1 before the first run)."""
+        return lib().aspen_dse_group_last_mode(self.h)
 
     def set_rpool(self, rpool: RPool):
         lib().dse_group_set_rpool(self.h, rpool.h)

@@ -40,6 +40,7 @@ struct aspen_hip_graph_t
     uint32_t epoch;         // tag of the last run's queue entries, cycles 1..255
     unsigned long long *d_prof;
     uint32_t default_workgroups;    // grid of a dataflow run when the caller names none, see graph_parallelism
+    double parallelism;             // average parallelism of the tile graph, see graph_parallelism
     int cached_loads;       // 1: no cache line of an activation is shared by two producer tiles
     unsigned long long *d_trace;    // [2*tile] start, [2*tile+1] end time stamps (allocated on first traced run)
 };
@@ -641,6 +642,7 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     {
         // default grid: a whole number of workgroups per compute unit, no more than the graph can keep busy
         const double par = graph_parallelism (layers, ninst_layer, child_off, child_idx, num_ninst);
+        g->parallelism = par;
         uint32_t per_cu = (uint32_t)g_resident_wg;
         // measured on 256 compute units (ResNet-50 batch 1 / 32, VGG-16, BERT, GPT-2): one more workgroup per
         // unit pays once the average parallelism grows by another two tiles per unit
@@ -747,6 +749,8 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     CHECK (hipEventRecord (g_events[NUM_EVENTS - 1], g_stream));
     return 0;
 }
+
+extern "C" double aspen_hip_graph_parallelism (const aspen_hip_graph_t *g) { return g ? g->parallelism : 0.0; }
 
 extern "C" int aspen_hip_profile_layers (aspen_hip_graph_t *g, uint32_t iters, float *ms_per_layer)
 {

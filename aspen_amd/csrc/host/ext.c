@@ -5,7 +5,8 @@
 unsigned int aspen_rpool_num_ninst (rpool_t *rp);
 void aspen_nasm_tile_range_internal (const nasm_ldata_t *ld, unsigned int t, unsigned int *r);
 
-void aspen_dse_group_set_mode (dse_group_t *g, int mode) { if (g) g->mode = mode ? 1 : 0; }
+void aspen_dse_group_set_mode (dse_group_t *g, int mode) { if (g) g->mode = mode < 0 || mode > 2 ? 2 : mode; }
+int aspen_dse_group_last_mode (dse_group_t *g) { return g ? g->last_mode : -1; }
 void aspen_dse_group_set_workgroups (dse_group_t *g, unsigned int w) { if (g) g->workgroups = w; }
 
 static int keep_layer_outputs = -1;          /* -1: not set yet, take the environment's word */

@@ -115,7 +115,8 @@ struct dse_group_t
 {
     unsigned int num_dses;
     rpool_t *rpool;
-    int mode;                                /* 0 = one launch per layer, 1 = persistent dataflow kernel */
+    int mode;                                /* 0 = one launch per layer, 1 = persistent dataflow kernel, 2 = chosen per graph */
+    int last_mode;                           /* what the last dse_group_run used (0 / 1) */
     unsigned int workgroups;
 };
 

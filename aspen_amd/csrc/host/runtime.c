@@ -187,13 +187,17 @@ static int rebuild_graph (rpool_t *rp)
 }
 
 /* ---- scheduling engines ------------------------------------------------------------------------ */
+#define AUTO_LAYERS_BELOW 128.0    /* measured: ResNet-50 batch 1 (parallelism ~90) 0.90 vs 1.03 ms; YOLO-v3 batch 1
+                                      (~330) and BERT-base 1024 tokens (~260) are faster on the persistent kernel */
 dse_group_t *dse_group_init (unsigned int num_dse)
 {
     dse_group_t *g = calloc (1, sizeof (dse_group_t));
     g->num_dses = num_dse;
-    g->mode = 1;
-    const char *m = getenv ("ASPEN_GPU_MODE");           /* "layers" = one launch per layer, "dataflow" = persistent kernel */
+    g->mode = 2;
+    g->last_mode = -1;
+    const char *m = getenv ("ASPEN_GPU_MODE");           /* "layers" = one launch per layer, "dataflow" = persistent kernel, "auto" */
     if (m != NULL && strcmp (m, "layers") == 0) g->mode = 0;
+    if (m != NULL && strcmp (m, "dataflow") == 0) g->mode = 1;
     const char *w = getenv ("ASPEN_GPU_WORKGROUPS");
     g->workgroups = w ? (unsigned int)atoi (w) : 0;
     return g;
@@ -227,7 +231,13 @@ void dse_group_run (dse_group_t *dse_group)
     if (rp->graph_dirty && rebuild_graph (rp)) { ERROR_PRTF ("ERROR: dse_group_run: graph upload failed: %s\n", aspen_hip_last_error ()); return; }
     if (rp->graph == NULL) return;
     int rc;
-    if (dse_group->mode == 0)
+    /* auto: the persistent kernel, unless the graph offers so little parallelism (one image through a deep
+       network: under half a tile per compute unit on average) that its per-tile scheduling latency costs
+       more than the launch gaps of one kernel per layer */
+    int mode = dse_group->mode;
+    if (mode == 2) mode = aspen_hip_graph_parallelism (rp->graph) < AUTO_LAYERS_BELOW ? 0 : 1;
+    dse_group->last_mode = mode;
+    if (mode == 0)
     {
         uint32_t layers = 0;
         for (unsigned int i = 0; i < rp->num_nasms; i++) layers += rp->nasms[i]->num_ldata;

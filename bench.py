@@ -105,7 +105,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="resnet50_b32", choices=list(WORKLOADS))
-    ap.add_argument("--mode", default="dataflow", choices=["dataflow", "layers"])
+    ap.add_argument("--mode", default="auto", choices=["auto", "dataflow", "layers"],
+                    help="auto (the library's default): persistent dataflow kernel unless the graph has too little parallelism for it")
     ap.add_argument("--min-ninst", type=int, default=0, help="tiles wanted per layer (0: the workload's tuned value)")
     ap.add_argument("--workgroups", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -149,7 +150,7 @@ def main():
         args.min_ninst = tuned_min_ninst
 
     pool = api.RPool()
-    dse = api.DseGroup(1, api.MODE_DATAFLOW if args.mode == "dataflow" else api.MODE_LAYERS, args.workgroups)
+    dse = api.DseGroup(1, {"auto": api.MODE_AUTO, "dataflow": api.MODE_DATAFLOW, "layers": api.MODE_LAYERS}[args.mode], args.workgroups)
     dse.set_rpool(pool)
     nets = []
     for name in cfgs:
@@ -179,6 +180,8 @@ def main():
     for _, _, n, _ in nets:
         dse.wait(n)
     dse.stop()
+    # what "auto" resolved to for this graph
+    args.mode = "dataflow" if dse.last_mode() == api.MODE_DATAFLOW else "layers"
     for _ in range(args.warmup):
         step()
     L.aspen_hip_sync()

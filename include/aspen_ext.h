@@ -12,9 +12,13 @@
 extern "C" {
 #endif
 
-/* 0: one kernel launch per layer (layer-synchronous); 1: persistent dataflow kernel (default).
-   The environment variable ASPEN_GPU_MODE=layers|dataflow sets the initial value. */
+/* 0: one kernel launch per layer (layer-synchronous); 1: persistent dataflow kernel; 2 (default): the
+   persistent kernel unless the graph's average parallelism is below half a tile per compute unit (a
+   single image through a deep network), where one launch per layer is faster.
+   The environment variable ASPEN_GPU_MODE=layers|dataflow|auto sets the initial value. */
 void aspen_dse_group_set_mode (dse_group_t *dse_group, int mode);
+/* the mode the last dse_group_run used: 0 or 1 (-1 before the first run) */
+int aspen_dse_group_last_mode (dse_group_t *dse_group);
 /* persistent workgroups of the dataflow kernel; 0 = two per compute unit */
 void aspen_dse_group_set_workgroups (dse_group_t *dse_group, unsigned int workgroups);
 

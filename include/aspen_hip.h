@@ -119,6 +119,11 @@ aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *layers, uint
     const uint32_t *ninst_layer, const uint32_t *num_parents, const uint32_t *child_off,
     const uint32_t *child_idx, uint32_t num_ninst, const uint32_t *roots, uint32_t num_roots);
 void aspen_hip_graph_destroy (aspen_hip_graph_t *graph);
+/* Average parallelism of the uploaded graph: summed tile cost over the cost of the longest dependency
+   chain (cost = K slices of a contraction tile plus a constant).  The default grid of a dataflow run
+   is sized from it; a host runtime can use it to prefer one launch per layer for graphs that could
+   never keep a persistent grid busy (a single image through a deep network). */
+double aspen_hip_graph_parallelism (const aspen_hip_graph_t *graph);
 
 /* ---- execution (all asynchronous on the library's stream) -------------------------------------- */
 /* One launch per layer, layers [first, last] in index order: the per-operator baseline and the
