@@ -770,14 +770,16 @@ __device__ __forceinline__ void tile_softmax (const aspen_hip_layer_t &L, uint32
 // ---------------------------------------------------------------------------------------------
 // Attention tiles.
 // K tile: one (batch, head) x KATTN_BN queries x all keys.  scores = K.Q on the matrix cores, 128 keys at
-// a time; causal mask (-1e10 before the 1/sqrt(hd) scale), exp without max subtraction and the row
-// sums are fused into the epilogue; a second sweep over the tile's own output divides by the sums.
+// a time; causal mask (-1e10 before the 1/sqrt(hd) scale), exp without max subtraction.  A first pass over
+// the key blocks accumulates every query's sum, a second recomputes the scores, divides and stores.
 // in0 = Query matrix, in1 = Key matrix (reference cfg: parent = Query, from = Key).
 // ---------------------------------------------------------------------------------------------
 template <int COH>
 __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, uint32_t tn, float *smem)
 {
     constexpr int BM = 128, BN = KATTN_BN, WM = 2, WN = 2, TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int TROW = BM + 8;            // staging row of one query: (4 * TROW) % 64 == 32, see the contraction epilogue
+    static_assert (BN * TROW <= GEMM_SMEM_FLOATS, "probability staging fits the GEMM stage");
     __shared__ float rowsum[BN];
     const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
     const uint32_t S = L.seq, qtiles = (S + BN - 1) / BN;
@@ -788,67 +790,98 @@ __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, ui
     Q.init (L.in0, L.N / L.heads, L.ld0); Kmat.init (L.in1, L.N / L.heads, L.ld1); out.init (L.out, L.N, L.ld);
     const uint32_t obase = bh * S * L.ld;                // column (b*H + h)*S + q, rows = keys
     const float scale = 1.0f / sqrtf ((float)L.hd);
-    if (tid < BN) rowsum[tid] = 0.f;
+    const uint32_t nq = min ((uint32_t)BN, S - q0);
+    // with the causal mask every key beyond the tile's last query is masked for all of its queries:
+    // exp (-1e10 * scale) is exactly 0, so those key blocks add nothing to the sums and are written as zeros
+    const uint32_t kend = L.masked ? min (S, q0 + (uint32_t)BN) : S;
+    const int kiters = (int)(L.hd / GEMM_BK);
+    if (tid < BN) rowsum[tid] = 0.f;                     // ordered before the atomics below by the barriers of gemm_core
+
+    // The scores are computed twice: the first pass only accumulates every query's sum of exponentials, the
+    // second recomputes them, normalises and stores.  Recomputing 2*hd flops per score is far cheaper than
+    // keeping S scores per query in registers or writing them out and reading them back.
+    auto scores = [&] (uint32_t k0, floatx16 (&acc)[TN][TM])
+    {
+        ActRowLoader<BM, COH> al; al.init (Kmat, b * S + k0, b * S + S - 1, L.ld1, h * L.hd, tid);
+        ActRowLoader<BN, COH> bl; bl.init (Q, b * S + q0, b * S + S - 1, L.ld0, h * L.hd, tid);
+        gemm_core<BM, BN, WM, WN> (al, bl, 0, kiters, smem, acc);
+    };
+    // exponential of one score; reference order of operations: mask with -1e10, scale, exp, no max subtraction
+    auto weight = [&] (float sc, uint32_t key, uint32_t q) -> float
+    {
+        if (L.masked && key > q) sc = -1e10f;
+        return (key < S && q < S) ? expf (sc * scale) : 0.f;
+    };
+
     float part[TN][16];
     #pragma unroll
     for (int i = 0; i < TN; i++)
         #pragma unroll
         for (int v = 0; v < 16; v++) part[i][v] = 0.f;
-
-    const int kiters = (int)(L.hd / GEMM_BK);
-    for (uint32_t k0 = 0; k0 < S; k0 += BM)
+    constexpr uint32_t C4 = BM / 4, STEP = WG_THREADS / C4;
+    const uint32_t c = (tid % C4) * 4;
+    const uint32_t blocks = (kend + BM - 1) / BM;
+    // one loop for both passes, so that the matrix code exists once
+    for (uint32_t step = 0; step < 2 * blocks; step++)
     {
-        floatx16 acc[TN][TM];
-        ActRowLoader<BM, COH> al; al.init (Kmat, b * S + k0, b * S + S - 1, L.ld1, h * L.hd, tid);
-        ActRowLoader<BN, COH> bl; bl.init (Q, b * S + q0, b * S + S - 1, L.ld0, h * L.hd, tid);
-        gemm_core<BM, BN, WM, WN> (al, bl, 0, kiters, smem, acc);
-        #pragma unroll
-        for (int j = 0; j < TM; j++)
+        const bool second = step >= blocks;
+        const uint32_t k0 = (second ? step - blocks : step) * BM;
+        if (step == blocks)
         {
-            const uint32_t key = k0 + wm0 + 32 * j + (lane & 31);
+            // row sums: 32 lanes of a half-wave hold 32 different keys of the same query
             #pragma unroll
             for (int i = 0; i < TN; i++)
                 #pragma unroll
                 for (int v = 0; v < 16; v++)
                 {
-                    const uint32_t q = q0 + ACC_N (wn0, i, v, lane);
-                    float s = acc[i][j][v];
-                    if (L.masked && key > q) s = -1e10f;
-                    const float e = expf (s * scale);
-                    if (key < S && q < S) { out.st1 (obase + q * L.ld + key, e); part[i][v] += e; }
+                    float t = part[i][v];
+                    #pragma unroll
+                    for (int o = 16; o > 0; o >>= 1) t += __shfl_xor (t, o, 64);
+                    if ((lane & 31) == 0) atomicAdd (&rowsum[ACC_N (wn0, i, v, lane)], t);
                 }
+            __syncthreads ();
         }
-    }
-    // row sums: 32 lanes of a half-wave hold 32 different keys of the same query
-    #pragma unroll
-    for (int i = 0; i < TN; i++)
-        #pragma unroll
-        for (int v = 0; v < 16; v++)
+        floatx16 acc[TN][TM];
+        scores (k0, acc);                                // ends with a barrier: the stage is free
+        if (!second)
         {
-            float s = part[i][v];
             #pragma unroll
-            for (int o = 16; o > 0; o >>= 1) s += __shfl_xor (s, o, 64);
-            if ((lane & 31) == 0) atomicAdd (&rowsum[ACC_N (wn0, i, v, lane)], s);
+            for (int j = 0; j < TM; j++)
+                #pragma unroll
+                for (int i = 0; i < TN; i++)
+                    #pragma unroll
+                    for (int v = 0; v < 16; v++)
+                        part[i][v] += weight (acc[i][j][v], k0 + wm0 + 32 * j + (lane & 31), q0 + ACC_N (wn0, i, v, lane));
+            continue;
         }
-    __syncthreads ();
-    const uint32_t nq = min ((uint32_t)BN, S - q0);
-    const uint32_t S4 = S >> 2;
-    if ((S & 3) == 0)
-        for (uint32_t i = tid; i < nq * S4; i += WG_THREADS)
+        #pragma unroll
+        for (int i = 0; i < TN; i++)
+            #pragma unroll
+            for (int v = 0; v < 16; v++)
+            {
+                const uint32_t ql = ACC_N (wn0, i, v, lane);
+                const float sum = rowsum[ql];
+                #pragma unroll
+                for (int j = 0; j < TM; j++)
+                    smem[ql * TROW + wm0 + 32 * j + (lane & 31)] = weight (acc[i][j][v], k0 + wm0 + 32 * j + (lane & 31), q0 + ql) / sum;
+            }
+        __syncthreads ();
+        for (uint32_t r = tid / C4; r < nq; r += STEP)
         {
-            const uint32_t r = i / S4, c = (i - r * S4) * 4;
-            const uint32_t o = obase + (q0 + r) * L.ld + c;
-            const float sum = rowsum[r];
-            float4 v = out.ld4 (o);
-            v.x /= sum; v.y /= sum; v.z /= sum; v.w /= sum;
-            out.st4 (o, v);
+            const float4 p = ld4 (smem + r * TROW + c);
+            const uint32_t key = k0 + c, o = obase + (q0 + r) * L.ld + key;
+            if (key + 4 <= S) out.st4 (o, p);
+            else if (key < S) { out.st1 (o, p.x); if (key + 1 < S) out.st1 (o + 1, p.y); if (key + 2 < S) out.st1 (o + 2, p.z); }
         }
-    else
-        for (uint32_t i = tid; i < nq * S; i += WG_THREADS)
+        __syncthreads ();                                // the next block's operands overwrite the stage
+    }
+    // key blocks that are masked for every query of the tile
+    for (uint32_t k0 = (kend + BM - 1) / BM * BM; k0 < S; k0 += BM)
+        for (uint32_t r = tid / C4; r < nq; r += STEP)
         {
-            const uint32_t r = i / S, c = i - r * S;
-            const uint32_t o = obase + (q0 + r) * L.ld + c;
-            out.st1 (o, out.ld1 (o) / rowsum[r]);
+            const uint32_t key = k0 + c, o = obase + (q0 + r) * L.ld + key;
+            if (key + 4 <= S) out.st4 (o, make_float4 (0.f, 0.f, 0.f, 0.f));
+            else if (key < S) { out.st1 (o, 0.f); if (key + 1 < S) out.st1 (o + 1, 0.f); if (key + 2 < S) out.st1 (o + 2, 0.f); }
         }
     __syncthreads ();
 }
