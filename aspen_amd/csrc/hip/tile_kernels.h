@@ -770,8 +770,10 @@ __device__ __forceinline__ void tile_softmax (const aspen_hip_layer_t &L, uint32
 // ---------------------------------------------------------------------------------------------
 // Attention tiles.
 // K tile: one (batch, head) x KATTN_BN queries x all keys.  scores = K.Q on the matrix cores, 128 keys at
-// a time; causal mask (-1e10 before the 1/sqrt(hd) scale), exp without max subtraction.  A first pass over
-// the key blocks accumulates every query's sum, a second recomputes the scores, divides and stores.
+// a time; causal mask (-1e10 before the 1/sqrt(hd) scale), exp without max subtraction; every block's
+// exponentials are stored (staged through LDS for 16-byte stores) while the queries' sums accumulate,
+// then a sweep over the tile's own output divides by the sums.  Key blocks the causal mask zeroes for
+// every query of the tile are not computed at all.
 // in0 = Query matrix, in1 = Key matrix (reference cfg: parent = Query, from = Key).
 // ---------------------------------------------------------------------------------------------
 template <int COH>
@@ -820,50 +822,23 @@ __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, ui
         for (int v = 0; v < 16; v++) part[i][v] = 0.f;
     constexpr uint32_t C4 = BM / 4, STEP = WG_THREADS / C4;
     const uint32_t c = (tid % C4) * 4;
-    const uint32_t blocks = (kend + BM - 1) / BM;
-    // one loop for both passes, so that the matrix code exists once
-    for (uint32_t step = 0; step < 2 * blocks; step++)
+    for (uint32_t k0 = 0; k0 < kend; k0 += BM)
     {
-        const bool second = step >= blocks;
-        const uint32_t k0 = (second ? step - blocks : step) * BM;
-        if (step == blocks)
-        {
-            // row sums: 32 lanes of a half-wave hold 32 different keys of the same query
-            #pragma unroll
-            for (int i = 0; i < TN; i++)
-                #pragma unroll
-                for (int v = 0; v < 16; v++)
-                {
-                    float t = part[i][v];
-                    #pragma unroll
-                    for (int o = 16; o > 0; o >>= 1) t += __shfl_xor (t, o, 64);
-                    if ((lane & 31) == 0) atomicAdd (&rowsum[ACC_N (wn0, i, v, lane)], t);
-                }
-            __syncthreads ();
-        }
         floatx16 acc[TN][TM];
         scores (k0, acc);                                // ends with a barrier: the stage is free
-        if (!second)
-        {
-            #pragma unroll
-            for (int j = 0; j < TM; j++)
-                #pragma unroll
-                for (int i = 0; i < TN; i++)
-                    #pragma unroll
-                    for (int v = 0; v < 16; v++)
-                        part[i][v] += weight (acc[i][j][v], k0 + wm0 + 32 * j + (lane & 31), q0 + ACC_N (wn0, i, v, lane));
-            continue;
-        }
         #pragma unroll
         for (int i = 0; i < TN; i++)
             #pragma unroll
             for (int v = 0; v < 16; v++)
             {
                 const uint32_t ql = ACC_N (wn0, i, v, lane);
-                const float sum = rowsum[ql];
                 #pragma unroll
                 for (int j = 0; j < TM; j++)
-                    smem[ql * TROW + wm0 + 32 * j + (lane & 31)] = weight (acc[i][j][v], k0 + wm0 + 32 * j + (lane & 31), q0 + ql) / sum;
+                {
+                    const float e = weight (acc[i][j][v], k0 + wm0 + 32 * j + (lane & 31), q0 + ql);
+                    part[i][v] += e;
+                    smem[ql * TROW + wm0 + 32 * j + (lane & 31)] = e;
+                }
             }
         __syncthreads ();
         for (uint32_t r = tid / C4; r < nq; r += STEP)
@@ -875,6 +850,35 @@ __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, ui
         }
         __syncthreads ();                                // the next block's operands overwrite the stage
     }
+    // row sums: 32 lanes of a half-wave hold 32 different keys of the same query
+    #pragma unroll
+    for (int i = 0; i < TN; i++)
+        #pragma unroll
+        for (int v = 0; v < 16; v++)
+        {
+            float t = part[i][v];
+            #pragma unroll
+            for (int o = 16; o > 0; o >>= 1) t += __shfl_xor (t, o, 64);
+            if ((lane & 31) == 0) atomicAdd (&rowsum[ACC_N (wn0, i, v, lane)], t);
+        }
+    asm volatile ("s_waitcnt vmcnt(0)" ::: "memory");   // this workgroup's own stores, read back below
+    __syncthreads ();
+    // second sweep over the tile's own output: divide by the sums
+    const uint32_t kcov = min (S, (kend + BM - 1) / BM * BM);
+    for (uint32_t k0 = 0; k0 < kcov; k0 += BM)
+        for (uint32_t r = tid / C4; r < nq; r += STEP)
+        {
+            const uint32_t key = k0 + c, o = obase + (q0 + r) * L.ld + key;
+            const float sum = rowsum[r];
+            if (key + 4 <= S)
+            {
+                float4 p = out.ld4 (o);
+                p.x /= sum; p.y /= sum; p.z /= sum; p.w /= sum;
+                out.st4 (o, p);
+            }
+            else
+                for (uint32_t e = key; e < S; e++) out.st1 (o + e - key, out.ld1 (o + e - key) / sum);
+        }
     // key blocks that are masked for every query of the tile
     for (uint32_t k0 = (kend + BM - 1) / BM * BM; k0 < S; k0 += BM)
         for (uint32_t r = tid / C4; r < nq; r += STEP)
