@@ -90,11 +90,24 @@ template <int COH> struct ActView
     }
 };
 
-// Activations other than the three cheap ones follow the reference's C expressions, which evaluate
-// in double or call libm (reference src/naive_kernels.c:11-57).  Their code is large (erff, tanhf, exp,
-// double-precision constants), so they live in ONE real function: inlined into every epilogue copy they
-// multiplied the kernel's code far beyond the instruction cache, and their constants were set up in
-// front of the persistent loop and occupied registers during every tile.
+// The two GELU forms in single precision.  The reference's C expressions (src/naive_kernels.c:44-55)
+// promote to double around a single-precision erff / tanhf; the results agree to about 1e-7 relative,
+// three orders of magnitude inside the parity tolerance, and the transformer FFN epilogues spend a
+// quarter of their time here.  tanh (u) = 1 - 2 / (exp (2u) + 1) with the hardware exponential:
+// exp overflows to +inf for large u (-> 1) and underflows to 0 for very negative u (-> -1).
+__device__ __forceinline__ float gelu_erf (float x) { return 0.5f * x * (1.f + erff (x * 0.7071067811865475f)); }
+__device__ __forceinline__ float gelu_tanh (float x)
+{
+    const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+    const float t = 1.f - 2.f * __frcp_rn (__expf (2.f * u) + 1.f);
+    return 0.5f * x * (1.f + t);
+}
+
+// Activations other than the three cheap ones.  The rare ones follow the reference's C expressions, which
+// evaluate in double (reference src/naive_kernels.c:11-57).  Their code is large (erff, exp, double-precision
+// constants), so they live in real functions: inlined into every epilogue copy they multiplied the
+// kernel's code far beyond the instruction cache, and their constants were set up in front of the
+// persistent loop and occupied registers during every tile.
 __device__ __noinline__ float activate_slow (float x, int act)
 {
     switch (act)
@@ -103,10 +116,18 @@ __device__ __noinline__ float activate_slow (float x, int act)
     case SELU:          return x > 0 ? (float)(1.0507 * (double)x) : (float)(1.0507 * 1.67326 * (exp ((double)x) - 1));
     case SIGMOID:       return (float)(1 / (1 + exp (-(double)x)));
     case TANH:          return (float)tanh ((double)x);
-    case GELU:          return (float)(0.5 * (double)x * (double)(1 + erff (x * 0.7071067811865475f)));
-    case GELU_ACCURATE: return (float)(0.5 * (double)x * (double)(1 + tanhf (0.7978845608028654f * (float)((double)x + 0.044715 * (double)x * (double)x * (double)x))));
+    case GELU:          return gelu_erf (x);
+    case GELU_ACCURATE: return gelu_tanh (x);
     default:            return x;
     }
+}
+
+// four values per call: the epilogues work on 16-byte pieces
+__device__ __noinline__ float4 activate_slow4 (float4 v, int act)
+{
+    if (act == GELU) return make_float4 (gelu_erf (v.x), gelu_erf (v.y), gelu_erf (v.z), gelu_erf (v.w));
+    if (act == GELU_ACCURATE) return make_float4 (gelu_tanh (v.x), gelu_tanh (v.y), gelu_tanh (v.z), gelu_tanh (v.w));
+    return make_float4 (activate_slow (v.x, act), activate_slow (v.y, act), activate_slow (v.z, act), activate_slow (v.w, act));
 }
 
 __device__ __forceinline__ float activate (float x, int act)
@@ -122,8 +143,13 @@ __device__ __forceinline__ float activate (float x, int act)
 
 __device__ __forceinline__ float4 act4 (float4 v, int act)
 {
-    v.x = activate (v.x, act); v.y = activate (v.y, act); v.z = activate (v.z, act); v.w = activate (v.w, act);
-    return v;
+    switch (act)
+    {
+    case NO_ACTIVATION: case LINEAR: return v;
+    case RELU:          return make_float4 (v.x > 0 ? v.x : 0, v.y > 0 ? v.y : 0, v.z > 0 ? v.z : 0, v.w > 0 ? v.w : 0);
+    case LEAKY_RELU:    return make_float4 (activate (v.x, act), activate (v.y, act), activate (v.z, act), activate (v.w, act));
+    default:            return activate_slow4 (v, act);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
