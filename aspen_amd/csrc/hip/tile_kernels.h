@@ -228,9 +228,14 @@ template <int ROWS, int COH> struct ConvLoader
     const aspen_hip_ktab_t *ktab;
     int32_t base[R], ih0[R], iw0[R];
     uint32_t IH, IW, chunk, row0;
+    uint32_t slices_per_tap, KW, ld0;       // slices_per_tap != 0: a K slice never straddles taps, no table needed
+    int next_it;                            // slice the running tap position (kh, kw, c) below belongs to
+    uint32_t kh, kw, c;
     __device__ __forceinline__ void init (const aspen_hip_layer_t &L, const ActView<COH> &v, uint32_t first_row, uint32_t tid)
     {
         in = v; ktab = L.ktab; IH = L.IH; IW = L.IW;
+        slices_per_tap = L.IC % GEMM_BK == 0 ? L.IC / GEMM_BK : 0; KW = L.KW; ld0 = L.ld0;
+        next_it = -1; kh = kw = c = 0;
         chunk = tid & 7; row0 = tid >> 3;
         const uint32_t ohw = L.OH * L.OW;
         #pragma unroll
@@ -246,7 +251,27 @@ template <int ROWS, int COH> struct ConvLoader
     }
     __device__ __forceinline__ void load (int it, float4 (&v)[R])
     {
-        const aspen_hip_ktab_t e = ktab[it * 8 + chunk];
+        aspen_hip_ktab_t e;
+        if (slices_per_tap)
+        {
+            // channel counts that are multiples of the slice width (every layer but a network's first):
+            // the whole slice belongs to one tap, found with a few scalar operations.  Fetching the table
+            // entry instead puts a dependent memory access in front of the operand loads of every slice.
+            // Slices are asked for in ascending order, so the position is stepped, not divided out.
+            if (it != next_it)
+            {
+                const uint32_t tap = (uint32_t)it / slices_per_tap;
+                c = ((uint32_t)it - tap * slices_per_tap) * GEMM_BK;
+                kh = tap / KW; kw = tap - kh * KW;
+            }
+            e.offset = (int32_t)((kh * IW + kw) * ld0 + c + chunk * 4);
+            e.kh = (uint16_t)kh; e.kw = (uint16_t)kw;
+            next_it = it + 1;
+            c += GEMM_BK;
+            if (c == slices_per_tap * GEMM_BK) { c = 0; if (++kw == KW) { kw = 0; ++kh; } }
+        }
+        else
+            e = ktab[it * 8 + chunk];
         #pragma unroll
         for (int i = 0; i < R; i++)
         {
