@@ -79,6 +79,7 @@ def lib() -> C.CDLL:
         # aspen_ext.h
         "aspen_dse_group_set_mode": (None, [_vp, C.c_int]),
         "aspen_dse_group_last_mode": (C.c_int, [_vp]),
+        "aspen_dse_group_set_spin_limit": (None, [_vp, C.c_uint64]),
         "aspen_dse_group_set_workgroups": (None, [_vp, C.c_uint]),
         "aspen_keep_layer_outputs": (None, [C.c_int]),
         "aspen_nasm_num_ldata": (C.c_uint, [_vp]),

@@ -37,6 +37,7 @@ struct aspen_hip_graph_t
                             // [ST_ABORT] abort flag, [ST_TWICE] tiles executed more than once
     uint32_t *d_ran;        // per-tile execution count (sanity: every tile exactly once)
     uint32_t *d_arrivals;   // split-K arrival counters, see run_tile
+    uint32_t stall_gen;     // value of g_stall_gen when the arrival counters were last known to be whole multiples of the group sizes
     uint32_t epoch;         // tag of the last run's queue entries, cycles 1..255
     unsigned long long *d_prof;
     uint32_t default_workgroups;    // grid of a dataflow run when the caller names none, see graph_parallelism
@@ -52,6 +53,7 @@ static int g_num_cu = 0;
 static int g_resident_wg = WG_PER_CU;     // workgroups of the dataflow kernel that fit one compute unit
 static char g_err[512] = "";
 static uint32_t g_flags = 0;
+static uint32_t g_stall_gen = 0;            // counts aborted dataflow runs: they leave split-K arrival counters mid-group
 static uint32_t *g_host_abort = nullptr;    // pinned host word the persistent kernel raises when it gives up waiting
 
 static int fail (hipError_t e, const char *what)
@@ -713,6 +715,12 @@ static void launch_layer (const aspen_hip_graph_t *g, uint32_t l)
 extern "C" int aspen_hip_run_layers (aspen_hip_graph_t *g, uint32_t first_layer, uint32_t last_layer)
 {
     if (!g || first_layer > last_layer || last_layer >= g->num_layers) { snprintf (g_err, sizeof (g_err), "run_layers: bad range"); return -1; }
+    if (g->stall_gen != g_stall_gen)
+    {
+        // a dataflow run was aborted since: its groups may be half counted (a dataflow run re-arms them itself)
+        CHECK (hipMemsetAsync (g->d_arrivals, 0, sizeof (uint32_t) * (g->num_ninst + 1), g_stream));
+        g->stall_gen = g_stall_gen;
+    }
     for (uint32_t l = first_layer; l <= last_layer; l++)
     {
         const aspen_hip_layer_t &L = g->h_layers[l];
@@ -781,6 +789,7 @@ extern "C" int aspen_hip_sync (void)
     if (*(volatile uint32_t *)g_host_abort != 0)
     {
         *g_host_abort = 0;
+        g_stall_gen++;
         snprintf (g_err, sizeof (g_err), "dataflow run stalled: a wait on the ready queue exceeded its spin limit and the run was aborted");
         fprintf (stderr, "aspen_hip: %s\n", g_err);
         return ASPEN_HIP_ERR_STALLED;

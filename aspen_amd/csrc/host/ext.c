@@ -7,6 +7,7 @@ void aspen_nasm_tile_range_internal (const nasm_ldata_t *ld, unsigned int t, uns
 
 void aspen_dse_group_set_mode (dse_group_t *g, int mode) { if (g) g->mode = mode < 0 || mode > 2 ? 2 : mode; }
 int aspen_dse_group_last_mode (dse_group_t *g) { return g ? g->last_mode : -1; }
+void aspen_dse_group_set_spin_limit (dse_group_t *g, uint64_t polls) { if (g) g->spin_limit = polls; }
 void aspen_dse_group_set_workgroups (dse_group_t *g, unsigned int w) { if (g) g->workgroups = w; }
 
 static int keep_layer_outputs = -1;          /* -1: not set yet, take the environment's word */

@@ -117,6 +117,7 @@ struct dse_group_t
     rpool_t *rpool;
     int mode;                                /* 0 = one launch per layer, 1 = persistent dataflow kernel, 2 = chosen per graph */
     int last_mode;                           /* what the last dse_group_run used (0 / 1) */
+    uint64_t spin_limit;                     /* watchdog of the persistent kernel, 0 = default */
     unsigned int workgroups;
 };
 

@@ -244,7 +244,7 @@ void dse_group_run (dse_group_t *dse_group)
         rc = aspen_hip_run_layers (rp->graph, 0, layers - 1);
     }
     else
-        rc = aspen_hip_run_dataflow (rp->graph, dse_group->workgroups, 0);
+        rc = aspen_hip_run_dataflow (rp->graph, dse_group->workgroups, dse_group->spin_limit);
     if (rc) { ERROR_PRTF ("ERROR: dse_group_run: launch failed: %s\n", aspen_hip_last_error ()); return; }
     for (unsigned int i = 0; i < rp->num_nasms; i++) { rp->nasms[i]->armed = 0; rp->nasms[i]->completed = 2; }   /* 2 = in flight */
     rp->running = 1;

@@ -19,6 +19,10 @@ extern "C" {
 void aspen_dse_group_set_mode (dse_group_t *dse_group, int mode);
 /* the mode the last dse_group_run used: 0 or 1 (-1 before the first run) */
 int aspen_dse_group_last_mode (dse_group_t *dse_group);
+/* Watchdog of the persistent kernel: polls a workgroup may spend waiting for one ready tile before the
+   run is given up (every workgroup then leaves, the run reports ASPEN_HIP_ERR_STALLED and the next run
+   starts from re-armed state).  0 = the library's default (2^26 polls, minutes). */
+void aspen_dse_group_set_spin_limit (dse_group_t *dse_group, uint64_t polls);
 /* persistent workgroups of the dataflow kernel; 0 = two per compute unit */
 void aspen_dse_group_set_workgroups (dse_group_t *dse_group, unsigned int workgroups);
 

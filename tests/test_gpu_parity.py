@@ -299,3 +299,33 @@ def test_default_discards_outputs_only_a_fused_shortcut_reads(gpu):
                 net.close()
     finally:
         api.lib().aspen_keep_layer_outputs(1)
+
+
+@pytest.mark.gpu
+def test_stalled_run_is_reported_and_the_next_runs_recover(gpu, capfd):
+    """The persistent kernel's watchdog, forced from the host with a spin limit of one poll: the first
+    workgroup that finds its queue slot still empty gives the run up, every workgroup leaves, the run
+    reports the stall.  The following runs (persistent kernel, then one launch per layer, whose split-K
+    groups count arrivals in the same counters) must be complete and correct again."""
+    name = "resnet_mini_b2"
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()[name])
+    gold = np.load(os.path.join(H.GOLDEN, f"micro_{name}.npz"))
+    net = H.GpuNet(cfg, tens, batch, seq, min_ninst=1024, mode=api.MODE_DATAFLOW)    # 1024: split-K layers
+    try:
+        assert any(net.nasm.info(l)["splits"] > 1 for l in range(net.nasm.num_ldata))
+        api.lib().aspen_dse_group_set_spin_limit(net.dse.h, 1)
+        net.run(x)
+        st = net.rpool.run_stats()
+        assert st["aborted"] == 1 and st["executed"] < net.nasm.num_ninst, st
+        assert "stalled" in capfd.readouterr().err
+        api.lib().aspen_dse_group_set_spin_limit(net.dse.h, 0)
+        for mode in (api.MODE_DATAFLOW, api.MODE_LAYERS, api.MODE_DATAFLOW):
+            net.dse.set_mode(mode)
+            net.run(x)
+            if mode == api.MODE_DATAFLOW:
+                st = net.rpool.run_stats()
+                assert st == {"executed": net.nasm.num_ninst, "double_runs": 0, "aborted": 0}, st
+            for l in range(net.nasm.num_ldata):
+                assert H.rel_l2(net.layer(l), gold[f"layer{l}"]) <= H.REL_L2_TOL, (mode, l)
+    finally:
+        net.close()
