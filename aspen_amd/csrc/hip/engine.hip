@@ -498,6 +498,7 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
         if (L.variant < 0 || L.variant >= ASPEN_HIP_NUM_GEMM_VARIANTS) { snprintf (g_err, sizeof (g_err), "layer %u rejected: GEMM variant", idx); return -1; }
         const uint32_t bm = shp[2 * L.variant], bn = shp[2 * L.variant + 1];
         if (!L.weight) why = "missing weight";
+        else if ((uint64_t)((L.M + 127) / 128 * 128) * L.Kp * 4 >= 0xffffff00ull) why = "weight matrix larger than 4 GiB";
         else if (L.Kp == 0 || L.Kp % GEMM_BK) why = "Kp must be a positive multiple of 32";
         else if (L.tile_m != bm || L.tile_n != bn) why = "tile extent does not match the GEMM variant";
         else if ((uint64_t)L.tiles_m * bm < L.M || (uint64_t)L.tiles_n * bn < L.N) why = "tile grid does not cover the matrix";

@@ -45,7 +45,7 @@ __device__ __forceinline__ float4 ld4 (const float *p) { return *reinterpret_cas
 __device__ __forceinline__ void st4 (float *p, float4 v) { *reinterpret_cast<float4 *> (p) = v; }
 
 // View of one activation matrix.  COH selects how it is accessed:
-//   0  plain cached loads and stores: the one-launch-per-layer path, where kernel boundaries provide
+//   0  cached loads and write-back stores: the one-launch-per-layer path, where kernel boundaries provide
 //      coherence.
 //   1  every access is device-scope coherent (buffer instructions with sc1): loads bypass the per-CU
 //      L1 and the per-XCD L2 (which are not coherent across the 8 XCDs), stores write through, so
@@ -55,38 +55,46 @@ __device__ __forceinline__ void st4 (float *p, float4 v) { *reinterpret_cast<flo
 //      shared by two producer tiles (the host checks strides and tile heights): a line is first
 //      fetched after its only producer has finished, every element is written once per launch, and
 //      the caches start a launch invalidated, so a cached line can never be stale.
-// Offsets are in floats from the start of the matrix; the descriptor bounds-checks them in hardware
-// (out-of-range loads return 0, out-of-range stores are dropped).
+// Offsets are in floats from the start of the matrix.  In modes 1 and 2 the buffer descriptor bounds-checks
+// them in hardware (out-of-range loads return 0, out-of-range stores are dropped); mode 0 relies on the slack
+// every allocation carries for the few floats an edge tile reads past a row.
 typedef uint32_t u32x4 __attribute__ ((ext_vector_type (4)));
 #define CPOL_SC1 16
+typedef float floatx4 __attribute__ ((ext_vector_type (4)));
 template <int COH> struct ActView
 {
-    const float *base;
+    // COH != 0: buffer descriptor.  COH == 0: uniform base address for global loads / stores with 32-bit
+    // offsets (measured: lower latency than buffer instructions, which counts when a single image runs
+    // through one launch per layer; 64-bit pointers per row instead cost that kernel enough registers
+    // to spill the weight pointers into the middle of its first loads).
     __amdgpu_buffer_rsrc_t rsrc;
+    char __attribute__ ((address_space (1))) *base;
+    static constexpr int LOAD_POLICY = COH == 1 ? CPOL_SC1 : 0, STORE_POLICY = COH ? CPOL_SC1 : 0;
     __device__ __forceinline__ void init (const float *p, uint32_t columns, uint32_t ld)
     {
-        base = p;
         if (COH) rsrc = __builtin_amdgcn_make_buffer_rsrc ((void *)p, 0, (int)(columns * ld * 4u + 256u), 0x00020000);
+        else base = (char __attribute__ ((address_space (1))) *)p;
     }
     __device__ __forceinline__ float4 ld4 (uint32_t off) const
     {
-        if (COH) return __builtin_bit_cast (float4, __builtin_amdgcn_raw_buffer_load_b128 (rsrc, (int)(off * 4u), 0, COH == 1 ? CPOL_SC1 : 0));
-        return *reinterpret_cast<const float4 *> (base + off);
+        if (COH) return __builtin_bit_cast (float4, __builtin_amdgcn_raw_buffer_load_b128 (rsrc, (int)(off * 4u), 0, LOAD_POLICY));
+        const floatx4 x = *(const floatx4 __attribute__ ((address_space (1))) *)(base + off * 4u);
+        return make_float4 (x[0], x[1], x[2], x[3]);
     }
     __device__ __forceinline__ float ld1 (uint32_t off) const
     {
-        if (COH) return __builtin_bit_cast (float, __builtin_amdgcn_raw_buffer_load_b32 (rsrc, (int)(off * 4u), 0, COH == 1 ? CPOL_SC1 : 0));
-        return base[off];
+        if (COH) return __builtin_bit_cast (float, __builtin_amdgcn_raw_buffer_load_b32 (rsrc, (int)(off * 4u), 0, LOAD_POLICY));
+        return *(const float __attribute__ ((address_space (1))) *)(base + off * 4u);
     }
     __device__ __forceinline__ void st4 (uint32_t off, float4 v) const
     {
-        if (COH) __builtin_amdgcn_raw_buffer_store_b128 (__builtin_bit_cast (u32x4, v), rsrc, (int)(off * 4u), 0, CPOL_SC1);
-        else *reinterpret_cast<float4 *> (const_cast<float *> (base) + off) = v;
+        if (COH) __builtin_amdgcn_raw_buffer_store_b128 (__builtin_bit_cast (u32x4, v), rsrc, (int)(off * 4u), 0, STORE_POLICY);
+        else *(floatx4 __attribute__ ((address_space (1))) *)(base + off * 4u) = (floatx4){v.x, v.y, v.z, v.w};
     }
     __device__ __forceinline__ void st1 (uint32_t off, float v) const
     {
-        if (COH) __builtin_amdgcn_raw_buffer_store_b32 (__builtin_bit_cast (uint32_t, v), rsrc, (int)(off * 4u), 0, CPOL_SC1);
-        else const_cast<float *> (base)[off] = v;
+        if (COH) __builtin_amdgcn_raw_buffer_store_b32 (__builtin_bit_cast (uint32_t, v), rsrc, (int)(off * 4u), 0, STORE_POLICY);
+        else *(float __attribute__ ((address_space (1))) *)(base + off * 4u) = v;
     }
 };
 
@@ -162,23 +170,30 @@ __device__ __forceinline__ float4 act4 (float4 v, int act)
 template <int ROWS> struct RowLoader
 {
     static constexpr int R = ROWS / 32;
-    const float *ptr[R];
-    uint32_t chunk, row0;
-    __device__ __forceinline__ void init (const float *base, uint32_t first_row, uint32_t max_row, uint32_t ld, uint32_t tid)
+    // One uniform base pointer plus 32-bit byte offsets: global loads with a scalar base address need one
+    // vector register per row instead of a 64-bit pointer.
+    const char *base;
+    uint32_t off[R], chunk, row0;
+    // `rows` x `ld` floats at `p`, rows padded so that a tile never runs past them
+    __device__ __forceinline__ void init (const float *p, uint32_t first_row, uint32_t rows, uint32_t ld, uint32_t tid)
     {
+        (void)rows;
         chunk = tid & 7; row0 = tid >> 3;
+        base = reinterpret_cast<const char *> (p);
         #pragma unroll
-        for (int i = 0; i < R; i++)
-        {
-            uint32_t r = first_row + row0 + 32 * i;
-            r = r < max_row ? r : max_row;          // clamp: rows past the edge re-read the last row, never stored
-            ptr[i] = base + (size_t)r * ld + chunk * 4;
-        }
+        for (int i = 0; i < R; i++) off[i] = ((first_row + row0 + 32u * i) * ld + chunk * 4u) * 4u;
     }
     __device__ __forceinline__ void load (int it, float4 (&v)[R])
     {
         #pragma unroll
-        for (int i = 0; i < R; i++) v[i] = ld4 (ptr[i] + it * GEMM_BK);
+        for (int i = 0; i < R; i++)
+        {
+            // the address space makes this a global (not flat) load whose 64-bit base stays in scalar registers
+            typedef const floatx4 __attribute__ ((address_space (1))) global_floatx4;
+            const char __attribute__ ((address_space (1))) *g = (const char __attribute__ ((address_space (1))) *)base;
+            const floatx4 x = *(global_floatx4 *)(g + (off[i] + (uint32_t)it * (GEMM_BK * 4u)));
+            v[i] = make_float4 (x[0], x[1], x[2], x[3]);
+        }
     }
     __device__ __forceinline__ void store (float *lds, const float4 (&v)[R])
     {
@@ -501,7 +516,7 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
         kiters = min ((int)L.kiters_per_split, kiters - kbase);
     }
     RowLoader<BM> al;
-    al.init (L.weight, m0, 0xffffffffu, L.Kp, tid);
+    al.init (L.weight, m0, (L.M + 127u) / 128u * 128u, L.Kp, tid);
     if (L.direct)
     {
         ActRowLoader<BN, COH> bl;
