@@ -320,7 +320,9 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
         id = __builtin_amdgcn_readfirstlane (schedule_step (id, rec));
         if (id == QUEUE_EMPTY) break;           // all tickets taken, or aborted
         // wavefront 0 requests this tile's child record now; it arrives while the tile runs
-        if (threadIdx.x < CHILD_REC) rec = s_sched.a.child_rec[(size_t)id * CHILD_REC + threadIdx.x];
+        // (a global, not a flat load: a flat one would also count as LDS traffic the tile's first fragment wait sits out)
+        if (threadIdx.x < CHILD_REC)
+            rec = *(const qentry_t __attribute__ ((address_space (1))) *)(s_sched.a.child_rec + (size_t)id * CHILD_REC + threadIdx.x);
         if ((s_sched.a.flags & ASPEN_HIP_FLAG_TRACE) && threadIdx.x == 0) s_sched.a.trace[2 * (size_t)id] = wall_clock64 ();
         const aspen_hip_layer_t *L = &s_sched.desc[__builtin_amdgcn_readfirstlane (s_sched.desc_slot)];
         bool complete;

@@ -44,6 +44,17 @@ typedef float floatx16 __attribute__ ((ext_vector_type (16)));
 __device__ __forceinline__ float4 ld4 (const float *p) { return *reinterpret_cast<const float4 *> (p); }
 __device__ __forceinline__ void st4 (float *p, float4 v) { *reinterpret_cast<float4 *> (p) = v; }
 
+// Loads from device memory through pointers the compiler cannot prove to be global (descriptor fields)
+// would be FLAT instructions, which count as LDS traffic too: every wait for an LDS fragment would
+// then also wait for them.  These go through the global address space explicitly.
+typedef float floatx4 __attribute__ ((ext_vector_type (4)));
+__device__ __forceinline__ float4 gld4 (const float *p)
+{
+    const floatx4 x = *(const floatx4 __attribute__ ((address_space (1))) *)p;
+    return make_float4 (x[0], x[1], x[2], x[3]);
+}
+__device__ __forceinline__ float gld1 (const float *p) { return *(const float __attribute__ ((address_space (1))) *)p; }
+
 // View of one activation matrix.  COH selects how it is accessed:
 //   0  cached loads and write-back stores: the one-launch-per-layer path, where kernel boundaries provide
 //      coherence.
@@ -60,7 +71,6 @@ __device__ __forceinline__ void st4 (float *p, float4 v) { *reinterpret_cast<flo
 // every allocation carries for the few floats an edge tile reads past a row.
 typedef uint32_t u32x4 __attribute__ ((ext_vector_type (4)));
 #define CPOL_SC1 16
-typedef float floatx4 __attribute__ ((ext_vector_type (4)));
 template <int COH> struct ActView
 {
     // COH != 0: buffer descriptor.  COH == 0: uniform base address for global loads / stores with 32-bit
@@ -286,7 +296,11 @@ template <int ROWS, int COH> struct ConvLoader
             if (c == slices_per_tap * GEMM_BK) { c = 0; if (++kw == KW) { kw = 0; ++kh; } }
         }
         else
-            e = ktab[it * 8 + chunk];
+        {
+            typedef unsigned int uintx2 __attribute__ ((ext_vector_type (2)));
+            const uintx2 raw = *(const uintx2 __attribute__ ((address_space (1))) *)(ktab + it * 8 + chunk);
+            e.offset = (int32_t)raw[0]; e.kh = (uint16_t)(raw[1] & 0xffffu); e.kw = (uint16_t)(raw[1] >> 16);
+        }
         #pragma unroll
         for (int i = 0; i < R; i++)
         {
@@ -565,8 +579,8 @@ __device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L
         float4 b = make_float4 (0.f, 0.f, 0.f, 0.f);
         if (L.bias && slice < 0)
         {
-            if (c + 4 <= mrem) b = ld4 (L.bias + m0 + c);
-            else { b.x = L.bias[m0 + c]; if (c + 1 < mrem) b.y = L.bias[m0 + c + 1]; if (c + 2 < mrem) b.z = L.bias[m0 + c + 2]; }
+            if (c + 4 <= mrem) b = gld4 (L.bias + m0 + c);
+            else { b.x = gld1 (L.bias + m0 + c); if (c + 1 < mrem) b.y = gld1 (L.bias + m0 + c + 1); if (c + 2 < mrem) b.z = gld1 (L.bias + m0 + c + 2); }
         }
         const bool fuse = L.fuse_out != nullptr && slice < 0;
         const bool keep = !(fuse && L.fuse_discard);        // the pre-shortcut sums are stored unless the host has no use for them
@@ -648,10 +662,10 @@ __device__ __forceinline__ void tile_splitk_finish (const aspen_hip_layer_t &L, 
         }
         if (L.bias)
         {
-            v.x += L.bias[m0 + c];
-            if (c + 1 < mrem) v.y += L.bias[m0 + c + 1];
-            if (c + 2 < mrem) v.z += L.bias[m0 + c + 2];
-            if (c + 3 < mrem) v.w += L.bias[m0 + c + 3];
+            v.x += gld1 (L.bias + m0 + c);
+            if (c + 1 < mrem) v.y += gld1 (L.bias + m0 + c + 1);
+            if (c + 2 < mrem) v.z += gld1 (L.bias + m0 + c + 2);
+            if (c + 3 < mrem) v.w += gld1 (L.bias + m0 + c + 3);
         }
         v = act4 (v, L.act);
         const uint32_t o = (n0 + r) * L.ld + m0 + c;
@@ -736,8 +750,8 @@ __device__ __forceinline__ void tile_yolo (const aspen_hip_layer_t &L, uint32_t 
         float r;
         if (j == 0) r = (1.0f / (1.0f + expf (-x)) + (float)w) * (float)L.stride;
         else if (j == 1) r = (1.0f / (1.0f + expf (-x)) + (float)h) * (float)L.stride;
-        else if (j == 2) r = expf (x) * L.weight[2 * a];
-        else if (j == 3) r = expf (x) * L.weight[2 * a + 1];
+        else if (j == 2) r = expf (x) * gld1 (L.weight + 2 * a);
+        else if (j == 3) r = expf (x) * gld1 (L.weight + 2 * a + 1);
         else r = 1.0f / (1.0f + expf (-x));
         out.st1 (n * L.ld + j, r);
     }
@@ -800,15 +814,15 @@ __device__ __forceinline__ void tile_layernorm (const aspen_hip_layer_t &L, uint
         const float rstd = 1.0f / sqrtf (var + 1e-6f);
         for (uint32_t m = lane; m < M4; m += 64)
         {
-            const float4 v = in.ld4 (x + m * 4), g = ld4 (L.weight + m * 4);
+            const float4 v = in.ld4 (x + m * 4), g = gld4 (L.weight + m * 4);
             float4 r;
             r.x = (v.x - mean) * rstd * g.x; r.y = (v.y - mean) * rstd * g.y;
             r.z = (v.z - mean) * rstd * g.z; r.w = (v.w - mean) * rstd * g.w;
-            if (L.bias) { const float4 b = ld4 (L.bias + m * 4); r.x += b.x; r.y += b.y; r.z += b.z; r.w += b.w; }
+            if (L.bias) { const float4 b = gld4 (L.bias + m * 4); r.x += b.x; r.y += b.y; r.z += b.z; r.w += b.w; }
             out.st4 (o + m * 4, r);
         }
         for (uint32_t m = M4 * 4 + lane; m < L.M; m += 64)
-            out.st1 (o + m, (in.ld1 (x + m) - mean) * rstd * L.weight[m] + (L.bias ? L.bias[m] : 0.f));
+            out.st1 (o + m, (in.ld1 (x + m) - mean) * rstd * gld1 (L.weight + m) + (L.bias ? gld1 (L.bias + m) : 0.f));
     }
 }
 
