@@ -329,3 +329,63 @@ def test_stalled_run_is_reported_and_the_next_runs_recover(gpu, capfd):
                 assert H.rel_l2(net.layer(l), gold[f"layer{l}"]) <= H.REL_L2_TOL, (mode, l)
     finally:
         net.close()
+
+
+@pytest.mark.gpu
+def test_reference_main_call_sequence(gpu, tmp_path):
+    """The call sequence of the reference's main.c:60-151 through the raw C ABI (no Python wrapper objects):
+    create dnn / nasm, rpool, engine group, add the input, run until completion, check completion, fetch
+    the result in {BATCH, OUT_C, OUT_H, OUT_W} order; then the reset / run / wait / stop loop, reading
+    the input from an NCHW file the second time; the print_* dumps and the teardown."""
+    import ctypes as C
+    from oracle import cpu
+    L = api.lib()
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()["custom_b3"])
+    cfg_path, w_path, in_path = str(tmp_path / "net.cfg"), str(tmp_path / "net.bin"), str(tmp_path / "in.bin")
+    open(cfg_path, "w").write(cfg)
+    M.write_aspen_data(w_path, tens)
+    want = cpu.run_network(layers, tens, x, batch, seq)[-1]            # [batch][classes]
+    dnn = L.apu_create_dnn(cfg_path.encode(), w_path.encode())
+    assert dnn
+    L.print_dnn_info(dnn, 0)
+    nasm = L.apu_create_nasm(dnn, 64, batch)
+    assert nasm
+    L.print_nasm_info(nasm, 0, 0)
+    rpool = L.rpool_init()
+    dse = L.dse_group_init(8)                                           # thread count: accepted, not used
+    L.dse_group_set_rpool(dse, rpool)
+    xin = np.ascontiguousarray(x, dtype=np.float32)
+    L.rpool_add_nasm_raw_input(rpool, nasm, xin.ctypes.data_as(C.c_void_p))
+    L.print_rpool_info(rpool)
+    assert L.dse_check_nasm_completion(nasm) == 0
+    L.dse_group_run_until_nasm_completion(dse, nasm)
+    assert L.dse_check_nasm_completion(nasm) == 1
+    order = (C.c_int * 4)(api.BATCH, api.OUT_C, api.OUT_H, api.OUT_W)
+
+    def fetch():
+        out = C.c_void_p()
+        n = L.dse_get_nasm_result(nasm, order, C.byref(out))
+        assert n == want.size * 4
+        a = np.ctypeslib.as_array(C.cast(out, C.POINTER(C.c_float)), shape=(n // 4,)).copy()
+        L._free(out)
+        return a.reshape(want.shape)
+
+    assert H.rel_l2(fetch(), want) <= H.REL_L2_TOL
+    # second inference: the reference's loop, input from a raw NCHW file this time
+    chw = [l for l in layers if l["type"] == "input"][0]
+    nchw = xin.reshape(batch, chw["H"], chw["W"], chw["C"]).transpose(0, 3, 1, 2)
+    np.ascontiguousarray(nchw).tofile(in_path)
+    for _ in range(2):
+        L.rpool_reset_queue(rpool)
+        L.apu_reset_nasm(nasm)
+        L.rpool_add_nasm(rpool, nasm, in_path.encode())
+        assert L.dse_check_nasm_completion(nasm) == 0
+        L.dse_group_run(dse)
+        L.dse_wait_for_nasm_completion(nasm)
+        L.dse_group_stop(dse)
+        assert H.rel_l2(fetch(), want) <= H.REL_L2_TOL
+    L.aspen_flush_dynamic_memory()
+    L.dse_group_destroy(dse)
+    L.rpool_destroy(rpool)
+    L.apu_destroy_nasm(nasm)
+    L.apu_destroy_dnn(dnn)
