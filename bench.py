@@ -99,6 +99,21 @@ def cpu_baseline(cfgname, budget_s=20.0):
                 "sample": f"{cfgname}: 1 full pass of the oracle port ({exc})", "ms_per_step": sec * 1e3}
 
 
+def quiet_stdout():
+    """The C library reports what it parses on stdout, as the reference does.  The benchmark's stdout
+    carries exactly one JSON line, so everything else written to file descriptor 1 goes to stderr; returns
+    the function that writes the final line to the real stdout."""
+    sys.stdout.flush()
+    real = os.dup(1)
+    os.dup2(2, 1)
+
+    def emit(line: str) -> None:
+        sys.stdout.flush()
+        os.write(real, (line + "\n").encode())
+
+    return emit
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -118,6 +133,7 @@ def main():
                     help="instead of a workload: run the library's streaming copy kernel over MIB MiB (--steps launches); "
                          "under a profiler this calibrates the HBM byte counters")
     args = ap.parse_args()
+    emit = quiet_stdout()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
         sys.exit(2)
@@ -140,7 +156,7 @@ def main():
         L.aspen_hip_sync()
         ms = api.C.c_float()
         L.aspen_hip_event_elapsed_ms(0, 1, api.C.byref(ms))
-        print(json.dumps({"copy_probe_bytes_read": nbytes, "copy_probe_bytes_written": nbytes, "launches": args.steps,
+        emit(json.dumps({"copy_probe_bytes_read": nbytes, "copy_probe_bytes_written": nbytes, "launches": args.steps,
                           "ms_per_launch": ms.value / args.steps,
                           "GB_per_s": 2 * nbytes * args.steps / (ms.value * 1e-3) / 1e9}))
         return
@@ -291,7 +307,7 @@ def main():
     pool.destroy()
     for _, dnn, nasm, _ in nets:
         dnn.destroy()
-    print(json.dumps(out))
+    emit(json.dumps(out))
 
 
 if __name__ == "__main__":
