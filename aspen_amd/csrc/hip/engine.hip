@@ -37,7 +37,6 @@ struct aspen_hip_graph_t
                             // [ST_ABORT] abort flag, [ST_TWICE] tiles executed more than once
     uint32_t *d_ran;        // per-tile execution count (sanity: every tile exactly once)
     uint32_t *d_arrivals;   // split-K arrival counters, see run_tile
-    uint32_t stall_gen;     // value of g_stall_gen when the arrival counters were last known to be whole multiples of the group sizes
     uint32_t epoch;         // tag of the last run's queue entries, cycles 1..255
     unsigned long long *d_prof;
     uint32_t default_workgroups;    // grid of a dataflow run when the caller names none, see graph_parallelism
@@ -53,7 +52,6 @@ static int g_num_cu = 0;
 static int g_resident_wg = WG_PER_CU;     // workgroups of the dataflow kernel that fit one compute unit
 static char g_err[512] = "";
 static uint32_t g_flags = 0;
-static uint32_t g_stall_gen = 0;            // counts aborted dataflow runs: they leave split-K arrival counters mid-group
 static uint32_t *g_host_abort = nullptr;    // pinned host word the persistent kernel raises when it gives up waiting
 
 static int fail (hipError_t e, const char *what)
@@ -78,6 +76,12 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) layer_kernel (const as
     const uint32_t xcd = bid & 7, local = bid >> 3, chunk = nt >> 3, rem = nt & 7;
     const uint32_t t = first_tile + xcd * chunk + (xcd < rem ? xcd : rem) + local;
     run_tile<0> (L, t, smem, [=] () { return arrivals; });
+}
+
+// Second launch of a split-K layer in launch-per-layer mode: one workgroup per output tile adds the slices up.
+__global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) finish_kernel (const aspen_hip_layer_t *layers, uint32_t l)
+{
+    finish_tile<0> (layers[l], blockIdx.x);
 }
 
 // Re-arm: counters back to the parent counts, queue seeded with the roots.  A queue entry is 64 bits:
@@ -707,23 +711,20 @@ extern "C" void aspen_hip_graph_destroy (aspen_hip_graph_t *g)
 // ------------------------------------------------------------------------------------------------
 // execution
 // ------------------------------------------------------------------------------------------------
-// One layer in launch mode (split-K needs no second launch: the slice of a group that finishes last
-// adds the group's partial sums up).
+// One layer in launch mode.  A split-K layer takes two launches: within one launch the plain (write-back)
+// stores of a workgroup are not visible to workgroups on other XCDs, so the slices cannot be added up by
+// whichever slice finishes last, as the persistent kernel (write-through stores) does.
 static void launch_layer (const aspen_hip_graph_t *g, uint32_t l)
 {
     const aspen_hip_layer_t &L = g->h_layers[l];
-    hipLaunchKernelGGL (layer_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, g->d_layers, l, 0u, g->d_arrivals);
+    hipLaunchKernelGGL (layer_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, g->d_layers, l, 0u, (uint32_t *)nullptr);
+    if (L.splits > 1)
+        hipLaunchKernelGGL (finish_kernel, dim3 (L.tiles_m * L.tiles_n), dim3 (WG_THREADS), 0, g_stream, g->d_layers, l);
 }
 
 extern "C" int aspen_hip_run_layers (aspen_hip_graph_t *g, uint32_t first_layer, uint32_t last_layer)
 {
     if (!g || first_layer > last_layer || last_layer >= g->num_layers) { snprintf (g_err, sizeof (g_err), "run_layers: bad range"); return -1; }
-    if (g->stall_gen != g_stall_gen)
-    {
-        // a dataflow run was aborted since: its groups may be half counted (a dataflow run re-arms them itself)
-        CHECK (hipMemsetAsync (g->d_arrivals, 0, sizeof (uint32_t) * (g->num_ninst + 1), g_stream));
-        g->stall_gen = g_stall_gen;
-    }
     for (uint32_t l = first_layer; l <= last_layer; l++)
     {
         const aspen_hip_layer_t &L = g->h_layers[l];
@@ -792,7 +793,6 @@ extern "C" int aspen_hip_sync (void)
     if (*(volatile uint32_t *)g_host_abort != 0)
     {
         *g_host_abort = 0;
-        g_stall_gen++;
         snprintf (g_err, sizeof (g_err), "dataflow run stalled: a wait on the ready queue exceeded its spin limit and the run was aborted");
         fprintf (stderr, "aspen_hip: %s\n", g_err);
         return ASPEN_HIP_ERR_STALLED;

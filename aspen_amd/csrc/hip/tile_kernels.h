@@ -1039,6 +1039,16 @@ __device__ __forceinline__ bool splitk_arrived_last (uint32_t *counter, uint32_t
     return before % splits == splits - 1;
 }
 
+// Split-K reduction of output tile t of the layer as a tile of its own (launch-per-layer mode).
+template <int COH>
+__device__ __forceinline__ void finish_tile (const aspen_hip_layer_t &Lg, uint32_t t)
+{
+    const aspen_hip_layer_t L = uniform_layer (Lg);
+    t = __builtin_amdgcn_readfirstlane (t);
+    const uint32_t tn = t / L.tiles_m;
+    tile_splitk_finish<COH> (L, tn, t - tn * L.tiles_m);
+}
+
 // Runs tile t of the layer.  `arrivals ()` yields the graph's array of zero-initialised counters, one per
 // tile (used at the index of a split-K group's first tile); it is a callable so that the pointer is
 // fetched where it is needed instead of occupying registers while the tile runs.  Returns false for
@@ -1070,8 +1080,11 @@ __device__ __forceinline__ bool run_tile (const aspen_hip_layer_t &Lg, uint32_t 
         contraction_epilogue<COH> (L, tn, tm, slice, smem, c4_log2, bn);
         if (slice >= 0)
         {
-            // split-K: every slice has written its partial sums; whoever arrives last adds them up
-            if (!splitk_arrived_last (arrivals () + group, L.splits, smem)) return false;
+            // split-K: every slice has written its partial sums; whoever arrives last adds them up.  Without
+            // counters (one launch per layer: stores of a launch are not visible across XCDs before it ends)
+            // the sums are added up by a second launch, see finish_tile.
+            uint32_t *counters = arrivals ();
+            if (counters == nullptr || !splitk_arrived_last (counters + group, L.splits, smem)) return false;
             tile_splitk_finish<COH> (L, tn, tm);
         }
         break;

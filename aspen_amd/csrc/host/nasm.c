@@ -160,11 +160,13 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
         /* still short of tiles with the smallest shape: cut the K axis (at least 8 slices of 32 per part) */
         const unsigned int kiters = aspen_layer_kiters (L), T = ld->num_ninst;
         ld->kiters_per_split = kiters;
-        if (T < want && kiters >= 16 && getenv ("ASPEN_GPU_NO_SPLITK") == NULL)
+        /* kiters_cap (graphs bound by their dependency chains, see create_nasm): no tile longer than that many K slices */
+        const unsigned int cap = nasm->kiters_cap;
+        if ((T < want || (cap && kiters > cap)) && kiters >= 16 && getenv ("ASPEN_GPU_NO_SPLITK") == NULL)
         {
             const char *e1 = getenv ("ASPEN_GPU_MAX_SPLITS"), *e2 = getenv ("ASPEN_GPU_MIN_KITERS");
             const unsigned int max_splits = e1 ? (unsigned int)atoi (e1) : 8, min_kiters = e2 ? (unsigned int)atoi (e2) : 8;
-            unsigned int s = umin (umin (cdiv (want, T), kiters / umax (min_kiters, 1)), umax (max_splits, 1));
+            unsigned int s = umin (umin (umax (cdiv (want, T), cap ? cdiv (kiters, cap) : 1), kiters / umax (min_kiters, 1)), umax (max_splits, 1));
             ld->kiters_per_split = cdiv (kiters, s);
             ld->splits = cdiv (kiters, ld->kiters_per_split);
             if (ld->splits > 1) ld->num_ninst = T * ld->splits;
@@ -432,11 +434,13 @@ static void fuse_shortcuts (nasm_t *nasm)
     }
 }
 
-static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned int batch, unsigned int seq)
+static nasm_t *build_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned int batch, unsigned int seq, unsigned int kiters_cap)
 {
     if (dnn == NULL) { ERROR_PRTF ("apu_create_nasm: dnn is NULL\n"); return NULL; }
     if (min_ninst < 1) { ERROR_PRTF ("ERROR: min_ninst_per_ldata should be at least 1\n"); return NULL; }
     nasm_t *nasm = calloc (1, sizeof (nasm_t));
+    nasm->kiters_cap = kiters_cap;
+    nasm->preferred_mode = -1;
     nasm->dnn = dnn; nasm->nasm_id = nasm_counter++;
     nasm->batch_size = batch > 0 ? batch : 1;
     nasm->tr_seq_len = seq; nasm->min_ninst_per_ldata = min_ninst;
@@ -485,6 +489,51 @@ static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned i
     return nasm;
 }
 
+/* Average parallelism of a tile graph: summed tile cost over the cost of the longest dependency chain
+   (cost = K slices of a contraction tile + a constant; the device library sizes its grid with the same
+   estimate). */
+static double nasm_parallelism (const nasm_t *nasm)
+{
+    const uint32_t n = nasm->num_ninst;
+    if (n == 0) return 0.0;
+    float *dist = calloc (n, sizeof (float));
+    double total = 0.0, longest = 0.0;
+    for (uint32_t t = 0; t < n; t++)
+    {
+        const nasm_ldata_t *ld = &nasm->ldata_arr[nasm->ninst_ldata[t]];
+        const LAYER_TYPE ty = ld->layer->type;
+        float cost = 4.f;
+        if (is_contraction (ty)) cost = 8.f + (float)(ld->splits > 1 ? ld->kiters_per_split : aspen_layer_kiters (ld->layer));
+        else if (ty == K_ATTENTION_LAYER || ty == V_ATTENTION_LAYER) cost = 16.f;
+        dist[t] += cost;
+        total += cost;
+        if (dist[t] > longest) longest = dist[t];
+        for (uint32_t e = nasm->child_off[t]; e < nasm->child_off[t + 1]; e++)
+            if (dist[nasm->child_idx[e]] < dist[t]) dist[nasm->child_idx[e]] = dist[t];      /* children have larger indices */
+    }
+    free (dist);
+    return longest > 0.0 ? total / longest : 0.0;
+}
+
+/* A graph that offers less parallelism than a 256-CU device has resident workgroups is bound by its
+   dependency chains, not by throughput: workgroups idle while the longest tiles of each stage finish
+   (BERT / GPT-2 with one or two thousand tokens: FFN tiles of 48-96 K slices).  Such a graph is rebuilt
+   with no tile longer than 48 K slices (more split-K): GPT-2 -6 %, BERT -3 %.  Throughput-bound graphs
+   (batch-32 vision nets) lose 2-3 % with the same cap (more partial sums to move) and keep long tiles. */
+#define CHAIN_BOUND_BELOW 1024.0
+#define CHAIN_BOUND_KITERS_CAP 48
+static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned int batch, unsigned int seq)
+{
+    const char *e = getenv ("ASPEN_GPU_MAX_KITERS");            /* experiments: fixed cap, 0 = none */
+    if (e != NULL) return build_nasm (dnn, min_ninst, batch, seq, (unsigned int)atoi (e));
+    nasm_t *nasm = build_nasm (dnn, min_ninst, batch, seq, 0);
+    if (nasm == NULL || nasm_parallelism (nasm) >= CHAIN_BOUND_BELOW) return nasm;
+    nasm_t *capped = build_nasm (dnn, min_ninst, batch, seq, CHAIN_BOUND_KITERS_CAP);
+    if (capped == NULL) return nasm;
+    apu_destroy_nasm (nasm);
+    return capped;
+}
+
 nasm_t *apu_create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst_per_ldata, unsigned int batch_size)
 {
     return create_nasm (dnn, min_ninst_per_ldata, batch_size, 0);
@@ -506,12 +555,13 @@ nasm_t *apu_create_transformer_nasm (aspen_dnn_t *dnn, unsigned int min_ninst_pe
 #include <time.h>
 /* large batches of vision nets like 1024-2048; transformers with a few hundred columns and batch 1 like
    few, large tiles (128-384) on one workgroup per compute unit */
-static const unsigned int tuner_candidates[] = {DEFAULT_MIN_NINST, 384, 128, 768, 1024, 2048, 256, 512, 3072};
+static const unsigned int tuner_candidates[] = {DEFAULT_MIN_NINST, 384, 128, 768, 192, 1024, 2048, 256, 512, 3072};
 
-static double test_nasm_time_sec (nasm_t *nasm, unsigned int iters)
+static double test_nasm_time_sec (nasm_t *nasm, unsigned int iters, int mode)
 {
     rpool_t *rpool = rpool_init ();
     dse_group_t *dse = dse_group_init (1);
+    dse->mode = mode;
     dse_group_set_rpool (dse, rpool);
     rpool_add_nasm (rpool, nasm, NULL);
     struct timespec t0, t1;
@@ -540,20 +590,28 @@ static nasm_t *generate_nasm (aspen_dnn_t *dnn, unsigned int batch, unsigned int
     const unsigned int ncand = sizeof (tuner_candidates) / sizeof (tuner_candidates[0]);
     if (num_iter == 0 || aspen_hip_init () != 0) return create_nasm (dnn, DEFAULT_MIN_NINST, batch, seq);
     unsigned int best = DEFAULT_MIN_NINST;
+    int best_mode = 1;
     double best_time = -1.0;
+    /* every candidate on both engines: the persistent kernel (1) and one launch per layer (0) */
     for (unsigned int c = 0; c < ncand && c <= num_iter; c++)
     {
         nasm_t *cand = create_nasm (dnn, tuner_candidates[c], batch, seq);
         if (cand == NULL) return NULL;
-        const double t = test_nasm_time_sec (cand, 10);
-        printf ("APU: min_ninst_per_ldata %u: %u tiles, %f sec per inference\n", tuner_candidates[c], cand->num_ninst, t);
-        fflush (stdout);
+        for (int mode = 1; mode >= 0; mode--)
+        {
+            const double t = test_nasm_time_sec (cand, 10, mode);
+            printf ("APU: min_ninst_per_ldata %u, %s: %u tiles, %f sec per inference\n", tuner_candidates[c],
+                mode ? "persistent kernel" : "one launch per layer", cand->num_ninst, t);
+            fflush (stdout);
+            if (t > 0 && (best_time < 0 || t < best_time)) { best_time = t; best = tuner_candidates[c]; best_mode = mode; }
+        }
         apu_destroy_nasm (cand);
-        if (t > 0 && (best_time < 0 || t < best_time)) { best_time = t; best = tuner_candidates[c]; }
     }
-    printf ("APU: NASM with min_ninst_per_ldata %u, time = %f sec selected.\n", best, best_time);
+    printf ("APU: NASM with min_ninst_per_ldata %u, %s, time = %f sec selected.\n", best, best_mode ? "persistent kernel" : "one launch per layer", best_time);
     fflush (stdout);
-    return create_nasm (dnn, best, batch, seq);
+    nasm_t *nasm = create_nasm (dnn, best, batch, seq);
+    if (nasm != NULL) nasm->preferred_mode = best_mode;      /* what an engine group in mode "auto" will run it with */
+    return nasm;
 }
 
 nasm_t *apu_generate_nasm (aspen_dnn_t *dnn, unsigned int batch_size, unsigned int num_iter)

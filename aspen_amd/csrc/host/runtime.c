@@ -235,7 +235,13 @@ void dse_group_run (dse_group_t *dse_group)
        network: under half a tile per compute unit on average) that its per-tile scheduling latency costs
        more than the launch gaps of one kernel per layer */
     int mode = dse_group->mode;
-    if (mode == 2) mode = aspen_hip_graph_parallelism (rp->graph) < AUTO_LAYERS_BELOW ? 0 : 1;
+    if (mode == 2)
+    {
+        /* graphs the timing tuner produced carry its verdict; it counts when all graphs of the pool agree */
+        int tuned = rp->num_nasms ? rp->nasms[0]->preferred_mode : -1;
+        for (unsigned int i = 1; i < rp->num_nasms; i++) if (rp->nasms[i]->preferred_mode != tuned) tuned = -1;
+        mode = tuned >= 0 ? tuned : (aspen_hip_graph_parallelism (rp->graph) < AUTO_LAYERS_BELOW ? 0 : 1);
+    }
     dse_group->last_mode = mode;
     if (mode == 0)
     {

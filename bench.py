@@ -34,18 +34,18 @@ FLOP_PER_UNIT = {
     "bert_base": 1.7459e8, "gpt2": 1.8877e8,
 }
 WORKLOADS = {
-    # name: (configs, unit, units per step, tiles wanted per layer)
-    # The last entry is what the library's timing tuner (apu_generate_nasm) settles on for the
-    # configuration, fixed here so that a bench run does not spend its time tuning; the reference ships
-    # its tile graphs tuned per model and batch in the same way.
-    "resnet50_b32": (["resnet50_b32"], "img/s", 32, 1536),
-    "resnet50_b1": (["resnet50_b1"], "img/s", 1, 128),
-    "vgg16_b32": (["vgg16_b32"], "img/s", 32, 1536),
-    "co_resnet50_vgg16_b16": (["resnet50_b16", "vgg16_b16"], "img/s", 32, 1536),
-    "bert_base_b8_s128": (["bert_base_b8_s128"], "tokens/s", 8 * 128, 128),
-    "gpt2_b4_s512": (["gpt2_b4_s512"], "tokens/s", 4 * 512, 384),
-    "yolov3_b1": (["yolov3_b1"], "img/s", 1, 512),
-    "yolov3_b8": (["yolov3_b8"], "img/s", 8, 1536),
+    # name: (configs, unit, units per step, tiles wanted per layer, engine)
+    # The last two entries are what the library's timing tuner (apu_generate_nasm: candidate tile counts on
+    # both engines) settles on for the configuration, fixed here so that a bench run does not spend its time
+    # tuning; the reference ships its tile graphs tuned per model and batch in the same way.
+    "resnet50_b32": (["resnet50_b32"], "img/s", 32, 1536, "dataflow"),
+    "resnet50_b1": (["resnet50_b1"], "img/s", 1, 128, "layers"),
+    "vgg16_b32": (["vgg16_b32"], "img/s", 32, 1536, "dataflow"),
+    "co_resnet50_vgg16_b16": (["resnet50_b16", "vgg16_b16"], "img/s", 32, 1536, "dataflow"),
+    "bert_base_b8_s128": (["bert_base_b8_s128"], "tokens/s", 8 * 128, 192, "dataflow"),
+    "gpt2_b4_s512": (["gpt2_b4_s512"], "tokens/s", 4 * 512, 384, "dataflow"),
+    "yolov3_b1": (["yolov3_b1"], "img/s", 1, 768, "layers"),
+    "yolov3_b8": (["yolov3_b8"], "img/s", 8, 1536, "dataflow"),
 }
 
 
@@ -121,7 +121,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="resnet50_b32", choices=list(WORKLOADS))
     ap.add_argument("--mode", default="auto", choices=["auto", "dataflow", "layers"],
-                    help="auto (the library's default): persistent dataflow kernel unless the graph has too little parallelism for it")
+                    help="auto: the engine the timing tuner picks for the workload (the persistent dataflow kernel except at batch 1)")
     ap.add_argument("--min-ninst", type=int, default=0, help="tiles wanted per layer (0: the workload's tuned value)")
     ap.add_argument("--workgroups", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -161,9 +161,11 @@ def main():
                           "GB_per_s": 2 * nbytes * args.steps / (ms.value * 1e-3) / 1e9}))
         return
     L.aspen_hip_set_flags((1 if args.skip_tiles else 0) | (4 if args.engine_profile else 0) | (8 if args.trace else 0))
-    cfgs, unit, units_per_step, tuned_min_ninst = WORKLOADS[args.workload]
+    cfgs, unit, units_per_step, tuned_min_ninst, tuned_engine = WORKLOADS[args.workload]
     if args.min_ninst <= 0:
         args.min_ninst = tuned_min_ninst
+    if args.mode == "auto":
+        args.mode = tuned_engine
 
     pool = api.RPool()
     dse = api.DseGroup(1, {"auto": api.MODE_AUTO, "dataflow": api.MODE_DATAFLOW, "layers": api.MODE_LAYERS}[args.mode], args.workgroups)
