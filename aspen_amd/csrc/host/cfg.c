@@ -67,6 +67,7 @@ static section_t *read_sections (const char *path, int *count)
     if (fp == NULL) { ERROR_PRTF ("Couldn't open cfg file %s\n", path); return NULL; }
     int cap = 64, n = 0, skipping = 0;
     section_t *secs = calloc (cap, sizeof (section_t));
+    if (secs == NULL) { ERROR_PRTF ("Out of host memory reading %s\n", path); fclose (fp); return NULL; }
     char line[512];
     while (fgets (line, sizeof (line), fp))
     {
@@ -76,7 +77,13 @@ static section_t *read_sections (const char *path, int *count)
         {
             if (section_type (p) == NO_LAYER_TYPE) { ERROR_PRTF ("Unsupported section type: %s\n", p); skipping = 1; continue; }
             skipping = 0;
-            if (n == cap) { cap *= 2; secs = realloc (secs, cap * sizeof (section_t)); memset (secs + n, 0, (cap - n) * sizeof (section_t)); }
+            if (n == cap)
+            {
+                section_t *grown = realloc (secs, 2 * (size_t)cap * sizeof (section_t));
+                if (grown == NULL) { ERROR_PRTF ("Out of host memory reading %s\n", path); free (secs); fclose (fp); return NULL; }
+                secs = grown; cap *= 2;
+                memset (secs + n, 0, (size_t)(cap - n) * sizeof (section_t));
+            }
             strncpy (secs[n].name, p, sizeof (secs[n].name) - 1);
             n++;
             continue;
@@ -216,10 +223,12 @@ aspen_dnn_t *aspen_parse_cfg (const char *path)
         return NULL;
     }
     aspen_dnn_t *dnn = calloc (1, sizeof (aspen_dnn_t));
+    if (dnn == NULL) { ERROR_PRTF ("Out of host memory reading %s\n", path); free (secs); return NULL; }
     strncpy (dnn->name, path, MAX_STRING_LEN - 1);
     dnn->element_size = sizeof (float);
     dnn->num_layers = n;
     dnn->layers = calloc (n, sizeof (aspen_layer_t));
+    if (dnn->layers == NULL) { ERROR_PRTF ("Out of host memory reading %s\n", path); free (dnn); free (secs); return NULL; }
     int bad = 0;
     for (int i = 0; i < n && !bad; i++)
     {

@@ -27,7 +27,7 @@ static void fill_uniform (aspen_tensor_t *t, uint64_t *state, float range)
     }
 }
 
-static void create_layer_tensors (aspen_layer_t *L, uint64_t *rng)
+static int create_layer_tensors (aspen_layer_t *L, uint64_t *rng)
 {
     const unsigned int *p = L->params;
     switch (L->type)
@@ -36,21 +36,30 @@ static void create_layer_tensors (aspen_layer_t *L, uint64_t *rng)
     case FC_LAYER:      L->gemm_m = p[OUT_C]; L->gemm_k = p[IN_H] * p[IN_W] * p[IN_C]; break;
     case MATMUL_LAYER:  L->gemm_m = p[MAT_M]; L->gemm_k = p[MAT_K]; break;
     case LAYERNORM_LAYER: L->gemm_m = p[MAT_M]; L->gemm_k = 1; break;
-    default: return;
+    default: return 0;
     }
     alloc_tensor (&L->weight, (size_t)L->gemm_m * L->gemm_k);
     alloc_tensor (&L->bias, L->gemm_m);
+    if (L->weight.data == NULL || L->bias.data == NULL)
+    {
+        ERROR_PRTF ("layer %u: out of host memory for %zu weights\n", L->layer_idx, (size_t)L->gemm_m * L->gemm_k);
+        free (L->weight.data); free (L->bias.data);
+        L->weight.data = L->bias.data = NULL; L->weight.num_elements = L->bias.num_elements = 0;
+        return -1;
+    }
     fill_uniform (&L->weight, rng, 0.3f);
     fill_uniform (&L->bias, rng, 0.3f);
+    return 0;
 }
 
 /* tensors of a layer whose parameters are known, zero filled (the .aspen reader fills them) */
-void aspen_create_layer_tensors (aspen_layer_t *L)
+int aspen_create_layer_tensors (aspen_layer_t *L)
 {
     uint64_t rng = 1;
-    create_layer_tensors (L, &rng);
+    if (create_layer_tensors (L, &rng)) return -1;
     if (L->weight.data) memset (L->weight.data, 0, L->weight.num_elements * sizeof (float));
     if (L->bias.data) memset (L->bias.data, 0, L->bias.num_elements * sizeof (float));
+    return 0;
 }
 
 aspen_dnn_t *apu_create_dnn (char *input_path, char *data_path)
@@ -60,7 +69,7 @@ aspen_dnn_t *apu_create_dnn (char *input_path, char *data_path)
     if (dnn == NULL) return NULL;
     uint64_t rng = 0x5851f42d4c957f2dull;
     for (unsigned int i = 0; i < dnn->num_layers; i++)
-        create_layer_tensors (&dnn->layers[i], &rng);
+        if (create_layer_tensors (&dnn->layers[i], &rng)) { apu_destroy_dnn (dnn); return NULL; }
     if (data_path != NULL)
         aspen_load_weight_file (dnn, data_path);   /* a missing or broken file only prints, as in the reference */
     return dnn;
@@ -288,6 +297,7 @@ int aspen_layer_to_device (aspen_layer_t *L, unsigned int parent_ld)
     if (!L->d_bias || aspen_hip_h2d (L->d_bias, L->bias.data, L->gemm_m * sizeof (float))) return -1;
     /* k-chunk table: chunk c covers K positions [4c, 4c+4) = tap (4c / icp), channels (4c % icp).. */
     aspen_hip_ktab_t *tab = calloc (kp / 4, sizeof (aspen_hip_ktab_t));
+    if (tab == NULL) return -1;
     for (unsigned int c = 0; c < kp / 4; c++)
     {
         const unsigned int tap = (c * 4) / icp, ch = (c * 4) % icp;
@@ -302,5 +312,3 @@ int aspen_layer_to_device (aspen_layer_t *L, unsigned int parent_ld)
     L->dev_kp = kp; L->dev_icp = icp; L->dev_in_ld = parent_ld;
     return rc;
 }
-
-

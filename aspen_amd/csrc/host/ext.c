@@ -178,5 +178,5 @@ void print_rpool_info (rpool_t *rp)
         rp->num_nasms, rp->ref_dses, aspen_rpool_num_ninst (rp));
     for (unsigned int i = 0; i < rp->num_nasms; i++)
         printf ("\tnasm %u (%s): %u ninsts, %s\n", rp->nasms[i]->nasm_id, rp->nasms[i]->dnn->name, rp->nasms[i]->num_ninst,
-            rp->nasms[i]->completed == 1 ? "completed" : rp->nasms[i]->completed == 2 ? "in flight" : rp->nasms[i]->armed ? "armed" : "idle");
+            rp->nasms[i]->completed == 1 ? "completed" : rp->nasms[i]->completed == 2 ? "in flight" : rp->nasms[i]->completed == 3 ? "failed" : rp->nasms[i]->armed ? "armed" : "idle");
 }

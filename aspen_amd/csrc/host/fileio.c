@@ -81,6 +81,12 @@ void apu_save_dnn_to_file (aspen_dnn_t *dnn, char *filename)
                 /* [M/8][K][8], K in the order the dimension list spells out */
                 const unsigned int M = L->gemm_m, K = L->gemm_k, G = (M + VEC_M - 1) / VEC_M;
                 float *packed = calloc ((size_t)G * K * VEC_M, sizeof (float));
+                if (packed == NULL)
+                {
+                    ERROR_PRTF ("Error: apu_save_dnn_to_file: out of host memory; %s is incomplete.\n", filename);
+                    fclose (fp);
+                    return;
+                }
                 for (unsigned int m = 0; m < M; m++)
                     for (unsigned int k = 0; k < K; k++)
                         packed[((size_t)(m / VEC_M) * K + k) * VEC_M + m % VEC_M] = L->weight.data[(size_t)m * K + k];
@@ -180,7 +186,7 @@ static int place_tensor (aspen_layer_t *L, int slot, const int *order, int num_d
     return 0;    /* tensors this build has no use for (anchors, BN statistics already folded) are skipped */
 }
 
-void aspen_create_layer_tensors (aspen_layer_t *L);     /* dnn.c */
+int aspen_create_layer_tensors (aspen_layer_t *L);      /* dnn.c */
 
 aspen_dnn_t *apu_load_dnn_from_file (char *filename)
 {
@@ -194,6 +200,7 @@ aspen_dnn_t *apu_load_dnn_from_file (char *filename)
     if (next_line (fp, line, "ASPEN_DNN") == NULL || next_line (fp, line, "ASPEN_BUILD:") == NULL) goto fail;
     if ((ptr = next_line (fp, line, "DNN_NAME:")) == NULL) goto fail;
     dnn = calloc (1, sizeof (aspen_dnn_t));
+    if (dnn == NULL) goto fail;
     strncpy (dnn->name, ptr, MAX_STRING_LEN - 1);
     if ((ptr = next_line (fp, line, "DNN_ELEMENT_SIZE:")) == NULL) goto fail;
     dnn->element_size = (unsigned int)atoi (ptr);
@@ -202,6 +209,7 @@ aspen_dnn_t *apu_load_dnn_from_file (char *filename)
     dnn->num_layers = (unsigned int)atoi (ptr);
     if (dnn->num_layers == 0 || dnn->num_layers > 65535) goto fail;
     dnn->layers = calloc (dnn->num_layers, sizeof (aspen_layer_t));
+    if (dnn->layers == NULL) { dnn->num_layers = 0; goto fail; }
     for (unsigned int i = 0; i < dnn->num_layers; i++)
     {
         aspen_layer_t *L = &dnn->layers[i];
@@ -210,8 +218,10 @@ aspen_dnn_t *apu_load_dnn_from_file (char *filename)
         L->layer_idx = (unsigned int)atoi (ptr);
         if ((ptr = next_line (fp, line, "LAYER_TYPE:")) == NULL) goto fail;
         L->type = (LAYER_TYPE)atoi (ptr);
+        if ((int)L->type < 0 || (int)L->type >= NUM_LAYER_ELEMENTS) { ERROR_PRTF ("ASPEN DNN file %s: layer %u has unknown type %d.\n", filename, i, (int)L->type); goto fail; }
         if ((ptr = next_line (fp, line, "LAYER_ACTIVATION:")) == NULL) goto fail;
         L->activation = (LAYER_ACT)atoi (ptr);
+        if ((int)L->activation < 0 || (int)L->activation >= NUM_ACTIVATIONS) { ERROR_PRTF ("ASPEN DNN file %s: layer %u has unknown activation %d.\n", filename, i, (int)L->activation); goto fail; }
         if (next_line (fp, line, "LAYER_PARENTS:") == NULL) goto fail;
         for (int j = 0; j < NUM_PARENT_ELEMENTS; j++)
         {
@@ -227,7 +237,7 @@ aspen_dnn_t *apu_load_dnn_from_file (char *filename)
             L->params[a] = (unsigned int)b;
         }
         if (next_line (fp, line, "LAYER_PARAMS_END") == NULL || next_line (fp, line, "LAYER_TENSORS:") == NULL) goto fail;
-        aspen_create_layer_tensors (L);
+        if (aspen_create_layer_tensors (L)) goto fail;
         for (int j = 0; j < NUM_TENSORS; j++)
         {
             int slot, present;
@@ -283,8 +293,10 @@ static void parent_lists (const nasm_t *nasm, uint32_t **off_out, uint32_t **idx
 {
     const uint32_t n = nasm->num_ninst;
     uint32_t *off = calloc ((size_t)n + 2, sizeof (uint32_t)), *idx = calloc (nasm->num_edges ? nasm->num_edges : 1, sizeof (uint32_t));
-    for (uint32_t t = 0; t < n; t++) off[t + 1] = off[t] + nasm->num_parents[t];
     uint32_t *cur = calloc (n ? n : 1, sizeof (uint32_t));
+    *off_out = *idx_out = NULL;
+    if (off == NULL || idx == NULL || cur == NULL) { free (off); free (idx); free (cur); return; }
+    for (uint32_t t = 0; t < n; t++) off[t + 1] = off[t] + nasm->num_parents[t];
     for (uint32_t t = 0; t < n; t++)                       /* parents in increasing order, as tiles are visited in order */
         for (uint32_t c = nasm->child_off[t]; c < nasm->child_off[t + 1]; c++)
         {
@@ -303,6 +315,7 @@ void apu_save_nasm_to_file (nasm_t *nasm, char *filename)
     if (fp == NULL) { ERROR_PRTF ("Error: apu_save_nasm_to_file Failed to open file %s for writing\n", filename); return; }
     uint32_t *poff, *pidx;
     parent_lists (nasm, &poff, &pidx);
+    if (poff == NULL) { ERROR_PRTF ("Error: apu_save_nasm_to_file: out of host memory.\n"); fclose (fp); return; }
     fprintf (fp, "ASPEN_NASM\n");
     fprintf (fp, "DNN_NAME:%s\n", nasm->dnn->name);
     fprintf (fp, "NUM_BATCH:%u\n", nasm->batch_size);
@@ -359,6 +372,7 @@ nasm_t *apu_load_nasm_from_file (char *filename, aspen_dnn_t *dnn)
     }
     /* the tile list: cross-checked when it is this build's grid, skipped when it is another build's */
     parent_lists (nasm, &poff, &pidx);
+    if (poff == NULL) goto fail;
     uint32_t count = 0;
     int own_grid = 1, mismatch = 0;
     for (;;)

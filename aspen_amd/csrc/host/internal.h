@@ -99,7 +99,7 @@ struct nasm_t
     float *d_arena;
     rpool_t *rpool;                          /* pool this nasm is attached to */
     int armed;                               /* input present and counters to be re-armed at the next run */
-    int completed;
+    int completed;                           /* 0 not run, 1 completed, 2 in flight, 3 the run failed (stall, launch error) */
 };
 
 #define RPOOL_MAX_NASMS 64

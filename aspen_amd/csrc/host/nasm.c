@@ -57,10 +57,12 @@ static int set_out_mat (nasm_t *nasm, nasm_ldata_t *ld)
         ld->out_mat_dims[OUT_H] = p[MAT_M]; ld->out_mat_dims[OUT_W] = S * B;
         break;
     case K_ATTENTION_LAYER:
+        if (p[NUM_HEAD] == 0) { ERROR_PRTF ("layer %u: attention layer without heads\n", L->layer_idx); return -1; }
         flop_per_out = 2ull * p[NUM_HIDDEN] / p[NUM_HEAD];
         ld->out_mat_dims[OUT_H] = S; ld->out_mat_dims[OUT_W] = S * p[NUM_HEAD] * B;
         break;
     case V_ATTENTION_LAYER:
+        if (p[NUM_HEAD] == 0) { ERROR_PRTF ("layer %u: attention layer without heads\n", L->layer_idx); return -1; }
         flop_per_out = 2ull * S;
         ld->out_mat_dims[OUT_H] = p[MAT_M]; ld->out_mat_dims[OUT_W] = S * B;
         break;
@@ -212,7 +214,13 @@ void aspen_nasm_tile_range_internal (const nasm_ldata_t *ld, unsigned int t, uns
 typedef struct { uint32_t *v; size_t n, cap; } u32vec;
 static void push (u32vec *a, uint32_t x)
 {
-    if (a->n == a->cap) { a->cap = a->cap ? a->cap * 2 : 1024; a->v = realloc (a->v, a->cap * sizeof (uint32_t)); }
+    if (a->n == a->cap)
+    {
+        const size_t cap = a->cap ? a->cap * 2 : 1024;
+        uint32_t *v = realloc (a->v, cap * sizeof (uint32_t));
+        if (v == NULL) { ERROR_PRTF ("ERROR: out of host memory while building the tile graph.\n"); abort (); }
+        a->v = v; a->cap = cap;
+    }
     a->v[a->n++] = x;
 }
 
@@ -362,6 +370,7 @@ static int build_graph (nasm_t *nasm)
     nasm->num_parents = calloc (n ? n : 1, sizeof (uint32_t));
     nasm->child_off = calloc ((size_t)n + 2, sizeof (uint32_t));
     u32vec edges_parent = {0}, edges_child = {0}, tmp = {0};
+    if (nasm->ninst_ldata == NULL || nasm->num_parents == NULL || nasm->child_off == NULL) return -1;
     for (unsigned int l = 0; l < nasm->num_ldata; l++)
     {
         const nasm_ldata_t *ld = &nasm->ldata_arr[l];
@@ -377,7 +386,12 @@ static int build_graph (nasm_t *nasm)
             {
                 if (tmp.v[i] == prev) continue;         /* the two parents of a shortcut may be the same tile */
                 prev = tmp.v[i];
-                if (prev >= id) { ERROR_PRTF ("tile %u depends on a later tile %u\n", id, prev); return -1; }
+                if (prev >= id)
+                {
+                    ERROR_PRTF ("tile %u depends on a later tile %u\n", id, prev);
+                    free (edges_parent.v); free (edges_child.v); free (tmp.v);
+                    return -1;
+                }
                 /* A parent in a split layer stands for its group of `splits` partial tiles: the member
                    that finishes last completes the output and releases the children, so every member
                    carries the child list and the child counts the group once. */
@@ -395,6 +409,11 @@ static int build_graph (nasm_t *nasm)
     nasm->num_edges = (uint32_t)edges_parent.n;
     nasm->child_idx = calloc (edges_parent.n ? edges_parent.n : 1, sizeof (uint32_t));
     uint32_t *cursor = calloc (n ? n : 1, sizeof (uint32_t));
+    if (nasm->child_idx == NULL || cursor == NULL)
+    {
+        free (cursor); free (edges_parent.v); free (edges_child.v); free (tmp.v);
+        return -1;
+    }
     for (size_t e = 0; e < edges_parent.n; e++)
     {
         const uint32_t pnt = edges_parent.v[e];
@@ -439,13 +458,15 @@ static nasm_t *build_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned in
     if (dnn == NULL) { ERROR_PRTF ("apu_create_nasm: dnn is NULL\n"); return NULL; }
     if (min_ninst < 1) { ERROR_PRTF ("ERROR: min_ninst_per_ldata should be at least 1\n"); return NULL; }
     nasm_t *nasm = calloc (1, sizeof (nasm_t));
+    if (nasm == NULL) { ERROR_PRTF ("apu_create_nasm: out of host memory\n"); return NULL; }
     nasm->kiters_cap = kiters_cap;
     nasm->preferred_mode = -1;
     nasm->dnn = dnn; nasm->nasm_id = nasm_counter++;
     nasm->batch_size = batch > 0 ? batch : 1;
     nasm->tr_seq_len = seq; nasm->min_ninst_per_ldata = min_ninst;
     nasm->num_ldata = dnn->num_layers;
-    nasm->ldata_arr = calloc (nasm->num_ldata, sizeof (nasm_ldata_t));
+    nasm->ldata_arr = calloc (nasm->num_ldata ? nasm->num_ldata : 1, sizeof (nasm_ldata_t));
+    if (nasm->ldata_arr == NULL) { ERROR_PRTF ("apu_create_nasm: out of host memory\n"); free (nasm); return NULL; }
     size_t arena = 0;
     unsigned int total = 0;
     int bad = 0;
@@ -497,6 +518,7 @@ static double nasm_parallelism (const nasm_t *nasm)
     const uint32_t n = nasm->num_ninst;
     if (n == 0) return 0.0;
     float *dist = calloc (n, sizeof (float));
+    if (dist == NULL) return 0.0;
     double total = 0.0, longest = 0.0;
     for (uint32_t t = 0; t < n; t++)
     {
@@ -638,6 +660,7 @@ void apu_destroy_nasm (nasm_t *nasm)
                 break;
             }
     }
+    if (nasm->d_arena != NULL) aspen_hip_sync ();      /* a run still in flight reads and writes the arena */
     aspen_hip_free (nasm->d_arena);
     free (nasm->ninst_ldata); free (nasm->num_parents); free (nasm->child_off); free (nasm->child_idx);
     free (nasm->ldata_arr);
@@ -651,8 +674,6 @@ void apu_reset_nasm (nasm_t *nasm)
     nasm->completed = 0;
     nasm->armed = 1;
 }
-
-
 
 /* ---- device ------------------------------------------------------------------------------------ */
 int aspen_nasm_to_device (nasm_t *nasm)

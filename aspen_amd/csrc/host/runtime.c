@@ -17,6 +17,7 @@
 rpool_t *rpool_init (void)
 {
     rpool_t *rp = calloc (1, sizeof (rpool_t));
+    if (rp == NULL) { ERROR_PRTF ("ERROR: rpool_init: out of host memory.\n"); return NULL; }
     rp->graph_dirty = 1;
     return rp;
 }
@@ -84,6 +85,12 @@ void rpool_add_nasm (rpool_t *rpool, nasm_t *nasm, char *input_filename)
     const unsigned int *p = ld->layer->params;
     const size_t H = ld->out_mat_dims[OUT_H], W = ld->out_mat_dims[OUT_W], n = H * W;
     float *file = calloc (n, sizeof (float)), *dense = calloc (n, sizeof (float));
+    if (file == NULL || dense == NULL)
+    {
+        ERROR_PRTF ("ERROR: rpool_add_nasm: out of host memory.\n");
+        free (file); free (dense);
+        return;
+    }
     if (input_filename != NULL)
     {
         FILE *fp = fopen (input_filename, "rb");
@@ -146,6 +153,11 @@ static int rebuild_graph (rpool_t *rp)
     uint32_t *roots = calloc (ninst + 1, sizeof (uint32_t));
     uint32_t lbase = 0, nbase = 0, ebase = 0, nroots = 0;
     int rc = 0;
+    if (L == NULL || nl == NULL || np == NULL || co == NULL || ci == NULL || roots == NULL)
+    {
+        ERROR_PRTF ("ERROR: out of host memory while merging the graphs of the pool.\n");
+        rc = -1;
+    }
     for (unsigned int i = 0; i < rp->num_nasms && !rc; i++)
     {
         nasm_t *g = rp->nasms[i];
@@ -160,7 +172,7 @@ static int rebuild_graph (rpool_t *rp)
         for (uint32_t e = 0; e < g->num_edges; e++) ci[ebase + e] = nbase + g->child_idx[e];
         lbase += g->num_ldata; nbase += g->num_ninst; ebase += g->num_edges;
     }
-    co[ninst] = edges;
+    if (!rc) co[ninst] = edges;
     /* roots of the attached graphs taken in turns, so co-scheduled networks start together */
     if (!rc)
     {
@@ -192,6 +204,7 @@ static int rebuild_graph (rpool_t *rp)
 dse_group_t *dse_group_init (unsigned int num_dse)
 {
     dse_group_t *g = calloc (1, sizeof (dse_group_t));
+    if (g == NULL) { ERROR_PRTF ("ERROR: dse_group_init: out of host memory.\n"); return NULL; }
     g->num_dses = num_dse;
     g->mode = 2;
     g->last_mode = -1;
@@ -259,12 +272,12 @@ void dse_group_run (dse_group_t *dse_group)
 static void finish (rpool_t *rp)
 {
     if (rp == NULL || !rp->running) return;
-    if (aspen_hip_sync ()) ERROR_PRTF ("ERROR: device run failed: %s\n", aspen_hip_last_error ());
-    uint32_t executed = 0, twice = 0, aborted = 0;
+    /* a run the device gave up (watchdog, launch error) leaves its graphs NOT completed: 3 = failed */
+    int state = 1;
+    if (aspen_hip_sync ()) { ERROR_PRTF ("ERROR: device run failed: %s\n", aspen_hip_last_error ()); state = 3; }
     rp->running = 0;
     for (unsigned int i = 0; i < rp->num_nasms; i++)
-        if (rp->nasms[i]->completed == 2) rp->nasms[i]->completed = 1;
-    (void)executed; (void)twice; (void)aborted;
+        if (rp->nasms[i]->completed == 2) rp->nasms[i]->completed = state;
 }
 
 void dse_group_stop (dse_group_t *dse_group)
@@ -317,6 +330,7 @@ ssize_t dse_get_ldata_result (nasm_t *nasm, unsigned int ldata_idx, LAYER_PARAMS
         total += bytes[n++];
     }
     char *outp = calloc (total ? (size_t)total : 1, 1);
+    if (outp == NULL) { for (int i = 0; i < n; i++) free (parts[i]); return -1; }
     size_t off = 0;
     const size_t B = nasm->batch_size;
     for (size_t b = 0; b < B; b++)
@@ -337,6 +351,11 @@ static ssize_t get_ldata_output (nasm_t *nasm, unsigned int ldata_idx, LAYER_PAR
     if (out_ptr == NULL) { ERROR_PRTF ("Error in get_ldata_output: out_ptr is NULL.\n"); return -1; }
     if (nasm->d_arena == NULL) { ERROR_PRTF ("Error in get_ldata_output: nasm has not been run.\n"); return -1; }
     if (nasm->completed == 2) finish (nasm->rpool);
+    if (nasm->completed == 3 && ldata_idx != 0)
+    {
+        ERROR_PRTF ("Error in get_ldata_output: the last run of this nasm failed; its layers hold no valid result.\n");
+        return -1;
+    }
     const nasm_ldata_t *ld = &nasm->ldata_arr[ldata_idx];
     const aspen_layer_t *L = ld->layer;
     if (ld->out_discarded)
@@ -404,6 +423,7 @@ static ssize_t get_ldata_output (nasm_t *nasm, unsigned int ldata_idx, LAYER_PAR
     size_t nstride[NUM_PARAM_ELEMENTS] = {0}, s = 1;
     for (int i = nd - 1; i >= 0; i--) { nstride[native[i]] = s; s *= dim[native[i]]; }
     float *out = calloc (H * W, sizeof (float));
+    if (out == NULL) { free (dense); return -1; }
     size_t idx[4] = {0, 0, 0, 0};
     for (size_t o = 0; o < H * W; o++)
     {

@@ -324,6 +324,11 @@ def test_stalled_run_is_reported_and_the_next_runs_recover(gpu, capfd):
         st = net.rpool.run_stats()
         assert st["aborted"] == 1 and st["executed"] < net.nasm.num_ninst, st
         assert "stalled" in capfd.readouterr().err
+        # a run that was given up does not count as completed and hands out no results
+        assert api.lib().dse_check_nasm_completion(net.nasm.h) == 0
+        with pytest.raises(RuntimeError):
+            net.layer(net.nasm.num_ldata - 1)
+        capfd.readouterr()
         api.lib().aspen_dse_group_set_spin_limit(net.dse.h, 0)
         for mode in (api.MODE_DATAFLOW, api.MODE_LAYERS, api.MODE_DATAFLOW):
             net.dse.set_mode(mode)
