@@ -489,6 +489,13 @@ template <class T> static T *upload (const T *src, size_t n)
 static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
 {
     const char *why = nullptr;
+    // buffer descriptors carry 32-bit sizes: this holds for every matrix, also one no tile of its own layer writes
+    if ((uint64_t)L.N * L.ld * 4 * (L.splits > 1 ? L.splits : 1) >= 0xffffff00ull)
+    {
+        snprintf (g_err, sizeof (g_err), "layer %u rejected: matrix larger than 4 GiB", idx);
+        fprintf (stderr, "aspen_hip: %s\n", g_err);
+        return -1;
+    }
     if (L.type == INPUT_LAYER || L.num_ninst == 0) return 0;     // no tiles: written by the host, or by another layer's epilogue
     if (!L.out || !L.in0) why = "missing buffers";
     else if (L.ld % 4 || L.ld0 % 4 || (L.in1 && L.ld1 % 4)) why = "strides must be multiples of 4 floats";
@@ -496,7 +503,8 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
         || L.num_ninst != L.tiles_m * L.tiles_n * L.splits) why = "tile grid";
     else if (L.splits > 1 && (!L.partial || L.kiters_per_split == 0 || (uint64_t)L.splits * L.kiters_per_split * GEMM_BK < L.Kp
         || !(L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER))) why = "split-K geometry";
-    else if ((uint64_t)L.N * L.ld * 4 * L.splits >= 0xffffff00ull) why = "matrix larger than 4 GiB";
+    else if ((L.type == CONV_LAYER || L.type == MAXPOOL_LAYER || L.type == AVGPOOL_LAYER)
+        && (L.stride == 0 || L.KH == 0 || L.KW == 0 || L.IH == 0 || L.IW == 0 || L.OH == 0 || L.OW == 0 || L.N % (L.OH * L.OW))) why = "window geometry";
     else if (L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER)
     {
         uint32_t shp[9];
@@ -531,12 +539,12 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
     }
     else if (L.type == YOLO_LAYER)
     {
-        if (!L.weight || L.M < 5 || L.IC % L.M || L.IC / L.M > 3 || L.tiles_m != 1 || L.ld0 < L.IC) why = "yolo geometry";
+        if (!L.weight || L.M < 5 || L.IC % L.M || L.IC / L.M > 3 || L.IC == 0 || L.IH == 0 || L.IW == 0 || L.tiles_m != 1 || L.ld0 < L.IC) why = "yolo geometry";
         else if (L.N % (L.IH * L.IW * (L.IC / L.M))) why = "yolo columns";
     }
     else if (L.type == APPEND_LAYER)
     {
-        if (!L.in1 || L.stride == 0 || L.OH % L.stride || L.OW % L.stride || L.IC >= L.M || L.tiles_m != 1
+        if (!L.in1 || L.stride == 0 || L.OH == 0 || L.OW == 0 || L.OH % L.stride || L.OW % L.stride || L.IC >= L.M || L.tiles_m != 1
             || L.ld0 < L.IC || L.ld1 < L.M - L.IC || L.N % (L.OH * L.OW)) why = "append geometry";
     }
     else if (L.type == RESIDUAL_LAYER) { if (!L.in1 || L.tiles_m != 1) why = "missing second parent, or row tiles"; }
@@ -587,6 +595,7 @@ static double graph_parallelism (const aspen_hip_layer_t *layers, const uint32_t
 {
     if (num_ninst == 0) return 0.0;
     float *dist = (float *)calloc (num_ninst, sizeof (float));
+    if (!dist) return 1e30;
     double total = 0.0, longest = 0.0;
     bool ordered = true;
     for (uint32_t t = 0; t < num_ninst && ordered; t++)
@@ -625,6 +634,7 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     const uint32_t num_edges = child_off[num_ninst];
     {
         uint32_t *seen = (uint32_t *)calloc (num_ninst ? num_ninst : 1, sizeof (uint32_t));
+        if (!seen) { snprintf (g_err, sizeof (g_err), "out of host memory"); return nullptr; }
         bool ok = true;
         // the members of a split-K group carry the same child list and count as one parent
         for (uint32_t t = 0; t < num_ninst && ok; t++)
@@ -646,6 +656,7 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
         if (!ok) { snprintf (g_err, sizeof (g_err), "inconsistent dependency arrays"); fprintf (stderr, "aspen_hip: %s\n", g_err); return nullptr; }
     }
     aspen_hip_graph_t *g = (aspen_hip_graph_t *)calloc (1, sizeof (aspen_hip_graph_t));
+    if (!g) { snprintf (g_err, sizeof (g_err), "out of host memory"); return nullptr; }
     g->cached_loads = lines_have_one_producer (layers, num_layers) && getenv ("ASPEN_GPU_COHERENT_LOADS") == nullptr;
     g->num_layers = num_layers; g->num_ninst = num_ninst; g->num_roots = num_roots; g->num_edges = num_edges;
     {
@@ -661,7 +672,8 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
         if (getenv ("ASPEN_GPU_VERBOSE"))
             fprintf (stderr, "aspen_hip: %u tiles, average parallelism %.0f: %u workgroups by default\n", num_ninst, par, g->default_workgroups);
     }
-    g->h_layers = (aspen_hip_layer_t *)malloc (sizeof (aspen_hip_layer_t) * num_layers);
+    g->h_layers = (aspen_hip_layer_t *)malloc (sizeof (aspen_hip_layer_t) * (num_layers ? num_layers : 1));
+    if (!g->h_layers) { snprintf (g_err, sizeof (g_err), "out of host memory"); free (g); return nullptr; }
     memcpy (g->h_layers, layers, sizeof (aspen_hip_layer_t) * num_layers);
     g->d_layers = upload (layers, num_layers);
     g->d_ninst_layer = upload (ninst_layer, num_ninst);
@@ -674,14 +686,14 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     {
         // child records: what the publishing wavefront fetches with one 64-lane load
         qentry_t *rec = (qentry_t *)calloc ((size_t)(num_ninst ? num_ninst : 1) * CHILD_REC, sizeof (qentry_t));
-        for (uint32_t t = 0; t < num_ninst; t++)
+        for (uint32_t t = 0; rec && t < num_ninst; t++)
         {
             const uint32_t c0 = child_off[t], n = child_off[t + 1] - c0;
             rec[(size_t)t * CHILD_REC] = n;
             for (uint32_t c = 0; c < n && c < CHILD_REC - 1; c++)
                 rec[(size_t)t * CHILD_REC + 1 + c] = ((qentry_t)ninst_layer[child_idx[c0 + c]] << 32) | child_idx[c0 + c];
         }
-        g->d_child_rec = upload (rec, (size_t)num_ninst * CHILD_REC);
+        g->d_child_rec = rec ? upload (rec, (size_t)num_ninst * CHILD_REC) : nullptr;
         free (rec);
     }
     g->d_ran = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
@@ -689,7 +701,7 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     g->d_arrivals = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
     g->d_prof = (unsigned long long *)aspen_hip_alloc (sizeof (unsigned long long) * 8);
     if (!g->d_layers || !g->d_ninst_layer || !g->d_num_parents || !g->d_child_off || !g->d_child_idx || !g->d_roots
-        || !g->d_dep || !g->d_queue || !g->d_ran || !g->d_state || !g->d_child_rec || !g->d_arrivals)
+        || !g->d_dep || !g->d_queue || !g->d_ran || !g->d_state || !g->d_child_rec || !g->d_arrivals || !g->d_prof)
     {
         aspen_hip_graph_destroy (g);
         return nullptr;

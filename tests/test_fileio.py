@@ -71,6 +71,20 @@ def test_aspen_file_errors(tmp_path, capfd):
     assert capfd.readouterr().err != ""
 
 
+@pytest.mark.parametrize("field, value", [(b"LAYER_TYPE:", b"99"), (b"LAYER_TYPE:", b"-3"), (b"LAYER_ACTIVATION:", b"42")])
+def test_aspen_file_with_unknown_ids_is_rejected(tmp_path, field, value, capfd):
+    """A model file whose second layer names a layer type or activation the enumerations do not have
+    (they index the tables of the print_* dumps and select device code) does not load."""
+    raw = open(REF_ASPEN, "rb").read()
+    first = raw.index(field)
+    at = raw.index(field, first + 1) + len(field)
+    end = raw.index(b"\n", at)
+    bad = tmp_path / "bad.aspen"
+    bad.write_bytes(raw[:at] + value + raw[end:])
+    assert not api.lib().apu_load_dnn_from_file(str(bad).encode())
+    assert "unknown" in capfd.readouterr().err
+
+
 def test_nasm_file_round_trip_and_cross_check(tmp_path, capfd):
     L = api.lib()
     d = dnn_from_cfg(tmp_path)
