@@ -25,7 +25,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the persistent kernel, measured with rocprofv3 FETCH_SIZE / WRITE_SIZE passes
 # calibrated on the library's copy kernel (summary: profiles/dataflow_kernel_resnet50_b32_hbm_traffic.txt);
 # valid for the default configuration of that workload only
-MEASURED_TRAFFIC_BYTES = {("resnet50_b32", "dataflow", 1536): 10.29e9}
+MEASURED_TRAFFIC_BYTES = {("resnet50_b32", "dataflow", 1536): 10.54e9}
 
 # algorithmic GEMM-class flops per unit (2*M*N*K with the reference's K: padding taps counted, full
 # S x S attention): per image for the vision nets, per token for the transformers
