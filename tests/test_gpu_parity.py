@@ -67,6 +67,26 @@ def test_micro_nets_match_oracle(gpu, name, loads, monkeypatch):
         net.close()
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["resnet_mini_b2", "bert_mini_b2_s24", "yolo_mini_b2"])
+def test_launch_per_layer_reruns_match_oracle(gpu, name):
+    """One launch per layer, six runs on the same graph with changing inputs, each followed by downloads of
+    every layer, every one checked against the oracle; split-K layers (two launches each) included."""
+    from oracle import cpu
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()[name])
+    net = H.GpuNet(cfg, tens, batch, seq, min_ninst=1024, mode=api.MODE_LAYERS)
+    try:
+        for rep in range(6):
+            xin = (x * (1.0 - 0.25 * rep) + 0.125 * rep).astype(np.float32)
+            outs = cpu.run_network(layers, tens, xin, batch, seq)
+            net.run(xin)
+            for l in range(net.nasm.num_ldata):
+                err = H.rel_l2(net.layer(l), outs[l])
+                assert err <= H.REL_L2_TOL, f"run {rep} layer {l} ({layers[l]['type']}): rel L2 {err:.3g}"
+    finally:
+        net.close()
+
+
 def test_engine_rearm_many_runs(gpu):
     """Re-arm and re-run one graph many times: every run must execute each tile exactly once, never
     stall, and reproduce the first run bit for bit (tiles are deterministic; only their order varies)."""
