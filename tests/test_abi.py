@@ -69,3 +69,47 @@ def test_tile_shapes_are_constants():
 def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "ONE GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_error_conventions_of_the_reference_api(tmp_path, capfd):
+    """Constructors return NULL on failure, read-outs return -1 on NULL arguments, other calls print and
+    return (reference main.c:67-71, src/apu.c:229-238); an object that is still referenced is not
+    destroyed (reference src/apu.c:49-54, src/rpool.c:62-66).  No call here touches the GPU."""
+    import ctypes as C
+    from aspen_amd import models as M
+    from tests import helpers as H
+    L = api.lib()
+    assert not L.apu_create_dnn(None, None)
+    assert not L.apu_create_dnn(b"/nonexistent/net.cfg", None)
+    assert not L.apu_create_dnn(b"/nonexistent/net.txt", None)          # only .cfg descriptions are read
+    assert not L.apu_create_nasm(None, 8, 1)
+    assert not L.apu_load_dnn_from_file(None) and not L.apu_load_nasm_from_file(None, None)
+    out = C.c_void_p()
+    assert L.dse_get_nasm_result(None, None, C.byref(out)) == -1
+    assert L.dse_get_ldata_result(None, 0, None, C.byref(out)) == -1
+    assert L.dse_check_nasm_completion(None) == 0
+    for call in (lambda: L.rpool_add_nasm_raw_input(None, None, None), lambda: L.dse_group_run(None),
+                 lambda: L.dse_group_stop(None), lambda: L.dse_group_set_rpool(None, None),
+                 lambda: L.rpool_reset_nasm(None, None), lambda: L.apu_destroy_nasm(None), lambda: L.apu_destroy_dnn(None),
+                 lambda: L.rpool_destroy(None), lambda: L.dse_group_destroy(None), lambda: L.apu_save_nasm_to_file(None, None)):
+        call()                                                           # must return, not crash
+    cfg, layers, tens, x, batch, seq = H.tiny_case()
+    wp = str(tmp_path / "w.bin")
+    M.write_aspen_data(wp, tens)
+    d = api.Dnn(cfg, wp)
+    assert not L.apu_create_nasm(d.h, 0, batch)                          # min_ninst_per_ldata must be at least 1
+    n = api.Nasm(d, batch, seq, 8)
+    L.apu_destroy_dnn(d.h)                                               # refused: a nasm still references it
+    assert "still referencing" in capfd.readouterr().err
+    assert api.Nasm(d, batch, seq, 8).num_ninst == n.num_ninst           # ... and the dnn is still usable
+    assert L.dse_get_ldata_result(n.h, 10 ** 6, None, C.byref(out)) == -1   # layer index out of range
+    assert L.dse_get_nasm_result(n.h, None, C.byref(out)) == -1          # never run: nothing on the device
+    rp, g = L.rpool_init(), L.dse_group_init(4)
+    L.dse_group_set_rpool(g, rp)
+    L.rpool_destroy(rp)                                                  # refused: an engine group still references it
+    assert "still referencing" in capfd.readouterr().err
+    L.dse_group_run(g)                                                   # nothing attached: returns without a launch
+    L.rpool_reset_nasm(rp, n.h)                                          # not in this pool: prints
+    assert "not in rpool" in capfd.readouterr().err
+    L.dse_group_destroy(g)
+    L.rpool_destroy(rp)
