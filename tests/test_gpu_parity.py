@@ -87,6 +87,42 @@ def test_launch_per_layer_reruns_match_oracle(gpu, name):
         net.close()
 
 
+def activation_zoo_cfg():
+    """Every activation the reference's naive_activate knows (reference src/naive_kernels.c:11-57) on a
+    contraction epilogue or a shortcut, a padded max pool and average pool, a [softmax] layer at the end."""
+    s = "[net]\nheight=12\nwidth=12\nchannels=5\n\n"
+    for act in ("logistic", "tanh", "elu", "selu", "leaky", "gelu", "gelu_acc", "relu", "linear"):
+        s += f"[convolutional]\nfilters=24\nsize=3\nstride=1\npad=1\nactivation={act}\n\n"
+    s += "[shortcut]\nfrom=-3\nactivation=tanh\n\n"
+    s += "[maxpool]\nsize=3\nstride=2\npad=1\n\n"
+    s += "[avgpool]\nsize=3\nstride=1\npad=1\n\n"
+    s += "[connected]\noutput=40\nactivation=logistic\n\n[connected]\noutput=17\nactivation=linear\n\n[softmax]\n\n"
+    return s
+
+
+@pytest.mark.parametrize("mode", [api.MODE_LAYERS, api.MODE_DATAFLOW], ids=["layers", "dataflow"])
+def test_every_activation_and_softmax_match_oracle(gpu, mode):
+    from oracle import cpu
+    cfg = activation_zoo_cfg()
+    layers = M.parse_cfg(cfg)
+    tens = M.synth_weights(layers, 21, "he")
+    batch = 3
+    x = M.synth_input(layers, 21, batch, 0, "token_ids")
+    x = (x * 2.0 - 1.0).astype(np.float32)                 # both signs, so the negative branches are exercised
+    outs = cpu.run_network(layers, tens, x, batch, 0)
+    assert [L["type"] for L in layers].count("softmax") == 1 and np.allclose(outs[-1].sum(axis=1), 1.0, atol=1e-5)
+    assert min(float(o.min()) for o in outs[1:6]) < 0                     # negative pre-activations did occur
+    net = H.GpuNet(cfg, tens, batch, 0, min_ninst=64, mode=mode)
+    try:
+        net.run(x)
+        for l in range(net.nasm.num_ldata):
+            err = H.rel_l2(net.layer(l), outs[l])
+            assert err <= H.REL_L2_TOL, f"layer {l} ({layers[l]['type']}, {layers[l].get('act')}): rel L2 {err:.3g}"
+        assert np.array_equal(net.layer(net.nasm.num_ldata - 1).argmax(axis=1), outs[-1].argmax(axis=1))
+    finally:
+        net.close()
+
+
 def test_engine_rearm_many_runs(gpu):
     """Re-arm and re-run one graph many times: every run must execute each tile exactly once, never
     stall, and reproduce the first run bit for bit (tiles are deterministic; only their order varies)."""
