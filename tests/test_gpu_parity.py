@@ -123,6 +123,56 @@ def test_every_activation_and_softmax_match_oracle(gpu, mode):
         net.close()
 
 
+def test_results_in_the_callers_dimension_order(gpu):
+    """dse_get_ldata_result permutes a layer's native tensor into the order the caller names (reference
+    get_ldata_output, src/apu.c:227-297): matrices of a transformer are (BATCH, MAT_N, MAT_M), attention
+    probabilities (BATCH, NUM_HEAD, MAT_N, MAT_M), images (BATCH, OUT_H, OUT_W, OUT_C), vectors (BATCH, OUT_C).
+    Checked against numpy transpositions of the native [columns][rows] read-out."""
+    import itertools
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()["bert_mini_b2_s24"])
+    net = H.GpuNet(cfg, tens, batch, seq, min_ninst=64, mode=api.MODE_DATAFLOW)
+    try:
+        net.run(x)
+        kinds = {L["type"]: i for i, L in enumerate(layers)}                  # last layer of every kind
+        for t in ("matmul", "layernorm", "attn_v", "residual"):
+            l = kinds[t]
+            native = net.layer(l)                                            # [batch*seq][M]
+            cube = native.reshape(batch, seq, native.shape[1])
+            names = (api.BATCH, api.MAT_N, api.MAT_M)
+            for perm in itertools.permutations(range(3)):
+                got = net.nasm.layer_output(l, order=[names[p] for p in perm])
+                assert np.array_equal(got, cube.transpose(perm).ravel()), (t, perm)
+        l = kinds["attn_k"]
+        native = net.layer(l)                                                # [batch*heads*seq][seq]
+        heads = native.shape[0] // (batch * seq)
+        cube = native.reshape(batch, heads, seq, seq)
+        names = (api.BATCH, api.NUM_HEAD, api.MAT_N, api.MAT_M)
+        for perm in ((0, 1, 2, 3), (0, 1, 3, 2), (1, 0, 2, 3), (3, 2, 1, 0)):
+            got = net.nasm.layer_output(l, order=[names[p] for p in perm])
+            assert np.array_equal(got, cube.transpose(perm).ravel()), perm
+    finally:
+        net.close()
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()["custom_b3"])
+    net = H.GpuNet(cfg, tens, batch, seq, min_ninst=64, mode=api.MODE_DATAFLOW)
+    try:
+        net.run(x)
+        l = [i for i, L in enumerate(layers) if L["type"] == "maxpool"][0]
+        native = net.layer(l)
+        hw = int(round((native.shape[0] // batch) ** 0.5))
+        cube = native.reshape(batch, hw, hw, native.shape[1])
+        names = (api.BATCH, api.OUT_H, api.OUT_W, api.OUT_C)
+        for perm in ((0, 3, 1, 2), (0, 1, 2, 3), (3, 0, 2, 1)):
+            got = net.nasm.layer_output(l, order=[names[p] for p in perm])
+            assert np.array_equal(got, cube.transpose(perm).ravel()), perm
+        l = net.nasm.num_ldata - 1                                           # connected layer: (BATCH, OUT_C)
+        native = net.layer(l)
+        assert np.array_equal(net.nasm.layer_output(l, order=[api.OUT_C, api.BATCH]), native.T.ravel())
+        # an order that is no permutation of the layer's dimensions yields the native tensor
+        assert np.array_equal(net.nasm.layer_output(l, order=[api.OUT_H, api.OUT_W]), native.ravel())
+    finally:
+        net.close()
+
+
 def test_engine_rearm_many_runs(gpu):
     """Re-arm and re-run one graph many times: every run must execute each tile exactly once, never
     stall, and reproduce the first run bit for bit (tiles are deterministic; only their order varies)."""
