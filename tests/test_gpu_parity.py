@@ -221,6 +221,40 @@ def test_full_config_matches_reference_summary(gpu, name, mode):
         net.close()
 
 
+@pytest.mark.parametrize("mode", [api.MODE_LAYERS, api.MODE_DATAFLOW], ids=["layers", "dataflow"])
+def test_two_nasms_of_one_dnn_share_a_pool(gpu, mode, tmp_path):
+    """The reference's second example runs two graphs of ONE model side by side (reference
+    examples/2. vgg16_example/aspen_execute.c:38-50): both share the model's device weights, each has its own
+    activations and input.  Here with different batch sizes and inputs; then one graph is destroyed and the
+    pool runs on with the other."""
+    from oracle import cpu
+    cfg, layers, tens, x3, _, _ = H.build_case(H.micro_cases()["custom_b3"])
+    wp = str(tmp_path / "w.bin")
+    M.write_aspen_data(wp, tens)
+    dnn = api.Dnn(cfg, wp)
+    x2 = (1.0 - x3[: 2 * (x3.shape[0] // 3)]).astype(np.float32)          # two images, different content
+    na, nb = api.Nasm(dnn, 3, 0, 64), api.Nasm(dnn, 2, 0, 16)
+    pool, dse = api.RPool(), api.DseGroup(1, mode)
+    dse.set_rpool(pool)
+    try:
+        pool.add_nasm_raw_input(na, x3)
+        pool.add_nasm_raw_input(nb, x2)
+        dse.run(); dse.wait(na); dse.wait(nb); dse.stop()
+        ref_a, ref_b = cpu.run_network(layers, tens, x3, 3, 0), cpu.run_network(layers, tens, x2, 2, 0)
+        for l in range(na.num_ldata):
+            assert H.rel_l2(na.layer_output(l), ref_a[l]) <= H.REL_L2_TOL, ("a", l)
+            assert H.rel_l2(nb.layer_output(l), ref_b[l]) <= H.REL_L2_TOL, ("b", l)
+        na.destroy()                                                         # leaves the pool; the weights stay
+        x2b = (x2 * 0.5).astype(np.float32)
+        pool.add_nasm_raw_input(nb, x2b)
+        dse.run(); dse.wait(nb); dse.stop()
+        ref_b = cpu.run_network(layers, tens, x2b, 2, 0)
+        for l in range(nb.num_ldata):
+            assert H.rel_l2(nb.layer_output(l), ref_b[l]) <= H.REL_L2_TOL, ("b again", l)
+    finally:
+        dse.destroy(); pool.destroy(); nb.destroy(); dnn.destroy()
+
+
 def test_co_inference_resnet50_vgg16_b16(gpu):
     """ResNet-50 batch 16 and VGG-16 batch 16 in one ready pool / one engine launch; each must equal
     its solo-run reference summary."""
