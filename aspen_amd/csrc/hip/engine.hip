@@ -455,6 +455,76 @@ extern "C" int aspen_hip_zero (void *dst, size_t bytes)
     return 0;
 }
 
+// Dense <-> strided columns.  dense[c * rows + r] <-> strided[c * ld + r]; padding rows [rows, ld) are written as zeros.
+__global__ void __launch_bounds__ (WG_THREADS) spread_columns_kernel (const float *__restrict__ dense, float *__restrict__ strided, uint32_t rows, uint32_t ld, size_t n)
+{
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += step)
+    {
+        const size_t c = i / ld;
+        const uint32_t r = (uint32_t)(i - c * ld);
+        strided[i] = r < rows ? dense[c * rows + r] : 0.f;
+    }
+}
+__global__ void __launch_bounds__ (WG_THREADS) gather_columns_kernel (const float *__restrict__ strided, float *__restrict__ dense, uint32_t rows, uint32_t ld, size_t n)
+{
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += step)
+    {
+        const size_t c = i / rows;
+        dense[i] = strided[c * ld + (i - c * rows)];
+    }
+}
+
+// staging buffer for the two functions below; grows on demand and lives as long as the process
+static float *g_stage = nullptr;
+static size_t g_stage_bytes = 0;
+static int stage_reserve (size_t bytes)
+{
+    if (bytes <= g_stage_bytes) return 0;
+    CHECK (hipStreamSynchronize (g_stream));
+    if (g_stage) { (void)hipFree (g_stage); g_stage = nullptr; g_stage_bytes = 0; }
+    CHECK (hipMalloc ((void **)&g_stage, bytes));
+    g_stage_bytes = bytes;
+    return 0;
+}
+static unsigned stream_grid (size_t n)
+{
+    const size_t want = (n + WG_THREADS - 1) / WG_THREADS, cap = (size_t)g_num_cu * 16;
+    return (unsigned)(want < cap ? (want ? want : 1) : cap);
+}
+
+extern "C" int aspen_hip_dense_host_to_device (float *dst, uint32_t ld, const float *src_host, uint32_t rows, size_t columns)
+{
+    if (aspen_hip_init ()) return -1;
+    if (!dst || !src_host || rows == 0 || ld < rows) { snprintf (g_err, sizeof (g_err), "dense_host_to_device: bad arguments"); return -1; }
+    if (columns == 0) return 0;
+    if (ld == rows) return aspen_hip_h2d (dst, src_host, (size_t)rows * columns * sizeof (float));
+    const size_t bytes = (size_t)rows * columns * sizeof (float);
+    if (stage_reserve (bytes)) return -1;
+    CHECK (hipMemcpyAsync (g_stage, src_host, bytes, hipMemcpyHostToDevice, g_stream));
+    const size_t n = (size_t)ld * columns;
+    hipLaunchKernelGGL (spread_columns_kernel, dim3 (stream_grid (n)), dim3 (WG_THREADS), 0, g_stream, g_stage, dst, rows, ld, n);
+    CHECK (hipGetLastError ());
+    CHECK (hipStreamSynchronize (g_stream));       // the caller may reuse its buffer, and the next call the staging buffer
+    return 0;
+}
+
+extern "C" int aspen_hip_dense_device_to_host (float *dst_host, const float *src, uint32_t ld, uint32_t rows, size_t columns)
+{
+    if (aspen_hip_init ()) return -1;
+    if (!dst_host || !src || rows == 0 || ld < rows) { snprintf (g_err, sizeof (g_err), "dense_device_to_host: bad arguments"); return -1; }
+    if (columns == 0) return 0;
+    if (ld == rows) return aspen_hip_d2h (dst_host, src, (size_t)rows * columns * sizeof (float));
+    const size_t bytes = (size_t)rows * columns * sizeof (float), n = (size_t)rows * columns;
+    if (stage_reserve (bytes)) return -1;
+    hipLaunchKernelGGL (gather_columns_kernel, dim3 (stream_grid (n)), dim3 (WG_THREADS), 0, g_stream, src, g_stage, rows, ld, n);
+    CHECK (hipGetLastError ());
+    CHECK (hipMemcpyAsync (dst_host, g_stage, bytes, hipMemcpyDeviceToHost, g_stream));
+    CHECK (hipStreamSynchronize (g_stream));
+    return 0;
+}
+
 // plain streaming copy, 16 bytes per lane per step; also the yardstick the HBM byte counters of a
 // profiler are calibrated with (its traffic is known: `bytes` read + `bytes` written)
 __global__ void __launch_bounds__ (WG_THREADS) copy_kernel (const float4 *__restrict__ src, float4 *__restrict__ dst, size_t n4)

@@ -59,19 +59,10 @@ void rpool_add_nasm_raw_input (rpool_t *rpool, nasm_t *nasm, void *input_data)
         const nasm_ldata_t *ld = &nasm->ldata_arr[0];
         const size_t H = ld->out_mat_dims[OUT_H], W = ld->out_mat_dims[OUT_W];
         aspen_hip_sync ();
-        /* one contiguous transfer: a strided copy of millions of 12-byte columns (3-channel images) is
-           orders of magnitude slower than repacking on the host first */
-        const size_t ldf = ld->out_mat_stride;
-        int rc;
-        if (ldf == H) rc = aspen_hip_h2d (nasm->d_arena + ld->out_mat_offset, input_data, H * W * sizeof (float));
-        else
-        {
-            float *staged = calloc (ldf * W, sizeof (float));
-            if (staged == NULL) { ERROR_PRTF ("ERROR: rpool_add_nasm_raw_input: out of host memory.\n"); return; }
-            for (size_t c = 0; c < W; c++) memcpy (staged + c * ldf, (const float *)input_data + c * H, H * sizeof (float));
-            rc = aspen_hip_h2d (nasm->d_arena + ld->out_mat_offset, staged, ldf * W * sizeof (float));
-            free (staged);
-        }
+        /* one contiguous transfer, then a kernel that spreads the columns to the matrix's stride: a strided
+           copy of millions of 12-byte columns (3-channel images) is orders of magnitude slower, and
+           repacking on the host costs more than the transfer */
+        const int rc = aspen_hip_dense_host_to_device (nasm->d_arena + ld->out_mat_offset, ld->out_mat_stride, input_data, (uint32_t)H, W);
         if (rc) ERROR_PRTF ("ERROR: rpool_add_nasm_raw_input: input upload failed: %s\n", aspen_hip_last_error ());
     }
     nasm->armed = 1;
@@ -367,22 +358,12 @@ static ssize_t get_ldata_output (nasm_t *nasm, unsigned int ldata_idx, LAYER_PAR
     const size_t H = ld->out_mat_dims[OUT_H], W = ld->out_mat_dims[OUT_W];
     float *dense = malloc (H * W * sizeof (float));
     if (dense == NULL) return -1;
+    /* padding rows stripped on the device, one contiguous transfer */
+    if (aspen_hip_dense_device_to_host (dense, nasm->d_arena + ld->out_mat_offset, ld->out_mat_stride, (uint32_t)H, W))
     {
-        /* one contiguous transfer of the strided matrix, padding rows stripped on the host */
-        const size_t ldf = ld->out_mat_stride;
-        float *strided = ldf == H ? dense : malloc (ldf * W * sizeof (float));
-        if (strided == NULL || aspen_hip_d2h (strided, nasm->d_arena + ld->out_mat_offset, ldf * W * sizeof (float)))
-        {
-            ERROR_PRTF ("Error in get_ldata_output: download failed: %s\n", aspen_hip_last_error ());
-            if (strided != dense) free (strided);
-            free (dense);
-            return -1;
-        }
-        if (strided != dense)
-        {
-            for (size_t c = 0; c < W; c++) memcpy (dense + c * H, strided + c * ldf, H * sizeof (float));
-            free (strided);
-        }
+        ERROR_PRTF ("Error in get_ldata_output: download failed: %s\n", aspen_hip_last_error ());
+        free (dense);
+        return -1;
     }
     /* native dimension list, slowest first */
     LAYER_PARAMS native[4];

@@ -104,6 +104,12 @@ int aspen_hip_d2h (void *dst, const void *src, size_t bytes);
 int aspen_hip_h2d_2d (void *dst, size_t dpitch, const void *src, size_t spitch, size_t width, size_t rows);
 int aspen_hip_d2h_2d (void *dst, size_t dpitch, const void *src, size_t spitch, size_t width, size_t rows);
 int aspen_hip_zero (void *dst, size_t bytes);
+/* dense host matrix (`columns` runs of `rows` floats) -> device matrix with column stride `ld` >= rows floats,
+   the padding rows zeroed: one contiguous upload into a staging buffer the library keeps, then a kernel
+   that spreads the columns (what the reference's copy_buffer_to_ldata_out_mat, src/apu_nasm.c:809-826, does
+   on the host).  dense_device_to_host is the inverse (reference get_packed_ldata_output_colwise). */
+int aspen_hip_dense_host_to_device (float *dst, uint32_t ld, const float *src_host, uint32_t rows, size_t columns);
+int aspen_hip_dense_device_to_host (float *dst_host, const float *src, uint32_t ld, uint32_t rows, size_t columns);
 /* device-to-device copy by a plain streaming kernel on the library's stream (asynchronous); size and
    addresses multiples of 16 bytes.  Its memory traffic is exactly 2 x bytes, which makes it the
    calibration point for a profiler's HBM byte counters. */
