@@ -879,9 +879,8 @@ __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, ui
     const int kiters = (int)(L.hd / GEMM_BK);
     if (tid < BN) rowsum[tid] = 0.f;                     // ordered before the atomics below by the barriers of gemm_core
 
-    // The scores are computed twice: the first pass only accumulates every query's sum of exponentials, the
-    // second recomputes them, normalises and stores.  Recomputing 2*hd flops per score is far cheaper than
-    // keeping S scores per query in registers or writing them out and reading them back.
+    // The scores are computed once: every key block's exponentials are stored unnormalised while the queries'
+    // sums accumulate, and a second sweep over the tile's own output (still in this XCD's L2) divides by them.
     auto scores = [&] (uint32_t k0, floatx16 (&acc)[TN][TM])
     {
         ActRowLoader<BM, COH> al; al.init (Kmat, b * S + k0, b * S + S - 1, L.ld1, h * L.hd, tid);

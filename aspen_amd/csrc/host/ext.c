@@ -90,13 +90,6 @@ unsigned int aspen_rpool_num_ninst (rpool_t *rp)
 }
 
 /* ---- dumps (reference include/aspen.h:124-133) -------------------------------------------------- */
-static const char *layer_type_name[NUM_LAYER_ELEMENTS] = {
-    "NO_LAYER_TYPE", "INPUT_LAYER", "CONV_LAYER", "FC_LAYER", "RESIDUAL_LAYER", "BATCHNORM_LAYER", "YOLO_LAYER",
-    "APPEND_LAYER", "ACTIVATION_LAYER", "MAXPOOL_LAYER", "AVGPOOL_LAYER", "ROUTE_LAYER", "SOFTMAX_LAYER",
-    "MATMUL_LAYER", "LAYERNORM_LAYER", "K_ATTENTION_LAYER", "V_ATTENTION_LAYER" };
-static const char *act_name[NUM_ACTIVATIONS] = {
-    "NO_ACTIVATION", "SIGMOID", "LINEAR", "TANH", "RELU", "LEAKY_RELU", "ELU", "SELU", "GELU", "GELU_ACCURATE" };
-
 void print_aspen_build_info (void)
 {
     printf ("ASPEN for AMD Instinct MI355X (gfx950): HIP tile kernels + device-side dataflow engine\n");
@@ -116,8 +109,8 @@ void print_tensor_info (aspen_tensor_t *t, int print_data)
 void print_layer_info (aspen_layer_t *L, int print_data)
 {
     if (L == NULL) { printf ("Error: layer is NULL.\n"); return; }
-    printf ("\tLayer %u: %s, activation %s, parents %d %d\n", L->layer_idx, layer_type_name[L->type],
-        act_name[L->activation], L->parent_idx[PARENT_0], L->parent_idx[PARENT_1]);
+    printf ("\tLayer %u: %s, activation %s, parents %d %d\n", L->layer_idx, layer_type_str[L->type],
+        activation_type_str[L->activation], L->parent_idx[PARENT_0], L->parent_idx[PARENT_1]);
     printf ("\t\tout C/H/W %u/%u/%u  in C/H/W %u/%u/%u  kernel %ux%u stride %u pad %u  M/K %u/%u heads %u\n",
         L->params[OUT_C], L->params[OUT_H], L->params[OUT_W], L->params[IN_C], L->params[IN_H], L->params[IN_W],
         L->params[WEIGHT_H], L->params[WEIGHT_W], L->params[STRIDE], L->params[PADDING],
@@ -139,7 +132,7 @@ void print_ldata_info (nasm_ldata_t *ld, int print_ninst, int print_data)
     (void)print_data;
     if (ld == NULL) { printf ("Error: ldata is NULL.\n"); return; }
     printf ("\tLdata %u (%s): matrix %u rows x %u columns, stride %u, tiles %u x %u of %u x %u, %u ninsts from %u, %.3f GFLOP\n",
-        ld->layer->layer_idx, layer_type_name[ld->layer->type], ld->out_mat_dims[OUT_H], ld->out_mat_dims[OUT_W],
+        ld->layer->layer_idx, layer_type_str[ld->layer->type], ld->out_mat_dims[OUT_H], ld->out_mat_dims[OUT_W],
         ld->out_mat_stride, ld->tiles_h, ld->tiles_w, ld->tile_dims[OUT_H], ld->tile_dims[OUT_W], ld->num_ninst,
         ld->ninst_start, (double)ld->flops * 1e-9);
     if (print_ninst)

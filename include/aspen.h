@@ -12,8 +12,26 @@
 #ifndef ASPEN_AMD_ASPEN_H
 #define ASPEN_AMD_ASPEN_H
 
+/* System headers a caller gets through the reference header (reference include/aspen.h:4-18) and relies
+   on: the reference's main.c and examples include nothing but aspen.h, yet use FILE, printf, strcpy,
+   atoi, gettimeofday and friends. */
+#ifndef _GNU_SOURCE
+#define _GNU_SOURCE
+#endif
 #include <stddef.h>
+#include <string.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <ctype.h>
+#include <math.h>
+#include <float.h>
+#include <limits.h>
+#include <stdint.h>
+#include <time.h>
+#include <sys/time.h>
 #include <sys/types.h>
+#include <assert.h>
+#include <unistd.h>
 
 #ifdef __cplusplus
 extern "C" {
@@ -21,6 +39,29 @@ extern "C" {
 
 #define MAX_TENSOR_DIMS 8      /* reference include/aspen.h:26 */
 #define MAX_STRING_LEN 256     /* reference include/aspen.h:27 */
+
+/* Console macros of the reference header (reference include/aspen.h:34-48): same names and colours, silenced
+   by SUPPRESS_OUTPUT != 0.  No shipped caller uses them; they are here so that code written against the
+   reference header compiles unchanged. */
+#ifndef SUPPRESS_OUTPUT
+#define SUPPRESS_OUTPUT 0
+#endif
+#define ASPEN_COLOUR_PRTF_(stream, colour, ...) do { fprintf (stream, "\033[0;" colour "m"); fprintf (stream, __VA_ARGS__); fprintf (stream, "\033[0m"); } while (0)
+#if SUPPRESS_OUTPUT == 0
+#define PRTF(...) printf (__VA_ARGS__)
+#define ERROR_PRTF(...) do { fprintf (stderr, "\033[0;31m(%s:%d)", __FILE__, __LINE__); fprintf (stderr, __VA_ARGS__); fprintf (stderr, "\033[0m"); } while (0)
+#define RED_PRTF(...) ASPEN_COLOUR_PRTF_ (stdout, "31", __VA_ARGS__)
+#define GREEN_PRTF(...) ASPEN_COLOUR_PRTF_ (stdout, "32", __VA_ARGS__)
+#define YELLOW_PRTF(...) ASPEN_COLOUR_PRTF_ (stdout, "33", __VA_ARGS__)
+#define BLUE_PRTF(...) ASPEN_COLOUR_PRTF_ (stdout, "34", __VA_ARGS__)
+#else
+#define PRTF(...) ((void)0)
+#define ERROR_PRTF(...) fprintf (stderr, "\033[0;31mASPEN: An error has occured.\033[0m")
+#define RED_PRTF(...) ((void)0)
+#define GREEN_PRTF(...) ((void)0)
+#define YELLOW_PRTF(...) ((void)0)
+#define BLUE_PRTF(...) ((void)0)
+#endif
 
 /* reference include/aspen.h:50 */
 typedef enum { NINST_NOT_READY, NINST_READY, NINST_COMPLETED, NUM_NINST_STATES } NINST_STATE;
@@ -54,6 +95,20 @@ typedef enum {
     NO_ACTIVATION, SIGMOID, LINEAR, TANH, RELU, LEAKY_RELU, ELU, SELU, GELU, GELU_ACCURATE,
     NUM_ACTIVATIONS
 } LAYER_ACT;
+
+/* reference include/aspen.h:65.  Ready-pool routing conditions: kept for source compatibility; this
+   library has one device-side ready queue and routes nothing. */
+typedef enum { RPOOL_DNN, RPOOL_LAYER_TYPE, RPOOL_LAYER_IDX, RPOOL_NASM, RPOOL_DSE, NUM_RPOOL_CONDS } RPOOL_CONDS;
+
+/* Printable names of the enumerators above, indexed by value (reference include/aspen.h:67-73, tables in
+   src/util.c:3-41). */
+extern char *ninst_state_str[NUM_NINST_STATES];
+extern char *layer_type_str[NUM_LAYER_ELEMENTS];
+extern char *param_type_str[NUM_PARAM_ELEMENTS];
+extern char *tensor_type_str[NUM_TENSORS];
+extern char *parent_type_str[NUM_PARENT_ELEMENTS];
+extern char *activation_type_str[NUM_ACTIVATIONS];
+extern char *rpool_cond_str[NUM_RPOOL_CONDS];
 
 typedef struct aspen_dnn_t aspen_dnn_t;       /* model: layers + weights          (include/aspen.h:74) */
 typedef struct aspen_layer_t aspen_layer_t;

@@ -23,7 +23,7 @@ int aspen_dse_group_last_mode (dse_group_t *dse_group);
    run is given up (every workgroup then leaves, the run reports ASPEN_HIP_ERR_STALLED and the next run
    starts from re-armed state).  0 = the library's default (2^26 polls, minutes). */
 void aspen_dse_group_set_spin_limit (dse_group_t *dse_group, uint64_t polls);
-/* persistent workgroups of the dataflow kernel; 0 = two per compute unit */
+/* persistent workgroups of the dataflow kernel; 0 = sized from the graph's average parallelism (1 to 4 per compute unit) */
 void aspen_dse_group_set_workgroups (dse_group_t *dse_group, unsigned int workgroups);
 
 /* Graphs created AFTER this call keep (1) or do not keep (0, the default) the matrix of a contraction

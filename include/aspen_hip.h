@@ -136,7 +136,8 @@ double aspen_hip_graph_parallelism (const aspen_hip_graph_t *graph);
    per-kernel profiling mode. */
 int aspen_hip_run_layers (aspen_hip_graph_t *graph, uint32_t first_layer, uint32_t last_layer);
 /* Barrier-free execution: re-arms the dependency counters and the ready queue, then one persistent
-   kernel of `workgroups` workgroups (0 = two per compute unit) pops ready tiles until all are done.
+   kernel of `workgroups` workgroups (0 = a whole number per compute unit, 1 to 4, sized from the graph's
+   average parallelism) pops ready tiles until all are done.
    spin_limit bounds every wait on the ready queue (0 = default); a wait that exceeds it raises the
    abort flag, all workgroups exit and aspen_hip_sync returns ASPEN_HIP_ERR_STALLED. */
 int aspen_hip_run_dataflow (aspen_hip_graph_t *graph, uint32_t workgroups, uint64_t spin_limit);
@@ -164,7 +165,9 @@ void aspen_hip_set_flags (uint32_t flags);
 int aspen_hip_sync (void);
 /* 1 when everything enqueued so far has finished, 0 when still running */
 int aspen_hip_idle (void);
-/* Tiles executed / executed-twice / executed-before-ready counters of the last dataflow run. */
+/* Counters of the last dataflow run (kept under ASPEN_HIP_FLAG_COUNT_TILES): tiles executed, tiles executed
+   more than once, and the abort flag.  That no tile starts before its parents have ended is checked from
+   the time stamps of a traced run (ASPEN_HIP_FLAG_TRACE), not counted on the device. */
 int aspen_hip_dataflow_stats (aspen_hip_graph_t *graph, uint32_t *executed, uint32_t *double_runs, uint32_t *abort_flag);
 
 /* ---- timing ------------------------------------------------------------------------------------- */
