@@ -376,6 +376,22 @@ CONFIGS = {
     "gpt2_b4_s512": (gpt2_cfg, "gpt", 4, 512, 404, "token_ids"),
 }
 
+# The graphs the benchmark times AND the full-size parity tests check (one table, so they cannot drift apart):
+#   name: (configurations co-run in one ready pool, unit, units per step, tiles wanted per layer, engine)
+# The last two entries are what the library's timing tuner (apu_generate_nasm: candidate tile counts on both
+# engines) settles on for the configuration, fixed here so that a run does not spend its time tuning; the
+# reference ships its tile graphs tuned per model and batch in the same way.
+WORKLOADS = {
+    "resnet50_b32": (["resnet50_b32"], "img/s", 32, 1536, "dataflow"),
+    "resnet50_b1": (["resnet50_b1"], "img/s", 1, 128, "layers"),
+    "vgg16_b32": (["vgg16_b32"], "img/s", 32, 1536, "dataflow"),
+    "co_resnet50_vgg16_b16": (["resnet50_b16", "vgg16_b16"], "img/s", 32, 1536, "dataflow"),
+    "bert_base_b8_s128": (["bert_base_b8_s128"], "tokens/s", 8 * 128, 192, "dataflow"),
+    "gpt2_b4_s512": (["gpt2_b4_s512"], "tokens/s", 4 * 512, 384, "dataflow"),
+    "yolov3_b1": (["yolov3_b1"], "img/s", 1, 768, "layers"),
+    "yolov3_b8": (["yolov3_b8"], "img/s", 8, 1536, "dataflow"),
+}
+
 
 def make_config(name: str):
     """(cfg text, parsed layers, weight tensors, dense input, batch, seq) of a named configuration."""

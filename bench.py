@@ -33,20 +33,7 @@ FLOP_PER_UNIT = {
     "resnet50": 8.178369e9, "vgg16": 3.069326e10 + 2.47267e8,
     "bert_base": 1.7459e8, "gpt2": 1.8877e8,
 }
-WORKLOADS = {
-    # name: (configs, unit, units per step, tiles wanted per layer, engine)
-    # The last two entries are what the library's timing tuner (apu_generate_nasm: candidate tile counts on
-    # both engines) settles on for the configuration, fixed here so that a bench run does not spend its time
-    # tuning; the reference ships its tile graphs tuned per model and batch in the same way.
-    "resnet50_b32": (["resnet50_b32"], "img/s", 32, 1536, "dataflow"),
-    "resnet50_b1": (["resnet50_b1"], "img/s", 1, 128, "layers"),
-    "vgg16_b32": (["vgg16_b32"], "img/s", 32, 1536, "dataflow"),
-    "co_resnet50_vgg16_b16": (["resnet50_b16", "vgg16_b16"], "img/s", 32, 1536, "dataflow"),
-    "bert_base_b8_s128": (["bert_base_b8_s128"], "tokens/s", 8 * 128, 192, "dataflow"),
-    "gpt2_b4_s512": (["gpt2_b4_s512"], "tokens/s", 4 * 512, 384, "dataflow"),
-    "yolov3_b1": (["yolov3_b1"], "img/s", 1, 768, "layers"),
-    "yolov3_b8": (["yolov3_b8"], "img/s", 8, 1536, "dataflow"),
-}
+from aspen_amd.models import WORKLOADS      # noqa: E402  (shared with the full-size parity tests)
 
 
 def gemm_flops(nasm, api):
@@ -97,6 +84,25 @@ def cpu_baseline(cfgname, budget_s=20.0):
         sec = time.time() - t0
         return {"value": units / sec, "unit": unit, "cores": threads, "kind": "port",
                 "sample": f"{cfgname}: 1 full pass of the oracle port ({exc})", "ms_per_step": sec * 1e3}
+
+
+def verify_final_layer(name, nasm):
+    """Final layer of the graph that was just timed against the fixture the compiled reference wrote for this
+    configuration (tests/golden/<name>.npz: strided samples, norm and per-column argmax).  Returns None when
+    no fixture exists for the configuration."""
+    path = os.path.join(ROOT, "tests", "golden", f"{name}.npz")
+    if not os.path.exists(path):
+        return None
+    gold = np.load(path)
+    l = int(gold["num_layers"]) - 1
+    got = nasm.layer_output(l)
+    flat = got.reshape(-1).astype(np.float64)
+    ref_val = gold[f"val{l}"].astype(np.float64)
+    err = float(np.linalg.norm(flat[gold[f"idx{l}"]] - ref_val) / max(np.linalg.norm(ref_val), 1e-30))
+    norm = float(np.sqrt((flat ** 2).sum()))
+    ref_norm = float(gold[f"l2_{l}"])
+    ok = err <= 1e-4 and abs(norm - ref_norm) <= 1e-4 * ref_norm and bool((got.argmax(axis=1) == gold["argmax"]).all())
+    return {"ok": ok, "sampled_rel_l2": err, "argmax_equal": bool((got.argmax(axis=1) == gold["argmax"]).all())}
 
 
 def quiet_stdout():
@@ -298,6 +304,14 @@ def main():
         out["layer_profile"] = per_type
         out["layer_ms"] = [round(float(v), 4) for v in lms]
 
+    # the graph that was timed must also have computed the right thing: its final layer against the
+    # compiled reference's fixture (outside the timed region)
+    if not args.skip_tiles:
+        checks = {name: verify_final_layer(name, n) for name, _, n, _ in nets}
+        have = [c for c in checks.values() if c is not None]
+        out["verified"] = all(c["ok"] for c in have) if have else None
+        out["verification"] = checks
+
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfgs[0])
 
@@ -310,6 +324,9 @@ def main():
     for _, dnn, nasm, _ in nets:
         dnn.destroy()
     emit(json.dumps(out))
+    if out.get("verified") is False:
+        print("bench.py: the timed graph's output does not match the reference fixture", file=sys.stderr)
+        sys.exit(3)
 
 
 if __name__ == "__main__":

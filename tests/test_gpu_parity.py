@@ -221,6 +221,74 @@ def test_full_config_matches_reference_summary(gpu, name, mode):
         net.close()
 
 
+@pytest.mark.timeout(900)
+@pytest.mark.parametrize("workload", list(M.WORKLOADS))
+def test_timed_graphs_match_oracle_on_whole_tensors(gpu, workload):
+    """Exactly the graphs bench.py times (models.WORKLOADS: same tile counts, same engine, one ready pool for the
+    co-scheduled pair), first with the library's default of not writing matrices that only a fused shortcut
+    reads -- the setting the benchmark runs -- then with every matrix kept.  EVERY element of every layer is
+    compared with the CPU oracle run on the same inputs (relative L2 <= 1e-4 per layer, identical argmax of
+    the final layer); a single wrong tile anywhere fails its layer."""
+    from oracle import cpu
+    cfgs, _, _, min_ninst, engine = M.WORKLOADS[workload]
+    mode = api.MODE_DATAFLOW if engine == "dataflow" else api.MODE_LAYERS
+    cases, want = [], []
+    for name in cfgs:
+        cfg, layers, tens, x, batch, seq = H.full_config(name)
+        want.append(cpu.run_network(layers, tens, x, batch, seq))
+        cases.append((name, cfg, layers, tens, x, batch, seq))
+        print(f"oracle done: {name}", flush=True)
+    try:
+        for keep in (0, 1):
+            api.lib().aspen_keep_layer_outputs(keep)
+            pool = api.RPool()
+            dse = api.DseGroup(1, mode)
+            dse.set_rpool(pool)
+            nets = []
+            try:
+                for name, cfg, layers, tens, x, batch, seq in cases:
+                    net = H.GpuNet(cfg, tens, batch, seq, min_ninst=min_ninst, mode=mode)
+                    net.rpool.destroy()
+                    net.rpool = pool
+                    pool.add_nasm_raw_input(net.nasm, x)
+                    nets.append(net)
+                print(f"{workload} keep={keep}: {sum(n.nasm.num_ninst for n in nets)} tiles", flush=True)
+                dse.run()
+                for net in nets:
+                    dse.wait(net.nasm)
+                dse.stop()
+                if mode == api.MODE_DATAFLOW:
+                    st = pool.run_stats()
+                    assert st == {"executed": sum(n.nasm.num_ninst for n in nets), "double_runs": 0, "aborted": 0}, st
+                worst = 0.0
+                for (name, _, layers, *_), net, outs in zip(cases, nets, want):
+                    dropped = 0
+                    for l in range(net.nasm.num_ldata):
+                        if keep == 0 and net.nasm.info(l)["fused_residual"] >= 0:
+                            with pytest.raises(RuntimeError):
+                                net.layer(l)
+                            dropped += 1
+                            continue
+                        got = net.layer(l)
+                        assert got.shape == outs[l].shape, (name, l, got.shape, outs[l].shape)
+                        err = H.rel_l2(got, outs[l])
+                        worst = max(worst, err)
+                        assert err <= H.REL_L2_TOL, f"{name} keep={keep} layer {l} ({layers[l]['type']}): rel L2 {err:.3g}"
+                    last = net.nasm.num_ldata - 1
+                    assert np.array_equal(net.layer(last).argmax(axis=1), outs[last].argmax(axis=1)), f"{name}: argmax differs"
+                    assert keep == 1 or dropped or not any(L["type"] == "residual" for L in layers)
+                print(f"{workload} keep={keep}: worst rel L2 {worst:.3g}", flush=True)
+            finally:
+                for net in nets:
+                    net.dse.destroy()
+                    net.nasm.destroy()
+                    net.dnn.destroy()
+                dse.destroy()
+                pool.destroy()
+    finally:
+        api.lib().aspen_keep_layer_outputs(1)
+
+
 @pytest.mark.parametrize("mode", [api.MODE_LAYERS, api.MODE_DATAFLOW], ids=["layers", "dataflow"])
 def test_two_nasms_of_one_dnn_share_a_pool(gpu, mode, tmp_path):
     """The reference's second example runs two graphs of ONE model side by side (reference
@@ -540,3 +608,45 @@ def test_reference_main_call_sequence(gpu, tmp_path):
     L.rpool_destroy(rpool)
     L.apu_destroy_nasm(nasm)
     L.apu_destroy_dnn(dnn)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,min_ninst,workgroups", [("resnet_mini_b2", 1024, 0), ("gpt_mini_b2_s20", 64, 16), ("yolo_mini_b2", 16, 0),
+                                                      ("resnet50_b1", 128, 0), ("bert_base_b8_s128", 192, 0)])
+def test_no_tile_starts_before_its_parents_have_ended(gpu, name, min_ninst, workgroups):
+    """The scheduler's invariant (reference src/dse.c:32-38, 311-317: a ninst runs only once all its parents are
+    completed), checked from the per-tile start / end stamps of a traced run of the persistent kernel: along
+    every dependency edge the child's start stamp is not earlier than the parent's end stamp, which is taken
+    after the parent's stores were acknowledged.  The members of a split-K group release their children
+    together, through whichever member finishes last: a child waits for the group's last end."""
+    micro = name in H.micro_cases()
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()[name]) if micro else H.full_config(name)
+    api.lib().aspen_hip_set_flags(2 | 8)
+    net = H.GpuNet(cfg, tens, batch, seq, min_ninst=min_ninst, mode=api.MODE_DATAFLOW, workgroups=workgroups)
+    try:
+        for rep in range(2):                                     # also on a re-armed graph
+            net.run(x if rep == 0 else None)
+            st = net.rpool.run_stats()
+            assert st == {"executed": net.nasm.num_ninst, "double_runs": 0, "aborted": 0}, st
+            stamps = net.rpool.dataflow_trace().astype(np.int64)
+            start, end = stamps[:, 0], stamps[:, 1].copy()
+            assert (start > 0).all() and (end >= start).all()
+            tile_layer, num_parents, child_off, child_idx = net.nasm.graph()
+            grouped = 0
+            for l in range(net.nasm.num_ldata):
+                i = net.nasm.info(l)
+                if i["splits"] > 1:
+                    seg = end[i["ninst_start"]: i["ninst_start"] + i["num_ninst"]].reshape(-1, i["splits"])
+                    seg[:] = seg.max(axis=1, keepdims=True)          # a view into `end`
+                    grouped += 1
+            parent_of_edge = np.repeat(np.arange(net.nasm.num_ninst), np.diff(child_off.astype(np.int64)))
+            assert len(parent_of_edge) == len(child_idx) > 0
+            early = start[child_idx] < end[parent_of_edge]
+            assert not early.any(), (f"{int(early.sum())} of {len(early)} edges violated, first: parent "
+                                     f"{parent_of_edge[early][0]} -> child {child_idx[early][0]}")
+            # roots start without waiting, everything else after at least one parent
+            assert (num_parents[child_idx] > 0).all()
+            print(f"{name} run {rep}: {len(child_idx)} edges hold, {grouped} split-K layers", flush=True)
+    finally:
+        api.lib().aspen_hip_set_flags(2)
+        net.close()
