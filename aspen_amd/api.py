@@ -82,6 +82,8 @@ def lib() -> C.CDLL:
         "aspen_dse_group_set_spin_limit": (None, [_vp, C.c_uint64]),
         "aspen_dse_group_set_workgroups": (None, [_vp, C.c_uint]),
         "aspen_keep_layer_outputs": (None, [C.c_int]),
+        "apu_load_dnn_data_from_file": (None, [_vp, C.c_char_p]),
+        "aspen_dnn_device_generation": (C.c_uint, [_vp]),
         "aspen_nasm_num_ldata": (C.c_uint, [_vp]),
         "aspen_nasm_num_ninst": (C.c_uint, [_vp]),
         "aspen_nasm_num_edges": (C.c_uint, [_vp]),
@@ -106,6 +108,7 @@ def lib() -> C.CDLL:
         "aspen_hip_copy": (C.c_int, [_vp, _vp, C.c_size_t]),
         "aspen_hip_zero": (C.c_int, [_vp, C.c_size_t]),
         "aspen_hip_sync": (C.c_int, []),
+        "aspen_hip_graph_sync": (C.c_int, [_vp]),
         "aspen_hip_set_flags": (None, [C.c_uint32]),
         "aspen_hip_idle": (C.c_int, []),
         "aspen_hip_event_record": (C.c_int, [C.c_int]),

@@ -43,6 +43,7 @@ struct aspen_hip_graph_t
     double parallelism;             // average parallelism of the tile graph, see graph_parallelism
     int cached_loads;       // 1: no cache line of an activation is shared by two producer tiles
     unsigned long long *d_trace;    // [2*tile] start, [2*tile+1] end time stamps (allocated on first traced run)
+    uint32_t *h_abort;              // pinned host word the persistent kernel raises when it gives this graph's run up
 };
 
 static hipStream_t g_stream = nullptr;
@@ -52,7 +53,6 @@ static int g_num_cu = 0;
 static int g_resident_wg = WG_PER_CU;     // workgroups of the dataflow kernel that fit one compute unit
 static char g_err[512] = "";
 static uint32_t g_flags = 0;
-static uint32_t *g_host_abort = nullptr;    // pinned host word the persistent kernel raises when it gives up waiting
 
 static int fail (hipError_t e, const char *what)
 {
@@ -363,8 +363,6 @@ extern "C" int aspen_hip_init (void)
     CHECK (hipGetDeviceProperties (&prop, 0));
     g_num_cu = prop.multiProcessorCount;
     CHECK (hipStreamCreate (&g_stream));
-    CHECK (hipHostMalloc ((void **)&g_host_abort, 64, hipHostMallocDefault));
-    *g_host_abort = 0;
     for (int i = 0; i < NUM_EVENTS; i++) CHECK (hipEventCreate (&g_events[i]));
     CHECK (hipFuncSetAttribute ((const void *)layer_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
     CHECK (hipFuncSetAttribute ((const void *)dataflow_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
@@ -770,7 +768,9 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     g->d_state = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * ST_WORDS);
     g->d_arrivals = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
     g->d_prof = (unsigned long long *)aspen_hip_alloc (sizeof (unsigned long long) * 8);
-    if (!g->d_layers || !g->d_ninst_layer || !g->d_num_parents || !g->d_child_off || !g->d_child_idx || !g->d_roots
+    if (hipHostMalloc ((void **)&g->h_abort, 64, hipHostMallocDefault) != hipSuccess) g->h_abort = nullptr;
+    else *g->h_abort = 0;
+    if (!g->h_abort || !g->d_layers || !g->d_ninst_layer || !g->d_num_parents || !g->d_child_off || !g->d_child_idx || !g->d_roots
         || !g->d_dep || !g->d_queue || !g->d_ran || !g->d_state || !g->d_child_rec || !g->d_arrivals || !g->d_prof)
     {
         aspen_hip_graph_destroy (g);
@@ -786,6 +786,7 @@ extern "C" void aspen_hip_graph_destroy (aspen_hip_graph_t *g)
     aspen_hip_free (g->d_layers); aspen_hip_free (g->d_ninst_layer); aspen_hip_free (g->d_num_parents);
     aspen_hip_free (g->d_child_off); aspen_hip_free (g->d_child_idx); aspen_hip_free (g->d_roots);
     aspen_hip_free (g->d_child_rec); aspen_hip_free (g->d_dep); aspen_hip_free (g->d_queue); aspen_hip_free (g->d_ran); aspen_hip_free (g->d_arrivals); aspen_hip_free (g->d_state); aspen_hip_free (g->d_prof); aspen_hip_free (g->d_trace);
+    if (g->h_abort) (void)hipHostFree (g->h_abort);
     free (g->h_layers);
     free (g);
 }
@@ -828,7 +829,7 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     CHECK (hipGetLastError ());
     dataflow_args_t a;
     a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx; a.child_rec = g->d_child_rec;
-    a.dep = g->d_dep; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran; a.arrivals = g->d_arrivals; a.prof = g->d_prof; a.host_abort = g_host_abort;
+    a.dep = g->d_dep; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran; a.arrivals = g->d_arrivals; a.prof = g->d_prof; a.host_abort = g->h_abort;
     if ((g_flags & ASPEN_HIP_FLAG_TRACE) && !g->d_trace)
     {
         g->d_trace = (unsigned long long *)aspen_hip_alloc (sizeof (unsigned long long) * 2 * (size_t)g->num_ninst);
@@ -872,9 +873,16 @@ extern "C" int aspen_hip_sync (void)
 {
     if (aspen_hip_init ()) return -1;
     CHECK (hipStreamSynchronize (g_stream));
-    if (*(volatile uint32_t *)g_host_abort != 0)
+    return 0;
+}
+
+extern "C" int aspen_hip_graph_sync (aspen_hip_graph_t *g)
+{
+    if (aspen_hip_init ()) return -1;
+    CHECK (hipStreamSynchronize (g_stream));
+    if (g && *(volatile uint32_t *)g->h_abort != 0)
     {
-        *g_host_abort = 0;
+        *g->h_abort = 0;
         snprintf (g_err, sizeof (g_err), "dataflow run stalled: a wait on the ready queue exceeded its spin limit and the run was aborted");
         fprintf (stderr, "aspen_hip: %s\n", g_err);
         return ASPEN_HIP_ERR_STALLED;

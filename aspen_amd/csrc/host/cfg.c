@@ -209,6 +209,50 @@ static int set_inout (aspen_dnn_t *dnn, aspen_layer_t *L)
     }
 }
 
+/* Checks a layer whose parents and parameters came from a file instead of a cfg section: parent indices
+   point at earlier layers, no dimension is absurd, and the geometry the file states is the one the layer's
+   parents and window parameters imply (the same derivation a cfg section goes through).  Layers
+   0 .. layer_idx-1 of the model must already have passed. */
+int aspen_layer_validate (aspen_dnn_t *dnn, aspen_layer_t *L)
+{
+    const unsigned int i = L->layer_idx;
+    if (L->type == INPUT_LAYER ? i != 0 : (i == 0 || L->parent_idx[PARENT_0] < 0 || L->parent_idx[PARENT_0] >= (int)i))
+    { ERROR_PRTF ("layer %u: bad first parent %d\n", i, L->parent_idx[PARENT_0]); return -1; }
+    if (L->parent_idx[PARENT_1] >= (int)i || L->parent_idx[PARENT_1] < -1)
+    { ERROR_PRTF ("layer %u: bad second parent %d\n", i, L->parent_idx[PARENT_1]); return -1; }
+    for (int k = 0; k < NUM_PARAM_ELEMENTS; k++)
+        if (L->params[k] > (1u << 24)) { ERROR_PRTF ("layer %u: parameter %d = %u is out of range\n", i, k, L->params[k]); return -1; }
+    unsigned int filed[NUM_PARAM_ELEMENTS];
+    memcpy (filed, L->params, sizeof (filed));
+    if (set_inout (dnn, L)) return -1;
+    static const int geometry[] = { OUT_H, OUT_W, OUT_C, IN_H, IN_W, IN_C, STRIDE };
+    /* layer kinds whose geometry follows from their parents' (image layers; the transformer kinds carry their
+       matrix extents as parameters of their own) */
+    const int derived = L->type == CONV_LAYER || L->type == MAXPOOL_LAYER || L->type == AVGPOOL_LAYER || L->type == FC_LAYER
+        || L->type == YOLO_LAYER || L->type == APPEND_LAYER
+        || ((L->type == INPUT_LAYER || L->type == RESIDUAL_LAYER || L->type == SOFTMAX_LAYER) && filed[MAT_M] == 0);
+    for (unsigned int k = 0; derived && k < sizeof (geometry) / sizeof (geometry[0]); k++)
+    {
+        const int g = geometry[k];
+        if (g == STRIDE && filed[STRIDE] == 0) continue;                       /* 0 means 1, as in a cfg section */
+        if (g == OUT_C && (L->type == CONV_LAYER || L->type == FC_LAYER)) continue;      /* free: the number of filters */
+        if (L->type == INPUT_LAYER && g >= IN_W) continue;
+        if (filed[g] != L->params[g])
+        {
+            ERROR_PRTF ("layer %u: the file states parameter %s = %u, the layer's parents and window imply %u\n",
+                i, param_type_str[g], filed[g], L->params[g]);
+            return -1;
+        }
+    }
+    if ((L->type == MATMUL_LAYER || L->type == K_ATTENTION_LAYER) && filed[MAT_K] != L->params[MAT_K])
+    { ERROR_PRTF ("layer %u: the file states K = %u, the layer's parent implies %u\n", i, filed[MAT_K], L->params[MAT_K]); return -1; }
+    /* what was compared is equal; everything else stays as the file has it */
+    const unsigned int stride = L->params[STRIDE];
+    memcpy (L->params, filed, sizeof (filed));
+    if (derived && filed[STRIDE] == 0) L->params[STRIDE] = stride;
+    return 0;
+}
+
 aspen_dnn_t *aspen_parse_cfg (const char *path)
 {
     const char *ext = strrchr (path, '.');

@@ -75,6 +75,16 @@ aspen_dnn_t *apu_create_dnn (char *input_path, char *data_path)
     return dnn;
 }
 
+/* reference include/apu.h:46 (src/apu_file_io.c:48): loads an ASPEN_DATA weight file into an existing model,
+   also one whose graphs have already run: the layers' device copies are dropped, and every ready pool that
+   holds a graph of this model rebuilds its device graph before its next run. */
+void apu_load_dnn_data_from_file (aspen_dnn_t *dnn, char *input_path)
+{
+    if (dnn == NULL || input_path == NULL) { ERROR_PRTF ("apu_load_dnn_data_from_file: NULL argument\n"); return; }
+    aspen_hip_sync ();                 /* nothing in flight may still read the buffers about to be released */
+    aspen_load_weight_file (dnn, input_path);
+}
+
 void apu_destroy_dnn (aspen_dnn_t *dnn)
 {
     if (dnn == NULL) return;
@@ -126,6 +136,8 @@ static void ochw_to_ohwc (const float *src, float *dst, unsigned int O, unsigned
 
 static void invalidate_device (aspen_layer_t *L)
 {
+    /* device graphs that were built from these buffers must not run again as they are */
+    if ((L->d_weight || L->d_bias || L->d_ktab) && L->dnn != NULL) L->dnn->dev_generation++;
     aspen_hip_free (L->d_weight); aspen_hip_free (L->d_bias); aspen_hip_free (L->d_ktab);
     L->d_weight = NULL; L->d_bias = NULL; L->d_ktab = NULL;
 }
@@ -158,12 +170,39 @@ int aspen_load_weight_file (aspen_dnn_t *dnn, const char *path)
         if ((p = expect_line (fp, line, sizeof (line), "DATA_SIZE:", 0)) == NULL) goto done;
         const size_t bytes = (size_t)atoll (p);
         if (expect_line (fp, line, sizeof (line), "DATA_START:", 0) == NULL) goto done;
-        float *buf = malloc (bytes ? bytes : 1);
-        if (buf == NULL || fread (buf, 1, bytes, fp) != bytes)
+        /* the size the tensor must have is known from the layer: checked BEFORE anything is allocated, so a
+           file cannot ask for an arbitrary amount of memory */
+        size_t expect;
+        int skip = 0;
+        if (strcmp (kind, "WEIGHT") == 0) expect = L->weight.num_elements * sizeof (float);
+        else if (strcmp (kind, "BIAS") == 0) expect = L->bias.num_elements * sizeof (float);
+        else if (strcmp (kind, "BN_VAR") == 0 || strcmp (kind, "BN_MEAN") == 0 || strcmp (kind, "BN_WEIGHT") == 0) expect = L->gemm_m * sizeof (float);
+        else if (strcmp (kind, "INPUT") == 0 || strcmp (kind, "OUTPUT") == 0) { expect = bytes; skip = 1; }
+        else
         {
-            ERROR_PRTF ("ASPEN DNN file %s parse error: Failed to read data.\n", path);
-            free (buf);
+            ERROR_PRTF ("ASPEN DNN file %s file layer %d parse error: Invalid TENSOR_TYPE %s.\n", path, file_layer, kind);
             goto done;
+        }
+        if (bytes != expect)
+        {
+            ERROR_PRTF ("ASPEN DNN file %s parse error: Layer %u %s_TENSOR size mismatch. Tensor: %zu, File: %zu.\n",
+                path, L->layer_idx, kind, expect, bytes);
+            goto done;
+        }
+        float *buf = NULL;
+        if (skip)
+        {
+            if (fseek (fp, (long)bytes, SEEK_CUR) != 0) { ERROR_PRTF ("ASPEN DNN file %s parse error: Failed to read data.\n", path); goto done; }
+        }
+        else
+        {
+            buf = malloc (bytes ? bytes : 1);
+            if (buf == NULL || fread (buf, 1, bytes, fp) != bytes)
+            {
+                ERROR_PRTF ("ASPEN DNN file %s parse error: Failed to read data.\n", path);
+                free (buf);
+                goto done;
+            }
         }
         if (expect_line (fp, line, sizeof (line), "DATA_END", 0) == NULL) { free (buf); goto done; }
         const unsigned int *q = L->params;

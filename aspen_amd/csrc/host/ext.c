@@ -82,6 +82,8 @@ int aspen_rpool_dataflow_trace (rpool_t *rp, uint64_t *start_end)
     return aspen_hip_dataflow_trace (rp->graph, start_end, aspen_rpool_num_ninst (rp));
 }
 
+unsigned int aspen_dnn_device_generation (aspen_dnn_t *dnn) { return dnn ? dnn->dev_generation : 0; }
+
 unsigned int aspen_rpool_num_ninst (rpool_t *rp)
 {
     unsigned int n = 0;

@@ -237,6 +237,9 @@ aspen_dnn_t *apu_load_dnn_from_file (char *filename)
             L->params[a] = (unsigned int)b;
         }
         if (next_line (fp, line, "LAYER_PARAMS_END") == NULL || next_line (fp, line, "LAYER_TENSORS:") == NULL) goto fail;
+        if (L->layer_idx != i) { ERROR_PRTF ("ASPEN DNN file %s: layer %u carries index %u.\n", filename, i, L->layer_idx); goto fail; }
+        /* the tensors are sized from these parameters and the kernels index with them */
+        if (aspen_layer_validate (dnn, L)) { ERROR_PRTF ("ASPEN DNN file %s: layer %u has inconsistent parameters.\n", filename, i); goto fail; }
         if (aspen_create_layer_tensors (L)) goto fail;
         for (int j = 0; j < NUM_TENSORS; j++)
         {

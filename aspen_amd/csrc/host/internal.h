@@ -16,6 +16,7 @@
 #include "aspen.h"
 #include "aspen_hip.h"
 
+#undef ERROR_PRTF     /* the library's own messages carry file and line also under SUPPRESS_OUTPUT */
 #define ERROR_PRTF(...) do { fprintf (stderr, "\033[0;31m(%s:%d) ", __FILE__, __LINE__); fprintf (stderr, __VA_ARGS__); fprintf (stderr, "\033[0m"); } while (0)
 
 struct aspen_tensor_t
@@ -50,6 +51,9 @@ struct aspen_dnn_t
     aspen_layer_t *layers;
     unsigned int num_layers;
     unsigned int ref_nasms;
+    /* grows whenever a layer's device buffers (weights, bias, k-chunk table) are released: a device graph
+       built before that holds stale pointers and is rebuilt before the next run, see dse_group_run */
+    unsigned int dev_generation;
 };
 
 struct nasm_ldata_t
@@ -110,6 +114,7 @@ struct rpool_t
     unsigned int ref_dses;
     aspen_hip_graph_t *graph;                /* merged device graph of all attached nasms */
     int graph_dirty;
+    uint64_t graph_generation;               /* sum of the attached models' dev_generation when the graph was built */
     int running;
 };
 
@@ -125,6 +130,7 @@ struct dse_group_t
 
 /* cfg.c */
 aspen_dnn_t *aspen_parse_cfg (const char *path);
+int aspen_layer_validate (aspen_dnn_t *dnn, aspen_layer_t *layer);
 /* dnn.c */
 int aspen_layer_to_device (aspen_layer_t *layer, unsigned int parent_ld);
 int aspen_load_weight_file (aspen_dnn_t *dnn, const char *path);

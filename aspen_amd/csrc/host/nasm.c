@@ -588,16 +588,18 @@ static double test_nasm_time_sec (nasm_t *nasm, unsigned int iters, int mode)
     rpool_add_nasm (rpool, nasm, NULL);
     struct timespec t0, t1;
     double sec = -1.0;
+    int ok = 1;
     for (unsigned int i = 0; i < 2 + iters; i++)
     {
         if (i == 2) { aspen_hip_sync (); clock_gettime (CLOCK_MONOTONIC, &t0); }
         dse_group_run (dse);
         dse_wait_for_nasm_completion (nasm);
         dse_group_stop (dse);
+        if (nasm->completed != 1) ok = 0;         /* a run the device gave up is no timing */
         rpool_reset_queue (rpool);
         rpool_reset_nasm (rpool, nasm);
     }
-    if (aspen_hip_sync () == 0)
+    if (aspen_hip_sync () == 0 && ok)
     {
         clock_gettime (CLOCK_MONOTONIC, &t1);
         sec = ((double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec)) / (double)iters;

@@ -126,6 +126,13 @@ void rpool_reset_nasm (rpool_t *rpool, nasm_t *nasm)
     apu_reset_nasm (nasm);
 }
 
+static uint64_t pool_generation (const rpool_t *rp)
+{
+    uint64_t g = 0;
+    for (unsigned int i = 0; i < rp->num_nasms; i++) g += rp->nasms[i]->dnn->dev_generation;
+    return g;
+}
+
 /* merged device graph of every nasm in the pool: layer and tile indices shifted, roots interleaved */
 static int rebuild_graph (rpool_t *rp)
 {
@@ -186,6 +193,7 @@ static int rebuild_graph (rpool_t *rp)
     }
     free (L); free (nl); free (np); free (co); free (ci); free (roots);
     rp->graph_dirty = rc != 0;
+    rp->graph_generation = pool_generation (rp);
     return rc;
 }
 
@@ -232,6 +240,9 @@ void dse_group_run (dse_group_t *dse_group)
     int armed = 0;
     for (unsigned int i = 0; i < rp->num_nasms; i++) armed |= rp->nasms[i]->armed;
     if (!armed) return;                                    /* nothing ready: the engines idle, as in the reference */
+    /* a model whose weights were loaded again since the graph was built has released the device buffers the
+       graph's layer descriptors point to */
+    if (rp->graph != NULL && rp->graph_generation != pool_generation (rp)) rp->graph_dirty = 1;
     if (rp->graph_dirty && rebuild_graph (rp)) { ERROR_PRTF ("ERROR: dse_group_run: graph upload failed: %s\n", aspen_hip_last_error ()); return; }
     if (rp->graph == NULL) return;
     int rc;
@@ -265,7 +276,7 @@ static void finish (rpool_t *rp)
     if (rp == NULL || !rp->running) return;
     /* a run the device gave up (watchdog, launch error) leaves its graphs NOT completed: 3 = failed */
     int state = 1;
-    if (aspen_hip_sync ()) { ERROR_PRTF ("ERROR: device run failed: %s\n", aspen_hip_last_error ()); state = 3; }
+    if (aspen_hip_graph_sync (rp->graph)) { ERROR_PRTF ("ERROR: device run failed: %s\n", aspen_hip_last_error ()); state = 3; }
     rp->running = 0;
     for (unsigned int i = 0; i < rp->num_nasms; i++)
         if (rp->nasms[i]->completed == 2) rp->nasms[i]->completed = state;

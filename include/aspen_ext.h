@@ -12,6 +12,14 @@
 extern "C" {
 #endif
 
+/* Loads an ASPEN_DATA weight file into an existing model (reference include/apu.h:46, src/apu_file_io.c:48; the
+   reference calls it from apu_create_dnn and keeps it out of its public header).  Allowed at any time
+   between runs: ready pools that hold a graph of the model pick the new weights up at their next run. */
+void apu_load_dnn_data_from_file (aspen_dnn_t *dnn, char *input_path);
+/* how often device copies of the model's weights have been released (by a reload); a ready pool compares it
+   with the value its device graph was built at */
+unsigned int aspen_dnn_device_generation (aspen_dnn_t *dnn);
+
 /* 0: one kernel launch per layer (layer-synchronous); 1: persistent dataflow kernel; 2 (default): the
    persistent kernel unless the graph's average parallelism is below half a tile per compute unit (a
    single image through a deep network), where one launch per layer is faster.

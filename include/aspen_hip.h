@@ -139,7 +139,7 @@ int aspen_hip_run_layers (aspen_hip_graph_t *graph, uint32_t first_layer, uint32
    kernel of `workgroups` workgroups (0 = a whole number per compute unit, 1 to 4, sized from the graph's
    average parallelism) pops ready tiles until all are done.
    spin_limit bounds every wait on the ready queue (0 = default); a wait that exceeds it raises the
-   abort flag, all workgroups exit and aspen_hip_sync returns ASPEN_HIP_ERR_STALLED. */
+   abort flag of THIS graph, all workgroups exit and aspen_hip_graph_sync (graph) returns ASPEN_HIP_ERR_STALLED. */
 int aspen_hip_run_dataflow (aspen_hip_graph_t *graph, uint32_t workgroups, uint64_t spin_limit);
 #define ASPEN_HIP_ERR_STALLED 0x7001
 /* Debug switches for later dataflow runs.  SKIP_TILES runs the whole dependency protocol with empty
@@ -162,7 +162,12 @@ int aspen_hip_dataflow_profile (aspen_hip_graph_t *graph, uint64_t ticks[8], int
 #define ASPEN_HIP_FLAG_TRACE 8u
 int aspen_hip_dataflow_trace (aspen_hip_graph_t *graph, uint64_t *start_end, uint32_t num_ninst);
 void aspen_hip_set_flags (uint32_t flags);
+/* Waits for everything enqueued on the library's stream.  Reports device errors only; whether a dataflow
+   run was given up is a property of its graph, see aspen_hip_graph_sync. */
 int aspen_hip_sync (void);
+/* aspen_hip_sync, then ASPEN_HIP_ERR_STALLED if the last dataflow run of `graph` was given up by its
+   watchdog (the flag is consumed).  A stall of one graph is never reported against another. */
+int aspen_hip_graph_sync (aspen_hip_graph_t *graph);
 /* 1 when everything enqueued so far has finished, 0 when still running */
 int aspen_hip_idle (void);
 /* Counters of the last dataflow run (kept under ASPEN_HIP_FLAG_COUNT_TILES): tiles executed, tiles executed

@@ -149,3 +149,69 @@ def test_shipped_resnet50_nasm_header_matches_model(capfd):
     assert not h
     capfd.readouterr()
     d.destroy()
+
+
+def _with_layer_param(raw: bytes, layer: int, param: int, value: int) -> bytes:
+    """The model file with parameter `param` of layer `layer` set to `value` (records are "\\t\\t<index> <value>")."""
+    at = -1
+    for _ in range(layer + 1):
+        at = raw.index(b"\tLAYER_PARAMS:\n", at + 1)
+    key = b"\t\t%d " % param
+    i = raw.index(key, at)
+    j = raw.index(b"\n", i)
+    return raw[:i] + key + b"%d" % value + raw[j:]
+
+
+@pytest.mark.parametrize("layer, param, value", [
+    (1, api.STRIDE, 7),             # window geometry no longer gives the stated output size
+    (1, api.OUT_H, 4000),           # output taller than its parent allows
+    (1, api.IN_C, 64),              # more input channels than the parent has
+    (1, api.PADDING, 1 << 30),      # absurd value
+    (2, api.IN_H, 1),               # pool reading a parent of another height
+    (4, api.IN_W, 9),               # FC layer over a wider image than its parent
+])
+def test_aspen_file_with_inconsistent_parameters_is_rejected(tmp_path, layer, param, value, capfd):
+    """The loader derives every layer's geometry from its parents and window, as the cfg parser does, and
+    refuses a file that states something else: tensors are sized and kernels index with these numbers."""
+    raw = open(REF_ASPEN, "rb").read()
+    assert api.lib().apu_load_dnn_from_file(str(REF_ASPEN).encode())     # untouched: loads
+    bad = tmp_path / "bad.aspen"
+    bad.write_bytes(_with_layer_param(raw, layer, param, value))
+    assert not api.lib().apu_load_dnn_from_file(str(bad).encode())
+    err = capfd.readouterr().err
+    assert "inconsistent parameters" in err
+
+
+def test_weight_file_cannot_ask_for_arbitrary_memory(tmp_path, capfd):
+    """ASPEN_DATA: a tensor's size is checked against the layer BEFORE anything is allocated."""
+    cfg, layers, tens, x, batch, seq = H.tiny_case()
+    wp = str(tmp_path / "w.bin")
+    M.write_aspen_data(wp, tens)
+    raw = open(wp, "rb").read()
+    i = raw.index(b"DATA_SIZE:") + len(b"DATA_SIZE:")
+    j = raw.index(b"\n", i)
+    huge = tmp_path / "huge.bin"
+    huge.write_bytes(raw[:i] + b"%d" % (1 << 46) + raw[j:])
+    d = api.Dnn(cfg, str(huge))                                    # prints, keeps the seeded weights (as the reference does)
+    assert "size mismatch" in capfd.readouterr().err
+    d.destroy()
+
+
+def test_reloading_weights_marks_device_graphs_stale(tmp_path):
+    """apu_load_dnn_data_from_file on a model advances its device generation only when device copies existed;
+    without a GPU no copies exist and the call just replaces the host weights."""
+    cfg, layers, tens, x, batch, seq = H.tiny_case()
+    wp = str(tmp_path / "w.bin")
+    M.write_aspen_data(wp, tens)
+    d = api.Dnn(cfg, wp)
+    before = str(tmp_path / "a.aspen"); after = str(tmp_path / "b.aspen")
+    api.lib().apu_save_dnn_to_file(d.h, before.encode())
+    tens2 = [(i, k, (a * 2).astype(np.float32)) for i, k, a in tens]
+    wp2 = str(tmp_path / "w2.bin")
+    M.write_aspen_data(wp2, tens2)
+    assert api.lib().aspen_dnn_device_generation(d.h) == 0
+    api.lib().apu_load_dnn_data_from_file(d.h, wp2.encode())
+    assert api.lib().aspen_dnn_device_generation(d.h) == 0          # nothing was on a device
+    api.lib().apu_save_dnn_to_file(d.h, after.encode())
+    assert lines_except_header(before) != lines_except_header(after)
+    d.destroy()

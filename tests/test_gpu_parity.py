@@ -650,3 +650,33 @@ def test_no_tile_starts_before_its_parents_have_ended(gpu, name, min_ninst, work
     finally:
         api.lib().aspen_hip_set_flags(2)
         net.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", [api.MODE_LAYERS, api.MODE_DATAFLOW], ids=["layers", "dataflow"])
+def test_weights_reloaded_between_runs_are_used_by_the_next_run(gpu, mode, tmp_path):
+    """apu_load_dnn_data_from_file on a model whose graph has already run releases the layers' device copies;
+    the pool notices (the model's device generation moved), rebuilds its device graph and the next
+    reset / run computes with the new weights -- checked against the oracle for both weight sets."""
+    from oracle import cpu
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()["resnet_mini_b2"])
+    tens2 = [(i, k, (a * (0.5 if k == "WEIGHT" else -1.0)).astype(np.float32)) for i, k, a in tens]
+    w2 = str(tmp_path / "w2.bin")
+    M.write_aspen_data(w2, tens2)
+    net = H.GpuNet(cfg, tens, batch, seq, min_ninst=256, mode=mode)
+    try:
+        net.run(x)
+        want = cpu.run_network(layers, tens, x, batch, seq)
+        for l in range(net.nasm.num_ldata):
+            assert H.rel_l2(net.layer(l), want[l]) <= H.REL_L2_TOL, l
+        gen = api.lib().aspen_dnn_device_generation(net.dnn.h)
+        api.lib().apu_load_dnn_data_from_file(net.dnn.h, w2.encode())
+        assert api.lib().aspen_dnn_device_generation(net.dnn.h) > gen
+        for rep in range(2):
+            net.run(x if rep == 0 else None)
+            want2 = cpu.run_network(layers, tens2, x, batch, seq)
+            for l in range(net.nasm.num_ldata):
+                assert H.rel_l2(net.layer(l), want2[l]) <= H.REL_L2_TOL, (rep, l)
+        assert H.rel_l2(want2[-1], want[-1]) > 1e-2           # the two weight sets do give different results
+    finally:
+        net.close()
