@@ -121,6 +121,21 @@ def check_against_summary(net, gold, layers, label):
     return worst
 
 
+def activation_zoo_cfg(softmax=True):
+    """Every activation the reference's naive_activate knows (reference src/naive_kernels.c:11-57) on a
+    contraction epilogue or a shortcut, a padded max pool and average pool, a [softmax] layer at the end."""
+    s = "[net]\nheight=12\nwidth=12\nchannels=5\n\n"
+    for act in ("logistic", "tanh", "elu", "selu", "leaky", "gelu", "gelu_acc", "relu", "linear"):
+        s += f"[convolutional]\nfilters=24\nsize=3\nstride=1\npad=1\nactivation={act}\n\n"
+    s += "[shortcut]\nfrom=-3\nactivation=tanh\n\n"
+    s += "[maxpool]\nsize=3\nstride=2\npad=1\n\n"
+    s += "[avgpool]\nsize=3\nstride=1\npad=1\n\n"
+    s += "[connected]\noutput=40\nactivation=logistic\n\n[connected]\noutput=17\nactivation=linear\n\n"
+    if softmax:
+        s += "[softmax]\n\n"
+    return s
+
+
 def tiny_cfg():
     """A few-kilobyte network for file-format fixtures: odd channel counts exercise the padding of the
     reference's 8-row weight interleave (the layer in front of the FC layer has 64 channels:

@@ -87,23 +87,10 @@ def test_launch_per_layer_reruns_match_oracle(gpu, name):
         net.close()
 
 
-def activation_zoo_cfg():
-    """Every activation the reference's naive_activate knows (reference src/naive_kernels.c:11-57) on a
-    contraction epilogue or a shortcut, a padded max pool and average pool, a [softmax] layer at the end."""
-    s = "[net]\nheight=12\nwidth=12\nchannels=5\n\n"
-    for act in ("logistic", "tanh", "elu", "selu", "leaky", "gelu", "gelu_acc", "relu", "linear"):
-        s += f"[convolutional]\nfilters=24\nsize=3\nstride=1\npad=1\nactivation={act}\n\n"
-    s += "[shortcut]\nfrom=-3\nactivation=tanh\n\n"
-    s += "[maxpool]\nsize=3\nstride=2\npad=1\n\n"
-    s += "[avgpool]\nsize=3\nstride=1\npad=1\n\n"
-    s += "[connected]\noutput=40\nactivation=logistic\n\n[connected]\noutput=17\nactivation=linear\n\n[softmax]\n\n"
-    return s
-
-
 @pytest.mark.parametrize("mode", [api.MODE_LAYERS, api.MODE_DATAFLOW], ids=["layers", "dataflow"])
 def test_every_activation_and_softmax_match_oracle(gpu, mode):
     from oracle import cpu
-    cfg = activation_zoo_cfg()
+    cfg = H.activation_zoo_cfg()
     layers = M.parse_cfg(cfg)
     tens = M.synth_weights(layers, 21, "he")
     batch = 3

@@ -38,11 +38,20 @@ def test_oracle_resnet50_b1_summary():
 
 
 @pytest.mark.skipif(not ref.available(), reason="oracle/_ref (reference build) not present")
-@pytest.mark.parametrize("name", ["custom_b3", "bert_mini_b2_s24"])
+@pytest.mark.parametrize("name", ["custom_b3", "bert_mini_b2_s24", "activation_zoo"])
 def test_oracle_matches_compiled_reference(name, tmp_path):
     """Layer by layer against the reference's own tiled_* kernels, including its packed weights
-    and its result unpacker."""
-    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()[name])
+    and its result unpacker.  "activation_zoo" runs every activation of naive_activate and padded pools
+    through the reference, with inputs of both signs (without the closing [softmax] layer: the reference's
+    tiler divides by zero on a softmax layer outside a transformer; the oracle's softmax is pinned by torch)."""
+    if name == "activation_zoo":
+        cfg = H.activation_zoo_cfg(softmax=False)
+        layers = M.parse_cfg(cfg)
+        tens = M.synth_weights(layers, 21, "he")
+        batch, seq = 3, 0
+        x = (M.synth_input(layers, 21, batch, 0, "token_ids") * 2.0 - 1.0).astype(np.float32)
+    else:
+        cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()[name])
     wp = str(tmp_path / "w.bin")
     M.write_aspen_data(wp, tens)
     net = ref.RefNet(cfg, wp, batch, seq, threads=2)

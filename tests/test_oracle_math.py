@@ -54,6 +54,11 @@ def test_activations_closed_forms():
     assert np.allclose(cpu.activate(x, 5), np.where(x > 0, x, 0.1 * x), rtol=1e-6)
     assert np.allclose(cpu.activate(x, 6), np.where(x > 0, x, 0.1 * (np.exp(x.astype(np.float64)) - 1)), rtol=1e-6)
     assert np.allclose(cpu.activate(x, 7), np.where(x > 0, 1.0507 * x, 1.0507 * 1.67326 * (np.exp(x.astype(np.float64)) - 1)), rtol=1e-6)
+    # the same two against the library forms: ELU with the reference's alpha 0.1; SELU, whose published
+    # constants (1.0507009873554805, 1.6732632423543772) the reference rounds to 1.0507 and 1.67326
+    assert np.allclose(cpu.activate(x, 6), F.elu(t, alpha=0.1).numpy(), rtol=1e-6, atol=1e-7)
+    assert np.allclose(cpu.activate(x, 7), F.selu(t).numpy(), rtol=3e-6, atol=1e-7)
+    assert not np.allclose(cpu.activate(x, 6), F.elu(t, alpha=1.0).numpy(), rtol=1e-3)       # alpha is discriminated
     assert np.allclose(cpu.activate(x, 1), torch.sigmoid(t).numpy(), rtol=1e-6)
     assert np.allclose(cpu.activate(x, 3), torch.tanh(t).numpy(), rtol=1e-6)
     assert np.allclose(cpu.activate(x, 8), F.gelu(t).numpy(), rtol=1e-5, atol=2e-6)      # float erff
