@@ -121,16 +121,16 @@ def check_against_summary(net, gold, layers, label):
     return worst
 
 
-def activation_zoo_cfg(softmax=True):
+def activation_zoo_cfg(softmax=True, filters=24, hidden=40):
     """Every activation the reference's naive_activate knows (reference src/naive_kernels.c:11-57) on a
     contraction epilogue or a shortcut, a padded max pool and average pool, a [softmax] layer at the end."""
     s = "[net]\nheight=12\nwidth=12\nchannels=5\n\n"
     for act in ("logistic", "tanh", "elu", "selu", "leaky", "gelu", "gelu_acc", "relu", "linear"):
-        s += f"[convolutional]\nfilters=24\nsize=3\nstride=1\npad=1\nactivation={act}\n\n"
+        s += f"[convolutional]\nfilters={filters}\nsize=3\nstride=1\npad=1\nactivation={act}\n\n"
     s += "[shortcut]\nfrom=-3\nactivation=tanh\n\n"
     s += "[maxpool]\nsize=3\nstride=2\npad=1\n\n"
     s += "[avgpool]\nsize=3\nstride=1\npad=1\n\n"
-    s += "[connected]\noutput=40\nactivation=logistic\n\n[connected]\noutput=17\nactivation=linear\n\n"
+    s += f"[connected]\noutput={hidden}\nactivation=logistic\n\n[connected]\noutput=17\nactivation=linear\n\n"
     if softmax:
         s += "[softmax]\n\n"
     return s

@@ -43,9 +43,11 @@ def test_oracle_matches_compiled_reference(name, tmp_path):
     """Layer by layer against the reference's own tiled_* kernels, including its packed weights
     and its result unpacker.  "activation_zoo" runs every activation of naive_activate and padded pools
     through the reference, with inputs of both signs (without the closing [softmax] layer: the reference's
-    tiler divides by zero on a softmax layer outside a transformer; the oracle's softmax is pinned by torch)."""
+    tiler divides by zero on a softmax layer outside a transformer; the oracle's softmax is pinned by torch;
+    64 channels in front of each connected layer, whose reference kernel assumes that its parent's column
+    stride equals its channel count)."""
     if name == "activation_zoo":
-        cfg = H.activation_zoo_cfg(softmax=False)
+        cfg = H.activation_zoo_cfg(softmax=False, filters=64, hidden=64)
         layers = M.parse_cfg(cfg)
         tens = M.synth_weights(layers, 21, "he")
         batch, seq = 3, 0
