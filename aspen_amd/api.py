@@ -115,6 +115,9 @@ def lib() -> C.CDLL:
         "aspen_hip_event_elapsed_ms": (C.c_int, [C.c_int, C.c_int, _fp]),
         "aspen_hip_sgemm": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, _vp, C.c_uint32, _vp, C.c_uint32, _vp,
                                       C.c_uint32, _vp, C.c_int]),
+        "aspen_hip_sgemm_static": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, _vp, C.c_uint32, _vp, C.c_uint32, _vp,
+                                             C.c_uint32, _vp, C.c_int]),
+        "aspen_hip_sgemm_static_max_bytes": (C.c_size_t, []),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)

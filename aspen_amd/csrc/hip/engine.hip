@@ -349,6 +349,8 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
     }
 }
 
+__global__ void sgemm_kernel (const aspen_hip_layer_t L);       // defined with aspen_hip_sgemm_static
+
 // ------------------------------------------------------------------------------------------------
 // device, memory
 // ------------------------------------------------------------------------------------------------
@@ -365,6 +367,7 @@ extern "C" int aspen_hip_init (void)
     CHECK (hipStreamCreate (&g_stream));
     for (int i = 0; i < NUM_EVENTS; i++) CHECK (hipEventCreate (&g_events[i]));
     CHECK (hipFuncSetAttribute ((const void *)layer_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
+    CHECK (hipFuncSetAttribute ((const void *)sgemm_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
     CHECK (hipFuncSetAttribute ((const void *)dataflow_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
     CHECK (hipFuncSetAttribute ((const void *)dataflow_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
     // how many persistent workgroups really fit a compute unit (registers, LDS): the default grid
@@ -964,5 +967,87 @@ extern "C" int aspen_hip_sgemm (uint32_t M, uint32_t N, uint32_t K, const float 
     if (e == hipSuccess) e = hipStreamSynchronize (g_stream);
     aspen_hip_free (dL); aspen_hip_free (Ap);
     if (e != hipSuccess) return fail (e, "sgemm launch");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+// SGEMM that allocates nothing (for callers that cannot call hipMalloc: code under stream capture, tight
+// serving loops).  aspen_hip_sgemm stages A into a zero-padded copy it allocates and frees per call; here that
+// staging copy lives in a file-scope device array, and the layer descriptor travels as a kernel argument.
+// Each device holds its own copy of the array at its own address: the address is looked up once per device
+// with hipGetSymbolAddress and only that pointer is ever handed to kernels.  Every call on a device shares the
+// array (it keeps the previous call's contents, so the padding rows are rewritten each time): calls are ordered
+// by the library's one stream; calls made concurrently from several host threads would race.
+// ------------------------------------------------------------------------------------------------
+#define SGEMM_SCRATCH_BYTES (8u << 20)
+#define MAX_DEVICES 16
+static __device__ __align__ (256) unsigned char scratch[SGEMM_SCRATCH_BYTES];
+static float *g_scratch_ptr[MAX_DEVICES];           // device address of `scratch` per device, see scratch_for_current_device
+
+static float *scratch_for_current_device (void)
+{
+    int dev = -1;
+    if (hipGetDevice (&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) { snprintf (g_err, sizeof (g_err), "sgemm_static: no current device"); return nullptr; }
+    if (g_scratch_ptr[dev] == nullptr)
+    {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress (&p, HIP_SYMBOL (scratch));
+        if (e != hipSuccess || p == nullptr) { fail (e, "hipGetSymbolAddress (scratch)"); return nullptr; }
+        g_scratch_ptr[dev] = (float *)p;
+    }
+    return g_scratch_ptr[dev];
+}
+
+// dst[r][0..K) = src[r][0..K) for r < M, zeros for M <= r < Mp; K % 4 == 0, lda % 4 == 0
+__global__ void __launch_bounds__ (WG_THREADS) pad_rows_kernel (const float *__restrict__ src, uint32_t lda, float *__restrict__ dst, uint32_t M, uint32_t Mp, uint32_t K)
+{
+    const uint32_t k4 = K >> 2;
+    const size_t n = (size_t)Mp * k4, step = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += step)
+    {
+        const uint32_t r = (uint32_t)(i / k4), c = (uint32_t)(i - (size_t)r * k4) * 4;
+        const float4 v = r < M ? gld4 (src + (size_t)r * lda + c) : make_float4 (0.f, 0.f, 0.f, 0.f);
+        st4 (dst + (size_t)r * K + c, v);
+    }
+}
+
+// one contraction tile per workgroup, the descriptor in the kernel-argument segment
+__global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) sgemm_kernel (const aspen_hip_layer_t L)
+{
+    extern __shared__ __align__ (16) float smem[];
+    run_tile<0> (L, blockIdx.x, smem, [] () { return (uint32_t *)nullptr; });
+}
+
+extern "C" size_t aspen_hip_sgemm_static_max_bytes (void) { return SGEMM_SCRATCH_BYTES; }
+
+extern "C" int aspen_hip_sgemm_static (uint32_t M, uint32_t N, uint32_t K, const float *A, uint32_t lda, const float *B,
+    uint32_t ldb, float *C, uint32_t ldc, const float *bias, int act)
+{
+    if (aspen_hip_init ()) return -1;
+    if (M == 0 || N == 0 || !A || !B || !C) { snprintf (g_err, sizeof (g_err), "sgemm_static: empty problem or null pointer"); return -1; }
+    if (K == 0 || K % GEMM_BK || lda % 4 || ldb % 4 || ldc % 4 || lda < K || ldb < K || ldc < M)
+    { snprintf (g_err, sizeof (g_err), "sgemm_static: K must be a multiple of 32, strides multiples of 4"); return -1; }
+    if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) % 16 || (bias && (uintptr_t)bias % 4))
+    { snprintf (g_err, sizeof (g_err), "sgemm_static: A, B and C must be 16-byte aligned"); return -1; }
+    const uint64_t Mp = ((uint64_t)M + 127) / 128 * 128;
+    if (Mp * K * sizeof (float) > SGEMM_SCRATCH_BYTES)
+    {
+        snprintf (g_err, sizeof (g_err), "sgemm_static: roundup (M, 128) * K * 4 = %llu bytes exceeds the static staging buffer of %u bytes; use aspen_hip_sgemm",
+            (unsigned long long)(Mp * K * sizeof (float)), SGEMM_SCRATCH_BYTES);
+        return -1;
+    }
+    if ((uint64_t)N * ldc * 4 >= 0xffffff00ull || (uint64_t)N * ldb * 4 >= 0xffffff00ull) { snprintf (g_err, sizeof (g_err), "sgemm_static: matrix larger than 4 GiB"); return -1; }
+    float *Ap = scratch_for_current_device ();
+    if (!Ap) return -1;
+    hipLaunchKernelGGL (pad_rows_kernel, dim3 (stream_grid ((size_t)Mp * (K / 4))), dim3 (WG_THREADS), 0, g_stream, A, lda, Ap, M, (uint32_t)Mp, K);
+    CHECK (hipGetLastError ());
+    aspen_hip_layer_t L;
+    memset (&L, 0, sizeof (L));
+    L.type = MATMUL_LAYER; L.act = act; L.variant = ASPEN_HIP_GEMM_SMALL; L.direct = 1;
+    L.M = M; L.N = N; L.ld = ldc; L.tile_m = VAR2_BM; L.tile_n = VAR2_BN;
+    L.tiles_m = (M + VAR2_BM - 1) / VAR2_BM; L.tiles_n = (N + VAR2_BN - 1) / VAR2_BN; L.num_ninst = L.tiles_m * L.tiles_n; L.splits = 1;
+    L.K = K; L.Kp = K; L.ld0 = ldb; L.out = C; L.in0 = B; L.weight = Ap; L.bias = bias;
+    hipLaunchKernelGGL (sgemm_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, L);
+    CHECK (hipGetLastError ());
     return 0;
 }

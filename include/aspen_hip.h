@@ -192,6 +192,17 @@ int aspen_hip_event_elapsed_ms (int slot_begin, int slot_end, float *ms);
 int aspen_hip_sgemm (uint32_t M, uint32_t N, uint32_t K, const float *A, uint32_t lda, const float *B,
     uint32_t ldb, float *C, uint32_t ldc, const float *bias, int act);
 
+/* The same SGEMM for callers that cannot allocate device memory (code under stream capture, tight serving
+   loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  It calls no hipMalloc / hipFree:
+   the zero-padded staging copy of A that aspen_hip_sgemm allocates per call lives in a static device array of
+   aspen_hip_sgemm_static_max_bytes () bytes (8 MiB per GPU, held until the process ends), so
+   roundup (M, 128) * K * 4 must not exceed that; larger problems are refused with a message.  Asynchronous on
+   the library's stream: C is complete after aspen_hip_sync ().  All calls on a GPU share the one staging
+   array; the library's stream orders them, calls issued concurrently from several host threads would race. */
+int aspen_hip_sgemm_static (uint32_t M, uint32_t N, uint32_t K, const float *A, uint32_t lda, const float *B,
+    uint32_t ldb, float *C, uint32_t ldc, const float *bias, int act);
+size_t aspen_hip_sgemm_static_max_bytes (void);
+
 #ifdef __cplusplus
 }
 #endif
