@@ -261,10 +261,14 @@ class RPool:
 
     def dataflow_profile(self, reset: bool = True) -> dict:
         """Summed workgroup time of dataflow runs since the last reset, in seconds (profile flag 4)."""
-        t = (C.c_uint64 * 8)()
+        t = (C.c_uint64 * 16)()
         if lib().aspen_rpool_dataflow_profile(self.h, t, 1 if reset else 0):
             raise RuntimeError("no dataflow profile")
-        return {k: t[i] * 1e-8 for i, k in enumerate(["tile", "drain", "sched", "total", "publish", "ticket", "slot_wait"])}
+        d = {k: t[i] * 1e-8 for i, k in enumerate(["tile", "drain", "sched", "total", "publish", "ticket", "slot_wait"])}
+        for i, k in enumerate(["gemm_setup", "gemm_kloop", "gemm_epilogue", "gemm_splitk"]):
+            d[k] = t[8 + i] * 1e-8
+        d["engine_clock_mhz"] = t[7] / max(t[3], 1) * 100.0
+        return d
 
     def dataflow_trace(self) -> np.ndarray:
         """[tiles][2] start / end stamps (100 MHz ticks) of the last run made with the trace flag (8)."""

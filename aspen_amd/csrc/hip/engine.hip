@@ -20,7 +20,8 @@ typedef unsigned long long qentry_t;      // ready-queue entry / child-record en
 #define ST_DONE 64
 #define ST_ABORT 96
 #define ST_TWICE 128
-#define ST_WORDS 160
+#define ST_SINKS 160
+#define ST_WORDS 192
 #define NUM_EVENTS 16
 #define DEFAULT_SPIN_LIMIT (1ull << 26)
 
@@ -34,9 +35,10 @@ struct aspen_hip_graph_t
     qentry_t *d_queue;      // ready queue: slot t is written once, by whoever makes a tile ready
     qentry_t *d_child_rec;  // per tile: child count + its first CHILD_REC-1 children with their layers
     uint32_t *d_state;      // one counter per 128-byte line: [ST_HEAD] pop tickets, [ST_TAIL] push cursor, [ST_DONE] tiles done,
-                            // [ST_ABORT] abort flag, [ST_TWICE] tiles executed more than once
+                            // [ST_ABORT] abort flag, [ST_TWICE] tiles executed more than once, [ST_SINKS] finished tiles without children
     uint32_t *d_ran;        // per-tile execution count (sanity: every tile exactly once)
     uint32_t *d_arrivals;   // split-K arrival counters, see run_tile
+    uint32_t num_sinks;     // tiles without children
     uint32_t epoch;         // tag of the last run's queue entries, cycles 1..255
     unsigned long long *d_prof;
     uint32_t default_workgroups;    // grid of a dataflow run when the caller names none, see graph_parallelism
@@ -129,6 +131,7 @@ __global__ void arm_kernel (uint32_t *dep, const uint32_t *num_parents, qentry_t
         __hip_atomic_store (&state[ST_DONE], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store (&state[ST_ABORT], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store (&state[ST_TWICE], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store (&state[ST_SINKS], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 
@@ -144,6 +147,7 @@ struct dataflow_args_t
     unsigned long long *trace;      // per-tile start / end time stamps when ASPEN_HIP_FLAG_TRACE is set
     unsigned long long *prof;       // 8 counters of summed 100 MHz ticks, see aspen_hip_dataflow_profile
     uint32_t num_ninst;
+    uint32_t num_sinks;             // tiles without children: when all of them have finished, so has every tile
     uint32_t epoch;                 // 1..255, tag of this run's queue entries
     uint32_t flags;                 // ASPEN_HIP_FLAG_*
     uint32_t queue_row;             // see queue_slot
@@ -153,8 +157,10 @@ struct dataflow_args_t
 #define CHILD_REC 64     // entries per child record: one per lane of the publishing wavefront
 #define QENTRY_EMPTY (~(qentry_t)0)
 
-// Waits until queue slot `ticket` holds a tile of this run and returns the entry; QENTRY_EMPTY when all
-// tickets are taken or the run was aborted.  The wait polls with relaxed device-scope loads (an
+// Waits until queue slot `ticket` holds an entry of this run and returns it; QENTRY_EMPTY when all tickets
+// are taken or the run was aborted.  An entry whose tile is QUEUE_EMPTY tells the workgroup to leave: the
+// workgroup that finishes the run's last tile writes it to the slots that will never be served, see
+// schedule_step.  The wait polls with relaxed device-scope loads (an
 // acquire here would invalidate this XCD's L2 on every poll).
 __device__ __forceinline__ qentry_t wait_for_slot (const dataflow_args_t &a, uint32_t ticket)
 {
@@ -186,11 +192,13 @@ struct sched_lds_t
     dataflow_args_t a;
     uint32_t tile, layer;                // tile to run next (QUEUE_EMPTY: leave) and its layer
     uint32_t complete;                   // 0: the tile just run was a split-K slice that did not finish its group
+    uint32_t may_keep;                   // the tile just run releases children, one of which this workgroup may run next
     // the descriptors of the last few layers this workgroup worked on: consecutive tiles mostly belong
     // to the same two or three layers, so most tiles find theirs here instead of fetching it from memory
     uint32_t desc_slot, desc_next, desc_id[DESC_CACHE];
     aspen_hip_layer_t desc[DESC_CACHE];
     unsigned long long t0, ticks[6];     // profiling: last time stamp; tile / drain / scheduling / publish / ticket / slot-wait ticks
+    unsigned long long p0, phase[4];     // profiling of contraction tiles: last phase stamp; set-up / K loop / epilogue / split-K ticks
 };
 __shared__ sched_lds_t s_sched;
 
@@ -203,70 +211,52 @@ __device__ __forceinline__ void prof_lap (int which)
     }
 }
 
-// Counts down one child; whoever takes its counter to zero puts it into the ready queue.
-__device__ __forceinline__ void release_child (const dataflow_args_t &a, uint32_t child, uint32_t layer)
+__device__ void tile_phase_lap (int which)
 {
-    const uint32_t before = __hip_atomic_fetch_sub (&a.dep[child], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (before == 1u)
+    if ((s_sched.a.flags & ASPEN_HIP_FLAG_PROFILE) && threadIdx.x == 0)
     {
-        const uint32_t slot = atomicAdd (&a.state[ST_TAIL], 1u);
-        __hip_atomic_store (&a.queue[queue_slot (slot, a.queue_row)], make_entry (a.epoch, layer, child), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned long long t = wall_clock64 ();
+        s_sched.phase[which - 8] += t - s_sched.p0; s_sched.p0 = t;
     }
 }
 
-// One scheduling step of a workgroup, as a real function call (it needs few registers, all of them
-// caller-saved, so the call costs no register traffic): wavefront 0 publishes the finished tile
-// (dependency countdown of its children, push of those that became ready) while wavefront 1 pops the
-// next one.  done == QUEUE_EMPTY: nothing to publish (first step).  `rec` is this lane's entry of the
-// finished tile's child record, fetched by wavefront 0 before the tile ran, so publishing starts
-// with the atomics right away.  Returns the tile to run next; its layer is left in s_sched.layer.
-// The reference's counterpart is dse_schedule / update_children (src/dse.c:20-108, :363-401).
-__device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
+// Puts a tile that has become ready into the queue.
+__device__ __forceinline__ void push_ready (const dataflow_args_t &a, uint32_t child, uint32_t layer)
 {
-    const dataflow_args_t &a = s_sched.a;
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    if (done != QUEUE_EMPTY)
+    const uint32_t slot = atomicAdd (&a.state[ST_TAIL], 1u);
+    __hip_atomic_store (&a.queue[queue_slot (slot, a.queue_row)], make_entry (a.epoch, layer, child), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// One scheduling step of a workgroup, as a real function call (it needs few registers, all of them
+// caller-saved, so the call costs no register traffic).  done == QUEUE_EMPTY: nothing to publish (first
+// step).  `rec` is this lane's entry of the finished tile's child record, fetched by wavefront 0 before the
+// tile ran, so publishing starts with the atomics right away.  Returns the tile to run next; its layer is
+// left in s_sched.layer.
+//
+// Publish: one child per lane of wavefront 0, a relaxed device-scope countdown of the child's counter.  The
+// FIRST child whose counter this brings to zero is kept: it is this workgroup's next tile, with no trip
+// through the queue (the reference's depth-first hand-off: the thread that completes a ninst's last parent
+// runs that ninst next and pushes only the others it made ready, src/dse.c:363-401).  It saves the two
+// atomic round trips and the poll of a pop on the chain parent -> child, and the child finds its parent's
+// output in this XCD's L2.  Only a workgroup that kept nothing draws a ticket and waits for its queue slot.
+// A tile that cannot release anything (no children, or a split-K slice that was not the last of its group)
+// pops while it is being accounted, as before.
+// Kept tiles never enter the queue, so fewer than num_ninst tickets are ever served.  Tiles without children
+// count themselves when they finish; the last of them (then every tile has finished, for every tile has a
+// descendant without children) writes a leave entry into the next gridDim.x slots behind the tail: every
+// workgroup holds at most one ticket, so these are all the slots anyone can still be waiting for.
+// The pop half of a scheduling step, run by one wavefront: draws a ticket, waits for its slot, and makes sure
+// the tile's layer descriptor is in the LDS cache.  kept != QUEUE_EMPTY: the tile to run is already known.
+__device__ __forceinline__ void pop_next (const dataflow_args_t &a, uint32_t lane, uint32_t kept, uint32_t kept_layer, bool prof)
+{
+    if (lane == 0)
     {
-        prof_lap (0);
-        // every wave waits until its (write-through, device-coherent) stores have been acknowledged.
-        // An explicit wait: a workgroup-scope fence does not have to wait for global stores.
-        asm volatile ("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads ();
-        prof_lap (1);
-        if ((a.flags & ASPEN_HIP_FLAG_TRACE) && threadIdx.x == 0) a.trace[2 * (size_t)done + 1] = wall_clock64 ();
-    }
-    const bool prof = (a.flags & ASPEN_HIP_FLAG_PROFILE) && lane == 0;
-    if (wave == 0 && done != QUEUE_EMPTY)
-    {
-        const unsigned long long tp = prof ? wall_clock64 () : 0;
-        // publish: relaxed device-scope atomics on the children's counters, one child per lane
-        // a split-K slice that was not the last of its group leaves the children to the one that is
-        const uint32_t count = s_sched.complete ? (uint32_t)__shfl (rec, 0, 64) : 0u;
-        if (lane >= 1 && lane <= count) release_child (a, (uint32_t)rec, (uint32_t)(rec >> 32));
-        if (count > CHILD_REC - 1)
+        if (kept != QUEUE_EMPTY) { s_sched.tile = kept; s_sched.layer = kept_layer; }
+        else
         {
-            // more children than the record holds: the rest comes from the CSR lists
-            const uint32_t c0 = a.child_off[done] + (CHILD_REC - 1), c1 = a.child_off[done + 1];
-            for (uint32_t c = c0 + lane; c < c1; c += 64)
-            {
-                const uint32_t child = a.child_idx[c];
-                release_child (a, child, a.ninst_layer[child]);
-            }
-        }
-        if (lane == 0 && (a.flags & ASPEN_HIP_FLAG_COUNT_TILES))
-        {
-            if (atomicAdd (&a.ran[done], 1u) != 0) atomicAdd (&a.state[ST_TWICE], 1u);
-            atomicAdd (&a.state[ST_DONE], 1u);
-        }
-        if (prof) { asm volatile ("s_waitcnt vmcnt(0)" ::: "memory"); s_sched.ticks[3] += wall_clock64 () - tp; }
-    }
-    else if (wave == 1)
-    {
-        if (lane == 0)
-        {
-            // pop: a ticket is drawn only now, when this workgroup is free.  Drawing it earlier would
-            // hide the atomic's round trip but binds a (possibly already ready) tile to a busy
-            // workgroup while idle ones wait on later slots.
+            // a ticket is drawn only now, when this workgroup is free.  Drawing it earlier would hide the
+            // atomic's round trip but binds a (possibly already ready) tile to a busy workgroup while idle
+            // ones wait on later slots.
             const unsigned long long t1 = prof ? wall_clock64 () : 0;
             const uint32_t ticket = atomicAdd (&a.state[ST_HEAD], 1u);
             const unsigned long long t2 = prof ? wall_clock64 () : 0;
@@ -275,24 +265,100 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
             s_sched.layer = (uint32_t)(e >> 32) & 0xffffu;
             if (prof) { s_sched.ticks[4] += t2 - t1; s_sched.ticks[5] += wall_clock64 () - t2; }
         }
-        // the popping wavefront also makes sure the tile's layer descriptor is in the LDS cache
-        // (same wavefront, program order: lane 0's LDS writes above are visible to all lanes here)
-        const uint32_t tile = __builtin_amdgcn_readfirstlane (s_sched.tile), layer = __builtin_amdgcn_readfirstlane (s_sched.layer);
-        if (tile != QUEUE_EMPTY)
-        {
-            uint32_t slot = DESC_CACHE;
-            for (uint32_t i = 0; i < DESC_CACHE; i++) if (s_sched.desc_id[i] == layer) slot = i;
-            slot = __builtin_amdgcn_readfirstlane (slot);
-            if (slot == DESC_CACHE)
-            {
-                slot = __builtin_amdgcn_readfirstlane (s_sched.desc_next);
-                if (lane < sizeof (aspen_hip_layer_t) / 4)
-                    reinterpret_cast<uint32_t *> (&s_sched.desc[slot])[lane] = reinterpret_cast<const uint32_t *> (&a.layers[layer])[lane];
-                if (lane == 0) { s_sched.desc_id[slot] = layer; s_sched.desc_next = (slot + 1) % DESC_CACHE; }
-            }
-            if (lane == 0) s_sched.desc_slot = slot;
-        }
     }
+    // (same wavefront, program order: lane 0's LDS writes above are visible to all lanes here)
+    const uint32_t tile = __builtin_amdgcn_readfirstlane (s_sched.tile), layer = __builtin_amdgcn_readfirstlane (s_sched.layer);
+    if (tile != QUEUE_EMPTY)
+    {
+        uint32_t slot = DESC_CACHE;
+        for (uint32_t i = 0; i < DESC_CACHE; i++) if (s_sched.desc_id[i] == layer) slot = i;
+        slot = __builtin_amdgcn_readfirstlane (slot);
+        if (slot == DESC_CACHE)
+        {
+            slot = __builtin_amdgcn_readfirstlane (s_sched.desc_next);
+            if (lane < sizeof (aspen_hip_layer_t) / 4)
+                reinterpret_cast<uint32_t *> (&s_sched.desc[slot])[lane] = reinterpret_cast<const uint32_t *> (&a.layers[layer])[lane];
+            if (lane == 0) { s_sched.desc_id[slot] = layer; s_sched.desc_next = (slot + 1) % DESC_CACHE; }
+        }
+        if (lane == 0) s_sched.desc_slot = slot;
+    }
+}
+
+__device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
+{
+    const dataflow_args_t &a = s_sched.a;
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (done != QUEUE_EMPTY)
+    {
+        prof_lap (0);
+        // a tile that releases children may keep one of them: then the pop waits for the outcome of the
+        // countdown; otherwise wavefront 1 pops while wavefront 0 does the accounting
+        if (threadIdx.x == 0)
+            s_sched.may_keep = s_sched.complete && (uint32_t)rec != 0u && !(a.flags & ASPEN_HIP_FLAG_NO_HANDOFF);
+        // every wave waits until its (write-through, device-coherent) stores have been acknowledged.
+        // An explicit wait: a workgroup-scope fence does not have to wait for global stores.
+        asm volatile ("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads ();
+        prof_lap (1);
+        if ((a.flags & ASPEN_HIP_FLAG_TRACE) && threadIdx.x == 0) a.trace[2 * (size_t)done + 1] = wall_clock64 ();
+    }
+    const bool prof = (a.flags & ASPEN_HIP_FLAG_PROFILE) && lane == 0;
+    const bool may_keep = done != QUEUE_EMPTY && __builtin_amdgcn_readfirstlane (s_sched.may_keep) != 0u;
+    if (wave == 0 && done != QUEUE_EMPTY)
+    {
+        const unsigned long long tp = prof ? wall_clock64 () : 0;
+        uint32_t kept = QUEUE_EMPTY, kept_layer = 0;
+        // a split-K slice that was not the last of its group leaves the children to the one that is
+        const uint32_t listed = (uint32_t)__shfl (rec, 0, 64), count = s_sched.complete ? listed : 0u;
+        const uint32_t child = (uint32_t)rec, layer = (uint32_t)(rec >> 32);
+        bool ready = false;
+        if (lane >= 1 && lane <= count)
+            ready = __hip_atomic_fetch_sub (&a.dep[child], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 1u;
+        if (may_keep)
+        {
+            const unsigned long long made_ready = __ballot (ready);
+            if (made_ready)
+            {
+                const int keeper = __builtin_ctzll (made_ready);
+                kept = (uint32_t)__shfl (child, keeper, 64);
+                kept_layer = (uint32_t)__shfl (layer, keeper, 64);
+                ready = ready && (int)lane != keeper;
+            }
+        }
+        if (ready) push_ready (a, child, layer);
+        if (count > CHILD_REC - 1)
+        {
+            // more children than the record holds: the rest comes from the CSR lists and goes through the queue
+            const uint32_t c0 = a.child_off[done] + (CHILD_REC - 1), c1 = a.child_off[done + 1];
+            for (uint32_t c = c0 + lane; c < c1; c += 64)
+            {
+                const uint32_t ch = a.child_idx[c];
+                if (__hip_atomic_fetch_sub (&a.dep[ch], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 1u) push_ready (a, ch, a.ninst_layer[ch]);
+            }
+        }
+        if (listed == 0u)
+        {
+            // a tile without children (no hand-off, so wavefront 1 is popping meanwhile): was it the run's last?
+            uint32_t last = 0;
+            if (lane == 0) last = __hip_atomic_fetch_add (&a.state[ST_SINKS], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u == a.num_sinks;
+            if (__shfl (last, 0, 64))
+            {
+                // the run is over and nothing will be pushed any more: tell everyone who waits, this workgroup's
+                // own popping wavefront included
+                const uint32_t tail = __hip_atomic_load (&a.state[ST_TAIL], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (uint32_t t = tail + lane; t < tail + gridDim.x && t < a.num_ninst; t += 64)
+                    __hip_atomic_store (&a.queue[queue_slot (t, a.queue_row)], make_entry (a.epoch, 0, QUEUE_EMPTY), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        if (lane == 0 && (a.flags & ASPEN_HIP_FLAG_COUNT_TILES))
+        {
+            if (atomicAdd (&a.ran[done], 1u) != 0) atomicAdd (&a.state[ST_TWICE], 1u);
+            atomicAdd (&a.state[ST_DONE], 1u);
+        }
+        if (prof) s_sched.ticks[3] += wall_clock64 () - tp;
+        if (may_keep) pop_next (a, lane, kept, kept_layer, prof);
+    }
+    else if (wave == 1 && !may_keep) pop_next (a, lane, QUEUE_EMPTY, 0, prof);
     __syncthreads ();
     const uint32_t next = s_sched.tile;
     prof_lap (2);
@@ -312,11 +378,13 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
         s_sched.a = args;
         s_sched.t0 = wall_clock64 ();
         for (int i = 0; i < 6; i++) s_sched.ticks[i] = 0;
+        for (int i = 0; i < 4; i++) s_sched.phase[i] = 0;
         s_sched.desc_next = 0;
+        s_sched.may_keep = 0;
         for (int i = 0; i < DESC_CACHE; i++) s_sched.desc_id[i] = 0xffffffffu;
     }
     __syncthreads ();
-    const unsigned long long t_begin = wall_clock64 ();
+    const unsigned long long t_begin = wall_clock64 (), c_begin = clock64 ();
     uint32_t id = QUEUE_EMPTY;
     qentry_t rec = 0;
     for (;;)
@@ -328,6 +396,7 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
         if (threadIdx.x < CHILD_REC)
             rec = *(const qentry_t __attribute__ ((address_space (1))) *)(s_sched.a.child_rec + (size_t)id * CHILD_REC + threadIdx.x);
         if ((s_sched.a.flags & ASPEN_HIP_FLAG_TRACE) && threadIdx.x == 0) s_sched.a.trace[2 * (size_t)id] = wall_clock64 ();
+        if ((s_sched.a.flags & ASPEN_HIP_FLAG_PROFILE) && threadIdx.x == 0) s_sched.p0 = wall_clock64 ();
         const aspen_hip_layer_t *L = &s_sched.desc[__builtin_amdgcn_readfirstlane (s_sched.desc_slot)];
         bool complete;
         if (!(s_sched.a.flags & ASPEN_HIP_FLAG_SKIP_TILES))
@@ -346,6 +415,8 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
         atomicAdd (&prof[0], s_sched.ticks[0]); atomicAdd (&prof[1], s_sched.ticks[1]); atomicAdd (&prof[2], s_sched.ticks[2]);
         atomicAdd (&prof[3], wall_clock64 () - t_begin);
         atomicAdd (&prof[4], s_sched.ticks[3]); atomicAdd (&prof[5], s_sched.ticks[4]); atomicAdd (&prof[6], s_sched.ticks[5]);
+        for (int i = 0; i < 4; i++) atomicAdd (&prof[8 + i], s_sched.phase[i]);
+        atomicAdd (&prof[7], (unsigned long long)(clock64 () - c_begin));     // engine clock cycles: [7] / [3] * 100 MHz = the clock the run had
     }
 }
 
@@ -730,6 +801,7 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     if (!g) { snprintf (g_err, sizeof (g_err), "out of host memory"); return nullptr; }
     g->cached_loads = lines_have_one_producer (layers, num_layers) && getenv ("ASPEN_GPU_COHERENT_LOADS") == nullptr;
     g->num_layers = num_layers; g->num_ninst = num_ninst; g->num_roots = num_roots; g->num_edges = num_edges;
+    for (uint32_t t = 0; t < num_ninst; t++) g->num_sinks += child_off[t + 1] == child_off[t];
     {
         // default grid: a whole number of workgroups per compute unit, no more than the graph can keep busy
         const double par = graph_parallelism (layers, ninst_layer, child_off, child_idx, num_ninst);
@@ -770,7 +842,7 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     g->d_ran = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
     g->d_state = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * ST_WORDS);
     g->d_arrivals = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
-    g->d_prof = (unsigned long long *)aspen_hip_alloc (sizeof (unsigned long long) * 8);
+    g->d_prof = (unsigned long long *)aspen_hip_alloc (sizeof (unsigned long long) * 16);
     if (hipHostMalloc ((void **)&g->h_abort, 64, hipHostMallocDefault) != hipSuccess) g->h_abort = nullptr;
     else *g->h_abort = 0;
     if (!g->h_abort || !g->d_layers || !g->d_ninst_layer || !g->d_num_parents || !g->d_child_off || !g->d_child_idx || !g->d_roots
@@ -839,7 +911,7 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
         if (!g->d_trace) return -1;
     }
     a.trace = g->d_trace;
-    a.num_ninst = g->num_ninst; a.epoch = g->epoch; a.flags = g_flags; a.queue_row = queue_row (g->num_ninst); a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
+    a.num_ninst = g->num_ninst; a.num_sinks = g->num_sinks; a.epoch = g->epoch; a.flags = g_flags; a.queue_row = queue_row (g->num_ninst); a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
     CHECK (hipEventRecord (g_events[NUM_EVENTS - 2], g_stream));
     if (g->cached_loads) hipLaunchKernelGGL (dataflow_kernel<2>, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);
     else hipLaunchKernelGGL (dataflow_kernel<1>, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);
@@ -910,12 +982,12 @@ extern "C" int aspen_hip_dataflow_stats (aspen_hip_graph_t *g, uint32_t *execute
     return 0;
 }
 
-extern "C" int aspen_hip_dataflow_profile (aspen_hip_graph_t *g, uint64_t ticks[8], int reset)
+extern "C" int aspen_hip_dataflow_profile (aspen_hip_graph_t *g, uint64_t ticks[16], int reset)
 {
     if (!g || !ticks) return -1;
-    unsigned long long h[8];
+    unsigned long long h[16];
     if (aspen_hip_d2h (h, g->d_prof, sizeof (h))) return -1;
-    for (int i = 0; i < 8; i++) ticks[i] = h[i];
+    for (int i = 0; i < 16; i++) ticks[i] = h[i];
     if (reset) { CHECK (hipMemsetAsync (g->d_prof, 0, sizeof (h), g_stream)); }
     return 0;
 }

@@ -16,6 +16,11 @@
 
 typedef float floatx16 __attribute__ ((ext_vector_type (16)));
 
+// Phase accounting of contraction tiles inside the persistent kernel (defined next to the kernel; costs one
+// LDS read per call when profiling is off): 8 = operand set-up and first loads, 9 = K loop, 10 = epilogue,
+// 11 = split-K arrival and reduction
+__device__ void tile_phase_lap (int which);
+
 #define WG_THREADS 256
 #define GEMM_BK 32            // K floats staged per iteration: one 128-byte line per operand row
 #define LDS_ROW 36            // floats per staged row: 32 + 4 padding -> conflict-free 128-bit reads
@@ -25,20 +30,40 @@ typedef float floatx16 __attribute__ ((ext_vector_type (16)));
 // wavefronts) share a compute unit and one workgroup's load latency, epilogue and scheduling gaps are
 // covered by the other three.  (128 x 128 tiles with two LDS stages and two workgroups per compute
 // unit were measured too: better for very large GEMMs only, worse for every network here.)
+#ifndef VAR0_BM
 #define VAR0_BM 128
 #define VAR0_BN 64
+#endif
+#ifndef WG_PER_CU
 #define WG_PER_CU 4
+#endif
 #define KATTN_BN 64
+#ifndef VAR1_BM
 #define VAR1_BM 64
 #define VAR1_BN 128
+#endif
 #define VAR2_BM 64
 #define VAR2_BN 64
+// K slices in flight from memory per tile shape (see gemm_core); overridable for experiments
+#ifndef VAR0_DEPTH
+#define VAR0_DEPTH 1
+#endif
+#ifndef VAR1_DEPTH
+#define VAR1_DEPTH 1
+#endif
+#ifndef VAR2_DEPTH
+#define VAR2_DEPTH 2
+#endif
 #define CMAX(a, b) ((a) > (b) ? (a) : (b))
 #define STAGE_FLOATS(bm, bn) (((bm) + (bn)) * LDS_ROW)
 #define EPI_FLOATS(bm, bn) ((bn) * ((bm) + 8))
 #define VAR_FLOATS(bm, bn) CMAX (STAGE_FLOATS (bm, bn), EPI_FLOATS (bm, bn))
+#ifdef NO_ATTENTION_TILES
+#define GEMM_SMEM_FLOATS CMAX (CMAX (VAR_FLOATS (VAR0_BM, VAR0_BN), VAR_FLOATS (VAR1_BM, VAR1_BN)), VAR_FLOATS (VAR2_BM, VAR2_BN))
+#else
 #define GEMM_SMEM_FLOATS CMAX (CMAX (VAR_FLOATS (VAR0_BM, VAR0_BN), VAR_FLOATS (VAR1_BM, VAR1_BN)), \
                                CMAX (VAR_FLOATS (VAR2_BM, VAR2_BN), STAGE_FLOATS (128, KATTN_BN)))
+#endif
 #define GEMM_SMEM_BYTES (GEMM_SMEM_FLOATS * 4)
 
 __device__ __forceinline__ float4 ld4 (const float *p) { return *reinterpret_cast<const float4 *> (p); }
@@ -379,10 +404,15 @@ __device__ __forceinline__ void lds_barrier ()
 #define SG_DS_READ 0x100
 #define SG_DS_WRITE 0x200
 
-template <int BM, int BN, int WM, int WN, class ALoader, class BLoader>
+// DEPTH = number of K slices in flight from memory (register sets): 1 = the slice after the staged one
+// waits in registers; 2 = the two slices after it do.  A slice cannot take less than the memory latency
+// divided by DEPTH, and when a compute unit runs fewer workgroups than it could hold (a graph bound by its
+// dependency chains) nothing else hides that latency; the second set costs 4 registers per 32 operand rows.
+template <int BM, int BN, int WM, int WN, int DEPTH, class ALoader, class BLoader>
 __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, int kiters, float *smem,
-    floatx16 (&acc)[BN / WN / 32][BM / WM / 32])
+    floatx16 (&acc)[BN / WN / 32][BM / WM / 32], bool phases = false)
 {
+    static_assert (DEPTH == 1 || DEPTH == 2, "one or two register sets");
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     constexpr int KK = GEMM_BK / 8;
     const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
@@ -401,6 +431,9 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
     float4 af[2][TM], bf[2][TN];
     auto read_frags = [&] (int buf, int sub)
     {
+#ifdef ABL_LDSR
+        if (sub != 0) return;
+#endif
         #pragma unroll
         for (int j = 0; j < TM; j++) af[buf][j] = ld4 (afrag + j * 32 * LDS_ROW + sub * 8);
         #pragma unroll
@@ -427,23 +460,28 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
             }
     };
 
-    float4 areg[ALoader::R], breg[BLoader::R];
-    al.load (kbase, areg); bl.load (kbase, breg);
-    al.store (smem, areg); bl.store (smem + BM * LDS_ROW, breg);
-    if (kiters > 1) { al.load (kbase + 1, areg); bl.load (kbase + 1, breg); }
+    // register set s holds slice it with (it - first) % DEPTH == s
+    float4 areg[DEPTH][ALoader::R], breg[DEPTH][BLoader::R];
+    al.load (kbase, areg[0]); bl.load (kbase, breg[0]);
+    if (DEPTH == 2 && kiters > 1) { al.load (kbase + 1, areg[DEPTH - 1]); bl.load (kbase + 1, breg[DEPTH - 1]); }
+    al.store (smem, areg[0]); bl.store (smem + BM * LDS_ROW, breg[0]);
+    if (kiters > DEPTH) { al.load (kbase + DEPTH, areg[0]); bl.load (kbase + DEPTH, breg[0]); }
     lds_barrier ();
+    if (phases) tile_phase_lap (8);
     read_frags (0, 0);
 
     // One K slice per iteration, single LDS stage, software-pipelined by hand:
     //   sub-steps 0 .. KK-2: the fragments of sub-step s+1 are fetched between the two halves of the
     //   MFMAs of sub-step s, so they have arrived even if the compiler waits for ALL LDS traffic before s+1;
     //   last sub-step: once every wave holds its last fragments (barrier), the next slice (waiting in
-    //   registers) overwrites the stage and the slice after it is requested from memory, all under
-    //   the first half of the sub-step's MFMAs; after the second barrier the first fragments of the new
-    //   slice are fetched under the second half.
+    //   registers) overwrites the stage and the slice DEPTH after it is requested from memory into the
+    //   registers just freed, all under the first half of the sub-step's MFMAs; after the second barrier the
+    //   first fragments of the new slice are fetched under the second half.
     // The scheduling-group hints pin that order; left alone, the compiler fetches each fragment right
     // before its use and the LDS latency shows.
-    for (int it = 0; it + 1 < kiters; it++)
+    // `set` (a literal at every call, so that the register arrays are indexed statically) = the register set
+    // that holds slice it + 1.
+    auto slice = [&] (int it, int set)
     {
         #pragma unroll
         for (int kk = 0; kk + 1 < KK; kk++)
@@ -456,18 +494,42 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
             __builtin_amdgcn_sched_group_barrier (SG_MFMA, 2 * TM * TN, 0);
         }
         __builtin_amdgcn_sched_barrier (0);
+#ifndef ABL_BARRIER
         lds_barrier ();
+#endif
         __builtin_amdgcn_sched_barrier (0);
-        al.store (smem, areg); bl.store (smem + BM * LDS_ROW, breg);
-        if (it + 2 < kiters) { al.load (kbase + it + 2, areg); bl.load (kbase + it + 2, breg); }
+#ifndef ABL_LDSW
+        al.store (smem, areg[set]); bl.store (smem + BM * LDS_ROW, breg[set]);
+#endif
+#ifndef ABL_GLOAD
+        if (DEPTH == 2)
+        {
+            // always issued (the last slices are requested again and never used): a request inside a branch makes
+            // the compiler lose count of what is in flight, and it then waits for everything before every store
+            const int nxt = kbase + min (it + 1 + DEPTH, kiters - 1);
+            al.load (nxt, areg[set]); bl.load (nxt, breg[set]);
+        }
+        else if (it + 1 + DEPTH < kiters) { al.load (kbase + it + 1 + DEPTH, areg[set]); bl.load (kbase + it + 1 + DEPTH, breg[set]); }
+#endif
         mfma_half ((KK - 1) & 1, 0);
         __builtin_amdgcn_sched_barrier (0);
+#ifndef ABL_BARRIER
         lds_barrier ();
+#endif
         __builtin_amdgcn_sched_barrier (0);
         read_frags (0, 0);
         mfma_half ((KK - 1) & 1, 1);
         __builtin_amdgcn_sched_group_barrier (SG_DS_READ, TM + TN, 0);
         __builtin_amdgcn_sched_group_barrier (SG_MFMA, 2 * TM * TN, 0);
+    };
+    if (DEPTH == 1)
+        for (int it = 0; it + 1 < kiters; it++) slice (it, 0);
+    else
+    {
+        // slice it + 1 sits in set (it + 1) % 2: two slices per trip keep the set a literal
+        int it = 0;
+        for (; it + 2 < kiters; it += 2) { slice (it, DEPTH - 1); slice (it + 1, 0); }
+        if (it + 1 < kiters) slice (it, DEPTH - 1);
     }
     // last slice: nothing left to stage
     #pragma unroll
@@ -514,7 +576,7 @@ __device__ __forceinline__ void fused_shortcut (const aspen_hip_layer_t &L, cons
 // K slices [slice*kiters_per_split, ...) only, raw sums to that slice's partial matrix.
 // This part (operand loaders, K loop, accumulators parked in LDS) exists once per tile shape; the
 // epilogue that follows it is shared by all shapes, which keeps the kernel's code small.
-template <int BM, int BN, int WM, int WN, int COH>
+template <int BM, int BN, int WM, int WN, int DEPTH, int COH>
 __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, int slice, float *smem)
 {
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
@@ -535,14 +597,15 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
     {
         ActRowLoader<BN, COH> bl;
         bl.init (in, n0, L.N - 1, L.ld0, 0, tid);
-        gemm_core<BM, BN, WM, WN> (al, bl, kbase, kiters, smem, acc);
+        gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0);
     }
     else
     {
         ConvLoader<BN, COH> bl;
         bl.init (L, in, n0, tid);
-        gemm_core<BM, BN, WM, WN> (al, bl, kbase, kiters, smem, acc);
+        gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0);
     }
+    if (COH) tile_phase_lap (9);
     const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);
     // Epilogue through LDS (free after the last K slice): the raw accumulators are parked as
     // [column][channel] for contraction_epilogue.
@@ -650,29 +713,61 @@ __device__ __forceinline__ void tile_splitk_finish (const aspen_hip_layer_t &L, 
     part.init (L.partial, L.N * L.splits, L.ld); out.init (L.out, L.N, L.ld);
     const bool fuse = L.fuse_out != nullptr, keep = !(fuse && L.fuse_discard);
     if (fuse) { fin.init (L.fuse_in, L.N, L.fuse_ld_in); fout.init (L.fuse_out, L.N, L.ld); }
-    for (uint32_t idx = tile_thread (); idx < rows * C4; idx += WG_THREADS)
+    // Two 16-byte pieces per thread and four slices of each at a time: eight loads in flight, so that their
+    // memory latencies overlap instead of adding up (the partial sums come from other XCDs' tiles and miss this
+    // XCD's L2).  The slices are added in slice order whoever runs this; a slice index past the last one
+    // re-reads the last slice and is not added.
+    constexpr uint32_t PIECES = 2, BATCH = 4;
+    const uint32_t total = rows * C4, pstride = L.N * L.ld, last = L.splits - 1;
+    for (uint32_t i0 = tile_thread (); i0 < total; i0 += PIECES * WG_THREADS)
     {
-        const uint32_t r = idx / C4, c = (idx - r * C4) * 4;
-        if (c >= mrem) continue;
-        float4 v = make_float4 (0.f, 0.f, 0.f, 0.f);
-        for (uint32_t s = 0; s < L.splits; s++)
+        uint32_t o[PIECES], cc[PIECES];
+        bool live[PIECES];
+        float4 v[PIECES];
+        #pragma unroll
+        for (uint32_t u = 0; u < PIECES; u++)
         {
-            const float4 p = part.ld4 ((s * L.N + n0 + r) * L.ld + m0 + c);
-            v.x += p.x; v.y += p.y; v.z += p.z; v.w += p.w;
+            const uint32_t idx = min (i0 + u * WG_THREADS, total - 1), r = idx / C4;
+            cc[u] = (idx - r * C4) * 4;
+            live[u] = i0 + u * WG_THREADS < total && cc[u] < mrem;
+            o[u] = (n0 + r) * L.ld + m0 + (cc[u] < mrem ? cc[u] : 0u);      // channels past the matrix: fetch something that exists
+            v[u] = make_float4 (0.f, 0.f, 0.f, 0.f);
         }
-        if (L.bias)
+        for (uint32_t s0 = 0; s0 < L.splits; s0 += BATCH)
         {
-            v.x += gld1 (L.bias + m0 + c);
-            if (c + 1 < mrem) v.y += gld1 (L.bias + m0 + c + 1);
-            if (c + 2 < mrem) v.z += gld1 (L.bias + m0 + c + 2);
-            if (c + 3 < mrem) v.w += gld1 (L.bias + m0 + c + 3);
+            float4 p[PIECES][BATCH];
+            #pragma unroll
+            for (uint32_t u = 0; u < PIECES; u++)
+                #pragma unroll
+                for (uint32_t j = 0; j < BATCH; j++) p[u][j] = part.ld4 (o[u] + min (s0 + j, last) * pstride);
+            #pragma unroll
+            for (uint32_t u = 0; u < PIECES; u++)
+                #pragma unroll
+                for (uint32_t j = 0; j < BATCH; j++)
+                {
+                    const bool use = s0 + j <= last;
+                    v[u].x += use ? p[u][j].x : 0.f; v[u].y += use ? p[u][j].y : 0.f; v[u].z += use ? p[u][j].z : 0.f; v[u].w += use ? p[u][j].w : 0.f;
+                }
         }
-        v = act4 (v, L.act);
-        const uint32_t o = (n0 + r) * L.ld + m0 + c;
-        if (!keep) { }
-        else if (c + 4 <= mrem) out.st4 (o, v);
-        else { out.st1 (o, v.x); if (c + 1 < mrem) out.st1 (o + 1, v.y); if (c + 2 < mrem) out.st1 (o + 2, v.z); }
-        if (fuse) fused_shortcut<COH> (L, fin, fout, v, n0 + r, m0 + c, mrem - c);
+        #pragma unroll
+        for (uint32_t u = 0; u < PIECES; u++)
+        {
+            if (!live[u]) continue;
+            const uint32_t c = cc[u];
+            float4 y = v[u];
+            if (L.bias)
+            {
+                y.x += gld1 (L.bias + m0 + c);
+                if (c + 1 < mrem) y.y += gld1 (L.bias + m0 + c + 1);
+                if (c + 2 < mrem) y.z += gld1 (L.bias + m0 + c + 2);
+                if (c + 3 < mrem) y.w += gld1 (L.bias + m0 + c + 3);
+            }
+            y = act4 (y, L.act);
+            if (!keep) { }
+            else if (c + 4 <= mrem) out.st4 (o[u], y);
+            else { out.st1 (o[u], y.x); if (c + 1 < mrem) out.st1 (o[u] + 1, y.y); if (c + 2 < mrem) out.st1 (o[u] + 2, y.z); }
+            if (fuse) fused_shortcut<COH> (L, fin, fout, y, (o[u] - m0 - c) / L.ld, m0 + c, mrem - c);
+        }
     }
 }
 
@@ -885,7 +980,7 @@ __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, ui
     {
         ActRowLoader<BM, COH> al; al.init (Kmat, b * S + k0, b * S + S - 1, L.ld1, h * L.hd, tid);
         ActRowLoader<BN, COH> bl; bl.init (Q, b * S + q0, b * S + S - 1, L.ld0, h * L.hd, tid);
-        gemm_core<BM, BN, WM, WN> (al, bl, 0, kiters, smem, acc);
+        gemm_core<BM, BN, WM, WN, 1> (al, bl, 0, kiters, smem, acc);
     };
     // exponential of one score; reference order of operations: mask with -1e10, scale, exp, no max subtraction
     auto weight = [&] (float sc, uint32_t key, uint32_t q) -> float
@@ -987,7 +1082,7 @@ __device__ __forceinline__ void tile_v_attention (const aspen_hip_layer_t &L, ui
     floatx16 acc[TN][TM];
     TransLoader64<COH> al; al.init (V, b * S * L.ld1 + m0, L.ld1, L.tile_m, S, tid);
     ActRowLoader<BN, COH> bl; bl.init (P, prow + q0, prow + S - 1, L.ld0, 0, tid);   // P's stride is a multiple of 32 with zero padding
-    gemm_core<BM, BN, WM, WN> (al, bl, 0, (int)((S + GEMM_BK - 1) / GEMM_BK), smem, acc);
+    gemm_core<BM, BN, WM, WN, 1> (al, bl, 0, (int)((S + GEMM_BK - 1) / GEMM_BK), smem, acc);
     const uint32_t mm = wm0 + (lane & 31);
     if (mm < L.tile_m)
         #pragma unroll
@@ -1072,19 +1167,21 @@ __device__ __forceinline__ bool run_tile (const aspen_hip_layer_t &Lg, uint32_t 
     case CONV_LAYER: case FC_LAYER: case MATMUL_LAYER:
     {
         uint32_t c4_log2, bn;
-        if (L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, COH> (L, tn, tm, slice, smem); c4_log2 = 5; bn = VAR0_BN; }
-        else if (L.variant == ASPEN_HIP_GEMM_WIDE) { contraction_mainloop<VAR1_BM, VAR1_BN, 2, 2, COH> (L, tn, tm, slice, smem); c4_log2 = 4; bn = VAR1_BN; }
-        else { contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, COH> (L, tn, tm, slice, smem); c4_log2 = 4; bn = VAR2_BN; }
-        static_assert (VAR0_BM == 128 && VAR1_BM == 64 && VAR2_BM == 64, "c4_log2 above");
+        if (L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, VAR0_DEPTH, COH> (L, tn, tm, slice, smem); c4_log2 = VAR0_BM == 128 ? 5 : 4; bn = VAR0_BN; }
+        else if (L.variant == ASPEN_HIP_GEMM_WIDE) { contraction_mainloop<VAR1_BM, VAR1_BN, 2, 2, VAR1_DEPTH, COH> (L, tn, tm, slice, smem); c4_log2 = 4; bn = VAR1_BN; }
+        else { contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, VAR2_DEPTH, COH> (L, tn, tm, slice, smem); c4_log2 = 4; bn = VAR2_BN; }
+        
         contraction_epilogue<COH> (L, tn, tm, slice, smem, c4_log2, bn);
+        if (COH) tile_phase_lap (10);
         if (slice >= 0)
         {
             // split-K: every slice has written its partial sums; whoever arrives last adds them up.  Without
             // counters (one launch per layer: stores of a launch are not visible across XCDs before it ends)
             // the sums are added up by a second launch, see finish_tile.
             uint32_t *counters = arrivals ();
-            if (counters == nullptr || !splitk_arrived_last (counters + group, L.splits, smem)) return false;
+            if (counters == nullptr || !splitk_arrived_last (counters + group, L.splits, smem)) { if (COH) tile_phase_lap (11); return false; }
             tile_splitk_finish<COH> (L, tn, tm);
+            if (COH) tile_phase_lap (11);
         }
         break;
     }
@@ -1095,8 +1192,10 @@ __device__ __forceinline__ bool run_tile (const aspen_hip_layer_t &Lg, uint32_t 
     case APPEND_LAYER:      tile_append<COH> (L, tn); break;
     case LAYERNORM_LAYER:   tile_layernorm<COH> (L, tn); break;
     case SOFTMAX_LAYER:     tile_softmax<COH> (L, tn); break;
+#ifndef NO_ATTENTION_TILES
     case K_ATTENTION_LAYER: tile_k_attention<COH> (L, tn, smem); break;
     case V_ATTENTION_LAYER: tile_v_attention<COH> (L, tn, tm, smem); break;
+#endif
     default: break;
     }
     return true;

@@ -70,7 +70,7 @@ int aspen_rpool_profile_layers (rpool_t *rp, unsigned int iters, float *ms)
     return aspen_hip_profile_layers (rp->graph, iters, ms);
 }
 
-int aspen_rpool_dataflow_profile (rpool_t *rp, uint64_t ticks[8], int reset)
+int aspen_rpool_dataflow_profile (rpool_t *rp, uint64_t ticks[16], int reset)
 {
     if (rp == NULL || rp->graph == NULL) return -1;
     return aspen_hip_dataflow_profile (rp->graph, ticks, reset);

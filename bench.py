@@ -132,6 +132,7 @@ def main():
     ap.add_argument("--workgroups", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--skip-tiles", action="store_true", help="scheduler-only run: dependency protocol with empty tiles")
+    ap.add_argument("--no-handoff", action="store_true", help="every ready tile goes through the queue (no parent -> child hand-off)")
     ap.add_argument("--engine-profile", action="store_true", help="report where the persistent workgroups spend their time")
     ap.add_argument("--trace", default="", metavar="NPZ", help="write per-tile start/end stamps of the last timed step (dataflow mode)")
     ap.add_argument("--layer-profile", action="store_true", help="also time every layer's kernel (layer-launch mode)")
@@ -166,7 +167,7 @@ def main():
                           "ms_per_launch": ms.value / args.steps,
                           "GB_per_s": 2 * nbytes * args.steps / (ms.value * 1e-3) / 1e9}))
         return
-    L.aspen_hip_set_flags((1 if args.skip_tiles else 0) | (4 if args.engine_profile else 0) | (8 if args.trace else 0))
+    L.aspen_hip_set_flags((1 if args.skip_tiles else 0) | (4 if args.engine_profile else 0) | (8 if args.trace else 0) | (16 if args.no_handoff else 0))
     cfgs, unit, units_per_step, tuned_min_ninst, tuned_engine = WORKLOADS[args.workload]
     if args.min_ninst <= 0:
         args.min_ninst = tuned_min_ninst
@@ -267,7 +268,8 @@ def main():
 
     if args.engine_profile and args.mode == "dataflow":
         prof = pool.dataflow_profile()
-        out["engine_profile"] = {k: v / max(prof["total"], 1e-12) for k, v in prof.items() if k != "total"}
+        out["engine_profile"] = {k: v / max(prof["total"], 1e-12) for k, v in prof.items() if k not in ("total", "engine_clock_mhz")}
+        out["engine_profile"]["engine_clock_mhz"] = prof["engine_clock_mhz"]
         out["engine_profile"]["workgroup_seconds_per_step"] = prof["total"] / args.steps
     if args.trace and args.mode == "dataflow":
         stamps = pool.dataflow_trace()

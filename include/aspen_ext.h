@@ -65,7 +65,7 @@ int aspen_rpool_run_stats (rpool_t *rpool, uint32_t *executed, uint32_t *double_
    ms must hold one float per layer of every attached nasm, in attachment order */
 int aspen_rpool_profile_layers (rpool_t *rpool, unsigned int iters, float *ms);
 /* where the workgroups of the dataflow kernel spent their time (needs ASPEN_HIP_FLAG_PROFILE) */
-int aspen_rpool_dataflow_profile (rpool_t *rpool, uint64_t ticks[8], int reset);
+int aspen_rpool_dataflow_profile (rpool_t *rpool, uint64_t ticks[16], int reset);
 /* start / end time stamps (100 MHz) of every tile of the pool's last run made with ASPEN_HIP_FLAG_TRACE;
    start_end holds 2 * aspen_rpool_num_ninst values, tiles in pool order (nasms in attachment order) */
 int aspen_rpool_dataflow_trace (rpool_t *rpool, uint64_t *start_end);

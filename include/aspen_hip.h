@@ -154,12 +154,17 @@ int aspen_hip_run_dataflow (aspen_hip_graph_t *graph, uint32_t workgroups, uint6
    the tile's stores to be acknowledged, [2] scheduling step (publish, pop, waiting for a ready tile),
    [3] total workgroup lifetime; detail of [2]: [4] publishing wavefront (countdown of the children,
    pushes), [5] popping wavefront drawing its ticket, [6] popping wavefront waiting for its queue slot
-   to be filled; [7] unused */
-int aspen_hip_dataflow_profile (aspen_hip_graph_t *graph, uint64_t ticks[8], int reset);
+   to be filled; [7] engine-clock cycles of the workgroups' lifetimes ([7] / [3] x 100 MHz = the
+   average engine clock during the run); contraction tiles only: [8] operand set-up up to the first staged
+   slice, [9] K loop, [10] epilogue, [11] split-K arrival and reduction; [12..15] unused */
+int aspen_hip_dataflow_profile (aspen_hip_graph_t *graph, uint64_t ticks[16], int reset);
 /* TRACE makes the dataflow kernel stamp every tile's start and end (100 MHz device clock);
    aspen_hip_dataflow_trace copies the stamps of the last traced run: start_end[2*i], [2*i+1] for tile i
    of the graph's num_ninst tiles. */
 #define ASPEN_HIP_FLAG_TRACE 8u
+/* NO_HANDOFF sends every tile that becomes ready through the queue, instead of letting the workgroup that
+   finished its last parent run it next (for comparisons). */
+#define ASPEN_HIP_FLAG_NO_HANDOFF 16u
 int aspen_hip_dataflow_trace (aspen_hip_graph_t *graph, uint64_t *start_end, uint32_t num_ninst);
 void aspen_hip_set_flags (uint32_t flags);
 /* Waits for everything enqueued on the library's stream.  Reports device errors only; whether a dataflow
