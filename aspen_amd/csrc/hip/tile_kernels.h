@@ -408,9 +408,12 @@ __device__ __forceinline__ void lds_barrier ()
 // waits in registers; 2 = the two slices after it do.  A slice cannot take less than the memory latency
 // divided by DEPTH, and when a compute unit runs fewer workgroups than it could hold (a graph bound by its
 // dependency chains) nothing else hides that latency; the second set costs 4 registers per 32 operand rows.
-template <int BM, int BN, int WM, int WN, int DEPTH, class ALoader, class BLoader>
+struct NoHook { __device__ __forceinline__ void operator() () const {} };
+// `before_last_slice` runs right before the MFMAs of the last K slice: the place to request what the epilogue
+// will need from memory, with the operand registers free and a whole slice of arithmetic to hide the latency.
+template <int BM, int BN, int WM, int WN, int DEPTH, class ALoader, class BLoader, class Hook = NoHook>
 __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, int kiters, float *smem,
-    floatx16 (&acc)[BN / WN / 32][BM / WM / 32], bool phases = false)
+    floatx16 (&acc)[BN / WN / 32][BM / WM / 32], bool phases = false, Hook before_last_slice = Hook ())
 {
     static_assert (DEPTH == 1 || DEPTH == 2, "one or two register sets");
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
@@ -532,6 +535,7 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
         if (it + 1 < kiters) slice (it, DEPTH - 1);
     }
     // last slice: nothing left to stage
+    before_last_slice ();
     #pragma unroll
     for (int kk = 0; kk < KK; kk++)
     {
@@ -576,8 +580,12 @@ __device__ __forceinline__ void fused_shortcut (const aspen_hip_layer_t &L, cons
 // K slices [slice*kiters_per_split, ...) only, raw sums to that slice's partial matrix.
 // This part (operand loaders, K loop, accumulators parked in LDS) exists once per tile shape; the
 // epilogue that follows it is shared by all shapes, which keeps the kernel's code small.
+// what the main loop already requested for the epilogue (threads whose four channels all exist): the bias, and all
+// of the thread's pieces of a fused shortcut's operand (a tile has at most 128 columns: 8 pieces per thread)
+struct shortcut_prefetch_t { float4 s[8]; float4 bias; bool have, have_shortcut; };
+
 template <int BM, int BN, int WM, int WN, int DEPTH, int COH>
-__device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, int slice, float *smem)
+__device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, int slice, float *smem, shortcut_prefetch_t &pre)
 {
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
@@ -593,20 +601,62 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
     }
     RowLoader<BM> al;
     al.init (L.weight, m0, (L.M + 127u) / 128u * 128u, L.Kp, tid);
+    // a fused shortcut's other operand comes from memory another XCD may have written: the first pieces this
+    // thread will need in the epilogue (see contraction_epilogue for the thread -> piece mapping) are
+    // requested under the last K slice
+    auto fetch_shortcut = [&] ()
+    {
+        constexpr uint32_t C4_LOG2 = BM == 128 ? 5 : 4, STEP = WG_THREADS >> C4_LOG2, PIECES = BN / STEP;
+        static_assert (PIECES <= 8, "pieces per thread");
+        const uint32_t c = (tid & ((1u << C4_LOG2) - 1)) * 4, rows = min ((uint32_t)BN, L.N - n0), r0 = tid >> C4_LOG2;
+        pre.have = slice < 0 && c + 4 <= L.M - m0;
+        pre.have_shortcut = pre.have && L.fuse_out != nullptr;
+        if (pre.have) pre.bias = L.bias ? gld4 (L.bias + m0 + c) : make_float4 (0.f, 0.f, 0.f, 0.f);
+        if (pre.have_shortcut)
+        {
+            ActView<COH> fin;
+            fin.init (L.fuse_in, L.N, L.fuse_ld_in);
+            #pragma unroll
+            for (uint32_t u = 0; u < PIECES; u++)
+                if (r0 + u * STEP < rows) pre.s[u] = fin.ld4 ((n0 + r0 + u * STEP) * L.fuse_ld_in + m0 + c);
+        }
+    };
     if (L.direct)
     {
         ActRowLoader<BN, COH> bl;
         bl.init (in, n0, L.N - 1, L.ld0, 0, tid);
-        gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0);
+        gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
     }
     else
     {
         ConvLoader<BN, COH> bl;
         bl.init (L, in, n0, tid);
-        gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0);
+        gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
     }
     if (COH) tile_phase_lap (9);
     const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);
+    if (slice >= 0)
+    {
+        // split-K: the raw sums go straight from the accumulators to this slice's partial matrix.  Register v of
+        // a block holds 32 consecutive channels of one column across a half-wave, so every store instruction
+        // writes two whole 128-byte lines; no bias, no activation, nothing to stage through LDS.
+        ActView<COH> part;
+        part.init (L.partial + (size_t)slice * L.N * L.ld, L.N, L.ld);
+        #pragma unroll
+        for (int j = 0; j < TM; j++)
+        {
+            const uint32_t m = m0 + wm0 + 32 * j + (lane & 31);
+            #pragma unroll
+            for (int i = 0; i < TN; i++)
+                #pragma unroll
+                for (int v = 0; v < 16; v++)
+                {
+                    const uint32_t n = n0 + ACC_N (wn0, i, v, lane);
+                    if (n < L.N && m < L.M) part.st1 (n * L.ld + m, acc[i][j][v]);
+                }
+        }
+        return;
+    }
     // Epilogue through LDS (free after the last K slice): the raw accumulators are parked as
     // [column][channel] for contraction_epilogue.
     constexpr int TROW = BM + 8;            // (4 * TROW) % 64 == 32: the two half-waves hit disjoint banks
@@ -624,28 +674,28 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
 // LDS as [column][BM + 8]: a rolled loop adds the bias, applies the activation and writes 128-bit pieces,
 // so a wavefront covers whole 512-byte (BM = 128) / 256-byte (BM = 64) runs of a column.
 template <int COH>
-__device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, int slice, float *smem,
-    uint32_t c4_log2, uint32_t BN)
+__device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, float *smem,
+    uint32_t c4_log2, uint32_t BN, const shortcut_prefetch_t &pre)
 {
     const uint32_t tid = tile_thread ();
     const uint32_t C4 = 1u << c4_log2, BM = 4u << c4_log2, TROW = BM + 8;
     const uint32_t m0 = tm * BM, n0 = tn * BN;
-    const int act = slice >= 0 ? NO_ACTIVATION : L.act;
+    const int act = L.act;
     ActView<COH> out;
-    if (slice >= 0) out.init (L.partial + (size_t)slice * L.N * L.ld, L.N, L.ld);
-    else out.init (L.out, L.N, L.ld);
+    out.init (L.out, L.N, L.ld);
     const uint32_t rows = min (BN, L.N - n0);
     const uint32_t mrem = L.M - m0;         // channels of this tile that exist (may exceed BM)
     const uint32_t c = (tid & (C4 - 1)) * 4;      // WG_THREADS is a multiple of C4: a thread keeps its channels
     if (c < mrem)
     {
         float4 b = make_float4 (0.f, 0.f, 0.f, 0.f);
-        if (L.bias && slice < 0)
+        if (pre.have) b = pre.bias;
+        else if (L.bias)
         {
             if (c + 4 <= mrem) b = gld4 (L.bias + m0 + c);
             else { b.x = gld1 (L.bias + m0 + c); if (c + 1 < mrem) b.y = gld1 (L.bias + m0 + c + 1); if (c + 2 < mrem) b.z = gld1 (L.bias + m0 + c + 2); }
         }
-        const bool fuse = L.fuse_out != nullptr && slice < 0;
+        const bool fuse = L.fuse_out != nullptr;
         const bool keep = !(fuse && L.fuse_discard);        // the pre-shortcut sums are stored unless the host has no use for them
         ActView<COH> fin, fout;
         if (fuse) { fin.init (L.fuse_in, L.N, L.fuse_ld_in); fout.init (L.fuse_out, L.N, L.ld); }
@@ -656,8 +706,12 @@ __device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L
             // whole float4 of channels: rows are handled U at a time, all LDS reads and shortcut loads of a
             // group issued before its first store.  Loads and stores share one in-order counter, so a
             // shortcut load issued after a (write-through) store waits for that store's acknowledgement.
-            for (uint32_t r0 = tid >> c4_log2; r0 < rows; r0 += U * STEP)
+            // The shortcut pieces were requested under the last K slice (pre); group g's are pre.s[4 g ..].
+            #pragma unroll
+            for (uint32_t g = 0; g < 2; g++)
             {
+                const uint32_t r0 = (tid >> c4_log2) + g * U * STEP;
+                if (r0 >= rows) break;
                 float4 v[U], s[U];
                 #pragma unroll
                 for (uint32_t u = 0; u < U; u++)
@@ -666,7 +720,7 @@ __device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L
                     if (r < rows)
                     {
                         v[u] = ld4 (smem + r * TROW + c);
-                        if (fuse) s[u] = fin.ld4 ((n0 + r) * L.fuse_ld_in + m0 + c);
+                        if (fuse) s[u] = pre.have_shortcut ? pre.s[g * U + u] : fin.ld4 ((n0 + r) * L.fuse_ld_in + m0 + c);
                     }
                 }
                 #pragma unroll
@@ -1167,11 +1221,13 @@ __device__ __forceinline__ bool run_tile (const aspen_hip_layer_t &Lg, uint32_t 
     case CONV_LAYER: case FC_LAYER: case MATMUL_LAYER:
     {
         uint32_t c4_log2, bn;
-        if (L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, VAR0_DEPTH, COH> (L, tn, tm, slice, smem); c4_log2 = VAR0_BM == 128 ? 5 : 4; bn = VAR0_BN; }
-        else if (L.variant == ASPEN_HIP_GEMM_WIDE) { contraction_mainloop<VAR1_BM, VAR1_BN, 2, 2, VAR1_DEPTH, COH> (L, tn, tm, slice, smem); c4_log2 = 4; bn = VAR1_BN; }
-        else { contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, VAR2_DEPTH, COH> (L, tn, tm, slice, smem); c4_log2 = 4; bn = VAR2_BN; }
+        shortcut_prefetch_t pre;
+        pre.have = pre.have_shortcut = false;
+        if (L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, VAR0_DEPTH, COH> (L, tn, tm, slice, smem, pre); c4_log2 = VAR0_BM == 128 ? 5 : 4; bn = VAR0_BN; }
+        else if (L.variant == ASPEN_HIP_GEMM_WIDE) { contraction_mainloop<VAR1_BM, VAR1_BN, 2, 2, VAR1_DEPTH, COH> (L, tn, tm, slice, smem, pre); c4_log2 = 4; bn = VAR1_BN; }
+        else { contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, VAR2_DEPTH, COH> (L, tn, tm, slice, smem, pre); c4_log2 = 4; bn = VAR2_BN; }
         
-        contraction_epilogue<COH> (L, tn, tm, slice, smem, c4_log2, bn);
+        if (slice < 0) contraction_epilogue<COH> (L, tn, tm, smem, c4_log2, bn, pre);
         if (COH) tile_phase_lap (10);
         if (slice >= 0)
         {
