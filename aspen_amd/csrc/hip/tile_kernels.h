@@ -30,40 +30,26 @@ __device__ void tile_phase_lap (int which);
 // wavefronts) share a compute unit and one workgroup's load latency, epilogue and scheduling gaps are
 // covered by the other three.  (128 x 128 tiles with two LDS stages and two workgroups per compute
 // unit were measured too: better for very large GEMMs only, worse for every network here.)
-#ifndef VAR0_BM
 #define VAR0_BM 128
 #define VAR0_BN 64
-#endif
-#ifndef WG_PER_CU
 #define WG_PER_CU 4
-#endif
 #define KATTN_BN 64
-#ifndef VAR1_BM
 #define VAR1_BM 64
 #define VAR1_BN 128
-#endif
 #define VAR2_BM 64
 #define VAR2_BN 64
-// K slices in flight from memory per tile shape (see gemm_core); overridable for experiments
-#ifndef VAR0_DEPTH
+// K slices in flight from memory per tile shape (see gemm_core).  Two for the small shape, whose tiles are the
+// short ones of layers cut along K; with two the larger shapes run out of registers (measured: ResNet-50 batch 32
+// 2.81 -> 2.89 ms, VGG-16 7.90 -> 8.83 ms).
 #define VAR0_DEPTH 1
-#endif
-#ifndef VAR1_DEPTH
 #define VAR1_DEPTH 1
-#endif
-#ifndef VAR2_DEPTH
 #define VAR2_DEPTH 2
-#endif
 #define CMAX(a, b) ((a) > (b) ? (a) : (b))
 #define STAGE_FLOATS(bm, bn) (((bm) + (bn)) * LDS_ROW)
 #define EPI_FLOATS(bm, bn) ((bn) * ((bm) + 8))
 #define VAR_FLOATS(bm, bn) CMAX (STAGE_FLOATS (bm, bn), EPI_FLOATS (bm, bn))
-#ifdef NO_ATTENTION_TILES
-#define GEMM_SMEM_FLOATS CMAX (CMAX (VAR_FLOATS (VAR0_BM, VAR0_BN), VAR_FLOATS (VAR1_BM, VAR1_BN)), VAR_FLOATS (VAR2_BM, VAR2_BN))
-#else
 #define GEMM_SMEM_FLOATS CMAX (CMAX (VAR_FLOATS (VAR0_BM, VAR0_BN), VAR_FLOATS (VAR1_BM, VAR1_BN)), \
                                CMAX (VAR_FLOATS (VAR2_BM, VAR2_BN), STAGE_FLOATS (128, KATTN_BN)))
-#endif
 #define GEMM_SMEM_BYTES (GEMM_SMEM_FLOATS * 4)
 
 __device__ __forceinline__ float4 ld4 (const float *p) { return *reinterpret_cast<const float4 *> (p); }
@@ -434,9 +420,6 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
     float4 af[2][TM], bf[2][TN];
     auto read_frags = [&] (int buf, int sub)
     {
-#ifdef ABL_LDSR
-        if (sub != 0) return;
-#endif
         #pragma unroll
         for (int j = 0; j < TM; j++) af[buf][j] = ld4 (afrag + j * 32 * LDS_ROW + sub * 8);
         #pragma unroll
@@ -497,14 +480,9 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
             __builtin_amdgcn_sched_group_barrier (SG_MFMA, 2 * TM * TN, 0);
         }
         __builtin_amdgcn_sched_barrier (0);
-#ifndef ABL_BARRIER
         lds_barrier ();
-#endif
         __builtin_amdgcn_sched_barrier (0);
-#ifndef ABL_LDSW
         al.store (smem, areg[set]); bl.store (smem + BM * LDS_ROW, breg[set]);
-#endif
-#ifndef ABL_GLOAD
         if (DEPTH == 2)
         {
             // always issued (the last slices are requested again and never used): a request inside a branch makes
@@ -513,12 +491,9 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
             al.load (nxt, areg[set]); bl.load (nxt, breg[set]);
         }
         else if (it + 1 + DEPTH < kiters) { al.load (kbase + it + 1 + DEPTH, areg[set]); bl.load (kbase + it + 1 + DEPTH, breg[set]); }
-#endif
         mfma_half ((KK - 1) & 1, 0);
         __builtin_amdgcn_sched_barrier (0);
-#ifndef ABL_BARRIER
         lds_barrier ();
-#endif
         __builtin_amdgcn_sched_barrier (0);
         read_frags (0, 0);
         mfma_half ((KK - 1) & 1, 1);
@@ -844,77 +819,130 @@ __device__ __forceinline__ void tile_residual (const aspen_hip_layer_t &L, uint3
     }
 }
 
+// One thread = four channels of TWO neighbouring output positions.  Where both lie in the same output row their
+// windows overlap by KW - stride input columns (a 3x3 / stride-2 pool fetches every input 2.25 times when each
+// output loads its own window): the union of the two windows is fetched once, 15 instead of 18 loads for 3x3 / 2.
 template <bool IS_MAX, int COH>
 __device__ __forceinline__ void tile_pool (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm)
 {
     // rows [r0, r1) of the tile; the last row tile also covers the padding rows up to the stride
     const uint32_t r0 = tm * L.tile_m, r1 = tm + 1 == L.tiles_m ? L.ld : r0 + L.tile_m;
     const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N), M4 = (r1 - r0) >> 2;
-    const uint32_t total = (n1 - n0) * M4, ohw = L.OH * L.OW;
+    // pairing pays only where neighbouring windows overlap; elsewhere a thread keeps to one position
+    const uint32_t per_thread = (L.KW > L.stride && L.OW > 1) ? 2u : 1u;
+    const uint32_t pairs = (n1 - n0 + per_thread - 1) / per_thread, total = pairs * M4, ohw = L.OH * L.OW;
     const float inv = 1.0f / (float)(L.KH * L.KW);
     ActView<COH> in, out;
     in.init (L.in0, (L.N / ohw) * L.IH * L.IW, L.ld0); out.init (L.out, L.N, L.ld);
-    for (uint32_t i = tile_thread (); i < total; i += WG_THREADS)
+    const float4 start = IS_MAX ? make_float4 (-INFINITY, -INFINITY, -INFINITY, -INFINITY) : make_float4 (0.f, 0.f, 0.f, 0.f);
+    auto combine = [] (float4 &r, const float4 &x)
     {
-        const uint32_t c = i / M4, m = r0 + (i - c * M4) * 4, n = n0 + c;
-        const uint32_t b = n / ohw, rem = n - b * ohw, oh = rem / L.OW, ow = rem - oh * L.OW;
-        float4 r = IS_MAX ? make_float4 (-INFINITY, -INFINITY, -INFINITY, -INFINITY) : make_float4 (0.f, 0.f, 0.f, 0.f);
-        for (uint32_t kh = 0; kh < L.KH; kh++)
-        {
-            const int ih = (int)(oh * L.stride + kh) - (int)L.pad;
-            if ((uint32_t)ih >= L.IH) continue;
-            for (uint32_t kw = 0; kw < L.KW; kw++)
-            {
-                const int iw = (int)(ow * L.stride + kw) - (int)L.pad;
-                if ((uint32_t)iw >= L.IW) continue;
-                const float4 x = in.ld4 (((b * L.IH + ih) * L.IW + iw) * L.ld0 + m);
-                if (IS_MAX) { r.x = r.x >= x.x ? r.x : x.x; r.y = r.y >= x.y ? r.y : x.y; r.z = r.z >= x.z ? r.z : x.z; r.w = r.w >= x.w ? r.w : x.w; }
-                else { r.x += x.x; r.y += x.y; r.z += x.z; r.w += x.w; }
-            }
-        }
+        if (IS_MAX) { r.x = r.x >= x.x ? r.x : x.x; r.y = r.y >= x.y ? r.y : x.y; r.z = r.z >= x.z ? r.z : x.z; r.w = r.w >= x.w ? r.w : x.w; }
+        else { r.x += x.x; r.y += x.y; r.z += x.z; r.w += x.w; }
+    };
+    auto finish = [&] (float4 r, uint32_t n, uint32_t m)
+    {
         if (!IS_MAX) { r.x *= inv; r.y *= inv; r.z *= inv; r.w *= inv; }
         r = act4 (r, L.act);
         // keep the zero padding rows [M, ld) intact
         if (m + 4 > L.M) { if (m + 0 >= L.M) r.x = 0.f; if (m + 1 >= L.M) r.y = 0.f; if (m + 2 >= L.M) r.z = 0.f; if (m + 3 >= L.M) r.w = 0.f; }
         out.st4 (n * L.ld + m, r);
+    };
+    for (uint32_t i = tile_thread (); i < total; i += WG_THREADS)
+    {
+        const uint32_t c = i / M4, m = r0 + (i - c * M4) * 4, n = n0 + per_thread * c;
+        const uint32_t b = n / ohw, rem = n - b * ohw, oh = rem / L.OW, ow = rem - oh * L.OW;
+        const bool second = per_thread == 2 && n + 1 < n1, same_row = second && ow + 1 < L.OW;
+        // windows of the two positions as one span of input columns when they share a row, else one window each
+        const uint32_t span = same_row ? L.KW + L.stride : L.KW;
+        for (uint32_t which = 0; which < (second && !same_row ? 2u : 1u); which++)
+        {
+            const uint32_t nn = n + which;
+            uint32_t bb = b, hh = oh, ww = ow;
+            if (which) { ww = ow + 1; if (ww == L.OW) { ww = 0; if (++hh == L.OH) { hh = 0; ++bb; } } }
+            float4 ra = start, rb = start;
+            for (uint32_t kh = 0; kh < L.KH; kh++)
+            {
+                const int ih = (int)(hh * L.stride + kh) - (int)L.pad;
+                if ((uint32_t)ih >= L.IH) continue;
+                for (uint32_t kw = 0; kw < span; kw++)
+                {
+                    const int iw = (int)(ww * L.stride + kw) - (int)L.pad;
+                    if ((uint32_t)iw >= L.IW) continue;
+                    const float4 x = in.ld4 (((bb * L.IH + ih) * L.IW + iw) * L.ld0 + m);
+                    if (kw < L.KW) combine (ra, x);
+                    if (same_row && kw >= L.stride) combine (rb, x);
+                }
+            }
+            finish (ra, nn, m);
+            if (same_row) finish (rb, nn + 1, m);
+        }
     }
 }
 
 // YOLO box decode (reference tiled_yolo, src/tiled_kernels.c:675-708).  Output column = (batch, anchor,
 // cell); rows = classes + 5 read from channels [anchor * M, anchor * M + M) of input column (batch, cell).
 // L.weight holds the three anchor boxes (w0, h0, w1, h1, w2, h2).
+// One thread per four consecutive rows of a column: the output piece is one aligned 16-byte store; the four
+// inputs start at channel anchor * M, which is not 16-byte aligned in general, and are fetched as four
+// dwords (neighbouring lanes read neighbouring dwords, so the wave still covers whole cache lines).
 template <int COH>
 __device__ __forceinline__ void tile_yolo (const aspen_hip_layer_t &L, uint32_t tn)
 {
     const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N);
-    const uint32_t cells = L.IH * L.IW, A = L.IC / L.M, total = (n1 - n0) * L.M;
+    const uint32_t cells = L.IH * L.IW, A = L.IC / L.M, pieces = (L.M + 3) >> 2, total = (n1 - n0) * pieces;
+    const float stride = (float)L.stride;
     ActView<COH> in, out;
     in.init (L.in0, (L.N / (cells * A)) * cells, L.ld0); out.init (L.out, L.N, L.ld);
     for (uint32_t i = tile_thread (); i < total; i += WG_THREADS)
     {
-        const uint32_t c = i / L.M, j = i - c * L.M, n = n0 + c;
+        const uint32_t c = i / pieces, j = (i - c * pieces) * 4, n = n0 + c;
         const uint32_t seg = n / cells, b = seg / A, a = seg - b * A, cell = n - seg * cells;
-        const uint32_t h = cell / L.IW, w = cell - h * L.IW;
-        const float x = in.ld1 ((b * cells + cell) * L.ld0 + a * L.M + j);
-        float r;
-        if (j == 0) r = (1.0f / (1.0f + expf (-x)) + (float)w) * (float)L.stride;
-        else if (j == 1) r = (1.0f / (1.0f + expf (-x)) + (float)h) * (float)L.stride;
-        else if (j == 2) r = expf (x) * gld1 (L.weight + 2 * a);
-        else if (j == 3) r = expf (x) * gld1 (L.weight + 2 * a + 1);
-        else r = 1.0f / (1.0f + expf (-x));
-        out.st1 (n * L.ld + j, r);
+        const uint32_t src = (b * cells + cell) * L.ld0 + a * L.M + j, left = L.M - j;
+        float x[4], r[4];
+        #pragma unroll
+        for (uint32_t k = 0; k < 4; k++) x[k] = k < left ? in.ld1 (src + k) : 0.f;
+        #pragma unroll
+        for (uint32_t k = 0; k < 4; k++) r[k] = 1.0f / (1.0f + expf (-x[k]));
+        if (j == 0)
+        {
+            const uint32_t h = cell / L.IW, w = cell - h * L.IW;
+            r[0] = (r[0] + (float)w) * stride;
+            r[1] = (r[1] + (float)h) * stride;
+            r[2] = expf (x[2]) * gld1 (L.weight + 2 * a);
+            r[3] = expf (x[3]) * gld1 (L.weight + 2 * a + 1);
+        }
+        const uint32_t dst = n * L.ld + j;
+        if (left >= 4) out.st4 (dst, make_float4 (r[0], r[1], r[2], r[3]));
+        else { out.st1 (dst, r[0]); if (left > 1) out.st1 (dst + 1, r[1]); if (left > 2) out.st1 (dst + 2, r[2]); }
     }
 }
 
 // Nearest-neighbour upsampling of the first parent by `stride`, concatenated along the channels with
 // the second parent (reference tiled_append, src/tiled_kernels.c:710-741).  IC = channels of the first parent.
+// Both parts of an output column are contiguous copies: 16 bytes per thread when the channel counts are
+// multiples of four (then every piece is aligned and lies within one part), one float per thread otherwise.
 template <int COH>
 __device__ __forceinline__ void tile_append (const aspen_hip_layer_t &L, uint32_t tn)
 {
-    const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N), total = (n1 - n0) * L.M;
+    const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N);
     const uint32_t ohw = L.OH * L.OW, iw = L.OW / L.stride, ih = L.OH / L.stride;
     ActView<COH> p0, p1, out;
     p0.init (L.in0, (L.N / ohw) * ih * iw, L.ld0); p1.init (L.in1, L.N, L.ld1); out.init (L.out, L.N, L.ld);
+    if (((L.IC | L.M) & 3u) == 0)
+    {
+        const uint32_t M4 = L.M >> 2, total = (n1 - n0) * M4;
+        for (uint32_t i = tile_thread (); i < total; i += WG_THREADS)
+        {
+            const uint32_t c = i / M4, m = (i - c * M4) * 4, n = n0 + c;
+            const uint32_t b = n / ohw, rem = n - b * ohw, oh = rem / L.OW, ow = rem - oh * L.OW;
+            const float4 v = m < L.IC ? p0.ld4 (((b * ih + oh / L.stride) * iw + ow / L.stride) * L.ld0 + m)
+                                      : p1.ld4 (n * L.ld1 + (m - L.IC));
+            out.st4 (n * L.ld + m, v);
+        }
+        return;
+    }
+    const uint32_t total = (n1 - n0) * L.M;
     for (uint32_t i = tile_thread (); i < total; i += WG_THREADS)
     {
         const uint32_t c = i / L.M, m = i - c * L.M, n = n0 + c;
@@ -938,9 +966,79 @@ __device__ __forceinline__ float wave_max (float v)
     return v;
 }
 
-// one wavefront per column: mean and E[x^2] in one pass, eps 1e-6f
+// One wavefront per column, the column kept in registers between the two passes (16 bytes x COLUMN_CACHE per
+// lane: columns of up to 64 * 4 * COLUMN_CACHE floats are read once; longer ones are read again).
+#define COLUMN_CACHE 4
+
+// mean and E[x^2] in one pass, eps 1e-6f (reference tiled_layernorm, src/tiled_kernels.c:743-783)
 template <int COH>
 __device__ __forceinline__ void tile_layernorm (const aspen_hip_layer_t &L, uint32_t tn)
+{
+    const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N);
+    const uint32_t lane = tile_thread () & 63, wave = tile_thread () >> 6, M4 = L.M >> 2;
+    ActView<COH> in, out;
+    in.init (L.in0, L.N, L.ld0); out.init (L.out, L.N, L.ld);
+    // this lane's scale and shift are the same for every column
+    float4 g[COLUMN_CACHE], b[COLUMN_CACHE];
+    #pragma unroll
+    for (uint32_t k = 0; k < COLUMN_CACHE; k++)
+    {
+        const uint32_t m = lane + 64 * k;
+        g[k] = m < M4 ? gld4 (L.weight + m * 4) : make_float4 (0.f, 0.f, 0.f, 0.f);
+        b[k] = (m < M4 && L.bias) ? gld4 (L.bias + m * 4) : make_float4 (0.f, 0.f, 0.f, 0.f);
+    }
+    for (uint32_t n = n0 + wave; n < n1; n += WG_THREADS / 64)
+    {
+        const uint32_t x = n * L.ld0, o = n * L.ld;
+        float4 v[COLUMN_CACHE];
+        #pragma unroll
+        for (uint32_t k = 0; k < COLUMN_CACHE; k++)
+            v[k] = lane + 64 * k < M4 ? in.ld4 (x + (lane + 64 * k) * 4) : make_float4 (0.f, 0.f, 0.f, 0.f);
+        float s = 0.f, q = 0.f;
+        #pragma unroll
+        for (uint32_t k = 0; k < COLUMN_CACHE; k++)
+        {
+            s += v[k].x + v[k].y + v[k].z + v[k].w;
+            q += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
+        }
+        for (uint32_t m = lane + 64 * COLUMN_CACHE; m < M4; m += 64)
+        {
+            const float4 w = in.ld4 (x + m * 4);
+            s += w.x + w.y + w.z + w.w;
+            q += w.x * w.x + w.y * w.y + w.z * w.z + w.w * w.w;
+        }
+        for (uint32_t m = M4 * 4 + lane; m < L.M; m += 64) { const float w = in.ld1 (x + m); s += w; q += w * w; }
+        s = wave_sum (s); q = wave_sum (q);
+        const float mean = s / (float)L.M;
+        float var = q / (float)L.M - mean * mean;
+        const float rstd = 1.0f / sqrtf (var + 1e-6f);
+        #pragma unroll
+        for (uint32_t k = 0; k < COLUMN_CACHE; k++)
+            if (lane + 64 * k < M4)
+            {
+                float4 r;
+                r.x = (v[k].x - mean) * rstd * g[k].x; r.y = (v[k].y - mean) * rstd * g[k].y;
+                r.z = (v[k].z - mean) * rstd * g[k].z; r.w = (v[k].w - mean) * rstd * g[k].w;
+                if (L.bias) { r.x += b[k].x; r.y += b[k].y; r.z += b[k].z; r.w += b[k].w; }
+                out.st4 (o + (lane + 64 * k) * 4, r);
+            }
+        for (uint32_t m = lane + 64 * COLUMN_CACHE; m < M4; m += 64)
+        {
+            const float4 w = in.ld4 (x + m * 4), gg = gld4 (L.weight + m * 4);
+            float4 r;
+            r.x = (w.x - mean) * rstd * gg.x; r.y = (w.y - mean) * rstd * gg.y;
+            r.z = (w.z - mean) * rstd * gg.z; r.w = (w.w - mean) * rstd * gg.w;
+            if (L.bias) { const float4 bb = gld4 (L.bias + m * 4); r.x += bb.x; r.y += bb.y; r.z += bb.z; r.w += bb.w; }
+            out.st4 (o + m * 4, r);
+        }
+        for (uint32_t m = M4 * 4 + lane; m < L.M; m += 64)
+            out.st1 (o + m, (in.ld1 (x + m) - mean) * rstd * gld1 (L.weight + m) + (L.bias ? gld1 (L.bias + m) : 0.f));
+    }
+}
+
+// max-subtracted softmax over the rows of a column (reference tiled_softmax, src/tiled_kernels.c:640-673)
+template <int COH>
+__device__ __forceinline__ void tile_softmax (const aspen_hip_layer_t &L, uint32_t tn)
 {
     const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N);
     const uint32_t lane = tile_thread () & 63, wave = tile_thread () >> 6, M4 = L.M >> 2;
@@ -949,50 +1047,34 @@ __device__ __forceinline__ void tile_layernorm (const aspen_hip_layer_t &L, uint
     for (uint32_t n = n0 + wave; n < n1; n += WG_THREADS / 64)
     {
         const uint32_t x = n * L.ld0, o = n * L.ld;
-        float s = 0.f, q = 0.f;
-        for (uint32_t m = lane; m < M4; m += 64)
-        {
-            const float4 v = in.ld4 (x + m * 4);
-            s += v.x + v.y + v.z + v.w;
-            q += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-        }
-        for (uint32_t m = M4 * 4 + lane; m < L.M; m += 64) { const float v = in.ld1 (x + m); s += v; q += v * v; }
-        s = wave_sum (s); q = wave_sum (q);
-        const float mean = s / (float)L.M;
-        float var = q / (float)L.M - mean * mean;
-        const float rstd = 1.0f / sqrtf (var + 1e-6f);
-        for (uint32_t m = lane; m < M4; m += 64)
-        {
-            const float4 v = in.ld4 (x + m * 4), g = gld4 (L.weight + m * 4);
-            float4 r;
-            r.x = (v.x - mean) * rstd * g.x; r.y = (v.y - mean) * rstd * g.y;
-            r.z = (v.z - mean) * rstd * g.z; r.w = (v.w - mean) * rstd * g.w;
-            if (L.bias) { const float4 b = gld4 (L.bias + m * 4); r.x += b.x; r.y += b.y; r.z += b.z; r.w += b.w; }
-            out.st4 (o + m * 4, r);
-        }
-        for (uint32_t m = M4 * 4 + lane; m < L.M; m += 64)
-            out.st1 (o + m, (in.ld1 (x + m) - mean) * rstd * gld1 (L.weight + m) + (L.bias ? gld1 (L.bias + m) : 0.f));
-    }
-}
-
-// one wavefront per column: max-subtracted softmax over the rows
-template <int COH>
-__device__ __forceinline__ void tile_softmax (const aspen_hip_layer_t &L, uint32_t tn)
-{
-    const uint32_t n0 = tn * L.tile_n, n1 = min (n0 + L.tile_n, L.N);
-    const uint32_t lane = tile_thread () & 63, wave = tile_thread () >> 6;
-    ActView<COH> in, out;
-    in.init (L.in0, L.N, L.ld0); out.init (L.out, L.N, L.ld);
-    for (uint32_t n = n0 + wave; n < n1; n += WG_THREADS / 64)
-    {
-        const uint32_t x = n * L.ld0, o = n * L.ld;
+        const float4 low = make_float4 (-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+        float4 v[COLUMN_CACHE];
+        #pragma unroll
+        for (uint32_t k = 0; k < COLUMN_CACHE; k++) v[k] = lane + 64 * k < M4 ? in.ld4 (x + (lane + 64 * k) * 4) : low;
         float mx = -INFINITY;
-        for (uint32_t m = lane; m < L.M; m += 64) mx = fmaxf (mx, in.ld1 (x + m));
+        #pragma unroll
+        for (uint32_t k = 0; k < COLUMN_CACHE; k++) mx = fmaxf (mx, fmaxf (fmaxf (v[k].x, v[k].y), fmaxf (v[k].z, v[k].w)));
+        for (uint32_t m = (lane + 64 * COLUMN_CACHE) * 4; m < M4 * 4; m += 256) { const float4 w = in.ld4 (x + m); mx = fmaxf (mx, fmaxf (fmaxf (w.x, w.y), fmaxf (w.z, w.w))); }
+        for (uint32_t m = M4 * 4 + lane; m < L.M; m += 64) mx = fmaxf (mx, in.ld1 (x + m));
         mx = wave_max (mx);
+        // the exponentials of the cached part are computed once; exp (-inf) = 0 for the lanes past the column
         float s = 0.f;
-        for (uint32_t m = lane; m < L.M; m += 64) s += expf (in.ld1 (x + m) - mx);
+        #pragma unroll
+        for (uint32_t k = 0; k < COLUMN_CACHE; k++)
+        {
+            v[k] = make_float4 (expf (v[k].x - mx), expf (v[k].y - mx), expf (v[k].z - mx), expf (v[k].w - mx));
+            s += v[k].x + v[k].y + v[k].z + v[k].w;
+        }
+        for (uint32_t m = (lane + 64 * COLUMN_CACHE) * 4; m < M4 * 4; m += 256)
+        { const float4 w = in.ld4 (x + m); s += expf (w.x - mx) + expf (w.y - mx) + expf (w.z - mx) + expf (w.w - mx); }
+        for (uint32_t m = M4 * 4 + lane; m < L.M; m += 64) s += expf (in.ld1 (x + m) - mx);
         s = wave_sum (s);
-        for (uint32_t m = lane; m < L.M; m += 64) out.st1 (o + m, expf (in.ld1 (x + m) - mx) / s);
+        #pragma unroll
+        for (uint32_t k = 0; k < COLUMN_CACHE; k++)
+            if (lane + 64 * k < M4) out.st4 (o + (lane + 64 * k) * 4, make_float4 (v[k].x / s, v[k].y / s, v[k].z / s, v[k].w / s));
+        for (uint32_t m = (lane + 64 * COLUMN_CACHE) * 4; m < M4 * 4; m += 256)
+        { const float4 w = in.ld4 (x + m); out.st4 (o + m, make_float4 (expf (w.x - mx) / s, expf (w.y - mx) / s, expf (w.z - mx) / s, expf (w.w - mx) / s)); }
+        for (uint32_t m = M4 * 4 + lane; m < L.M; m += 64) out.st1 (o + m, expf (in.ld1 (x + m) - mx) / s);
     }
 }
 
@@ -1223,7 +1305,7 @@ __device__ __forceinline__ bool run_tile (const aspen_hip_layer_t &Lg, uint32_t 
         uint32_t c4_log2, bn;
         shortcut_prefetch_t pre;
         pre.have = pre.have_shortcut = false;
-        if (L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, VAR0_DEPTH, COH> (L, tn, tm, slice, smem, pre); c4_log2 = VAR0_BM == 128 ? 5 : 4; bn = VAR0_BN; }
+        if (L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, VAR0_DEPTH, COH> (L, tn, tm, slice, smem, pre); c4_log2 = 5; bn = VAR0_BN; }
         else if (L.variant == ASPEN_HIP_GEMM_WIDE) { contraction_mainloop<VAR1_BM, VAR1_BN, 2, 2, VAR1_DEPTH, COH> (L, tn, tm, slice, smem, pre); c4_log2 = 4; bn = VAR1_BN; }
         else { contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, VAR2_DEPTH, COH> (L, tn, tm, slice, smem, pre); c4_log2 = 4; bn = VAR2_BN; }
         
@@ -1248,10 +1330,8 @@ __device__ __forceinline__ bool run_tile (const aspen_hip_layer_t &Lg, uint32_t 
     case APPEND_LAYER:      tile_append<COH> (L, tn); break;
     case LAYERNORM_LAYER:   tile_layernorm<COH> (L, tn); break;
     case SOFTMAX_LAYER:     tile_softmax<COH> (L, tn); break;
-#ifndef NO_ATTENTION_TILES
     case K_ATTENTION_LAYER: tile_k_attention<COH> (L, tn, smem); break;
     case V_ATTENTION_LAYER: tile_v_attention<COH> (L, tn, tm, smem); break;
-#endif
     default: break;
     }
     return true;
