@@ -265,7 +265,7 @@ class RPool:
         if lib().aspen_rpool_dataflow_profile(self.h, t, 1 if reset else 0):
             raise RuntimeError("no dataflow profile")
         d = {k: t[i] * 1e-8 for i, k in enumerate(["tile", "drain", "sched", "total", "publish", "ticket", "slot_wait"])}
-        for i, k in enumerate(["gemm_setup", "gemm_kloop", "gemm_epilogue", "gemm_splitk"]):
+        for i, k in enumerate(["gemm_first_loads", "gemm_kloop", "gemm_epilogue", "gemm_splitk", "gemm_init"]):
             d[k] = t[8 + i] * 1e-8
         d["engine_clock_mhz"] = t[7] / max(t[3], 1) * 100.0
         return d

@@ -198,7 +198,7 @@ struct sched_lds_t
     uint32_t desc_slot, desc_next, desc_id[DESC_CACHE];
     aspen_hip_layer_t desc[DESC_CACHE];
     unsigned long long t0, ticks[6];     // profiling: last time stamp; tile / drain / scheduling / publish / ticket / slot-wait ticks
-    unsigned long long p0, phase[4];     // profiling of contraction tiles: last phase stamp; set-up / K loop / epilogue / split-K ticks
+    unsigned long long p0, phase[5];     // profiling of contraction tiles: last phase stamp; set-up / K loop / epilogue / split-K ticks
 };
 __shared__ sched_lds_t s_sched;
 
@@ -378,7 +378,7 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
         s_sched.a = args;
         s_sched.t0 = wall_clock64 ();
         for (int i = 0; i < 6; i++) s_sched.ticks[i] = 0;
-        for (int i = 0; i < 4; i++) s_sched.phase[i] = 0;
+        for (int i = 0; i < 5; i++) s_sched.phase[i] = 0;
         s_sched.desc_next = 0;
         s_sched.may_keep = 0;
         for (int i = 0; i < DESC_CACHE; i++) s_sched.desc_id[i] = 0xffffffffu;
@@ -415,7 +415,7 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
         atomicAdd (&prof[0], s_sched.ticks[0]); atomicAdd (&prof[1], s_sched.ticks[1]); atomicAdd (&prof[2], s_sched.ticks[2]);
         atomicAdd (&prof[3], wall_clock64 () - t_begin);
         atomicAdd (&prof[4], s_sched.ticks[3]); atomicAdd (&prof[5], s_sched.ticks[4]); atomicAdd (&prof[6], s_sched.ticks[5]);
-        for (int i = 0; i < 4; i++) atomicAdd (&prof[8 + i], s_sched.phase[i]);
+        for (int i = 0; i < 5; i++) atomicAdd (&prof[8 + i], s_sched.phase[i]);
         atomicAdd (&prof[7], (unsigned long long)(clock64 () - c_begin));     // engine clock cycles: [7] / [3] * 100 MHz = the clock the run had
     }
 }

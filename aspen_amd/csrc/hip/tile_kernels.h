@@ -402,6 +402,7 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
     floatx16 (&acc)[BN / WN / 32][BM / WM / 32], bool phases = false, Hook before_last_slice = Hook ())
 {
     static_assert (DEPTH == 1 || DEPTH == 2, "one or two register sets");
+    if (phases) tile_phase_lap (12);
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     constexpr int KK = GEMM_BK / 8;
     const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
@@ -524,6 +525,83 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
     lds_barrier ();          // the caller reuses the stage (epilogue)
 }
 
+// The same for the 64 x 64 shape, whose four waves own ONE 32 x 32 block each, scheduled by hand for a
+// workgroup that has its compute unit (nearly) to itself -- the normal case for these tiles: they are the
+// short tiles of layers cut along K, and in a graph bound by its dependency chains only one or two
+// workgroups per compute unit are inside a K loop at any time.  Then nothing but this wave's own instruction
+// order hides the slice boundary (two barriers, the LDS refill, the next requests): in gemm_core the matrix
+// pipeline drains there, 16 MFMAs of 64 cycles each took ~1600 cycles per slice.
+// Here the fragments of all four sub-steps of a slice are resident (8 registers each, affordable with one
+// accumulator block), so every piece of boundary work sits between two MFMAs that do not depend on it:
+//   M00 M01 M02 |X| M03 wA M10 wB M11 gA M12 gB M13 M20 |Y| M21 r0 M22 r1 M23 M30 r2 M31 M32 M33 r3
+// Mij = MFMA on K pair j of sub-step i; X = barrier "everyone holds this slice's fragments", wA / wB = next
+// slice registers -> LDS, gA / gB = requests for the slice DEPTH ahead, Y = barrier "refill visible",
+// ri = fragments of sub-step i of the next slice (its buffer was released by Mi3).
+template <int DEPTH, class ALoader, class BLoader, class Hook = NoHook>
+__device__ __forceinline__ void gemm_core_single_block (ALoader &al, BLoader &bl, int kbase, int kiters, float *smem,
+    floatx16 (&accs)[1][1], bool phases = false, Hook before_last_slice = Hook ())
+{
+    static_assert (DEPTH == 1 || DEPTH == 2, "one or two register sets");
+    static_assert (ALoader::R == 2 && BLoader::R == 2 && GEMM_BK == 32, "64 x 64 tile, four sub-steps");
+    constexpr int BM = 64;
+    if (phases) tile_phase_lap (12);
+    const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
+    const uint32_t wm0 = (wave % 2) * 32, wn0 = (wave / 2) * 32;
+    const float *afrag = smem + wm0 * LDS_ROW + (lane & 31) * LDS_ROW + (lane >> 5) * 4;
+    const float *bfrag = smem + BM * LDS_ROW + wn0 * LDS_ROW + (lane & 31) * LDS_ROW + (lane >> 5) * 4;
+    floatx16 acc;
+    #pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = 0.f;
+    float4 fa[4], fb[4];
+#define SB __builtin_amdgcn_sched_barrier (0)
+#define RD(i) do { fa[i] = ld4 (afrag + (i) * 8); fb[i] = ld4 (bfrag + (i) * 8); SB; } while (0)
+#define MF(i, c) do { acc = __builtin_amdgcn_mfma_f32_32x32x2f32 (fb[i].c, fa[i].c, acc, 0, 0, 0); SB; } while (0)
+    float4 areg[DEPTH][2], breg[DEPTH][2];
+    al.load (kbase, areg[0]); bl.load (kbase, breg[0]);
+    if (DEPTH == 2 && kiters > 1) { al.load (kbase + 1, areg[DEPTH - 1]); bl.load (kbase + 1, breg[DEPTH - 1]); }
+    al.store (smem, areg[0]); bl.store (smem + BM * LDS_ROW, breg[0]);
+    if (kiters > DEPTH) { al.load (kbase + DEPTH, areg[0]); bl.load (kbase + DEPTH, breg[0]); }
+    lds_barrier ();
+    if (phases) tile_phase_lap (8);
+    SB; RD (0); RD (1); RD (2); RD (3);
+    // `set` (a literal at every call) = the register set that holds slice it + 1
+    auto slice = [&] (int it, int set)
+    {
+        // requests are always issued (the last slices are asked for again and never used): a request inside a
+        // branch makes the compiler lose count of what is in flight, and it then waits for everything
+        const int nxt = kbase + (DEPTH == 2 ? min (it + 1 + DEPTH, kiters - 1) : it + 2);
+        SB; MF (0, x); MF (0, y); MF (0, z);
+        lds_barrier (); SB;
+        MF (0, w); al.store (smem, areg[set]); SB;
+        MF (1, x); bl.store (smem + BM * LDS_ROW, breg[set]); SB;
+        MF (1, y); if (DEPTH == 2 || it + 2 < kiters) al.load (nxt, areg[set]); SB;
+        MF (1, z); if (DEPTH == 2 || it + 2 < kiters) bl.load (nxt, breg[set]); SB;
+        MF (1, w); MF (2, x);
+        lds_barrier (); SB;
+        MF (2, y); RD (0);
+        MF (2, z); RD (1);
+        MF (2, w); MF (3, x); RD (2);
+        MF (3, y); MF (3, z); MF (3, w); RD (3);
+    };
+    if (DEPTH == 1)
+        for (int it = 0; it + 1 < kiters; it++) slice (it, 0);
+    else
+    {
+        int it = 0;
+        for (; it + 2 < kiters; it += 2) { slice (it, DEPTH - 1); slice (it + 1, 0); }
+        if (it + 1 < kiters) slice (it, DEPTH - 1);
+    }
+    before_last_slice ();
+    SB;
+    MF (0, x); MF (0, y); MF (0, z); MF (0, w); MF (1, x); MF (1, y); MF (1, z); MF (1, w);
+    MF (2, x); MF (2, y); MF (2, z); MF (2, w); MF (3, x); MF (3, y); MF (3, z); MF (3, w);
+#undef SB
+#undef RD
+#undef MF
+    accs[0][0] = acc;
+    lds_barrier ();          // the caller reuses the stage (epilogue)
+}
+
 // Accumulator register v of MFMA block (i, j) holds output (row n, channel m):
 //   n = wn0 + 32 i + 8 (v / 4) + 4 (lane / 32) + v % 4,   m = wm0 + 32 j + lane % 32
 #define ACC_N(wn0, i, v, lane) ((wn0) + 32 * (i) + 8 * ((v) >> 2) + 4 * ((lane) >> 5) + ((v) & 3))
@@ -600,13 +678,15 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
     {
         ActRowLoader<BN, COH> bl;
         bl.init (in, n0, L.N - 1, L.ld0, 0, tid);
-        gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
+        if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
+        else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
     }
     else
     {
         ConvLoader<BN, COH> bl;
         bl.init (L, in, n0, tid);
-        gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
+        if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
+        else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
     }
     if (COH) tile_phase_lap (9);
     const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);

@@ -105,6 +105,87 @@ def verify_final_layer(name, nasm):
     return {"ok": ok, "sampled_rel_l2": err, "argmax_equal": bool((got.argmax(axis=1) == gold["argmax"]).all())}
 
 
+def cpu_description():
+    """CPU model, physical cores and hardware threads of this host (from /proc/cpuinfo)."""
+    model, phys, threads = "unknown", set(), 0
+    try:
+        pid = cid = None
+        for line in open("/proc/cpuinfo"):
+            k, _, v = line.partition(":")
+            k, v = k.strip(), v.strip()
+            if k == "model name":
+                model = v
+            elif k == "physical id":
+                pid = v
+            elif k == "core id":
+                cid = v
+            elif k == "processor":
+                threads += 1
+            elif not k and pid is not None:
+                phys.add((pid, cid)); pid = cid = None
+        if pid is not None:
+            phys.add((pid, cid))
+    except OSError:
+        pass
+    return {"model": model, "physical_cores": len(phys) or None, "hardware_threads": threads or (os.cpu_count() or 0)}
+
+
+def measure_workload(api, M, name, steps, warmup):
+    """One of the other benchmark configurations, in the same loop as the headline one: its tuned tile count and
+    engine (models.WORKLOADS), inputs resident, `warmup` untimed + `steps` timed steps, final layer checked
+    against the compiled reference's fixture afterwards.  Everything is torn down again."""
+    L = api.lib()
+    cfgs, unit, units_per_step, min_ninst, engine = WORKLOADS[name]
+    pool = api.RPool()
+    dse = api.DseGroup(1, api.MODE_DATAFLOW if engine == "dataflow" else api.MODE_LAYERS)
+    dse.set_rpool(pool)
+    nets = []
+    for cname in cfgs:
+        cfg, layers, tens, x, batch, seq = M.make_config(cname)
+        wp = tempfile.mktemp(suffix=".bin")
+        M.write_aspen_data(wp, tens)
+        dnn = api.Dnn(cfg, wp)
+        os.unlink(wp)
+        del tens
+        nasm = api.Nasm(dnn, batch, seq, min_ninst)
+        pool.add_nasm_raw_input(nasm, x)
+        nets.append((cname, dnn, nasm))
+    flops = sum(gemm_flops(n, api) for _, _, n in nets)
+
+    def one(first=False):
+        if not first:
+            pool.reset_queue()
+            for _, _, n in nets:
+                pool.reset_nasm(n)
+        dse.run()
+        for _, _, n in nets:
+            dse.wait(n)
+        dse.stop()
+
+    one(first=True)
+    for _ in range(warmup):
+        one()
+    L.aspen_hip_sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        one()
+    L.aspen_hip_sync()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    checks = [verify_final_layer(cname, n) for cname, _, n in nets]
+    have = [c for c in checks if c is not None]
+    ach = flops / (ms * 1e-3) / 1e12
+    out = {"ms_per_step": ms, "value": units_per_step / (ms * 1e-3), "unit": unit, "engine": engine, "min_ninst_per_ldata": min_ninst,
+           "tiles_per_step": sum(n.num_ninst for _, _, n in nets), "flops_per_step": flops,
+           "frac_of_fp32_mfma_peak": ach / PEAK_FP32_MFMA_TFLOPS, "verified": all(c["ok"] for c in have) if have else None}
+    dse.destroy()
+    for _, _, n in nets:
+        n.destroy()
+    pool.destroy()
+    for _, d, _ in nets:
+        d.destroy()
+    return out
+
+
 def quiet_stdout():
     """The C library reports what it parses on stdout, as the reference does.  The benchmark's stdout
     carries exactly one JSON line, so everything else written to file descriptor 1 goes to stderr; returns
@@ -131,6 +212,8 @@ def main():
     ap.add_argument("--min-ninst", type=int, default=0, help="tiles wanted per layer (0: the workload's tuned value)")
     ap.add_argument("--workgroups", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the `workloads` section (the other benchmark configurations, measured after the headline one)")
     ap.add_argument("--skip-tiles", action="store_true", help="scheduler-only run: dependency protocol with empty tiles")
     ap.add_argument("--no-handoff", action="store_true", help="every ready tile goes through the queue (no parent -> child hand-off)")
     ap.add_argument("--engine-profile", action="store_true", help="report where the persistent workgroups spend their time")
@@ -314,17 +397,27 @@ def main():
         out["verified"] = all(c["ok"] for c in have) if have else None
         out["verification"] = checks
 
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(cfgs[0])
-
-    for _, dnn, nasm, _ in nets:
-        pass
     dse.destroy()
     for _, dnn, nasm, _ in nets:
         nasm.destroy()
     pool.destroy()
     for _, dnn, nasm, _ in nets:
         dnn.destroy()
+    del nets
+
+    # the other configurations of the benchmark, each on its own tuned graph (value stays the headline workload's)
+    plain = not (args.skip_tiles or args.engine_profile or args.trace or args.layer_profile or args.no_handoff)
+    if not args.no_other_workloads and plain and args.workload == "resnet50_b32":
+        L.aspen_hip_set_flags(0)
+        out["workloads"] = {}
+        for name in ("resnet50_b1", "vgg16_b32", "co_resnet50_vgg16_b16", "bert_base_b8_s128", "gpt2_b4_s512"):
+            out["workloads"][name] = measure_workload(api, M, name, max(5, min(args.steps, 20)), args.warmup)
+        if not all(w["verified"] is not False for w in out["workloads"].values()):
+            out["verified"] = False
+
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfgs[0])
+        out["cpu_baseline"]["cpu"] = cpu_description()
     emit(json.dumps(out))
     if out.get("verified") is False:
         print("bench.py: the timed graph's output does not match the reference fixture", file=sys.stderr)

@@ -155,8 +155,9 @@ int aspen_hip_run_dataflow (aspen_hip_graph_t *graph, uint32_t workgroups, uint6
    [3] total workgroup lifetime; detail of [2]: [4] publishing wavefront (countdown of the children,
    pushes), [5] popping wavefront drawing its ticket, [6] popping wavefront waiting for its queue slot
    to be filled; [7] engine-clock cycles of the workgroups' lifetimes ([7] / [3] x 100 MHz = the
-   average engine clock during the run); contraction tiles only: [8] operand set-up up to the first staged
-   slice, [9] K loop, [10] epilogue, [11] split-K arrival and reduction; [12..15] unused */
+   average engine clock during the run); contraction tiles only: [12] descriptor and operand-address set-up, [8] from
+   there to the first staged slice (the first loads' latency), [9] K loop, [10] epilogue, [11] split-K arrival
+   and reduction; [13..15] unused */
 int aspen_hip_dataflow_profile (aspen_hip_graph_t *graph, uint64_t ticks[16], int reset);
 /* TRACE makes the dataflow kernel stamp every tile's start and end (100 MHz device clock);
    aspen_hip_dataflow_trace copies the stamps of the last traced run: start_end[2*i], [2*i+1] for tile i
