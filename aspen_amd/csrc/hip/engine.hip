@@ -621,6 +621,37 @@ extern "C" int aspen_hip_copy (void *dst, const void *src, size_t bytes)
 // ------------------------------------------------------------------------------------------------
 // graph
 // ------------------------------------------------------------------------------------------------
+// {multiplier, shift} for fast_div (tile_kernels.h): division by the invariant d in its branch-free round-up form
+// (T. Granlund, P. Montgomery, "Division by invariant integers using multiplication", 1994).
+static void divider_for (uint32_t d, uint32_t out[2])
+{
+    if (d <= 1) { out[0] = 0; out[1] = 0x80u; return; }
+    uint32_t lg = 31;
+    while (!(d >> lg)) lg--;                                 // floor (log2 (d))
+    if ((d & (d - 1)) == 0) { out[0] = 0; out[1] = lg - 1; return; }
+    const uint64_t two_k = (uint64_t)1 << (32 + lg);
+    uint64_t m = two_k / d;
+    const uint64_t rem = two_k - m * d;
+    m *= 2;
+    if (2 * rem >= d) m += 1;
+    out[0] = (uint32_t)(m + 1);
+    out[1] = lg;
+}
+
+// the values of a layer descriptor that aspen_hip_graph_create derives for the kernels
+static void fill_derived (aspen_hip_layer_t &L)
+{
+    divider_for (L.OH * L.OW, L.div_ohw);
+    divider_for (L.OW, L.div_ow);
+    divider_for (L.tiles_m, L.div_tiles_m);
+    divider_for (L.splits, L.div_splits);
+    if (L.type == FC_LAYER) L.in0_columns = L.N * L.IH * L.IW;
+    else if (L.type == CONV_LAYER && L.OH * L.OW != 0) L.in0_columns = (L.N / (L.OH * L.OW)) * L.IH * L.IW;
+    else L.in0_columns = L.N;
+}
+
+extern "C" void aspen_hip_divider_for (uint32_t d, uint32_t out[2]) { divider_for (d, out); }
+
 template <class T> static T *upload (const T *src, size_t n)
 {
     T *d = (T *)aspen_hip_alloc ((n ? n : 1) * sizeof (T));
@@ -818,7 +849,8 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     g->h_layers = (aspen_hip_layer_t *)malloc (sizeof (aspen_hip_layer_t) * (num_layers ? num_layers : 1));
     if (!g->h_layers) { snprintf (g_err, sizeof (g_err), "out of host memory"); free (g); return nullptr; }
     memcpy (g->h_layers, layers, sizeof (aspen_hip_layer_t) * num_layers);
-    g->d_layers = upload (layers, num_layers);
+    for (uint32_t l = 0; l < num_layers; l++) fill_derived (g->h_layers[l]);
+    g->d_layers = upload (g->h_layers, num_layers);
     g->d_ninst_layer = upload (ninst_layer, num_ninst);
     g->d_num_parents = upload (num_parents, num_ninst);
     g->d_child_off = upload (child_off, (size_t)num_ninst + 1);
@@ -1032,6 +1064,7 @@ extern "C" int aspen_hip_sgemm (uint32_t M, uint32_t N, uint32_t K, const float 
     L.M = M; L.N = N; L.ld = ldc; L.tile_m = 64; L.tile_n = 64;
     L.tiles_m = (M + 63) / 64; L.tiles_n = (N + 63) / 64; L.num_ninst = L.tiles_m * L.tiles_n; L.splits = 1;
     L.K = K; L.Kp = K; L.ld0 = ldb; L.out = C; L.in0 = B; L.weight = Ap; L.bias = bias;
+    fill_derived (L);
     aspen_hip_layer_t *dL = upload (&L, 1);
     if (!dL) { aspen_hip_free (Ap); return -1; }
     hipLaunchKernelGGL (layer_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, dL, 0u, 0u, (uint32_t *)nullptr);      // no split-K: the arrival counters are not touched
@@ -1119,6 +1152,7 @@ extern "C" int aspen_hip_sgemm_static (uint32_t M, uint32_t N, uint32_t K, const
     L.M = M; L.N = N; L.ld = ldc; L.tile_m = VAR2_BM; L.tile_n = VAR2_BN;
     L.tiles_m = (M + VAR2_BM - 1) / VAR2_BM; L.tiles_n = (N + VAR2_BN - 1) / VAR2_BN; L.num_ninst = L.tiles_m * L.tiles_n; L.splits = 1;
     L.K = K; L.Kp = K; L.ld0 = ldb; L.out = C; L.in0 = B; L.weight = Ap; L.bias = bias;
+    fill_derived (L);
     hipLaunchKernelGGL (sgemm_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, L);
     CHECK (hipGetLastError ());
     return 0;

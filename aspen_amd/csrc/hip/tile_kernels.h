@@ -52,6 +52,16 @@ __device__ void tile_phase_lap (int which);
                                CMAX (VAR_FLOATS (VAR2_BM, VAR2_BN), STAGE_FLOATS (128, KATTN_BN)))
 #define GEMM_SMEM_BYTES (GEMM_SMEM_FLOATS * 4)
 
+// n / d for any 32-bit n, with {multiplier, shift} prepared on the host by divider_for (engine.hip):
+// q = (((n - t) >> 1) + t) >> shift, t = high half of n * multiplier (the "round-up" method of division by an
+// invariant integer, in its branch-free form, which is exact for every n and every d >= 2); bit 7 of shift marks d = 1.
+__device__ __forceinline__ uint32_t fast_div (uint32_t n, const uint32_t (&dv)[2])
+{
+    const uint32_t t = __umulhi (n, dv[0]);
+    const uint32_t q = (((n - t) >> 1) + t) >> (dv[1] & 31u);
+    return (dv[1] & 0x80u) ? n : q;
+}
+
 __device__ __forceinline__ float4 ld4 (const float *p) { return *reinterpret_cast<const float4 *> (p); }
 __device__ __forceinline__ void st4 (float *p, float4 v) { *reinterpret_cast<float4 *> (p) = v; }
 
@@ -279,7 +289,7 @@ template <int ROWS, int COH> struct ConvLoader
         {
             uint32_t n = first_row + row0 + 32 * i;
             n = n < L.N ? n : L.N - 1;
-            uint32_t b = n / ohw, rem = n - b * ohw, oh = rem / L.OW, ow = rem - oh * L.OW;
+            uint32_t b = fast_div (n, L.div_ohw), rem = n - b * ohw, oh = fast_div (rem, L.div_ow), ow = rem - oh * L.OW;
             ih0[i] = (int32_t)(oh * L.stride) - (int32_t)L.pad;
             iw0[i] = (int32_t)(ow * L.stride) - (int32_t)L.pad;
             base[i] = ((int32_t)(b * L.IH) + ih0[i]) * (int32_t)L.IW * (int32_t)L.ld0 + iw0[i] * (int32_t)L.ld0;
@@ -645,7 +655,7 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
     const uint32_t m0 = tm * BM, n0 = tn * BN;
     floatx16 acc[TN][TM];
     ActView<COH> in;
-    in.init (L.in0, L.type == FC_LAYER ? L.N * L.IH * L.IW : (L.type == CONV_LAYER ? (L.N / (L.OH * L.OW)) * L.IH * L.IW : L.N), L.ld0);
+    in.init (L.in0, L.in0_columns, L.ld0);
     int kbase = 0, kiters = (int)(L.Kp / GEMM_BK);
     if (slice >= 0)
     {
@@ -1355,7 +1365,7 @@ __device__ __forceinline__ void finish_tile (const aspen_hip_layer_t &Lg, uint32
 {
     const aspen_hip_layer_t L = uniform_layer (Lg);
     t = __builtin_amdgcn_readfirstlane (t);
-    const uint32_t tn = t / L.tiles_m;
+    const uint32_t tn = fast_div (t, L.div_tiles_m);
     tile_splitk_finish<COH> (L, tn, t - tn * L.tiles_m);
 }
 
@@ -1373,11 +1383,12 @@ __device__ __forceinline__ bool run_tile (const aspen_hip_layer_t &Lg, uint32_t 
     uint32_t group = 0;
     if (L.splits > 1)
     {
-        slice = (int)(t % L.splits);
+        const uint32_t q = fast_div (t, L.div_splits);
+        slice = (int)(t - q * L.splits);
         group = L.ninst_start + t - (uint32_t)slice;
-        t /= L.splits;
+        t = q;
     }
-    const uint32_t tn = t / L.tiles_m, tm = t - tn * L.tiles_m;
+    const uint32_t tn = fast_div (t, L.div_tiles_m), tm = t - tn * L.tiles_m;
     switch (L.type)
     {
     case CONV_LAYER: case FC_LAYER: case MATMUL_LAYER:

@@ -87,6 +87,12 @@ typedef struct aspen_hip_layer_t
     const float *fuse_in;
     uint32_t fuse_ld_in;
     int32_t fuse_act;
+    /* Derived values, filled in by aspen_hip_graph_create (callers leave them zero): divisions by OH*OW, OW,
+       tiles_m and splits as multiply-and-shift pairs {multiplier, shift} (a tile's set-up is bound by
+       instruction issue, and an integer division costs some 25 instructions), and the number of columns of
+       the first parent's matrix. */
+    uint32_t div_ohw[2], div_ow[2], div_tiles_m[2], div_splits[2];
+    uint32_t in0_columns;
 } aspen_hip_layer_t;
 
 typedef struct aspen_hip_graph_t aspen_hip_graph_t;
@@ -191,6 +197,10 @@ int aspen_hip_profile_layers (aspen_hip_graph_t *graph, uint32_t iters, float *m
    kernel, so elapsed(14, 15) is that kernel's duration. */
 int aspen_hip_event_record (int slot);
 int aspen_hip_event_elapsed_ms (int slot_begin, int slot_end, float *ms);
+
+/* {multiplier, shift} with which the kernels divide by `d` (see aspen_hip_layer_t); pure arithmetic, callable
+   without a GPU. */
+void aspen_hip_divider_for (uint32_t d, uint32_t out[2]);
 
 /* ---- plain SGEMM seam (reference include/kernels.h:15-33 on device pointers) -------------------- */
 /* C[n*ldc + m] = act(bias[m] + sum_k A[m*lda + k] * B[n*ldb + k]); A row-major [M][K] (not packed),

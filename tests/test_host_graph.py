@@ -339,3 +339,33 @@ def test_generate_nasm_without_gpu_takes_the_default(capfd):
         assert g2.num_ninst == ref.num_ninst
         g2.destroy()
     g.destroy(); ref.destroy(); d.destroy()
+
+
+def test_kernel_dividers_are_exact():
+    """The kernels divide by layer constants (OH*OW, OW, tiles per row, K splits) with a multiplier and a shift that
+    aspen_hip_graph_create prepares (aspen_hip_divider_for): q = (((n - t) >> 1) + t) >> shift, t = high half of
+    n * multiplier.  Checked against integer division for small, large, power-of-two and odd divisors, at the
+    multiples of the divisor and their neighbours and at the ends of the 32-bit range."""
+    import ctypes
+    import random
+    L = api.lib()
+    L.aspen_hip_divider_for.argtypes = [ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint32)]
+
+    def divide(n, d):
+        o = (ctypes.c_uint32 * 2)()
+        L.aspen_hip_divider_for(d, o)
+        if o[1] & 0x80:
+            return n
+        t = (n * o[0]) >> 32
+        return ((((n - t) & 0xffffffff) >> 1) + t) >> (o[1] & 31)
+
+    rng = random.Random(7)
+    divisors = list(range(1, 200)) + [rng.randrange(1, 1 << 31) for _ in range(500)] + \
+        [12544, 3136, 784, 196, 49, 112, 56, 28, 14, 7, 224, 100352, 401408, 1605632, (1 << 31) - 1, 1 << 31, (1 << 31) + 1, (1 << 32) - 1]
+    for d in divisors:
+        ns = [0, 1, d - 1, d, d + 1, 2 * d - 1, 2 * d, (1 << 32) - 1, (1 << 32) - 2, 1 << 31, 123456789]
+        ns += [rng.randrange(0, 1 << 32) for _ in range(40)]
+        ns += [k * d + e for k in range(1, 20) for e in (-1, 0, 1)]
+        for n in ns:
+            if 0 <= n < (1 << 32):
+                assert divide(n, d) == n // d, (n, d)
