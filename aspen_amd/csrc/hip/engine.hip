@@ -73,17 +73,17 @@ static int fail (hipError_t e, const char *what)
 __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) layer_kernel (const aspen_hip_layer_t *layers, uint32_t l, uint32_t first_tile, uint32_t *arrivals)
 {
     extern __shared__ __align__ (16) float smem[];
-    const aspen_hip_layer_t &L = layers[l];
     const uint32_t nt = gridDim.x, bid = blockIdx.x;
     const uint32_t xcd = bid & 7, local = bid >> 3, chunk = nt >> 3, rem = nt & 7;
     const uint32_t t = first_tile + xcd * chunk + (xcd < rem ? xcd : rem) + local;
-    run_tile<0> (L, t, smem, [=] () { return arrivals; });
+    run_tile<0> ([=] () { return scalar_layer (layers + l); }, t, false, smem, [=] () { return arrivals; });
 }
 
 // Second launch of a split-K layer in launch-per-layer mode: one workgroup per output tile adds the slices up.
 __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) finish_kernel (const aspen_hip_layer_t *layers, uint32_t l)
 {
-    finish_tile<0> (layers[l], blockIdx.x);
+    const aspen_hip_layer_t L = scalar_layer (layers + l);
+    finish_tile<0> (L, blockIdx.x);
 }
 
 // Re-arm: counters back to the parent counts, queue seeded with the roots.  A queue entry is 64 bits:
@@ -182,9 +182,6 @@ __device__ __forceinline__ qentry_t wait_for_slot (const dataflow_args_t &a, uin
     }
 }
 
-#define DESC_CACHE 4
-static_assert (sizeof (aspen_hip_layer_t) % 4 == 0 && sizeof (aspen_hip_layer_t) / 4 <= 64, "one descriptor dword per lane of a wavefront");
-
 // Workgroup-local scheduler state.  It lives in LDS so that nothing of it occupies registers while a
 // tile runs: the tile code is inlined into the persistent loop and owns the whole register budget.
 struct sched_lds_t
@@ -193,10 +190,6 @@ struct sched_lds_t
     uint32_t tile, layer;                // tile to run next (QUEUE_EMPTY: leave) and its layer
     uint32_t complete;                   // 0: the tile just run was a split-K slice that did not finish its group
     uint32_t may_keep;                   // the tile just run releases children, one of which this workgroup may run next
-    // the descriptors of the last few layers this workgroup worked on: consecutive tiles mostly belong
-    // to the same two or three layers, so most tiles find theirs here instead of fetching it from memory
-    uint32_t desc_slot, desc_next, desc_id[DESC_CACHE];
-    aspen_hip_layer_t desc[DESC_CACHE];
     unsigned long long t0, ticks[6];     // profiling: last time stamp; tile / drain / scheduling / publish / ticket / slot-wait ticks
     unsigned long long p0, phase[5];     // profiling of contraction tiles: last phase stamp; set-up / K loop / epilogue / split-K ticks
 };
@@ -245,8 +238,8 @@ __device__ __forceinline__ void push_ready (const dataflow_args_t &a, uint32_t c
 // count themselves when they finish; the last of them (then every tile has finished, for every tile has a
 // descendant without children) writes a leave entry into the next gridDim.x slots behind the tail: every
 // workgroup holds at most one ticket, so these are all the slots anyone can still be waiting for.
-// The pop half of a scheduling step, run by one wavefront: draws a ticket, waits for its slot, and makes sure
-// the tile's layer descriptor is in the LDS cache.  kept != QUEUE_EMPTY: the tile to run is already known.
+// The pop half of a scheduling step, run by one wavefront: draws a ticket and waits for its slot.
+// kept != QUEUE_EMPTY: the tile to run is already known.
 __device__ __forceinline__ void pop_next (const dataflow_args_t &a, uint32_t lane, uint32_t kept, uint32_t kept_layer, bool prof)
 {
     if (lane == 0)
@@ -265,22 +258,6 @@ __device__ __forceinline__ void pop_next (const dataflow_args_t &a, uint32_t lan
             s_sched.layer = (uint32_t)(e >> 32) & 0xffffu;
             if (prof) { s_sched.ticks[4] += t2 - t1; s_sched.ticks[5] += wall_clock64 () - t2; }
         }
-    }
-    // (same wavefront, program order: lane 0's LDS writes above are visible to all lanes here)
-    const uint32_t tile = __builtin_amdgcn_readfirstlane (s_sched.tile), layer = __builtin_amdgcn_readfirstlane (s_sched.layer);
-    if (tile != QUEUE_EMPTY)
-    {
-        uint32_t slot = DESC_CACHE;
-        for (uint32_t i = 0; i < DESC_CACHE; i++) if (s_sched.desc_id[i] == layer) slot = i;
-        slot = __builtin_amdgcn_readfirstlane (slot);
-        if (slot == DESC_CACHE)
-        {
-            slot = __builtin_amdgcn_readfirstlane (s_sched.desc_next);
-            if (lane < sizeof (aspen_hip_layer_t) / 4)
-                reinterpret_cast<uint32_t *> (&s_sched.desc[slot])[lane] = reinterpret_cast<const uint32_t *> (&a.layers[layer])[lane];
-            if (lane == 0) { s_sched.desc_id[slot] = layer; s_sched.desc_next = (slot + 1) % DESC_CACHE; }
-        }
-        if (lane == 0) s_sched.desc_slot = slot;
     }
 }
 
@@ -379,9 +356,7 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
         s_sched.t0 = wall_clock64 ();
         for (int i = 0; i < 6; i++) s_sched.ticks[i] = 0;
         for (int i = 0; i < 5; i++) s_sched.phase[i] = 0;
-        s_sched.desc_next = 0;
         s_sched.may_keep = 0;
-        for (int i = 0; i < DESC_CACHE; i++) s_sched.desc_id[i] = 0xffffffffu;
     }
     __syncthreads ();
     const unsigned long long t_begin = wall_clock64 (), c_begin = clock64 ();
@@ -397,15 +372,18 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
             rec = *(const qentry_t __attribute__ ((address_space (1))) *)(s_sched.a.child_rec + (size_t)id * CHILD_REC + threadIdx.x);
         if ((s_sched.a.flags & ASPEN_HIP_FLAG_TRACE) && threadIdx.x == 0) s_sched.a.trace[2 * (size_t)id] = wall_clock64 ();
         if ((s_sched.a.flags & ASPEN_HIP_FLAG_PROFILE) && threadIdx.x == 0) s_sched.p0 = wall_clock64 ();
-        const aspen_hip_layer_t *L = &s_sched.desc[__builtin_amdgcn_readfirstlane (s_sched.desc_slot)];
+        // the layer's descriptor goes from memory into scalar registers (it is shared by all tiles of the layer
+        // and by all workgroups, so it sits in the scalar cache or in L2)
+        const auto descriptor = [] () { return scalar_layer (s_sched.a.layers + s_sched.layer); };
         bool complete;
         if (!(s_sched.a.flags & ASPEN_HIP_FLAG_SKIP_TILES))
-            complete = run_tile<COH> (*L, id - L->ninst_start, smem, [] () { return s_sched.a.arrivals; });
+            complete = run_tile<COH> (descriptor, id, true, smem, [] () { return s_sched.a.arrivals; });
         else
         {
             // scheduler-only run: the split-K groups still elect the member that releases the children
-            const uint32_t splits = __builtin_amdgcn_readfirstlane (L->splits), t = id - __builtin_amdgcn_readfirstlane (L->ninst_start);
-            complete = splits <= 1 || splitk_arrived_last (&s_sched.a.arrivals[id - t % splits], splits, smem);
+            const aspen_hip_layer_t L = descriptor ();
+            const uint32_t t = id - L.ninst_start;
+            complete = L.splits <= 1 || splitk_arrived_last (&s_sched.a.arrivals[id - t % L.splits], L.splits, smem);
         }
         if (threadIdx.x == 0) s_sched.complete = complete;      // read by schedule_step behind its barrier
     }
@@ -1120,7 +1098,7 @@ __global__ void __launch_bounds__ (WG_THREADS) pad_rows_kernel (const float *__r
 __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) sgemm_kernel (const aspen_hip_layer_t L)
 {
     extern __shared__ __align__ (16) float smem[];
-    run_tile<0> (L, blockIdx.x, smem, [] () { return (uint32_t *)nullptr; });
+    run_tile<0> ([&] () { return uniform_layer (L); }, blockIdx.x, false, smem, [] () { return (uint32_t *)nullptr; });
 }
 
 extern "C" size_t aspen_hip_sgemm_static_max_bytes (void) { return SGEMM_SCRATCH_BYTES; }

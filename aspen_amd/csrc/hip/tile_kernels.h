@@ -647,8 +647,8 @@ __device__ __forceinline__ void fused_shortcut (const aspen_hip_layer_t &L, cons
 // of the thread's pieces of a fused shortcut's operand (a tile has at most 128 columns: 8 pieces per thread)
 struct shortcut_prefetch_t { float4 s[8]; float4 bias; bool have, have_shortcut; };
 
-template <int BM, int BN, int WM, int WN, int DEPTH, int COH>
-__device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, int slice, float *smem, shortcut_prefetch_t &pre)
+template <int BM, int BN, int WM, int WN, int DEPTH, int COH, class Descriptor>
+__device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L, Descriptor descriptor, uint32_t tn, uint32_t tm, int slice, float *smem, shortcut_prefetch_t &pre)
 {
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
@@ -667,8 +667,10 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
     // a fused shortcut's other operand comes from memory another XCD may have written: the first pieces this
     // thread will need in the epilogue (see contraction_epilogue for the thread -> piece mapping) are
     // requested under the last K slice
+    // (`L` below is a fresh copy of the descriptor: what only this hook needs stays out of the K loop's registers)
     auto fetch_shortcut = [&] ()
     {
+        const aspen_hip_layer_t L = descriptor ();
         constexpr uint32_t C4_LOG2 = BM == 128 ? 5 : 4, STEP = WG_THREADS >> C4_LOG2, PIECES = BN / STEP;
         static_assert (PIECES <= 8, "pieces per thread");
         const uint32_t c = (tid & ((1u << C4_LOG2) - 1)) * 4, rows = min ((uint32_t)BN, L.N - n0), r0 = tid >> C4_LOG2;
@@ -705,6 +707,7 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
         // split-K: the raw sums go straight from the accumulators to this slice's partial matrix.  Register v of
         // a block holds 32 consecutive channels of one column across a half-wave, so every store instruction
         // writes two whole 128-byte lines; no bias, no activation, nothing to stage through LDS.
+        const aspen_hip_layer_t L = descriptor ();
         ActView<COH> part;
         part.init (L.partial + (size_t)slice * L.N * L.ld, L.N, L.ld);
         #pragma unroll
@@ -1326,14 +1329,36 @@ __device__ __forceinline__ void tile_v_attention (const aspen_hip_layer_t &L, ui
 // (reference src/dse.c:39-79).  `t` = tile index inside the layer, row-tile fastest
 // (reference src/apu_nasm.c:1218-1224).
 // ---------------------------------------------------------------------------------------------
-// A wave-uniform copy of a layer descriptor in scalar registers.  The descriptor sits in memory the
-// kernel also writes, so the compiler reads it with vector loads; without this copy every value
-// derived from it counts as per-lane data: buffer descriptors get rebuilt in a per-lane "waterfall"
-// loop around each access and all tile-level control flow runs on the vector unit.
-__device__ __forceinline__ aspen_hip_layer_t uniform_layer (const aspen_hip_layer_t &Lg)
+// A wave-uniform copy of a layer descriptor in scalar registers.  Every value derived from the descriptor must
+// be known to be uniform: otherwise buffer descriptors get rebuilt in a per-lane "waterfall" loop around each
+// access and all tile-level control flow runs on the vector unit.
+//
+// scalar_layer reads a descriptor in device memory through the scalar data cache (read-only use: descriptors
+// are written by the host before the launch and never by a kernel), 64 dwords in a handful of wide scalar
+// loads straight into scalar registers.  `g` must be the same for all lanes.
+__device__ __forceinline__ aspen_hip_layer_t scalar_layer (const aspen_hip_layer_t *g)
 {
     constexpr int W = sizeof (aspen_hip_layer_t) / 4;
     static_assert (sizeof (aspen_hip_layer_t) % 4 == 0, "descriptor is a whole number of dwords");
+    const uint64_t p = (uint64_t)g;
+    // (the builtin returns int: without the casts the low half would be sign-extended over the high one)
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane ((uint32_t)p), hi = (uint32_t)__builtin_amdgcn_readfirstlane ((uint32_t)(p >> 32));
+    uint64_t up = ((uint64_t)hi << 32) | (uint64_t)lo;
+    // Every call loads afresh: the compiler may not merge the loads of two calls (and so keep all 64 dwords in
+    // registers from the first use of a descriptor to the last), because it cannot see that `up` is unchanged.
+    asm volatile ("" : "+s" (up));
+    const uint32_t __attribute__ ((address_space (4))) *src = (const uint32_t __attribute__ ((address_space (4))) *)up;
+    uint32_t w[W];
+    #pragma unroll
+    for (int i = 0; i < W; i++) w[i] = src[i];
+    aspen_hip_layer_t L;
+    __builtin_memcpy (&L, w, sizeof (aspen_hip_layer_t));
+    return L;
+}
+// uniform_layer does the same for a descriptor the compiler already holds (a kernel argument).
+__device__ __forceinline__ aspen_hip_layer_t uniform_layer (const aspen_hip_layer_t &Lg)
+{
+    constexpr int W = sizeof (aspen_hip_layer_t) / 4;
     uint32_t w[W];
     __builtin_memcpy (w, &Lg, sizeof (aspen_hip_layer_t));
     #pragma unroll
@@ -1361,24 +1386,26 @@ __device__ __forceinline__ bool splitk_arrived_last (uint32_t *counter, uint32_t
 
 // Split-K reduction of output tile t of the layer as a tile of its own (launch-per-layer mode).
 template <int COH>
-__device__ __forceinline__ void finish_tile (const aspen_hip_layer_t &Lg, uint32_t t)
+__device__ __forceinline__ void finish_tile (const aspen_hip_layer_t &L, uint32_t t)
 {
-    const aspen_hip_layer_t L = uniform_layer (Lg);
     t = __builtin_amdgcn_readfirstlane (t);
     const uint32_t tn = fast_div (t, L.div_tiles_m);
     tile_splitk_finish<COH> (L, tn, t - tn * L.tiles_m);
 }
 
-// Runs tile t of the layer.  `arrivals ()` yields the graph's array of zero-initialised counters, one per
+// Runs tile t of the layer.  `descriptor ()` yields a wave-uniform copy of the layer's descriptor (scalar_layer /
+// uniform_layer); a contraction tile asks for it a second time behind its K loop, so that what only the
+// epilogue needs does not occupy scalar registers while the loop runs.  `arrivals ()` yields the graph's array of zero-initialised counters, one per
 // tile (used at the index of a split-K group's first tile); it is a callable so that the pointer is
 // fetched where it is needed instead of occupying registers while the tile runs.  Returns false for
 // a split-K partial tile that was not the last of its group to finish: the output tile is not
 // complete yet and nothing may be released.
-template <int COH, class Arrivals>
-__device__ __forceinline__ bool run_tile (const aspen_hip_layer_t &Lg, uint32_t t, float *smem, Arrivals arrivals)
+template <int COH, class Descriptor, class Arrivals>
+__device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, bool t_counts_from_graph_start, float *smem, Arrivals arrivals)
 {
-    const aspen_hip_layer_t L = uniform_layer (Lg);
+    const aspen_hip_layer_t L = descriptor ();
     t = __builtin_amdgcn_readfirstlane (t);
+    if (t_counts_from_graph_start) t -= L.ninst_start;
     int slice = -1;
     uint32_t group = 0;
     if (L.splits > 1)
@@ -1396,11 +1423,12 @@ __device__ __forceinline__ bool run_tile (const aspen_hip_layer_t &Lg, uint32_t 
         uint32_t c4_log2, bn;
         shortcut_prefetch_t pre;
         pre.have = pre.have_shortcut = false;
-        if (L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, VAR0_DEPTH, COH> (L, tn, tm, slice, smem, pre); c4_log2 = 5; bn = VAR0_BN; }
-        else if (L.variant == ASPEN_HIP_GEMM_WIDE) { contraction_mainloop<VAR1_BM, VAR1_BN, 2, 2, VAR1_DEPTH, COH> (L, tn, tm, slice, smem, pre); c4_log2 = 4; bn = VAR1_BN; }
-        else { contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, VAR2_DEPTH, COH> (L, tn, tm, slice, smem, pre); c4_log2 = 4; bn = VAR2_BN; }
+        if (L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, VAR0_DEPTH, COH> (L, descriptor, tn, tm, slice, smem, pre); c4_log2 = 5; bn = VAR0_BN; }
+        else if (L.variant == ASPEN_HIP_GEMM_WIDE) { contraction_mainloop<VAR1_BM, VAR1_BN, 2, 2, VAR1_DEPTH, COH> (L, descriptor, tn, tm, slice, smem, pre); c4_log2 = 4; bn = VAR1_BN; }
+        else { contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, VAR2_DEPTH, COH> (L, descriptor, tn, tm, slice, smem, pre); c4_log2 = 4; bn = VAR2_BN; }
         
-        if (slice < 0) contraction_epilogue<COH> (L, tn, tm, smem, c4_log2, bn, pre);
+        const aspen_hip_layer_t E = descriptor ();
+        if (slice < 0) contraction_epilogue<COH> (E, tn, tm, smem, c4_log2, bn, pre);
         if (COH) tile_phase_lap (10);
         if (slice >= 0)
         {
@@ -1408,8 +1436,8 @@ __device__ __forceinline__ bool run_tile (const aspen_hip_layer_t &Lg, uint32_t 
             // counters (one launch per layer: stores of a launch are not visible across XCDs before it ends)
             // the sums are added up by a second launch, see finish_tile.
             uint32_t *counters = arrivals ();
-            if (counters == nullptr || !splitk_arrived_last (counters + group, L.splits, smem)) { if (COH) tile_phase_lap (11); return false; }
-            tile_splitk_finish<COH> (L, tn, tm);
+            if (counters == nullptr || !splitk_arrived_last (counters + group, E.splits, smem)) { if (COH) tile_phase_lap (11); return false; }
+            tile_splitk_finish<COH> (E, tn, tm);
             if (COH) tile_phase_lap (11);
         }
         break;
