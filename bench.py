@@ -366,18 +366,23 @@ def main():
         # conv-tile MFMA utilisation and bandwidth of the elementwise tiles, one kernel per layer
         nl = sum(n.num_ldata for _, _, n, _ in nets)
         lms = pool.profile_layers(nl, 5)
-        per_type, base = {}, 0
+        per_type, per_layer, base = {}, [], 0
         for name, _, n, _ in nets:
-            for l in range(n.num_ldata):
-                i = n.info(l)
+            infos = [n.info(l) for l in range(n.num_ldata)]
+            for l, i in enumerate(infos):
                 t = api.LAYER_TYPE_NAMES[i["type"]]
                 d = per_type.setdefault(t, {"ms": 0.0, "flops": 0, "bytes": 0})
                 d["ms"] += float(lms[base + l])
-                d["flops"] += i["flops"] if t in ("conv", "fc", "matmul", "attn_k", "attn_v") else 0
-                if t == "residual":
-                    d["bytes"] += 12 * i["H"] * i["W"]
-                elif t == "layernorm" or t == "softmax":
-                    d["bytes"] += 8 * i["H"] * i["W"]
+                contraction = t in ("conv", "fc", "matmul", "attn_k", "attn_v")
+                d["flops"] += i["flops"] if contraction else 0
+                # algorithmic bytes of a bandwidth tile layer: its output once and each parent's matrix once
+                nbytes = 0
+                if not contraction and t != "input" and i["num_ninst"]:
+                    nbytes = 4 * (i["H"] * i["W"] + sum(infos[p]["H"] * infos[p]["W"] for p in (i["p0"], i["p1"]) if 0 <= p < len(infos)))
+                d["bytes"] += nbytes
+                per_layer.append({"net": name, "layer": l, "type": t, "rows": i["H"], "columns": i["W"], "tiles": i["num_ninst"],
+                                  "splits": i["splits"], "bytes": nbytes, "flops": i["flops"] if contraction else 0,
+                                  "ms": round(float(lms[base + l]), 5)})
             base += n.num_ldata
         for t, d in per_type.items():
             if d["flops"]:
@@ -387,7 +392,7 @@ def main():
                 d["gbs"] = d["bytes"] / max(d["ms"], 1e-9) / 1e6
                 d["hbm_frac"] = d["gbs"] / PEAK_HBM_GBS
         out["layer_profile"] = per_type
-        out["layer_ms"] = [round(float(v), 4) for v in lms]
+        out["layers"] = per_layer
 
     # the graph that was timed must also have computed the right thing: its final layer against the
     # compiled reference's fixture (outside the timed region)
