@@ -359,6 +359,7 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
         s_sched.may_keep = 0;
     }
     __syncthreads ();
+    __builtin_amdgcn_s_setprio (TILE_PRIO);
     const unsigned long long t_begin = wall_clock64 (), c_begin = clock64 ();
     uint32_t id = QUEUE_EMPTY;
     qentry_t rec = 0;

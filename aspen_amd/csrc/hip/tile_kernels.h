@@ -404,6 +404,12 @@ __device__ __forceinline__ void lds_barrier ()
 // waits in registers; 2 = the two slices after it do.  A slice cannot take less than the memory latency
 // divided by DEPTH, and when a compute unit runs fewer workgroups than it could hold (a graph bound by its
 // dependency chains) nothing else hides that latency; the second set costs 4 registers per 32 operand rows.
+// Instruction-arbiter priority of a wavefront everywhere but inside a K loop.  The workgroups of a compute unit share
+// its matrix pipeline; the ones in a K loop can keep it busy by themselves, while a workgroup in a tile's set-up,
+// first operand fetch, epilogue or scheduling step is on the graph's critical path with a handful of instructions:
+// those go first, and the K loops fill every slot they leave.  (The opposite order, K loops first, is slower than
+// no priorities at all.)
+#define TILE_PRIO 2
 struct NoHook { __device__ __forceinline__ void operator() () const {} };
 // `before_last_slice` runs right before the MFMAs of the last K slice: the place to request what the epilogue
 // will need from memory, with the operand registers free and a whole slice of arithmetic to hide the latency.
@@ -465,6 +471,7 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
     if (kiters > DEPTH) { al.load (kbase + DEPTH, areg[0]); bl.load (kbase + DEPTH, breg[0]); }
     lds_barrier ();
     if (phases) tile_phase_lap (8);
+    __builtin_amdgcn_s_setprio (0);
     read_frags (0, 0);
 
     // One K slice per iteration, single LDS stage, software-pipelined by hand:
@@ -532,6 +539,7 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
         if (kk + 1 < KK) __builtin_amdgcn_sched_group_barrier (SG_DS_READ, TM + TN, 0);
         __builtin_amdgcn_sched_group_barrier (SG_MFMA, 2 * TM * TN, 0);
     }
+    __builtin_amdgcn_s_setprio (TILE_PRIO);
     lds_barrier ();          // the caller reuses the stage (epilogue)
 }
 
@@ -573,6 +581,7 @@ __device__ __forceinline__ void gemm_core_single_block (ALoader &al, BLoader &bl
     if (kiters > DEPTH) { al.load (kbase + DEPTH, areg[0]); bl.load (kbase + DEPTH, breg[0]); }
     lds_barrier ();
     if (phases) tile_phase_lap (8);
+    __builtin_amdgcn_s_setprio (0);
     SB; RD (0); RD (1); RD (2); RD (3);
     // `set` (a literal at every call) = the register set that holds slice it + 1
     auto slice = [&] (int it, int set)
@@ -609,6 +618,7 @@ __device__ __forceinline__ void gemm_core_single_block (ALoader &al, BLoader &bl
 #undef RD
 #undef MF
     accs[0][0] = acc;
+    __builtin_amdgcn_s_setprio (TILE_PRIO);
     lds_barrier ();          // the caller reuses the stage (epilogue)
 }
 
