@@ -968,6 +968,34 @@ __device__ __forceinline__ void tile_pool (const aspen_hip_layer_t &L, uint32_t 
             {
                 const int ih = (int)(hh * L.stride + kh) - (int)L.pad;
                 if ((uint32_t)ih >= L.IH) continue;
+                if (span > 4)
+                {
+                    // a wide window (global average pooling): eight positions of the row are requested at once, so that
+                    // their memory latencies overlap; positions outside the window or the image are fetched from a
+                    // clamped, valid address and not used.  Same order of additions as the plain loop below.
+                    const uint32_t row = (bb * L.IH + ih) * L.IW;
+                    for (uint32_t kw0 = 0; kw0 < span; kw0 += 8)
+                    {
+                        float4 x[8];
+                        #pragma unroll
+                        for (uint32_t q = 0; q < 8; q++)
+                        {
+                            const int iw = (int)(ww * L.stride + kw0 + q) - (int)L.pad;
+                            const uint32_t iwc = (uint32_t)min (max (iw, 0), (int)L.IW - 1);
+                            x[q] = in.ld4 ((row + iwc) * L.ld0 + m);
+                        }
+                        #pragma unroll
+                        for (uint32_t q = 0; q < 8; q++)
+                        {
+                            const uint32_t kw = kw0 + q;
+                            const int iw = (int)(ww * L.stride + kw) - (int)L.pad;
+                            if (kw >= span || (uint32_t)iw >= L.IW) continue;
+                            if (kw < L.KW) combine (ra, x[q]);
+                            if (same_row && kw >= L.stride) combine (rb, x[q]);
+                        }
+                    }
+                    continue;
+                }
                 for (uint32_t kw = 0; kw < span; kw++)
                 {
                     const int iw = (int)(ww * L.stride + kw) - (int)L.pad;
