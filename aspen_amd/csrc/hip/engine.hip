@@ -15,13 +15,22 @@
 
 #define QUEUE_EMPTY 0xffffffffu
 typedef unsigned long long qentry_t;      // ready-queue entry / child-record entry, see arm_kernel
-#define ST_HEAD 0
-#define ST_TAIL 32
 #define ST_DONE 64
 #define ST_ABORT 96
 #define ST_TWICE 128
 #define ST_SINKS 160
-#define ST_WORDS 192
+// Up to one ready queue per XCD (NUM_QUEUES = 8), chosen per run (ASPEN_HIP_FLAG_XCD_QUEUES); by default all tiles go
+// through queue 0.  With XCD queues workgroup b, which the dispatcher places on XCD b % 8, serves queue b % 8, and a
+// tile's home queue is the eighth of its layer's tile range it lies in, i.e. a fixed eighth of the layer's columns for
+// all but the smallest layers.  Tiles that read the same activations (neighbouring output positions, the row tiles and
+// split-K slices of one column block, a tile and the tile below it) then run on one XCD and find them in its L2 instead
+// of fetching them over the fabric once per XCD: ResNet-50 batch 32 reads 4.9 instead of 8.7 GB per inference.  It is
+// not the default because a free workgroup can no longer take a ready tile of another XCD: the same run is 3 % slower
+// (transformer graphs, whose layers have fewer tiles than there are workgroups, 6-11 %).
+#define NUM_QUEUES 8u
+#define ST_QHEAD(q) (192u + 64u * (q))      // pop tickets of queue q
+#define ST_QTAIL(q) (224u + 64u * (q))      // push cursor of queue q
+#define ST_WORDS (192u + 64u * NUM_QUEUES)
 #define NUM_EVENTS 16
 #define DEFAULT_SPIN_LIMIT (1ull << 26)
 
@@ -31,10 +40,14 @@ struct aspen_hip_graph_t
     aspen_hip_layer_t *h_layers;
     aspen_hip_layer_t *d_layers;
     uint32_t *d_ninst_layer, *d_num_parents, *d_child_off, *d_child_idx, *d_roots;
+    uint32_t *d_ninst_home;         // per tile: its home queue (0 .. NUM_QUEUES - 1)
+    uint32_t *d_root_pos;           // per root: its position among the roots of its home queue
+    uint32_t root_count[NUM_QUEUES];
+    uint32_t queue_row, queue_cap;  // see queue_slot
     uint32_t *d_dep;        // remaining-parent counters, re-armed before every dataflow run
     qentry_t *d_queue;      // ready queue: slot t is written once, by whoever makes a tile ready
     qentry_t *d_child_rec;  // per tile: child count + its first CHILD_REC-1 children with their layers
-    uint32_t *d_state;      // one counter per 128-byte line: [ST_HEAD] pop tickets, [ST_TAIL] push cursor, [ST_DONE] tiles done,
+    uint32_t *d_state;      // one counter per 128-byte line: [ST_QHEAD (q)] pop tickets, [ST_QTAIL (q)] push cursor of queue q, [ST_DONE] tiles done,
                             // [ST_ABORT] abort flag, [ST_TWICE] tiles executed more than once, [ST_SINKS] finished tiles without children
     uint32_t *d_ran;        // per-tile execution count (sanity: every tile exactly once)
     uint32_t *d_arrivals;   // split-K arrival counters, see run_tile
@@ -86,9 +99,9 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) finish_kernel (const a
     finish_tile<0> (L, blockIdx.x);
 }
 
-// Re-arm: counters back to the parent counts, queue seeded with the roots.  A queue entry is 64 bits:
-// tile [31:0], layer [47:32], the run's epoch [63:56].  An entry left over from an earlier run never
-// matches the current epoch, so the queue needs no clearing and a poll can never mistake an old
+// Re-arm: counters back to the parent counts, queues seeded with the roots.  A queue entry is 64 bits:
+// tile [31:0], layer [47:32], the run's epoch [63:56] (a child record's entries carry the child's home queue in [55:48]).  An entry left over from an earlier run never
+// matches the current epoch, so the queues need no clearing and a poll can never mistake an old
 // entry for a new one; carrying the layer saves the consumer a dependent lookup.  All writes are
 // device-scope (write-through) stores, the same path the persistent kernel's polls and atomics use.
 #define QUEUE_ID_BITS 24
@@ -98,21 +111,30 @@ __device__ __forceinline__ qentry_t make_entry (uint32_t epoch, uint32_t layer, 
 {
     return ((qentry_t)epoch << 56) | ((qentry_t)layer << 32) | tile;
 }
-// Ticket t lives in queue entry (t % QUEUE_LANES) * row + t / QUEUE_LANES, row >= QUEUE_MIN_ROW entries:
-// the workgroups that wait hold consecutive tickets and each polls its entry, so neighbouring tickets
+// Ticket t of a queue lives in that queue's entry (t % QUEUE_LANES) * row + t / QUEUE_LANES, row >= QUEUE_MIN_ROW
+// entries: the workgroups that wait hold consecutive tickets and each polls its entry, so neighbouring tickets
 // are placed at least 4 KiB apart and the polls spread over all memory channels instead of
-// hammering the one or two that would hold a dense array's next few lines.
-#define QUEUE_LANES 1024u
+// hammering the one or two that would hold a dense array's next few lines.  Queue q starts QUEUE_LANES * row entries
+// behind queue q - 1.
+#define QUEUE_LANES 128u
 #define QUEUE_MIN_ROW 512u
-__device__ __forceinline__ size_t queue_slot (uint32_t ticket, uint32_t row) { return (size_t)(ticket % QUEUE_LANES) * row + ticket / QUEUE_LANES; }
-static uint32_t queue_row (uint32_t num_ninst)
+#define QUEUE_SLACK 8192u       // tickets beyond a queue's tiles: one "leave" entry per workgroup that may still wait
+__device__ __forceinline__ size_t queue_slot (uint32_t q, uint32_t ticket, uint32_t row)
 {
-    const uint32_t r = (num_ninst + QUEUE_LANES) / QUEUE_LANES;
+    return ((size_t)q * QUEUE_LANES + ticket % QUEUE_LANES) * row + ticket / QUEUE_LANES;
+}
+static uint32_t queue_row (uint32_t capacity)
+{
+    const uint32_t r = (capacity + QUEUE_LANES) / QUEUE_LANES;
     return r < QUEUE_MIN_ROW ? QUEUE_MIN_ROW : r;
 }
 
+struct queue_counts_t { uint32_t n[NUM_QUEUES]; };
+
+// nq_mask = number of queues in use - 1 (7 or 0); root_pos / counts describe the 8-queue seeding
 __global__ void arm_kernel (uint32_t *dep, const uint32_t *num_parents, qentry_t *queue, uint32_t *ran,
-    const uint32_t *roots, const uint32_t *ninst_layer, uint32_t num_ninst, uint32_t num_roots, uint32_t *state, uint32_t epoch, uint32_t qrow,
+    const uint32_t *roots, const uint32_t *ninst_layer, const uint32_t *ninst_home, const uint32_t *root_pos, queue_counts_t counts,
+    uint32_t num_ninst, uint32_t num_roots, uint32_t *state, uint32_t epoch, uint32_t qrow, uint32_t nq_mask,
     uint32_t *arrivals)
 {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -120,14 +142,20 @@ __global__ void arm_kernel (uint32_t *dep, const uint32_t *num_parents, qentry_t
     {
         __hip_atomic_store (&dep[i], num_parents[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (i < num_roots)
-            __hip_atomic_store (&queue[queue_slot (i, qrow)], make_entry (epoch, ninst_layer[roots[i]], roots[i]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        {
+            const uint32_t r = roots[i], q = ninst_home[r] & nq_mask, pos = nq_mask ? root_pos[i] : i;
+            __hip_atomic_store (&queue[queue_slot (q, pos, qrow)], make_entry (epoch, ninst_layer[r], r), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
         __hip_atomic_store (&ran[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store (&arrivals[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    if (i < NUM_QUEUES)
+    {
+        __hip_atomic_store (&state[ST_QHEAD (i)], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store (&state[ST_QTAIL (i)], nq_mask ? counts.n[i] : (i == 0 ? num_roots : 0u), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     if (i == 0)
     {
-        __hip_atomic_store (&state[ST_HEAD], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store (&state[ST_TAIL], num_roots, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store (&state[ST_DONE], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store (&state[ST_ABORT], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store (&state[ST_TWICE], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -138,8 +166,8 @@ __global__ void arm_kernel (uint32_t *dep, const uint32_t *num_parents, qentry_t
 struct dataflow_args_t
 {
     const aspen_hip_layer_t *layers;
-    const uint32_t *ninst_layer, *child_off, *child_idx;
-    const qentry_t *child_rec;      // [num_ninst][CHILD_REC]: [0] = number of children, then the first CHILD_REC-1 as (layer << 32 | tile)
+    const uint32_t *ninst_layer, *ninst_home, *child_off, *child_idx;
+    const qentry_t *child_rec;      // [num_ninst][CHILD_REC]: [0] = number of children, then the first CHILD_REC-1 as (home << 48 | layer << 32 | tile)
     qentry_t *queue;
     uint32_t *dep, *state, *ran;
     uint32_t *arrivals;             // per split-K group (at its first tile's index): slices that have finished, see run_tile
@@ -151,6 +179,8 @@ struct dataflow_args_t
     uint32_t epoch;                 // 1..255, tag of this run's queue entries
     uint32_t flags;                 // ASPEN_HIP_FLAG_*
     uint32_t queue_row;             // see queue_slot
+    uint32_t queue_cap;             // tickets a queue can hold
+    uint32_t nq_mask;               // queues in use - 1: NUM_QUEUES - 1, or 0 when the grid is not a multiple of NUM_QUEUES
     unsigned long long spin_limit;
 };
 
@@ -162,13 +192,13 @@ struct dataflow_args_t
 // workgroup that finishes the run's last tile writes it to the slots that will never be served, see
 // schedule_step.  The wait polls with relaxed device-scope loads (an
 // acquire here would invalidate this XCD's L2 on every poll).
-__device__ __forceinline__ qentry_t wait_for_slot (const dataflow_args_t &a, uint32_t ticket)
+__device__ __forceinline__ qentry_t wait_for_slot (const dataflow_args_t &a, uint32_t q, uint32_t ticket)
 {
-    if (ticket >= a.num_ninst) return QENTRY_EMPTY;
+    if (ticket >= a.queue_cap) return QENTRY_EMPTY;
     unsigned long long spins = 0;
     for (;;)
     {
-        const qentry_t e = __hip_atomic_load (&a.queue[queue_slot (ticket, a.queue_row)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const qentry_t e = __hip_atomic_load (&a.queue[queue_slot (q, ticket, a.queue_row)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if ((uint32_t)(e >> 56) == a.epoch) return e;
         ++spins;
         if ((spins & 63) == 0 && __hip_atomic_load (&a.state[ST_ABORT], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return QENTRY_EMPTY;
@@ -190,6 +220,7 @@ struct sched_lds_t
     uint32_t tile, layer;                // tile to run next (QUEUE_EMPTY: leave) and its layer
     uint32_t complete;                   // 0: the tile just run was a split-K slice that did not finish its group
     uint32_t may_keep;                   // the tile just run releases children, one of which this workgroup may run next
+    uint32_t my_queue;                   // the ready queue this workgroup serves
     unsigned long long t0, ticks[6];     // profiling: last time stamp; tile / drain / scheduling / publish / ticket / slot-wait ticks
     unsigned long long p0, phase[5];     // profiling of contraction tiles: last phase stamp; set-up / K loop / epilogue / split-K ticks
 };
@@ -214,10 +245,10 @@ __device__ void tile_phase_lap (int which)
 }
 
 // Puts a tile that has become ready into the queue.
-__device__ __forceinline__ void push_ready (const dataflow_args_t &a, uint32_t child, uint32_t layer)
+__device__ __forceinline__ void push_ready (const dataflow_args_t &a, uint32_t child, uint32_t layer, uint32_t home)
 {
-    const uint32_t slot = atomicAdd (&a.state[ST_TAIL], 1u);
-    __hip_atomic_store (&a.queue[queue_slot (slot, a.queue_row)], make_entry (a.epoch, layer, child), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t q = home & a.nq_mask, slot = atomicAdd (&a.state[ST_QTAIL (q)], 1u);
+    __hip_atomic_store (&a.queue[queue_slot (q, slot, a.queue_row)], make_entry (a.epoch, layer, child), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // One scheduling step of a workgroup, as a real function call (it needs few registers, all of them
@@ -251,9 +282,9 @@ __device__ __forceinline__ void pop_next (const dataflow_args_t &a, uint32_t lan
             // atomic's round trip but binds a (possibly already ready) tile to a busy workgroup while idle
             // ones wait on later slots.
             const unsigned long long t1 = prof ? wall_clock64 () : 0;
-            const uint32_t ticket = atomicAdd (&a.state[ST_HEAD], 1u);
+            const uint32_t q = s_sched.my_queue, ticket = atomicAdd (&a.state[ST_QHEAD (q)], 1u);
             const unsigned long long t2 = prof ? wall_clock64 () : 0;
-            const qentry_t e = wait_for_slot (a, ticket);
+            const qentry_t e = wait_for_slot (a, q, ticket);
             s_sched.tile = e == QENTRY_EMPTY ? QUEUE_EMPTY : (uint32_t)e;
             s_sched.layer = (uint32_t)(e >> 32) & 0xffffu;
             if (prof) { s_sched.ticks[4] += t2 - t1; s_sched.ticks[5] += wall_clock64 () - t2; }
@@ -287,13 +318,14 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
         uint32_t kept = QUEUE_EMPTY, kept_layer = 0;
         // a split-K slice that was not the last of its group leaves the children to the one that is
         const uint32_t listed = (uint32_t)__shfl (rec, 0, 64), count = s_sched.complete ? listed : 0u;
-        const uint32_t child = (uint32_t)rec, layer = (uint32_t)(rec >> 32);
+        const uint32_t child = (uint32_t)rec, layer = (uint32_t)(rec >> 32) & 0xffffu, home = (uint32_t)(rec >> 48) & 0xffu;
         bool ready = false;
         if (lane >= 1 && lane <= count)
             ready = __hip_atomic_fetch_sub (&a.dep[child], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 1u;
         if (may_keep)
         {
-            const unsigned long long made_ready = __ballot (ready);
+            // only a child at home in this workgroup's queue is kept
+            const unsigned long long made_ready = __ballot (ready && (home & a.nq_mask) == s_sched.my_queue);
             if (made_ready)
             {
                 const int keeper = __builtin_ctzll (made_ready);
@@ -302,7 +334,7 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
                 ready = ready && (int)lane != keeper;
             }
         }
-        if (ready) push_ready (a, child, layer);
+        if (ready) push_ready (a, child, layer, home);
         if (count > CHILD_REC - 1)
         {
             // more children than the record holds: the rest comes from the CSR lists and goes through the queue
@@ -310,7 +342,7 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
             for (uint32_t c = c0 + lane; c < c1; c += 64)
             {
                 const uint32_t ch = a.child_idx[c];
-                if (__hip_atomic_fetch_sub (&a.dep[ch], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 1u) push_ready (a, ch, a.ninst_layer[ch]);
+                if (__hip_atomic_fetch_sub (&a.dep[ch], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 1u) push_ready (a, ch, a.ninst_layer[ch], a.ninst_home[ch]);
             }
         }
         if (listed == 0u)
@@ -322,9 +354,12 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
             {
                 // the run is over and nothing will be pushed any more: tell everyone who waits, this workgroup's
                 // own popping wavefront included
-                const uint32_t tail = __hip_atomic_load (&a.state[ST_TAIL], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                for (uint32_t t = tail + lane; t < tail + gridDim.x && t < a.num_ninst; t += 64)
-                    __hip_atomic_store (&a.queue[queue_slot (t, a.queue_row)], make_entry (a.epoch, 0, QUEUE_EMPTY), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (uint32_t q = 0; q <= a.nq_mask; q++)
+                {
+                    const uint32_t tail = __hip_atomic_load (&a.state[ST_QTAIL (q)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    for (uint32_t t = tail + lane; t < tail + gridDim.x && t < a.queue_cap; t += 64)
+                        __hip_atomic_store (&a.queue[queue_slot (q, t, a.queue_row)], make_entry (a.epoch, 0, QUEUE_EMPTY), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
             }
         }
         if (lane == 0 && (a.flags & ASPEN_HIP_FLAG_COUNT_TILES))
@@ -357,6 +392,7 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
         for (int i = 0; i < 6; i++) s_sched.ticks[i] = 0;
         for (int i = 0; i < 5; i++) s_sched.phase[i] = 0;
         s_sched.may_keep = 0;
+        s_sched.my_queue = blockIdx.x & args.nq_mask;
     }
     __syncthreads ();
     __builtin_amdgcn_s_setprio (TILE_PRIO);
@@ -836,19 +872,40 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     g->d_child_idx = upload (child_idx, num_edges);
     g->d_roots = upload (roots, num_roots);
     g->d_dep = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
-    g->d_queue = (qentry_t *)aspen_hip_alloc (sizeof (qentry_t) * (size_t)QUEUE_LANES * queue_row (num_ninst));
+    g->queue_cap = num_ninst + QUEUE_SLACK;
+    g->queue_row = queue_row (g->queue_cap);
+    g->d_queue = (qentry_t *)aspen_hip_alloc (sizeof (qentry_t) * (size_t)NUM_QUEUES * QUEUE_LANES * g->queue_row);
     {
+        // home queues: the eighth of its layer's tile range a tile lies in (tiles are numbered column tile by column
+        // tile, the row tiles and split-K slices of a column tile next to each other)
+        uint32_t *home = (uint32_t *)malloc (sizeof (uint32_t) * (num_ninst ? num_ninst : 1));
+        uint32_t *pos = (uint32_t *)malloc (sizeof (uint32_t) * (num_roots ? num_roots : 1));
         // child records: what the publishing wavefront fetches with one 64-lane load
         qentry_t *rec = (qentry_t *)calloc ((size_t)(num_ninst ? num_ninst : 1) * CHILD_REC, sizeof (qentry_t));
-        for (uint32_t t = 0; rec && t < num_ninst; t++)
+        if (home && pos && rec)
         {
-            const uint32_t c0 = child_off[t], n = child_off[t + 1] - c0;
-            rec[(size_t)t * CHILD_REC] = n;
-            for (uint32_t c = 0; c < n && c < CHILD_REC - 1; c++)
-                rec[(size_t)t * CHILD_REC + 1 + c] = ((qentry_t)ninst_layer[child_idx[c0 + c]] << 32) | child_idx[c0 + c];
+            for (uint32_t t = 0; t < num_ninst; t++)
+            {
+                const aspen_hip_layer_t &L = layers[ninst_layer[t]];
+                const uint64_t in_layer = t >= L.ninst_start ? t - L.ninst_start : 0;
+                home[t] = L.num_ninst ? (uint32_t)(in_layer * NUM_QUEUES / L.num_ninst) % NUM_QUEUES : 0u;
+            }
+            for (uint32_t r = 0; r < num_roots; r++) pos[r] = g->root_count[home[roots[r]]]++;
+            for (uint32_t t = 0; t < num_ninst; t++)
+            {
+                const uint32_t c0 = child_off[t], n = child_off[t + 1] - c0;
+                rec[(size_t)t * CHILD_REC] = n;
+                for (uint32_t c = 0; c < n && c < CHILD_REC - 1; c++)
+                {
+                    const uint32_t ch = child_idx[c0 + c];
+                    rec[(size_t)t * CHILD_REC + 1 + c] = ((qentry_t)home[ch] << 48) | ((qentry_t)ninst_layer[ch] << 32) | ch;
+                }
+            }
+            g->d_ninst_home = upload (home, num_ninst);
+            g->d_root_pos = upload (pos, num_roots);
+            g->d_child_rec = upload (rec, (size_t)num_ninst * CHILD_REC);
         }
-        g->d_child_rec = rec ? upload (rec, (size_t)num_ninst * CHILD_REC) : nullptr;
-        free (rec);
+        free (home); free (pos); free (rec);
     }
     g->d_ran = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
     g->d_state = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * ST_WORDS);
@@ -857,7 +914,7 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     if (hipHostMalloc ((void **)&g->h_abort, 64, hipHostMallocDefault) != hipSuccess) g->h_abort = nullptr;
     else *g->h_abort = 0;
     if (!g->h_abort || !g->d_layers || !g->d_ninst_layer || !g->d_num_parents || !g->d_child_off || !g->d_child_idx || !g->d_roots
-        || !g->d_dep || !g->d_queue || !g->d_ran || !g->d_state || !g->d_child_rec || !g->d_arrivals || !g->d_prof)
+        || !g->d_dep || !g->d_queue || !g->d_ran || !g->d_state || !g->d_child_rec || !g->d_ninst_home || !g->d_root_pos || !g->d_arrivals || !g->d_prof)
     {
         aspen_hip_graph_destroy (g);
         return nullptr;
@@ -870,7 +927,7 @@ extern "C" void aspen_hip_graph_destroy (aspen_hip_graph_t *g)
     if (!g) return;
     (void)hipStreamSynchronize (g_stream);
     aspen_hip_free (g->d_layers); aspen_hip_free (g->d_ninst_layer); aspen_hip_free (g->d_num_parents);
-    aspen_hip_free (g->d_child_off); aspen_hip_free (g->d_child_idx); aspen_hip_free (g->d_roots);
+    aspen_hip_free (g->d_child_off); aspen_hip_free (g->d_child_idx); aspen_hip_free (g->d_roots); aspen_hip_free (g->d_ninst_home); aspen_hip_free (g->d_root_pos);
     aspen_hip_free (g->d_child_rec); aspen_hip_free (g->d_dep); aspen_hip_free (g->d_queue); aspen_hip_free (g->d_ran); aspen_hip_free (g->d_arrivals); aspen_hip_free (g->d_state); aspen_hip_free (g->d_prof); aspen_hip_free (g->d_trace);
     if (g->h_abort) (void)hipHostFree (g->h_abort);
     free (g->h_layers);
@@ -909,12 +966,20 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     if (!g) { snprintf (g_err, sizeof (g_err), "run_dataflow: null graph"); return -1; }
     if (g->num_ninst == 0) return 0;
     if (workgroups == 0) workgroups = g->default_workgroups;
+    if (workgroups > QUEUE_SLACK) workgroups = QUEUE_SLACK;         // every waiting workgroup must find a "leave" entry within its queue
     g->epoch = g->epoch % 255u + 1u;
+    // one queue per XCD on request, when every XCD gets the same number of workgroups (workgroup b runs on XCD b % 8)
+    static const bool xcd_queues_env = getenv ("ASPEN_GPU_XCD_QUEUES") != nullptr;
+    const bool xcd_queues = xcd_queues_env || (g_flags & ASPEN_HIP_FLAG_XCD_QUEUES);
+    const uint32_t nq_mask = (xcd_queues && workgroups % NUM_QUEUES == 0) ? NUM_QUEUES - 1u : 0u;
+    queue_counts_t counts;
+    for (uint32_t q = 0; q < NUM_QUEUES; q++) counts.n[q] = g->root_count[q];
     hipLaunchKernelGGL (arm_kernel, dim3 ((g->num_ninst + 255) / 256), dim3 (256), 0, g_stream,
-        g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->d_ninst_layer, g->num_ninst, g->num_roots, g->d_state, g->epoch, queue_row (g->num_ninst), g->d_arrivals);
+        g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->d_ninst_layer, g->d_ninst_home, g->d_root_pos, counts,
+        g->num_ninst, g->num_roots, g->d_state, g->epoch, g->queue_row, nq_mask, g->d_arrivals);
     CHECK (hipGetLastError ());
     dataflow_args_t a;
-    a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx; a.child_rec = g->d_child_rec;
+    a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.ninst_home = g->d_ninst_home; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx; a.child_rec = g->d_child_rec;
     a.dep = g->d_dep; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran; a.arrivals = g->d_arrivals; a.prof = g->d_prof; a.host_abort = g->h_abort;
     if ((g_flags & ASPEN_HIP_FLAG_TRACE) && !g->d_trace)
     {
@@ -922,7 +987,7 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
         if (!g->d_trace) return -1;
     }
     a.trace = g->d_trace;
-    a.num_ninst = g->num_ninst; a.num_sinks = g->num_sinks; a.epoch = g->epoch; a.flags = g_flags; a.queue_row = queue_row (g->num_ninst); a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
+    a.num_ninst = g->num_ninst; a.num_sinks = g->num_sinks; a.epoch = g->epoch; a.flags = g_flags; a.queue_row = g->queue_row; a.queue_cap = g->queue_cap; a.nq_mask = nq_mask; a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
     CHECK (hipEventRecord (g_events[NUM_EVENTS - 2], g_stream));
     if (g->cached_loads) hipLaunchKernelGGL (dataflow_kernel<2>, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);
     else hipLaunchKernelGGL (dataflow_kernel<1>, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);

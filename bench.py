@@ -218,6 +218,7 @@ def main():
                     help="skip the `workloads` section (the other benchmark configurations, measured after the headline one)")
     ap.add_argument("--skip-tiles", action="store_true", help="scheduler-only run: dependency protocol with empty tiles")
     ap.add_argument("--no-handoff", action="store_true", help="every ready tile goes through the queue (no parent -> child hand-off)")
+    ap.add_argument("--xcd-queues", action="store_true", help="one ready queue per XCD, tiles at home on a fixed eighth of the columns (less memory traffic, less balance)")
     ap.add_argument("--engine-profile", action="store_true", help="report where the persistent workgroups spend their time")
     ap.add_argument("--trace", default="", metavar="NPZ", help="write per-tile start/end stamps of the last timed step (dataflow mode)")
     ap.add_argument("--layer-profile", action="store_true", help="also time every layer's kernel (layer-launch mode)")
@@ -252,7 +253,7 @@ def main():
                           "ms_per_launch": ms.value / args.steps,
                           "GB_per_s": 2 * nbytes * args.steps / (ms.value * 1e-3) / 1e9}))
         return
-    L.aspen_hip_set_flags((1 if args.skip_tiles else 0) | (4 if args.engine_profile else 0) | (8 if args.trace else 0) | (16 if args.no_handoff else 0))
+    L.aspen_hip_set_flags((1 if args.skip_tiles else 0) | (4 if args.engine_profile else 0) | (8 if args.trace else 0) | (16 if args.no_handoff else 0) | (32 if args.xcd_queues else 0))
     cfgs, unit, units_per_step, tuned_min_ninst, tuned_engine = WORKLOADS[args.workload]
     if args.min_ninst <= 0:
         args.min_ninst = tuned_min_ninst
@@ -413,7 +414,7 @@ def main():
     del nets
 
     # the other configurations of the benchmark, each on its own tuned graph (value stays the headline workload's)
-    plain = not (args.skip_tiles or args.engine_profile or args.trace or args.layer_profile or args.no_handoff)
+    plain = not (args.skip_tiles or args.engine_profile or args.trace or args.layer_profile or args.no_handoff or args.xcd_queues)
     if not args.no_other_workloads and plain and args.workload == "resnet50_b32":
         L.aspen_hip_set_flags(0)
         out["workloads"] = {}

@@ -598,17 +598,31 @@ def test_reference_main_call_sequence(gpu, tmp_path):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name,min_ninst,workgroups", [("resnet_mini_b2", 1024, 0), ("gpt_mini_b2_s20", 64, 16), ("yolo_mini_b2", 16, 0),
-                                                      ("resnet50_b1", 128, 0), ("bert_base_b8_s128", 192, 0)])
-def test_no_tile_starts_before_its_parents_have_ended(gpu, name, min_ninst, workgroups):
+@pytest.mark.parametrize("name,min_ninst,workgroups,flags", [("resnet_mini_b2", 1024, 0, 0), ("gpt_mini_b2_s20", 64, 16, 0), ("yolo_mini_b2", 16, 0, 0),
+                                                            ("resnet50_b1", 128, 0, 0), ("bert_base_b8_s128", 192, 0, 0),
+                                                            ("resnet_mini_b2", 1024, 0, 32), ("gpt_mini_b2_s20", 64, 16, 32),
+                                                            ("resnet50_b1", 128, 0, 32), ("resnet_mini_b2", 1024, 0, 16)],
+                         ids=lambda v: str(v))
+def test_no_tile_starts_before_its_parents_have_ended(gpu, name, min_ninst, workgroups, flags):
     """The scheduler's invariant (reference src/dse.c:32-38, 311-317: a ninst runs only once all its parents are
     completed), checked from the per-tile start / end stamps of a traced run of the persistent kernel: along
     every dependency edge the child's start stamp is not earlier than the parent's end stamp, which is taken
     after the parent's stores were acknowledged.  The members of a split-K group release their children
-    together, through whichever member finishes last: a child waits for the group's last end."""
+    together, through whichever member finishes last: a child waits for the group's last end.
+    flags: 0 = the default engine, 32 = one ready queue per XCD, 16 = no parent -> child hand-off; the final layer must
+    come out bit-identical to the default engine's in every variant (tiles do the same arithmetic wherever they run)."""
     micro = name in H.micro_cases()
     cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()[name]) if micro else H.full_config(name)
-    api.lib().aspen_hip_set_flags(2 | 8)
+    expected = None
+    if flags:
+        api.lib().aspen_hip_set_flags(2)
+        plain = H.GpuNet(cfg, tens, batch, seq, min_ninst=min_ninst, mode=api.MODE_DATAFLOW, workgroups=workgroups)
+        try:
+            plain.run(x)
+            expected = plain.nasm.layer_output(plain.nasm.num_ldata - 1).copy()
+        finally:
+            plain.close()
+    api.lib().aspen_hip_set_flags(2 | 8 | flags)
     net = H.GpuNet(cfg, tens, batch, seq, min_ninst=min_ninst, mode=api.MODE_DATAFLOW, workgroups=workgroups)
     try:
         for rep in range(2):                                     # also on a re-armed graph
@@ -633,6 +647,8 @@ def test_no_tile_starts_before_its_parents_have_ended(gpu, name, min_ninst, work
                                      f"{parent_of_edge[early][0]} -> child {child_idx[early][0]}")
             # roots start without waiting, everything else after at least one parent
             assert (num_parents[child_idx] > 0).all()
+            if expected is not None:
+                assert np.array_equal(net.nasm.layer_output(net.nasm.num_ldata - 1), expected)
             print(f"{name} run {rep}: {len(child_idx)} edges hold, {grouped} split-K layers", flush=True)
     finally:
         api.lib().aspen_hip_set_flags(2)
