@@ -43,6 +43,7 @@ struct aspen_hip_graph_t
     uint32_t *d_ninst_home;         // per tile: its home queue (0 .. NUM_QUEUES - 1)
     uint32_t *d_root_pos;           // per root: its position among the roots of its home queue
     uint32_t root_count[NUM_QUEUES];
+    uint32_t root_shift;            // the XCD grouping (see nq_shift) d_root_pos / root_count were computed for
     uint32_t queue_row, queue_cap;  // see queue_slot
     uint32_t *d_dep;        // remaining-parent counters, re-armed before every dataflow run
     qentry_t *d_queue;      // ready queue: slot t is written once, by whoever makes a tile ready
@@ -134,7 +135,7 @@ struct queue_counts_t { uint32_t n[NUM_QUEUES]; };
 // nq_mask = number of queues in use - 1 (7 or 0); root_pos / counts describe the 8-queue seeding
 __global__ void arm_kernel (uint32_t *dep, const uint32_t *num_parents, qentry_t *queue, uint32_t *ran,
     const uint32_t *roots, const uint32_t *ninst_layer, const uint32_t *ninst_home, const uint32_t *root_pos, queue_counts_t counts,
-    uint32_t num_ninst, uint32_t num_roots, uint32_t *state, uint32_t epoch, uint32_t qrow, uint32_t nq_mask,
+    uint32_t num_ninst, uint32_t num_roots, uint32_t *state, uint32_t epoch, uint32_t qrow, uint32_t nq_mask, uint32_t nq_shift,
     uint32_t *arrivals)
 {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -143,7 +144,7 @@ __global__ void arm_kernel (uint32_t *dep, const uint32_t *num_parents, qentry_t
         __hip_atomic_store (&dep[i], num_parents[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (i < num_roots)
         {
-            const uint32_t r = roots[i], q = ninst_home[r] & nq_mask, pos = nq_mask ? root_pos[i] : i;
+            const uint32_t r = roots[i], q = (ninst_home[r] >> nq_shift) & nq_mask, pos = nq_mask ? root_pos[i] : i;
             __hip_atomic_store (&queue[queue_slot (q, pos, qrow)], make_entry (epoch, ninst_layer[r], r), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         __hip_atomic_store (&ran[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -181,6 +182,7 @@ struct dataflow_args_t
     uint32_t queue_row;             // see queue_slot
     uint32_t queue_cap;             // tickets a queue can hold
     uint32_t nq_mask;               // queues in use - 1: NUM_QUEUES - 1, or 0 when the grid is not a multiple of NUM_QUEUES
+    uint32_t nq_shift;              // XCDs per queue, as a power of two
     unsigned long long spin_limit;
 };
 
@@ -247,7 +249,7 @@ __device__ void tile_phase_lap (int which)
 // Puts a tile that has become ready into the queue.
 __device__ __forceinline__ void push_ready (const dataflow_args_t &a, uint32_t child, uint32_t layer, uint32_t home)
 {
-    const uint32_t q = home & a.nq_mask, slot = atomicAdd (&a.state[ST_QTAIL (q)], 1u);
+    const uint32_t q = (home >> a.nq_shift) & a.nq_mask, slot = atomicAdd (&a.state[ST_QTAIL (q)], 1u);
     __hip_atomic_store (&a.queue[queue_slot (q, slot, a.queue_row)], make_entry (a.epoch, layer, child), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
@@ -325,7 +327,7 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
         if (may_keep)
         {
             // only a child at home in this workgroup's queue is kept
-            const unsigned long long made_ready = __ballot (ready && (home & a.nq_mask) == s_sched.my_queue);
+            const unsigned long long made_ready = __ballot (ready && ((home >> a.nq_shift) & a.nq_mask) == s_sched.my_queue);
             if (made_ready)
             {
                 const int keeper = __builtin_ctzll (made_ready);
@@ -392,7 +394,7 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
         for (int i = 0; i < 6; i++) s_sched.ticks[i] = 0;
         for (int i = 0; i < 5; i++) s_sched.phase[i] = 0;
         s_sched.may_keep = 0;
-        s_sched.my_queue = blockIdx.x & args.nq_mask;
+        s_sched.my_queue = ((blockIdx.x & (NUM_QUEUES - 1u)) >> args.nq_shift) & args.nq_mask;
     }
     __syncthreads ();
     __builtin_amdgcn_s_setprio (TILE_PRIO);
@@ -971,12 +973,27 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     // one queue per XCD on request, when every XCD gets the same number of workgroups (workgroup b runs on XCD b % 8)
     static const bool xcd_queues_env = getenv ("ASPEN_GPU_XCD_QUEUES") != nullptr;
     const bool xcd_queues = xcd_queues_env || (g_flags & ASPEN_HIP_FLAG_XCD_QUEUES);
-    const uint32_t nq_mask = (xcd_queues && workgroups % NUM_QUEUES == 0) ? NUM_QUEUES - 1u : 0u;
+    static const uint32_t shift_env = getenv ("ASPEN_GPU_XCD_QUEUE_SHIFT") ? (uint32_t)atoi (getenv ("ASPEN_GPU_XCD_QUEUE_SHIFT")) : 0u;
+    const uint32_t nq_shift = shift_env > 2u ? 2u : shift_env;
+    const uint32_t nq_mask = (xcd_queues && workgroups % NUM_QUEUES == 0) ? (NUM_QUEUES >> nq_shift) - 1u : 0u;
     queue_counts_t counts;
+    if (nq_mask && g->root_shift != nq_shift)
+    {
+        // positions of the roots inside their queues for this grouping of the XCDs
+        uint32_t *home = (uint32_t *)malloc (sizeof (uint32_t) * g->num_ninst), *roots = (uint32_t *)malloc (sizeof (uint32_t) * g->num_roots), *pos = (uint32_t *)malloc (sizeof (uint32_t) * g->num_roots);
+        if (!home || !roots || !pos || aspen_hip_sync () || aspen_hip_d2h (home, g->d_ninst_home, sizeof (uint32_t) * g->num_ninst) || aspen_hip_d2h (roots, g->d_roots, sizeof (uint32_t) * g->num_roots))
+        { free (home); free (roots); free (pos); snprintf (g_err, sizeof (g_err), "run_dataflow: cannot regroup the roots"); return -1; }
+        memset (g->root_count, 0, sizeof (g->root_count));
+        for (uint32_t r = 0; r < g->num_roots; r++) pos[r] = g->root_count[(home[roots[r]] >> nq_shift) & nq_mask]++;
+        const int failed = aspen_hip_h2d (g->d_root_pos, pos, sizeof (uint32_t) * g->num_roots);
+        free (home); free (roots); free (pos);
+        if (failed) return -1;
+        g->root_shift = nq_shift;
+    }
     for (uint32_t q = 0; q < NUM_QUEUES; q++) counts.n[q] = g->root_count[q];
     hipLaunchKernelGGL (arm_kernel, dim3 ((g->num_ninst + 255) / 256), dim3 (256), 0, g_stream,
         g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->d_ninst_layer, g->d_ninst_home, g->d_root_pos, counts,
-        g->num_ninst, g->num_roots, g->d_state, g->epoch, g->queue_row, nq_mask, g->d_arrivals);
+        g->num_ninst, g->num_roots, g->d_state, g->epoch, g->queue_row, nq_mask, nq_shift, g->d_arrivals);
     CHECK (hipGetLastError ());
     dataflow_args_t a;
     a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.ninst_home = g->d_ninst_home; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx; a.child_rec = g->d_child_rec;
@@ -987,7 +1004,7 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
         if (!g->d_trace) return -1;
     }
     a.trace = g->d_trace;
-    a.num_ninst = g->num_ninst; a.num_sinks = g->num_sinks; a.epoch = g->epoch; a.flags = g_flags; a.queue_row = g->queue_row; a.queue_cap = g->queue_cap; a.nq_mask = nq_mask; a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
+    a.num_ninst = g->num_ninst; a.num_sinks = g->num_sinks; a.epoch = g->epoch; a.flags = g_flags; a.queue_row = g->queue_row; a.queue_cap = g->queue_cap; a.nq_mask = nq_mask; a.nq_shift = nq_shift; a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
     CHECK (hipEventRecord (g_events[NUM_EVENTS - 2], g_stream));
     if (g->cached_loads) hipLaunchKernelGGL (dataflow_kernel<2>, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);
     else hipLaunchKernelGGL (dataflow_kernel<1>, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);

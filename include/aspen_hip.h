@@ -175,7 +175,8 @@ int aspen_hip_dataflow_profile (aspen_hip_graph_t *graph, uint64_t ticks[16], in
 /* XCD_QUEUES gives every XCD a ready queue of its own and every tile a home XCD (a fixed eighth of its layer's
    columns), so that tiles reading the same activations share an L2: about 40 % less memory traffic on the
    convolutional networks, but free workgroups cannot help another XCD and runs take 0-11 % longer.  Also switched on
-   by ASPEN_GPU_XCD_QUEUES in the environment.  Needs a grid that is a multiple of 8 workgroups (else ignored). */
+   by ASPEN_GPU_XCD_QUEUES in the environment; ASPEN_GPU_XCD_QUEUE_SHIFT = 1 / 2 groups the XCDs in pairs / fours (4 / 2
+   queues).  Needs a grid that is a multiple of 8 workgroups (else ignored). */
 #define ASPEN_HIP_FLAG_XCD_QUEUES 32u
 int aspen_hip_dataflow_trace (aspen_hip_graph_t *graph, uint64_t *start_end, uint32_t num_ninst);
 void aspen_hip_set_flags (uint32_t flags);
