@@ -832,7 +832,8 @@ __device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L
                 if (fuse) fused_shortcut<COH> (L, fin, fout, v, n0 + r, m0 + c, mrem - c);
             }
     }
-    __syncthreads ();
+    // no barrier here: whatever runs next on this workgroup (the scheduling step of the persistent kernel) passes
+    // one before LDS is written again
 }
 
 // split-K, run by the slice that finishes last: sum of the slices (in slice order, whoever runs it) + bias, activation
