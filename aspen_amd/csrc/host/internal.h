@@ -89,6 +89,7 @@ struct nasm_t
     unsigned int batch_size, tr_seq_len, min_ninst_per_ldata;
     int preferred_mode;                      /* engine mode the timing tuner found fastest for this graph (0 / 1), -1: not tuned */
     unsigned int kiters_cap;                 /* 0, or the longest K loop (in slices of 32) a contraction tile may have, see create_nasm */
+    int small_tiles_only;                    /* every contraction layer uses the small tile shape, see create_nasm */
     nasm_ldata_t *ldata_arr;
     unsigned int num_ldata;
     unsigned int num_ninst;

@@ -112,6 +112,7 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
            shape when it would leave the layer with fewer tiles than wanted */
         int v = M <= 64 ? ASPEN_HIP_GEMM_WIDE : ASPEN_HIP_GEMM_LARGE;
         if (cdiv (M, bm[v]) * cdiv (N, bn[v]) < want || (N <= 64 && v == ASPEN_HIP_GEMM_WIDE)) v = ASPEN_HIP_GEMM_SMALL;
+        if (nasm->small_tiles_only) v = ASPEN_HIP_GEMM_SMALL;      /* graphs bound by their dependency chains, see create_nasm */
         ld->variant = v;
         ld->tile_dims[OUT_H] = bm[v]; ld->tile_dims[OUT_W] = bn[v];
     }
@@ -453,13 +454,14 @@ static void fuse_shortcuts (nasm_t *nasm)
     }
 }
 
-static nasm_t *build_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned int batch, unsigned int seq, unsigned int kiters_cap)
+static nasm_t *build_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned int batch, unsigned int seq, unsigned int kiters_cap, int small_tiles_only)
 {
     if (dnn == NULL) { ERROR_PRTF ("apu_create_nasm: dnn is NULL\n"); return NULL; }
     if (min_ninst < 1) { ERROR_PRTF ("ERROR: min_ninst_per_ldata should be at least 1\n"); return NULL; }
     nasm_t *nasm = calloc (1, sizeof (nasm_t));
     if (nasm == NULL) { ERROR_PRTF ("apu_create_nasm: out of host memory\n"); return NULL; }
     nasm->kiters_cap = kiters_cap;
+    nasm->small_tiles_only = small_tiles_only;
     nasm->preferred_mode = -1;
     nasm->dnn = dnn; nasm->nasm_id = nasm_counter++;
     nasm->batch_size = batch > 0 ? batch : 1;
@@ -538,22 +540,29 @@ static double nasm_parallelism (const nasm_t *nasm)
 }
 
 /* A graph that offers less parallelism than a 256-CU device has resident workgroups is bound by its
-   dependency chains, not by throughput: workgroups idle while the longest tiles of each stage finish
-   (BERT / GPT-2 with one or two thousand tokens: FFN tiles of 48-96 K slices).  Such a graph is rebuilt
-   with no tile longer than 48 K slices (more split-K): GPT-2 -6 %, BERT -3 %.  Throughput-bound graphs
-   (batch-32 vision nets) lose 2-3 % with the same cap (more partial sums to move) and keep long tiles. */
+   dependency chains, not by throughput: it runs on one or two workgroups per compute unit, and those idle while
+   the longest tiles of each stage finish (BERT / GPT-2 with one or two thousand tokens).  Such a graph is rebuilt
+   - with the small tile shape for every contraction layer: more and shorter tiles fill the rounds of a small grid
+     better than few long ones (the FFN layers of BERT as 768 tiles instead of 384: GPT-2 -2 %, BERT -0.5 %);
+   - if it still offers work for a second workgroup per compute unit, with no tile longer than 48 K slices (more
+     split-K): GPT-2 (average parallelism 529) -6 %.  With a single workgroup per compute unit the extra tiles only
+     queue up behind the others: BERT (265) is 2 % faster without the cap.
+   Throughput-bound graphs (batch-32 vision nets) lose 2-3 % with either and keep their large, long tiles. */
 #define CHAIN_BOUND_BELOW 1024.0
+#define CHAIN_BOUND_CAP_FROM 400.0
 #define CHAIN_BOUND_KITERS_CAP 48
 static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned int batch, unsigned int seq)
 {
     const char *e = getenv ("ASPEN_GPU_MAX_KITERS");            /* experiments: fixed cap, 0 = none */
-    if (e != NULL) return build_nasm (dnn, min_ninst, batch, seq, (unsigned int)atoi (e));
-    nasm_t *nasm = build_nasm (dnn, min_ninst, batch, seq, 0);
-    if (nasm == NULL || nasm_parallelism (nasm) >= CHAIN_BOUND_BELOW) return nasm;
-    nasm_t *capped = build_nasm (dnn, min_ninst, batch, seq, CHAIN_BOUND_KITERS_CAP);
-    if (capped == NULL) return nasm;
+    if (e != NULL) return build_nasm (dnn, min_ninst, batch, seq, (unsigned int)atoi (e), getenv ("ASPEN_GPU_SMALL_TILES") != NULL);
+    nasm_t *nasm = build_nasm (dnn, min_ninst, batch, seq, 0, 0);
+    if (nasm == NULL) return nasm;
+    const double parallelism = nasm_parallelism (nasm);
+    if (parallelism >= CHAIN_BOUND_BELOW) return nasm;
+    nasm_t *rebuilt = build_nasm (dnn, min_ninst, batch, seq, parallelism >= CHAIN_BOUND_CAP_FROM ? CHAIN_BOUND_KITERS_CAP : 0, 1);
+    if (rebuilt == NULL) return nasm;
     apu_destroy_nasm (nasm);
-    return capped;
+    return rebuilt;
 }
 
 nasm_t *apu_create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst_per_ldata, unsigned int batch_size)
