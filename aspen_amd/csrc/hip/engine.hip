@@ -53,6 +53,7 @@ struct aspen_hip_graph_t
     uint32_t *d_ran;        // per-tile execution count (sanity: every tile exactly once)
     uint32_t *d_arrivals;   // split-K arrival counters, see run_tile
     uint32_t num_sinks;     // tiles without children
+    unsigned features;      // TILES_* bits of the tile kinds the graph contains: picks the persistent kernel's variant
     uint32_t epoch;         // tag of the last run's queue entries, cycles 1..255
     unsigned long long *d_prof;
     uint32_t default_workgroups;    // grid of a dataflow run when the caller names none, see graph_parallelism
@@ -383,7 +384,7 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
 // No cache write-back / invalidate is needed anywhere: tiles store activations with device-scope
 // write-through instructions and load them either coherently (COH = 1) or, when the host has checked
 // that no cache line is shared between producer tiles, through the caches (COH = 2); see ActView.
-template <int COH>
+template <int COH, unsigned FEAT>
 __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataflow_args_t args)
 {
     extern __shared__ __align__ (16) float smem[];
@@ -416,7 +417,7 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
         const auto descriptor = [] () { return scalar_layer (s_sched.a.layers + s_sched.layer); };
         bool complete;
         if (!(s_sched.a.flags & ASPEN_HIP_FLAG_SKIP_TILES))
-            complete = run_tile<COH> (descriptor, id, true, smem, [] () { return s_sched.a.arrivals; });
+            complete = run_tile<COH, FEAT> (descriptor, id, true, smem, [] () { return s_sched.a.arrivals; });
         else
         {
             // scheduler-only run: the split-K groups still elect the member that releases the children
@@ -439,6 +440,40 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
 
 __global__ void sgemm_kernel (const aspen_hip_layer_t L);       // defined with aspen_hip_sgemm_static
 
+// The persistent kernel's variants, smallest first: [variant][0] coherent loads, [1] cached loads.  A graph runs on the
+// first variant that has all its tile kinds, see graph_features.
+#define NUM_KERNEL_VARIANTS 3
+static const unsigned kernel_variant_tiles[NUM_KERNEL_VARIANTS] = {TILES_TRANSFORMER, TILES_CONVNET, TILES_ALL};
+static const void *const dataflow_kernels[NUM_KERNEL_VARIANTS][2] = {
+    {(const void *)dataflow_kernel<1, TILES_TRANSFORMER>, (const void *)dataflow_kernel<2, TILES_TRANSFORMER>},
+    {(const void *)dataflow_kernel<1, TILES_CONVNET>, (const void *)dataflow_kernel<2, TILES_CONVNET>},
+    {(const void *)dataflow_kernel<1, TILES_ALL>, (const void *)dataflow_kernel<2, TILES_ALL>}};
+
+// The tile kinds a graph contains, as TILES_* bits.
+static unsigned graph_features (const aspen_hip_layer_t *layers, uint32_t num_layers)
+{
+    unsigned f = 0;
+    for (uint32_t l = 0; l < num_layers; l++)
+    {
+        const aspen_hip_layer_t &L = layers[l];
+        if (L.type == INPUT_LAYER || L.num_ninst == 0) continue;
+        switch (L.type)
+        {
+        case CONV_LAYER: case FC_LAYER: case MATMUL_LAYER:
+            f |= L.variant == ASPEN_HIP_GEMM_LARGE ? TILES_LARGE : L.variant == ASPEN_HIP_GEMM_WIDE ? TILES_WIDE : TILES_SMALL;
+            if (!L.direct) f |= TILES_GATHER;
+            break;
+        case K_ATTENTION_LAYER: case V_ATTENTION_LAYER: f |= TILES_ATTENTION; break;
+        case LAYERNORM_LAYER: case SOFTMAX_LAYER: f |= TILES_NORM; break;
+        case MAXPOOL_LAYER: case AVGPOOL_LAYER: f |= TILES_POOL; break;
+        case YOLO_LAYER: case APPEND_LAYER: f |= TILES_YOLO; break;
+        case RESIDUAL_LAYER: f |= TILES_RESIDUAL; break;
+        default: f |= TILES_ALL; break;
+        }
+    }
+    return f;
+}
+
 // ------------------------------------------------------------------------------------------------
 // device, memory
 // ------------------------------------------------------------------------------------------------
@@ -456,12 +491,13 @@ extern "C" int aspen_hip_init (void)
     for (int i = 0; i < NUM_EVENTS; i++) CHECK (hipEventCreate (&g_events[i]));
     CHECK (hipFuncSetAttribute ((const void *)layer_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
     CHECK (hipFuncSetAttribute ((const void *)sgemm_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
-    CHECK (hipFuncSetAttribute ((const void *)dataflow_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
-    CHECK (hipFuncSetAttribute ((const void *)dataflow_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
+    for (int v = 0; v < NUM_KERNEL_VARIANTS; v++)
+        for (int coh = 0; coh < 2; coh++)
+            CHECK (hipFuncSetAttribute (dataflow_kernels[v][coh], hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
     // how many persistent workgroups really fit a compute unit (registers, LDS): the default grid
     int occ1 = 0, occ2 = 0;
-    CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&occ1, dataflow_kernel<1>, WG_THREADS, GEMM_SMEM_BYTES));
-    CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&occ2, dataflow_kernel<2>, WG_THREADS, GEMM_SMEM_BYTES));
+    CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&occ1, dataflow_kernel<1, TILES_ALL>, WG_THREADS, GEMM_SMEM_BYTES));
+    CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&occ2, dataflow_kernel<2, TILES_ALL>, WG_THREADS, GEMM_SMEM_BYTES));
     g_resident_wg = occ1 < occ2 ? occ1 : occ2;
     if (g_resident_wg < 1) g_resident_wg = 1;
     if (getenv ("ASPEN_GPU_VERBOSE")) fprintf (stderr, "aspen_hip: %d resident dataflow workgroups per compute unit (built for %d)\n", g_resident_wg, WG_PER_CU);
@@ -849,6 +885,7 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     if (!g) { snprintf (g_err, sizeof (g_err), "out of host memory"); return nullptr; }
     g->cached_loads = lines_have_one_producer (layers, num_layers) && getenv ("ASPEN_GPU_COHERENT_LOADS") == nullptr;
     g->num_layers = num_layers; g->num_ninst = num_ninst; g->num_roots = num_roots; g->num_edges = num_edges;
+    g->features = graph_features (layers, num_layers);
     for (uint32_t t = 0; t < num_ninst; t++) g->num_sinks += child_off[t + 1] == child_off[t];
     {
         // default grid: a whole number of workgroups per compute unit, no more than the graph can keep busy
@@ -1006,8 +1043,13 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     a.trace = g->d_trace;
     a.num_ninst = g->num_ninst; a.num_sinks = g->num_sinks; a.epoch = g->epoch; a.flags = g_flags; a.queue_row = g->queue_row; a.queue_cap = g->queue_cap; a.nq_mask = nq_mask; a.nq_shift = nq_shift; a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
     CHECK (hipEventRecord (g_events[NUM_EVENTS - 2], g_stream));
-    if (g->cached_loads) hipLaunchKernelGGL (dataflow_kernel<2>, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);
-    else hipLaunchKernelGGL (dataflow_kernel<1>, dim3 (workgroups), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, a);
+    {
+        static const bool all_tiles = getenv ("ASPEN_GPU_ONE_KERNEL") != nullptr;       // comparisons: always the variant with every tile kind
+        int v = NUM_KERNEL_VARIANTS - 1;
+        for (int i = NUM_KERNEL_VARIANTS - 2; i >= 0 && !all_tiles; i--) if ((g->features & ~kernel_variant_tiles[i]) == 0) v = i;
+        void *kernel_args[] = {&a};
+        CHECK (hipLaunchKernel (dataflow_kernels[v][g->cached_loads ? 1 : 0], dim3 (workgroups), dim3 (WG_THREADS), kernel_args, GEMM_SMEM_BYTES, g_stream));
+    }
     CHECK (hipGetLastError ());
     CHECK (hipEventRecord (g_events[NUM_EVENTS - 1], g_stream));
     return 0;

@@ -411,6 +411,20 @@ __device__ __forceinline__ void lds_barrier ()
 // no priorities at all.)
 #define TILE_PRIO 2
 struct NoHook { __device__ __forceinline__ void operator() () const {} };
+
+// What a kernel that runs tiles is compiled for.  The persistent kernel exists in a few variants that leave out the
+// tile kinds a graph does not contain: four workgroups in different phases share a compute unit's 64 KB instruction
+// cache, and a transformer graph has no use for the convolution loaders' K loops, nor a ResNet for the attention tiles.
+enum : unsigned
+{
+    TILES_GATHER = 1u,          // contraction operands gathered through ConvLoader (convolutions, FC layers over images)
+    TILES_LARGE = 2u, TILES_WIDE = 4u, TILES_SMALL = 8u,       // contraction tile shapes
+    TILES_ATTENTION = 16u, TILES_NORM = 32u /* layernorm, softmax */, TILES_POOL = 64u, TILES_YOLO = 128u /* yolo, append */,
+    TILES_RESIDUAL = 256u,
+    TILES_ALL = 511u,
+    TILES_CONVNET = TILES_GATHER | TILES_LARGE | TILES_WIDE | TILES_SMALL | TILES_POOL | TILES_RESIDUAL,
+    TILES_TRANSFORMER = TILES_SMALL | TILES_ATTENTION | TILES_NORM | TILES_RESIDUAL
+};
 // `before_last_slice` runs right before the MFMAs of the last K slice: the place to request what the epilogue
 // will need from memory, with the operand registers free and a whole slice of arithmetic to hide the latency.
 template <int BM, int BN, int WM, int WN, int DEPTH, class ALoader, class BLoader, class Hook = NoHook>
@@ -657,7 +671,7 @@ __device__ __forceinline__ void fused_shortcut (const aspen_hip_layer_t &L, cons
 // of the thread's pieces of a fused shortcut's operand (a tile has at most 128 columns: 8 pieces per thread)
 struct shortcut_prefetch_t { float4 s[8]; float4 bias; bool have, have_shortcut; };
 
-template <int BM, int BN, int WM, int WN, int DEPTH, int COH, class Descriptor>
+template <int BM, int BN, int WM, int WN, int DEPTH, int COH, unsigned FEAT, class Descriptor>
 __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L, Descriptor descriptor, uint32_t tn, uint32_t tm, int slice, float *smem, shortcut_prefetch_t &pre)
 {
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
@@ -703,7 +717,7 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
         if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
         else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
     }
-    else
+    else if constexpr ((FEAT & TILES_GATHER) != 0)
     {
         ConvLoader<BN, COH> bl;
         bl.init (L, in, n0, tid);
@@ -1439,7 +1453,7 @@ __device__ __forceinline__ void finish_tile (const aspen_hip_layer_t &L, uint32_
 // fetched where it is needed instead of occupying registers while the tile runs.  Returns false for
 // a split-K partial tile that was not the last of its group to finish: the output tile is not
 // complete yet and nothing may be released.
-template <int COH, class Descriptor, class Arrivals>
+template <int COH, unsigned FEAT = TILES_ALL, class Descriptor, class Arrivals>
 __device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, bool t_counts_from_graph_start, float *smem, Arrivals arrivals)
 {
     const aspen_hip_layer_t L = descriptor ();
@@ -1462,9 +1476,10 @@ __device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, boo
         uint32_t c4_log2, bn;
         shortcut_prefetch_t pre;
         pre.have = pre.have_shortcut = false;
-        if (L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, VAR0_DEPTH, COH> (L, descriptor, tn, tm, slice, smem, pre); c4_log2 = 5; bn = VAR0_BN; }
-        else if (L.variant == ASPEN_HIP_GEMM_WIDE) { contraction_mainloop<VAR1_BM, VAR1_BN, 2, 2, VAR1_DEPTH, COH> (L, descriptor, tn, tm, slice, smem, pre); c4_log2 = 4; bn = VAR1_BN; }
-        else { contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, VAR2_DEPTH, COH> (L, descriptor, tn, tm, slice, smem, pre); c4_log2 = 4; bn = VAR2_BN; }
+        c4_log2 = 4; bn = VAR2_BN;
+        if ((FEAT & TILES_LARGE) && L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, VAR0_DEPTH, COH, FEAT> (L, descriptor, tn, tm, slice, smem, pre); c4_log2 = 5; bn = VAR0_BN; }
+        else if ((FEAT & TILES_WIDE) && L.variant == ASPEN_HIP_GEMM_WIDE) { contraction_mainloop<VAR1_BM, VAR1_BN, 2, 2, VAR1_DEPTH, COH, FEAT> (L, descriptor, tn, tm, slice, smem, pre); bn = VAR1_BN; }
+        else if (FEAT & TILES_SMALL) contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, VAR2_DEPTH, COH, FEAT> (L, descriptor, tn, tm, slice, smem, pre);
         
         const aspen_hip_layer_t E = descriptor ();
         if (slice < 0) contraction_epilogue<COH> (E, tn, tm, smem, c4_log2, bn, pre);
@@ -1481,15 +1496,15 @@ __device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, boo
         }
         break;
     }
-    case RESIDUAL_LAYER:    tile_residual<COH> (L, tn); break;
-    case MAXPOOL_LAYER:     tile_pool<true, COH> (L, tn, tm); break;
-    case AVGPOOL_LAYER:     tile_pool<false, COH> (L, tn, tm); break;
-    case YOLO_LAYER:        tile_yolo<COH> (L, tn); break;
-    case APPEND_LAYER:      tile_append<COH> (L, tn); break;
-    case LAYERNORM_LAYER:   tile_layernorm<COH> (L, tn); break;
-    case SOFTMAX_LAYER:     tile_softmax<COH> (L, tn); break;
-    case K_ATTENTION_LAYER: tile_k_attention<COH> (L, tn, smem); break;
-    case V_ATTENTION_LAYER: tile_v_attention<COH> (L, tn, tm, smem); break;
+    case RESIDUAL_LAYER:    if constexpr ((FEAT & TILES_RESIDUAL) != 0) tile_residual<COH> (L, tn); break;
+    case MAXPOOL_LAYER:     if constexpr ((FEAT & TILES_POOL) != 0) tile_pool<true, COH> (L, tn, tm); break;
+    case AVGPOOL_LAYER:     if constexpr ((FEAT & TILES_POOL) != 0) tile_pool<false, COH> (L, tn, tm); break;
+    case YOLO_LAYER:        if constexpr ((FEAT & TILES_YOLO) != 0) tile_yolo<COH> (L, tn); break;
+    case APPEND_LAYER:      if constexpr ((FEAT & TILES_YOLO) != 0) tile_append<COH> (L, tn); break;
+    case LAYERNORM_LAYER:   if constexpr ((FEAT & TILES_NORM) != 0) tile_layernorm<COH> (L, tn); break;
+    case SOFTMAX_LAYER:     if constexpr ((FEAT & TILES_NORM) != 0) tile_softmax<COH> (L, tn); break;
+    case K_ATTENTION_LAYER: if constexpr ((FEAT & TILES_ATTENTION) != 0) tile_k_attention<COH> (L, tn, smem); break;
+    case V_ATTENTION_LAYER: if constexpr ((FEAT & TILES_ATTENTION) != 0) tile_v_attention<COH> (L, tn, tm, smem); break;
     default: break;
     }
     return true;
