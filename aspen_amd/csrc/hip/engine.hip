@@ -442,11 +442,12 @@ __global__ void sgemm_kernel (const aspen_hip_layer_t L);       // defined with 
 
 // The persistent kernel's variants, smallest first: [variant][0] coherent loads, [1] cached loads.  A graph runs on the
 // first variant that has all its tile kinds, see graph_features.
-#define NUM_KERNEL_VARIANTS 3
-static const unsigned kernel_variant_tiles[NUM_KERNEL_VARIANTS] = {TILES_TRANSFORMER, TILES_CONVNET, TILES_ALL};
+#define NUM_KERNEL_VARIANTS 4
+static const unsigned kernel_variant_tiles[NUM_KERNEL_VARIANTS] = {TILES_TRANSFORMER, TILES_CONVNET, TILES_CONVNET | TILES_YOLO, TILES_ALL};
 static const void *const dataflow_kernels[NUM_KERNEL_VARIANTS][2] = {
     {(const void *)dataflow_kernel<1, TILES_TRANSFORMER>, (const void *)dataflow_kernel<2, TILES_TRANSFORMER>},
     {(const void *)dataflow_kernel<1, TILES_CONVNET>, (const void *)dataflow_kernel<2, TILES_CONVNET>},
+    {(const void *)dataflow_kernel<1, TILES_CONVNET | TILES_YOLO>, (const void *)dataflow_kernel<2, TILES_CONVNET | TILES_YOLO>},
     {(const void *)dataflow_kernel<1, TILES_ALL>, (const void *)dataflow_kernel<2, TILES_ALL>}};
 
 // The tile kinds a graph contains, as TILES_* bits.
@@ -461,7 +462,7 @@ static unsigned graph_features (const aspen_hip_layer_t *layers, uint32_t num_la
         {
         case CONV_LAYER: case FC_LAYER: case MATMUL_LAYER:
             f |= L.variant == ASPEN_HIP_GEMM_LARGE ? TILES_LARGE : L.variant == ASPEN_HIP_GEMM_WIDE ? TILES_WIDE : TILES_SMALL;
-            if (!L.direct) f |= TILES_GATHER;
+            if (L.direct != ASPEN_HIP_OPERAND_DIRECT) f |= TILES_GATHER;
             break;
         case K_ATTENTION_LAYER: case V_ATTENTION_LAYER: f |= TILES_ATTENTION; break;
         case LAYERNORM_LAYER: case SOFTMAX_LAYER: f |= TILES_NORM; break;
@@ -742,9 +743,11 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
         else if (L.Kp == 0 || L.Kp % GEMM_BK) why = "Kp must be a positive multiple of 32";
         else if (L.tile_m != bm || L.tile_n != bn) why = "tile extent does not match the GEMM variant";
         else if ((uint64_t)L.tiles_m * bm < L.M || (uint64_t)L.tiles_n * bn < L.N) why = "tile grid does not cover the matrix";
-        else if (!L.direct && !L.ktab) why = "missing k-chunk table";
+        else if (L.direct != ASPEN_HIP_OPERAND_DIRECT && !L.ktab) why = "missing k-chunk table";
         else if (L.fuse_out && (!L.fuse_in || L.fuse_ld_in % 4 || L.fuse_ld_in < L.M)) why = "fused shortcut operand";
-        else if (L.direct && (L.ld0 < L.Kp)) why = "direct operand shorter than Kp";
+        else if (L.direct == ASPEN_HIP_OPERAND_DIRECT && (L.ld0 < L.Kp)) why = "direct operand shorter than Kp";
+        else if (L.direct == ASPEN_HIP_OPERAND_DENSE3 && (L.IC != 3 || L.Kp > 512 || L.Kp < 3 * L.KH * L.KW || L.ld0 < 4 || bm != 64)) why = "dense three-channel operand";
+        else if (L.direct < 0 || L.direct > ASPEN_HIP_OPERAND_DENSE3) why = "operand kind";
     }
     else if (L.type == K_ATTENTION_LAYER)
     {

@@ -336,6 +336,61 @@ template <int ROWS, int COH> struct ConvLoader
     }
 };
 
+// Implicit-GEMM operand of a convolution over THREE input channels (a network's first layer on RGB images) with a
+// dense K axis: K order (tap, channel) without the padding to four channels per tap that ConvLoader's layout has
+// (ASPEN_HIP_OPERAND_DENSE3; the stem of ResNet-50 contracts 160 instead of 224, VGG-16's first layer 32 instead of
+// 64).  A chunk of four K positions spans two pixels: both are fetched (16 bytes each, the pixels of the matrix keep
+// their padded fourth float) and the chunk is put together from the last channels of the first and the first
+// channels of the second; chunk index % 3 says how many of each.  A loader of its own so that ConvLoader's code, which
+// every other convolution runs, stays as it is.
+template <int ROWS, int COH> struct Dense3Loader
+{
+    static constexpr int R = ROWS / 32;
+    ActView<COH> in;
+    const aspen_hip_ktab_t *ktab;
+    int32_t base[R], ih0[R], iw0[R];
+    uint32_t IH, IW, chunk, row0;
+    __device__ __forceinline__ void init (const aspen_hip_layer_t &L, const ActView<COH> &v, uint32_t first_row, uint32_t tid)
+    {
+        in = v; ktab = L.ktab; IH = L.IH; IW = L.IW;
+        chunk = tid & 7; row0 = tid >> 3;
+        const uint32_t ohw = L.OH * L.OW;
+        #pragma unroll
+        for (int i = 0; i < R; i++)
+        {
+            uint32_t n = first_row + row0 + 32 * i;
+            n = n < L.N ? n : L.N - 1;
+            uint32_t b = fast_div (n, L.div_ohw), rem = n - b * ohw, oh = fast_div (rem, L.div_ow), ow = rem - oh * L.OW;
+            ih0[i] = (int32_t)(oh * L.stride) - (int32_t)L.pad;
+            iw0[i] = (int32_t)(ow * L.stride) - (int32_t)L.pad;
+            base[i] = ((int32_t)(b * L.IH) + ih0[i]) * (int32_t)L.IW * (int32_t)L.ld0 + iw0[i] * (int32_t)L.ld0;
+        }
+    }
+    __device__ __forceinline__ void load (int it, float4 (&v)[R])
+    {
+        typedef unsigned int uintx4 __attribute__ ((ext_vector_type (4)));
+        const uint32_t kc = (uint32_t)it * 8 + chunk, sel = kc - 3 * ((kc * 43u) >> 7);        // kc % 3 for kc < 128
+        const uintx4 raw = *(const uintx4 __attribute__ ((address_space (1))) *)(ktab + 2 * kc);
+        #pragma unroll
+        for (int i = 0; i < R; i++)
+        {
+            const bool oka = (uint32_t)(ih0[i] + (int32_t)(raw[1] & 0xffffu)) < IH && (uint32_t)(iw0[i] + (int32_t)(raw[1] >> 16)) < IW;
+            const bool okb = (uint32_t)(ih0[i] + (int32_t)(raw[3] & 0xffffu)) < IH && (uint32_t)(iw0[i] + (int32_t)(raw[3] >> 16)) < IW;
+            const float4 z = make_float4 (0.f, 0.f, 0.f, 0.f);
+            const float4 a = oka ? in.ld4 ((uint32_t)(base[i] + (int32_t)raw[0])) : z, b = okb ? in.ld4 ((uint32_t)(base[i] + (int32_t)raw[2])) : z;
+            v[i].x = sel == 0 ? a.x : sel == 1 ? a.y : a.z;
+            v[i].y = sel == 0 ? a.y : sel == 1 ? a.z : b.x;
+            v[i].z = sel == 0 ? a.z : sel == 1 ? b.x : b.y;
+            v[i].w = sel == 0 ? b.x : sel == 1 ? b.y : b.z;
+        }
+    }
+    __device__ __forceinline__ void store (float *lds, const float4 (&v)[R])
+    {
+        #pragma unroll
+        for (int i = 0; i < R; i++) st4 (lds + (row0 + 32 * i) * LDS_ROW + chunk * 4, v[i]);
+    }
+};
+
 // K-strided operand (V of attention: rows = channels, K axis = sequence position with stride ld):
 // read 64 channels x 32 positions with 128-bit loads along the channels, transpose into LDS.
 template <int COH> struct TransLoader64
@@ -710,7 +765,7 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
                 if (r0 + u * STEP < rows) pre.s[u] = fin.ld4 ((n0 + r0 + u * STEP) * L.fuse_ld_in + m0 + c);
         }
     };
-    if (L.direct)
+    if (L.direct == ASPEN_HIP_OPERAND_DIRECT)
     {
         ActRowLoader<BN, COH> bl;
         bl.init (in, n0, L.N - 1, L.ld0, 0, tid);
@@ -719,10 +774,21 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
     }
     else if constexpr ((FEAT & TILES_GATHER) != 0)
     {
-        ConvLoader<BN, COH> bl;
-        bl.init (L, in, n0, tid);
-        if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
-        else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
+        // (the dense three-channel layout is only used for layers of up to 64 output channels, see aspen_layer_dense3)
+        if (BM == 64 && L.direct == ASPEN_HIP_OPERAND_DENSE3)
+        {
+            Dense3Loader<BN, COH> bl;
+            bl.init (L, in, n0, tid);
+            if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
+            else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
+        }
+        else
+        {
+            ConvLoader<BN, COH> bl;
+            bl.init (L, in, n0, tid);
+            if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
+            else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
+        }
     }
     if (COH) tile_phase_lap (9);
     const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);

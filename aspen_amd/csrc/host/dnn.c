@@ -281,6 +281,14 @@ done:
 /* ---------------------------------------------------------------------------------------------- */
 static unsigned int round_up (unsigned int v, unsigned int to) { return (v + to - 1) / to * to; }
 
+/* A convolution over three input channels (a network's first layer on RGB images) keeps its K axis dense on the
+   device: K = taps * 3 instead of taps * 4, see ASPEN_HIP_OPERAND_DENSE3.  (The stem of ResNet-50: 160 instead of 224.) */
+int aspen_layer_dense3 (const aspen_layer_t *L)
+{
+    return L->type == CONV_LAYER && L->params[IN_C] == 3 && L->params[WEIGHT_H] * L->params[WEIGHT_W] * 3 <= 508 && L->gemm_m <= 64
+        && getenv ("ASPEN_GPU_NO_DENSE3") == NULL;
+}
+
 /* padded K of the device layout / 32 (must agree with aspen_layer_to_device) */
 unsigned int aspen_layer_kiters (const aspen_layer_t *L)
 {
@@ -290,6 +298,7 @@ unsigned int aspen_layer_kiters (const aspen_layer_t *L)
     else if (L->type == FC_LAYER) { taps = p[IN_H] * p[IN_W]; ic = p[IN_C]; }
     else if (L->type == MATMUL_LAYER) { taps = 1; ic = p[MAT_K]; }
     else return 0;
+    if (aspen_layer_dense3 (L)) return round_up (taps * 3, 32) / 32;
     return round_up (taps * round_up (ic, 4), 32) / 32;
 }
 
@@ -320,7 +329,8 @@ int aspen_layer_to_device (aspen_layer_t *L, unsigned int parent_ld)
     if (L->type == CONV_LAYER) { taps = p[WEIGHT_H] * p[WEIGHT_W]; ic = p[IN_C]; kw_count = p[WEIGHT_W]; in_w = p[IN_W]; }
     else if (L->type == FC_LAYER) { taps = p[IN_H] * p[IN_W]; ic = p[IN_C]; kw_count = p[IN_W]; in_w = p[IN_W]; }
     else { taps = 1; ic = p[MAT_K]; kw_count = 1; in_w = 1; }
-    const unsigned int icp = round_up (ic, 4);
+    const int dense3 = aspen_layer_dense3 (L);
+    const unsigned int icp = dense3 ? 3 : round_up (ic, 4);
     const unsigned int kp = round_up (taps * icp, 32);
     const unsigned int mp = round_up (L->gemm_m, 128);
     float *staged = calloc ((size_t)mp * kp, sizeof (float));
@@ -334,6 +344,28 @@ int aspen_layer_to_device (aspen_layer_t *L, unsigned int parent_ld)
     if (rc) return rc;
     L->d_bias = aspen_hip_alloc (L->gemm_m * sizeof (float));
     if (!L->d_bias || aspen_hip_h2d (L->d_bias, L->bias.data, L->gemm_m * sizeof (float))) return -1;
+    if (dense3)
+    {
+        /* two entries per chunk: K positions [4c, 4c+4) lie in tap 4c / 3 and the tap after it; the entries point at
+           the first channel of the two pixels */
+        aspen_hip_ktab_t *tab2 = calloc (kp / 2, sizeof (aspen_hip_ktab_t));
+        if (tab2 == NULL) return -1;
+        for (unsigned int c = 0; c < kp / 4; c++)
+            for (unsigned int e = 0; e < 2; e++)
+            {
+                const unsigned int tap = (c * 4) / 3 + e;
+                aspen_hip_ktab_t *t = &tab2[2 * c + e];
+                if (tap >= taps) { t->offset = 0; t->kh = 0x4000; t->kw = 0; continue; }
+                const unsigned int kh = tap / kw_count, kw = tap % kw_count;
+                t->offset = (int32_t)((kh * in_w + kw) * parent_ld);
+                t->kh = (uint16_t)kh; t->kw = (uint16_t)kw;
+            }
+        L->d_ktab = aspen_hip_alloc (kp / 2 * sizeof (aspen_hip_ktab_t));
+        rc = L->d_ktab ? aspen_hip_h2d (L->d_ktab, tab2, kp / 2 * sizeof (aspen_hip_ktab_t)) : -1;
+        free (tab2);
+        L->dev_kp = kp; L->dev_icp = icp; L->dev_in_ld = parent_ld;
+        return rc;
+    }
     /* k-chunk table: chunk c covers K positions [4c, 4c+4) = tap (4c / icp), channels (4c % icp).. */
     aspen_hip_ktab_t *tab = calloc (kp / 4, sizeof (aspen_hip_ktab_t));
     if (tab == NULL) return -1;

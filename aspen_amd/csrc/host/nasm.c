@@ -743,6 +743,7 @@ int aspen_nasm_fill_device_layers (nasm_t *nasm, aspen_hip_layer_t *dst, uint32_
                 || (L->type == CONV_LAYER && p[WEIGHT_H] == 1 && p[WEIGHT_W] == 1 && p[STRIDE] == 1 && p[PADDING] == 0)
                 || (L->type == FC_LAYER && p[IN_H] == 1 && p[IN_W] == 1);
             d->direct = pointwise && (d->IC % 32 == 0) && d->ld0 >= d->Kp;
+            if (aspen_layer_dense3 (L)) d->direct = ASPEN_HIP_OPERAND_DENSE3;
         }
         if (ld->fused_residual >= 0)
         {

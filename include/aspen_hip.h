@@ -38,6 +38,13 @@ typedef struct aspen_hip_ktab_t
     uint16_t kh, kw;     /* tap; kh >= 0x4000 marks a chunk beyond the real K (reads as zero) */
 } aspen_hip_ktab_t;
 
+/* aspen_hip_layer_t.direct.  TABLE: K order (tap, channel padded to 4), one table entry per k-chunk.  DIRECT: the
+   parent's columns are the K axis.  DENSE3: a convolution over 3 input channels with K order (tap, channel) and NO
+   padding (weights [roundup(M,128)][Kp], Kp = roundup(3 * taps, 32) <= 512): k-chunk c = K positions 4c .. 4c+3 covers
+   the last 3 - c % 3 channels of tap 4c / 3 and the first c % 3 + 1 of the next tap; the table holds TWO entries per
+   chunk, 2c for the first tap and 2c + 1 for the second, each with the offset of that pixel's channel 0. */
+enum { ASPEN_HIP_OPERAND_TABLE = 0, ASPEN_HIP_OPERAND_DIRECT = 1, ASPEN_HIP_OPERAND_DENSE3 = 2 };
+
 /* GEMM tile shapes (rows of the weight matrix x activation columns per workgroup): LARGE = the
    biggest shape of the build (128 x 64 by default), WIDE = 64 x 128, SMALL = 64 x 64.  The graph
    builder asks aspen_hip_tile_shapes for the numbers instead of assuming them. */
@@ -55,7 +62,8 @@ typedef struct aspen_hip_layer_t
     int32_t type;            /* LAYER_TYPE of aspen.h */
     int32_t act;             /* LAYER_ACT of aspen.h */
     int32_t variant;         /* GEMM tile shape for contraction layers */
-    int32_t direct;          /* 1: B operand is read in place (1x1 stride-1 conv / matmul, K % 32 == 0) */
+    int32_t direct;          /* how the B operand is found, ASPEN_HIP_OPERAND_*: 0 k-chunk table, 1 read in place (1x1 stride-1
+                                conv / matmul, K % 32 == 0), 2 dense three-channel table */
     uint32_t M, N, ld;       /* output rows, columns, stride */
     uint32_t tile_m, tile_n; /* tile extent in rows / columns */
     uint32_t tiles_m, tiles_n;
@@ -78,7 +86,7 @@ typedef struct aspen_hip_layer_t
     const float *in1;        /* PARENT_1 */
     const float *weight;     /* [roundup(M,128)][Kp] row-major, zero padded; layernorm: gamma[M] */
     const float *bias;       /* [M] or NULL */
-    const aspen_hip_ktab_t *ktab; /* Kp/4 entries, NULL when direct */
+    const aspen_hip_ktab_t *ktab; /* Kp/4 entries (Kp/2 for DENSE3), NULL when direct */
     /* fused shortcut (contraction layers; reference tiled_residual, src/tiled_kernels.c:613-638, run in
        the epilogue): besides out = act(...) the tile also writes
        fuse_out = fuse_act (out + fuse_in) at the same rows / columns; fuse_out has stride ld.

@@ -110,6 +110,34 @@ def test_every_activation_and_softmax_match_oracle(gpu, mode):
         net.close()
 
 
+@pytest.mark.parametrize("mode", [api.MODE_LAYERS, api.MODE_DATAFLOW], ids=["layers", "dataflow"])
+@pytest.mark.parametrize("filters,size,stride,pad,min_ninst", [(16, 7, 2, 3, 16), (64, 3, 1, 1, 16), (64, 5, 1, 0, 2048), (96, 3, 2, 1, 16), (8, 1, 1, 0, 16)])
+def test_first_layer_over_three_channels_matches_oracle(gpu, mode, filters, size, stride, pad, min_ninst):
+    """A convolution over three input channels keeps its K axis dense on the device (K = 3 x taps, a chunk of four K
+    positions assembled from two neighbouring pixels) when it has at most 64 output channels, and the padded layout
+    otherwise: window sizes whose 3 x taps is and is not a multiple of 4, strides, padding on all four sides, all
+    three tile shapes (wide, small, split along K), against the oracle's convolution; the layer behind it checks
+    that nothing else of the network noticed."""
+    from oracle import cpu
+    cfg = ("[net]\nheight=19\nwidth=23\nchannels=3\n\n" + f"[convolutional]\nfilters={filters}\nsize={size}\nstride={stride}\npad={pad}\nactivation=leaky\n\n"
+           + "[convolutional]\nfilters=24\nsize=3\nstride=1\npad=1\nactivation=relu\n\n")
+    layers = M.parse_cfg(cfg)
+    tens = M.synth_weights(layers, 31, "he")
+    batch = 5
+    x = (M.synth_input(layers, 31, batch, 0, "token_ids") * 2.0 - 1.0).astype(np.float32)
+    outs = cpu.run_network(layers, tens, x, batch, 0)
+    net = H.GpuNet(cfg, tens, batch, 0, min_ninst=min_ninst, mode=mode)
+    try:
+        net.run(x)
+        dense = filters <= 64
+        assert net.nasm.info(1)["kiters_per_split"] * net.nasm.info(1)["splits"] >= -(-(size * size * (3 if dense else 4)) // 32)
+        for l in range(1, net.nasm.num_ldata):
+            err = H.rel_l2(net.layer(l), outs[l])
+            assert err <= H.REL_L2_TOL, f"layer {l}: rel L2 {err:.3g}"
+    finally:
+        net.close()
+
+
 def test_results_in_the_callers_dimension_order(gpu):
     """dse_get_ldata_result permutes a layer's native tensor into the order the caller names (reference
     get_ldata_output, src/apu.c:227-297): matrices of a transformer are (BATCH, MAT_N, MAT_M), attention

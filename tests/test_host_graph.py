@@ -260,6 +260,21 @@ def test_tile_graph_against_brute_force(name, min_ninst, fuse, monkeypatch):
     n.destroy(); d.destroy()
 
 
+def test_three_channel_first_layer_contracts_a_dense_k_axis():
+    """K slices (of 32) of a network's first convolution: 3 x taps without padding for up to 64 output channels (the
+    7x7 stem: 147 -> 160, five slices), taps x 4 as for every other layer beyond that."""
+    def first_conv_slices(filters, size):
+        cfg = f"[net]\nheight=32\nwidth=32\nchannels=3\n\n[convolutional]\nfilters={filters}\nsize={size}\nstride=1\npad=1\nactivation=relu\n\n"
+        layers = M.parse_cfg(cfg)
+        d = api.Dnn(cfg, None)
+        n = api.Nasm(d, 2, 0, 1)
+        i = n.info(1)
+        n.destroy(); d.destroy()
+        return i["kiters_per_split"] * i["splits"]
+    assert first_conv_slices(64, 7) == 5 and first_conv_slices(16, 3) == 1 and first_conv_slices(32, 5) == 3
+    assert first_conv_slices(96, 7) == 7 and first_conv_slices(128, 3) == 2
+
+
 def test_min_ninst_raises_tile_count():
     case = H.micro_cases()["resnet_mini_b2"]
     counts = []
