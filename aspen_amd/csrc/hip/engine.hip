@@ -97,8 +97,9 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) layer_kernel (const as
 // Second launch of a split-K layer in launch-per-layer mode: one workgroup per output tile adds the slices up.
 __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) finish_kernel (const aspen_hip_layer_t *layers, uint32_t l)
 {
+    extern __shared__ __align__ (16) float smem[];
     const aspen_hip_layer_t L = scalar_layer (layers + l);
-    finish_tile<0> (L, blockIdx.x);
+    finish_tile<0> (L, blockIdx.x, smem);
 }
 
 // Re-arm: counters back to the parent counts, queues seeded with the roots.  A queue entry is 64 bits:
@@ -717,7 +718,8 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
 {
     const char *why = nullptr;
     // buffer descriptors carry 32-bit sizes: this holds for every matrix, also one no tile of its own layer writes
-    if ((uint64_t)L.N * L.ld * 4 * (L.splits > 1 ? L.splits : 1) >= 0xffffff00ull)
+    if ((uint64_t)L.N * L.ld * 4 >= 0xffffff00ull
+        || (L.splits > 1 && (uint64_t)L.splits * L.tiles_m * L.tiles_n * SPLITK_TILE_FLOATS * 4 >= 0xffffff00ull))
     {
         snprintf (g_err, sizeof (g_err), "layer %u rejected: matrix larger than 4 GiB", idx);
         fprintf (stderr, "aspen_hip: %s\n", g_err);
@@ -729,7 +731,7 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
     else if (L.tiles_m == 0 || L.tiles_n == 0 || L.splits == 0
         || L.num_ninst != L.tiles_m * L.tiles_n * L.splits) why = "tile grid";
     else if (L.splits > 1 && (!L.partial || L.kiters_per_split == 0 || (uint64_t)L.splits * L.kiters_per_split * GEMM_BK < L.Kp
-        || !(L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER))) why = "split-K geometry";
+        || !(L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER) || L.variant != ASPEN_HIP_GEMM_SMALL)) why = "split-K geometry";
     else if ((L.type == CONV_LAYER || L.type == MAXPOOL_LAYER || L.type == AVGPOOL_LAYER)
         && (L.stride == 0 || L.KH == 0 || L.KW == 0 || L.IH == 0 || L.IW == 0 || L.OH == 0 || L.OW == 0 || L.N % (L.OH * L.OW))) why = "window geometry";
     else if (L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER)
@@ -987,7 +989,7 @@ static void launch_layer (const aspen_hip_graph_t *g, uint32_t l)
     const aspen_hip_layer_t &L = g->h_layers[l];
     hipLaunchKernelGGL (layer_kernel, dim3 (L.num_ninst), dim3 (WG_THREADS), GEMM_SMEM_BYTES, g_stream, g->d_layers, l, 0u, (uint32_t *)nullptr);
     if (L.splits > 1)
-        hipLaunchKernelGGL (finish_kernel, dim3 (L.tiles_m * L.tiles_n), dim3 (WG_THREADS), 0, g_stream, g->d_layers, l);
+        hipLaunchKernelGGL (finish_kernel, dim3 (L.tiles_m * L.tiles_n), dim3 (WG_THREADS), EPI_FLOATS (VAR2_BM, VAR2_BN) * sizeof (float), g_stream, g->d_layers, l);
 }
 
 extern "C" int aspen_hip_run_layers (aspen_hip_graph_t *g, uint32_t first_layer, uint32_t last_layer)

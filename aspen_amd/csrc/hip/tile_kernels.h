@@ -44,6 +44,7 @@ __device__ void tile_phase_lap (int which);
 #define VAR0_DEPTH 1
 #define VAR1_DEPTH 1
 #define VAR2_DEPTH 2
+#define SPLITK_TILE_FLOATS (VAR2_BM * VAR2_BN)     // one slice's sums of one output tile: a block of its own in `partial`
 #define CMAX(a, b) ((a) > (b) ? (a) : (b))
 #define STAGE_FLOATS(bm, bn) (((bm) + (bn)) * LDS_ROW)
 #define EPI_FLOATS(bm, bn) ((bn) * ((bm) + 8))
@@ -794,24 +795,20 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
     const uint32_t wm0 = (wave % WM) * (BM / WM), wn0 = (wave / WM) * (BN / WN);
     if (slice >= 0)
     {
-        // split-K: the raw sums go straight from the accumulators to this slice's partial matrix.  Register v of
-        // a block holds 32 consecutive channels of one column across a half-wave, so every store instruction
-        // writes two whole 128-byte lines; no bias, no activation, nothing to stage through LDS.
-        const aspen_hip_layer_t L = descriptor ();
-        ActView<COH> part;
-        part.init (L.partial + (size_t)slice * L.N * L.ld, L.N, L.ld);
-        #pragma unroll
-        for (int j = 0; j < TM; j++)
+        // split-K: the raw sums go straight from the accumulators to this slice's block of the output tile, in the
+        // accumulators' own layout (splitk_gather reads them back the same way): four 16-byte stores per lane, each
+        // instruction 1 KB in one piece; no bias, no activation, no bounds, nothing to stage through LDS.  Only the
+        // 64 x 64 shape is ever cut along K.
+        if constexpr (BM == VAR2_BM && BN == VAR2_BN)
         {
-            const uint32_t m = m0 + wm0 + 32 * j + (lane & 31);
+            const aspen_hip_layer_t L = descriptor ();
+            const uint32_t tiles = L.tiles_m * L.tiles_n;
+            ActView<COH> part;
+            part.init (L.partial, L.splits * tiles, SPLITK_TILE_FLOATS);
+            const uint32_t base = ((uint32_t)slice * tiles + tn * L.tiles_m + tm) * SPLITK_TILE_FLOATS + tid * 4;
             #pragma unroll
-            for (int i = 0; i < TN; i++)
-                #pragma unroll
-                for (int v = 0; v < 16; v++)
-                {
-                    const uint32_t n = n0 + ACC_N (wn0, i, v, lane);
-                    if (n < L.N && m < L.M) part.st1 (n * L.ld + m, acc[i][j][v]);
-                }
+            for (int q = 0; q < 4; q++)
+                part.st4 (base + q * 4 * WG_THREADS, make_float4 (acc[0][0][4 * q], acc[0][0][4 * q + 1], acc[0][0][4 * q + 2], acc[0][0][4 * q + 3]));
         }
         return;
     }
@@ -916,72 +913,50 @@ __device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L
     // one before LDS is written again
 }
 
-// split-K, run by the slice that finishes last: sum of the slices (in slice order, whoever runs it) + bias, activation
+// split-K, run by the slice that finishes last: the sum of the slices' blocks (in slice order, whoever runs it) in
+// the accumulator layout they were stored in, parked in LDS as [column][channel] like the accumulators of an unsplit
+// tile, so that contraction_epilogue finishes both alike.  Eight 16-byte loads in flight per thread: their memory
+// latencies overlap instead of adding up (the blocks come from other XCDs' tiles and miss this XCD's L2); a slice
+// index past the last one re-reads the last slice and is not added.
 template <int COH>
-__device__ __forceinline__ void tile_splitk_finish (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm)
+__device__ __forceinline__ void splitk_gather (const aspen_hip_layer_t &L, uint32_t t, float *smem)
 {
-    const uint32_t m0 = tm * L.tile_m, n0 = tn * L.tile_n, C4 = L.tile_m >> 2;
-    const uint32_t rows = min (L.tile_n, L.N - n0), mrem = L.M - m0;
-    ActView<COH> part, out, fin, fout;
-    part.init (L.partial, L.N * L.splits, L.ld); out.init (L.out, L.N, L.ld);
-    const bool fuse = L.fuse_out != nullptr, keep = !(fuse && L.fuse_discard);
-    if (fuse) { fin.init (L.fuse_in, L.N, L.fuse_ld_in); fout.init (L.fuse_out, L.N, L.ld); }
-    // Two 16-byte pieces per thread and four slices of each at a time: eight loads in flight, so that their
-    // memory latencies overlap instead of adding up (the partial sums come from other XCDs' tiles and miss this
-    // XCD's L2).  The slices are added in slice order whoever runs this; a slice index past the last one
-    // re-reads the last slice and is not added.
-    constexpr uint32_t PIECES = 2, BATCH = 4;
-    const uint32_t total = rows * C4, pstride = L.N * L.ld, last = L.splits - 1;
-    for (uint32_t i0 = tile_thread (); i0 < total; i0 += PIECES * WG_THREADS)
+    const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
+    const uint32_t tiles = L.tiles_m * L.tiles_n, sstride = tiles * SPLITK_TILE_FLOATS, last = L.splits - 1;
+    ActView<COH> part;
+    part.init (L.partial, L.splits * tiles, SPLITK_TILE_FLOATS);
+    const uint32_t base = t * SPLITK_TILE_FLOATS + tid * 4;
+    constexpr uint32_t BATCH = 2;       // (1 and 4 measured: no better)
+    float4 v[4];
+    #pragma unroll
+    for (int q = 0; q < 4; q++) v[q] = make_float4 (0.f, 0.f, 0.f, 0.f);
+    for (uint32_t s0 = 0; s0 < L.splits; s0 += BATCH)
     {
-        uint32_t o[PIECES], cc[PIECES];
-        bool live[PIECES];
-        float4 v[PIECES];
+        float4 p[BATCH][4];
         #pragma unroll
-        for (uint32_t u = 0; u < PIECES; u++)
-        {
-            const uint32_t idx = min (i0 + u * WG_THREADS, total - 1), r = idx / C4;
-            cc[u] = (idx - r * C4) * 4;
-            live[u] = i0 + u * WG_THREADS < total && cc[u] < mrem;
-            o[u] = (n0 + r) * L.ld + m0 + (cc[u] < mrem ? cc[u] : 0u);      // channels past the matrix: fetch something that exists
-            v[u] = make_float4 (0.f, 0.f, 0.f, 0.f);
-        }
-        for (uint32_t s0 = 0; s0 < L.splits; s0 += BATCH)
-        {
-            float4 p[PIECES][BATCH];
+        for (uint32_t j = 0; j < BATCH; j++)
             #pragma unroll
-            for (uint32_t u = 0; u < PIECES; u++)
-                #pragma unroll
-                for (uint32_t j = 0; j < BATCH; j++) p[u][j] = part.ld4 (o[u] + min (s0 + j, last) * pstride);
-            #pragma unroll
-            for (uint32_t u = 0; u < PIECES; u++)
-                #pragma unroll
-                for (uint32_t j = 0; j < BATCH; j++)
-                {
-                    const bool use = s0 + j <= last;
-                    v[u].x += use ? p[u][j].x : 0.f; v[u].y += use ? p[u][j].y : 0.f; v[u].z += use ? p[u][j].z : 0.f; v[u].w += use ? p[u][j].w : 0.f;
-                }
-        }
+            for (int q = 0; q < 4; q++) p[j][q] = part.ld4 (base + min (s0 + j, last) * sstride + q * 4 * WG_THREADS);
         #pragma unroll
-        for (uint32_t u = 0; u < PIECES; u++)
+        for (uint32_t j = 0; j < BATCH; j++)
         {
-            if (!live[u]) continue;
-            const uint32_t c = cc[u];
-            float4 y = v[u];
-            if (L.bias)
-            {
-                y.x += gld1 (L.bias + m0 + c);
-                if (c + 1 < mrem) y.y += gld1 (L.bias + m0 + c + 1);
-                if (c + 2 < mrem) y.z += gld1 (L.bias + m0 + c + 2);
-                if (c + 3 < mrem) y.w += gld1 (L.bias + m0 + c + 3);
-            }
-            y = act4 (y, L.act);
-            if (!keep) { }
-            else if (c + 4 <= mrem) out.st4 (o[u], y);
-            else { out.st1 (o[u], y.x); if (c + 1 < mrem) out.st1 (o[u] + 1, y.y); if (c + 2 < mrem) out.st1 (o[u] + 2, y.z); }
-            if (fuse) fused_shortcut<COH> (L, fin, fout, y, (o[u] - m0 - c) / L.ld, m0 + c, mrem - c);
+            const bool use = s0 + j <= last;
+            #pragma unroll
+            for (int q = 0; q < 4; q++)
+            { v[q].x += use ? p[j][q].x : 0.f; v[q].y += use ? p[j][q].y : 0.f; v[q].z += use ? p[j][q].z : 0.f; v[q].w += use ? p[j][q].w : 0.f; }
         }
     }
+    constexpr int TROW = VAR2_BM + 8;
+    const uint32_t wm0 = (wave % 2) * 32, wn0 = (wave / 2) * 32, m = wm0 + (lane & 31);
+    #pragma unroll
+    for (int q = 0; q < 4; q++)
+    {
+        smem[ACC_N (wn0, 0, 4 * q, lane) * TROW + m] = v[q].x;
+        smem[ACC_N (wn0, 0, 4 * q + 1, lane) * TROW + m] = v[q].y;
+        smem[ACC_N (wn0, 0, 4 * q + 2, lane) * TROW + m] = v[q].z;
+        smem[ACC_N (wn0, 0, 4 * q + 3, lane) * TROW + m] = v[q].w;
+    }
+    __syncthreads ();
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1505,11 +1480,14 @@ __device__ __forceinline__ bool splitk_arrived_last (uint32_t *counter, uint32_t
 
 // Split-K reduction of output tile t of the layer as a tile of its own (launch-per-layer mode).
 template <int COH>
-__device__ __forceinline__ void finish_tile (const aspen_hip_layer_t &L, uint32_t t)
+__device__ __forceinline__ void finish_tile (const aspen_hip_layer_t &L, uint32_t t, float *smem)
 {
     t = __builtin_amdgcn_readfirstlane (t);
     const uint32_t tn = fast_div (t, L.div_tiles_m);
-    tile_splitk_finish<COH> (L, tn, t - tn * L.tiles_m);
+    shortcut_prefetch_t pre;
+    pre.have = pre.have_shortcut = false;
+    splitk_gather<COH> (L, t, smem);
+    contraction_epilogue<COH> (L, tn, t - tn * L.tiles_m, smem, 4, VAR2_BN, pre);
 }
 
 // Runs tile t of the layer.  `descriptor ()` yields a wave-uniform copy of the layer's descriptor (scalar_layer /
@@ -1548,18 +1526,18 @@ __device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, boo
         else if (FEAT & TILES_SMALL) contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, VAR2_DEPTH, COH, FEAT> (L, descriptor, tn, tm, slice, smem, pre);
         
         const aspen_hip_layer_t E = descriptor ();
-        if (slice < 0) contraction_epilogue<COH> (E, tn, tm, smem, c4_log2, bn, pre);
-        if (COH) tile_phase_lap (10);
         if (slice >= 0)
         {
-            // split-K: every slice has written its partial sums; whoever arrives last adds them up.  Without
-            // counters (one launch per layer: stores of a launch are not visible across XCDs before it ends)
-            // the sums are added up by a second launch, see finish_tile.
+            // split-K: every slice has written its sums; whoever arrives last adds them up and finishes the tile.
+            // Without counters (one launch per layer: stores of a launch are not visible across XCDs before it
+            // ends) that is left to a second launch, see finish_tile.
+            if (COH) tile_phase_lap (10);
             uint32_t *counters = arrivals ();
             if (counters == nullptr || !splitk_arrived_last (counters + group, E.splits, smem)) { if (COH) tile_phase_lap (11); return false; }
-            tile_splitk_finish<COH> (E, tn, tm);
-            if (COH) tile_phase_lap (11);
+            splitk_gather<COH> (E, t, smem);
         }
+        contraction_epilogue<COH> (E, tn, tm, smem, c4_log2, bn, pre);
+        if (COH) tile_phase_lap (slice >= 0 ? 11 : 10);
         break;
     }
     case RESIDUAL_LAYER:    if constexpr ((FEAT & TILES_RESIDUAL) != 0) tile_residual<COH> (L, tn); break;

@@ -113,6 +113,7 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
         int v = M <= 64 ? ASPEN_HIP_GEMM_WIDE : ASPEN_HIP_GEMM_LARGE;
         if (cdiv (M, bm[v]) * cdiv (N, bn[v]) < want || (N <= 64 && v == ASPEN_HIP_GEMM_WIDE)) v = ASPEN_HIP_GEMM_SMALL;
         if (nasm->small_tiles_only) v = ASPEN_HIP_GEMM_SMALL;      /* graphs bound by their dependency chains, see create_nasm */
+        if (nasm->kiters_cap && aspen_layer_kiters (L) > nasm->kiters_cap) v = ASPEN_HIP_GEMM_SMALL;   /* only the small shape is cut along K */
         ld->variant = v;
         ld->tile_dims[OUT_H] = bm[v]; ld->tile_dims[OUT_W] = bn[v];
     }
@@ -498,7 +499,8 @@ static nasm_t *build_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned in
         if (ld->splits > 1)
         {
             ld->partial_offset = arena;
-            arena += ((size_t)ld->splits * ld->out_mat_stride * ld->out_mat_dims[OUT_W] + 63) / 64 * 64;
+            /* one block of tile_m x tile_n sums per slice and output tile (edge tiles included whole) */
+            arena += (size_t)ld->splits * ld->tiles_h * ld->tiles_w * ld->tile_dims[OUT_H] * ld->tile_dims[OUT_W];
         }
         ld->ninst_start = total;
         total += ld->num_ninst;

@@ -75,7 +75,8 @@ typedef struct aspen_hip_layer_t
     uint32_t heads, seq, hd, masked;
     /* split-K (contraction layers): the layer has T*splits tiles, T = tiles_m*tiles_n; tile
        (tile*splits + slice) computes the partial products over kiters_per_split K slices and writes
-       them to `partial` ([splits][N][ld]).  The `splits` tiles of one output tile form a group: the
+       them to `partial` ([splits][T] blocks of tile_m*tile_n floats in the kernel's own register order;
+       64 x 64 tiles only).  The `splits` tiles of one output tile form a group: the
        member that finishes last (an arrival counter decides) sums the slices in slice order, adds
        the bias, activates and writes the output; only it releases the group's children */
     uint32_t splits, kiters_per_split;
