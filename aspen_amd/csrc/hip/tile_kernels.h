@@ -276,13 +276,19 @@ template <int ROWS, int COH> struct ConvLoader
     int32_t base[R], ih0[R], iw0[R];
     uint32_t IH, IW, chunk, row0;
     uint32_t slices_per_tap, KW, ld0;       // slices_per_tap != 0: a K slice never straddles taps, no table needed
-    int next_it;                            // slice the running tap position (kh, kw, c) below belongs to
-    uint32_t kh, kw, c;
-    __device__ __forceinline__ void init (const aspen_hip_layer_t &L, const ActView<COH> &v, uint32_t first_row, uint32_t tid)
+    uint32_t kh, kw, c;                     // tap and channel the next slice asked for starts at (slices_per_tap != 0)
+    // first_it: the first K slice that will be asked for
+    __device__ __forceinline__ void init (const aspen_hip_layer_t &L, const ActView<COH> &v, uint32_t first_row, uint32_t tid, int first_it)
     {
         in = v; ktab = L.ktab; IH = L.IH; IW = L.IW;
         slices_per_tap = L.IC % GEMM_BK == 0 ? L.IC / GEMM_BK : 0; KW = L.KW; ld0 = L.ld0;
-        next_it = -1; kh = kw = c = 0;
+        kh = kw = c = 0;
+        if (slices_per_tap && first_it)
+        {
+            const uint32_t tap = (uint32_t)first_it / slices_per_tap;
+            c = ((uint32_t)first_it - tap * slices_per_tap) * GEMM_BK;
+            kh = tap / KW; kw = tap - kh * KW;
+        }
         chunk = tid & 7; row0 = tid >> 3;
         const uint32_t ohw = L.OH * L.OW;
         #pragma unroll
@@ -304,16 +310,12 @@ template <int ROWS, int COH> struct ConvLoader
             // channel counts that are multiples of the slice width (every layer but a network's first):
             // the whole slice belongs to one tap, found with a few scalar operations.  Fetching the table
             // entry instead puts a dependent memory access in front of the operand loads of every slice.
-            // Slices are asked for in ascending order, so the position is stepped, not divided out.
-            if (it != next_it)
-            {
-                const uint32_t tap = (uint32_t)it / slices_per_tap;
-                c = ((uint32_t)it - tap * slices_per_tap) * GEMM_BK;
-                kh = tap / KW; kw = tap - kh * KW;
-            }
+            // Slices are asked for in ascending order from the one init was told, so the position is stepped, not
+            // divided out, and `it` is not looked at.  (The K loops ask for the last slice once more than they need
+            // and drop the answer: that request is one step past the K axis, where a tap either lies inside the
+            // image, so the address exists, or fails the bounds test below and nothing is loaded.)
             e.offset = (int32_t)((kh * IW + kw) * ld0 + c + chunk * 4);
             e.kh = (uint16_t)kh; e.kw = (uint16_t)kw;
-            next_it = it + 1;
             c += GEMM_BK;
             if (c == slices_per_tap * GEMM_BK) { c = 0; if (++kw == KW) { kw = 0; ++kh; } }
         }
@@ -735,7 +737,9 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
     const uint32_t m0 = tm * BM, n0 = tn * BN;
     floatx16 acc[TN][TM];
     ActView<COH> in;
-    in.init (L.in0, L.in0_columns, L.ld0);
+    // (the operands' addresses come from loads of their own: taken from `L` they are parts of an 8-register piece of
+    // the descriptor, which the compiler then keeps alive, spills and restores as a whole around every K slice)
+    in.init (descriptor ().in0, L.in0_columns, L.ld0);
     int kbase = 0, kiters = (int)(L.Kp / GEMM_BK);
     if (slice >= 0)
     {
@@ -743,7 +747,7 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
         kiters = min ((int)L.kiters_per_split, kiters - kbase);
     }
     RowLoader<BM> al;
-    al.init (L.weight, m0, (L.M + 127u) / 128u * 128u, L.Kp, tid);
+    al.init (descriptor ().weight, m0, (L.M + 127u) / 128u * 128u, L.Kp, tid);
     // a fused shortcut's other operand comes from memory another XCD may have written: the first pieces this
     // thread will need in the epilogue (see contraction_epilogue for the thread -> piece mapping) are
     // requested under the last K slice
@@ -786,7 +790,7 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
         else
         {
             ConvLoader<BN, COH> bl;
-            bl.init (L, in, n0, tid);
+            bl.init (L, in, n0, tid, kbase);
             if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
             else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
         }
@@ -1521,8 +1525,8 @@ __device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, boo
         shortcut_prefetch_t pre;
         pre.have = pre.have_shortcut = false;
         c4_log2 = 4; bn = VAR2_BN;
-        if ((FEAT & TILES_LARGE) && L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, VAR0_DEPTH, COH, FEAT> (L, descriptor, tn, tm, slice, smem, pre); c4_log2 = 5; bn = VAR0_BN; }
-        else if ((FEAT & TILES_WIDE) && L.variant == ASPEN_HIP_GEMM_WIDE) { contraction_mainloop<VAR1_BM, VAR1_BN, 2, 2, VAR1_DEPTH, COH, FEAT> (L, descriptor, tn, tm, slice, smem, pre); bn = VAR1_BN; }
+        if ((FEAT & TILES_LARGE) && L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, VAR0_DEPTH, COH, FEAT> (L, descriptor, tn, tm, -1, smem, pre); c4_log2 = 5; bn = VAR0_BN; }
+        else if ((FEAT & TILES_WIDE) && L.variant == ASPEN_HIP_GEMM_WIDE) { contraction_mainloop<VAR1_BM, VAR1_BN, 2, 2, VAR1_DEPTH, COH, FEAT> (L, descriptor, tn, tm, -1, smem, pre); bn = VAR1_BN; }
         else if (FEAT & TILES_SMALL) contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, VAR2_DEPTH, COH, FEAT> (L, descriptor, tn, tm, slice, smem, pre);
         
         const aspen_hip_layer_t E = descriptor ();
