@@ -113,6 +113,13 @@ template <int COH> struct ActView
         const floatx4 x = *(const floatx4 __attribute__ ((address_space (1))) *)(base + off * 4u);
         return make_float4 (x[0], x[1], x[2], x[3]);
     }
+    // ok ? ld4 (off) : zeros.  With a buffer descriptor the choice is made on the offset (one past anything the
+    // descriptor covers reads as zeros): no branch around the load, so a K loop that uses it stays one basic block.
+    __device__ __forceinline__ float4 ld4_if (uint32_t off, bool ok) const
+    {
+        if (COH) return __builtin_bit_cast (float4, __builtin_amdgcn_raw_buffer_load_b128 (rsrc, ok ? (int)(off * 4u) : (int)0xfffffff0u, 0, LOAD_POLICY));
+        return ok ? ld4 (off) : make_float4 (0.f, 0.f, 0.f, 0.f);
+    }
     __device__ __forceinline__ float ld1 (uint32_t off) const
     {
         if (COH) return __builtin_bit_cast (float, __builtin_amdgcn_raw_buffer_load_b32 (rsrc, (int)(off * 4u), 0, LOAD_POLICY));
@@ -329,7 +336,7 @@ template <int ROWS, int COH> struct ConvLoader
         for (int i = 0; i < R; i++)
         {
             const bool ok = (uint32_t)(ih0[i] + (int32_t)e.kh) < IH && (uint32_t)(iw0[i] + (int32_t)e.kw) < IW;
-            v[i] = ok ? in.ld4 ((uint32_t)(base[i] + e.offset)) : make_float4 (0.f, 0.f, 0.f, 0.f);
+            v[i] = in.ld4_if ((uint32_t)(base[i] + e.offset), ok);
         }
     }
     __device__ __forceinline__ void store (float *lds, const float4 (&v)[R])
@@ -379,8 +386,7 @@ template <int ROWS, int COH> struct Dense3Loader
         {
             const bool oka = (uint32_t)(ih0[i] + (int32_t)(raw[1] & 0xffffu)) < IH && (uint32_t)(iw0[i] + (int32_t)(raw[1] >> 16)) < IW;
             const bool okb = (uint32_t)(ih0[i] + (int32_t)(raw[3] & 0xffffu)) < IH && (uint32_t)(iw0[i] + (int32_t)(raw[3] >> 16)) < IW;
-            const float4 z = make_float4 (0.f, 0.f, 0.f, 0.f);
-            const float4 a = oka ? in.ld4 ((uint32_t)(base[i] + (int32_t)raw[0])) : z, b = okb ? in.ld4 ((uint32_t)(base[i] + (int32_t)raw[2])) : z;
+            const float4 a = in.ld4_if ((uint32_t)(base[i] + (int32_t)raw[0]), oka), b = in.ld4_if ((uint32_t)(base[i] + (int32_t)raw[2]), okb);
             v[i].x = sel == 0 ? a.x : sel == 1 ? a.y : a.z;
             v[i].y = sel == 0 ? a.y : sel == 1 ? a.z : b.x;
             v[i].z = sel == 0 ? a.z : sel == 1 ? b.x : b.y;
