@@ -275,28 +275,37 @@ template <int ROWS, int COH> struct ActRowLoader
 // Implicit-GEMM activation operand of conv / FC: row n = output position (b, oh, ow); the K axis runs
 // over (kh, kw, ic) and is resolved through the layer's k-chunk table.  Replaces the reference's
 // pointer table + panel gather (prepare_input / load_im2col_ptr, reference src/tiled_kernels.c:3-159).
-template <int ROWS, int COH> struct ConvLoader
+// TABLE: the K axis is resolved through the layer's k-chunk table (channel counts that are not multiples of the slice
+// width, where a slice straddles taps; 64 x 64 tiles only, the host's tile policy sees to that).  Otherwise a whole
+// slice belongs to one tap, found with a few scalar operations: fetching the table entry instead puts a dependent
+// memory access in front of the operand loads of every slice.  Two loaders, not one with a branch: with both
+// paths in one K loop the compiler waits for ALL outstanding loads wherever they join.
+template <int ROWS, int COH, bool TABLE> struct ConvLoader
 {
     static constexpr int R = ROWS / 32;
     ActView<COH> in;
     const aspen_hip_ktab_t *ktab;
     int32_t base[R], ih0[R], iw0[R];
     uint32_t IH, IW, chunk, row0;
-    uint32_t slices_per_tap, KW, ld0;       // slices_per_tap != 0: a K slice never straddles taps, no table needed
-    uint32_t kh, kw, c;                     // tap and channel the next slice asked for starts at (slices_per_tap != 0)
+    uint32_t slices_per_tap, KW, ld0;
+    uint32_t kh, kw, c;                     // tap and channel the next slice asked for starts at (!TABLE)
     // first_it: the first K slice that will be asked for
     __device__ __forceinline__ void init (const aspen_hip_layer_t &L, const ActView<COH> &v, uint32_t first_row, uint32_t tid, int first_it)
     {
-        in = v; ktab = L.ktab; IH = L.IH; IW = L.IW;
-        slices_per_tap = L.IC % GEMM_BK == 0 ? L.IC / GEMM_BK : 0; KW = L.KW; ld0 = L.ld0;
-        kh = kw = c = 0;
-        if (slices_per_tap && first_it)
-        {
-            const uint32_t tap = (uint32_t)first_it / slices_per_tap;
-            c = ((uint32_t)first_it - tap * slices_per_tap) * GEMM_BK;
-            kh = tap / KW; kw = tap - kh * KW;
-        }
+        in = v; IH = L.IH; IW = L.IW;
         chunk = tid & 7; row0 = tid >> 3;
+        if (TABLE) ktab = L.ktab;
+        else
+        {
+            slices_per_tap = L.IC / GEMM_BK; KW = L.KW; ld0 = L.ld0;
+            kh = kw = c = 0;
+            if (first_it)
+            {
+                const uint32_t tap = (uint32_t)first_it / slices_per_tap;
+                c = ((uint32_t)first_it - tap * slices_per_tap) * GEMM_BK;
+                kh = tap / KW; kw = tap - kh * KW;
+            }
+        }
         const uint32_t ohw = L.OH * L.OW;
         #pragma unroll
         for (int i = 0; i < R; i++)
@@ -312,11 +321,14 @@ template <int ROWS, int COH> struct ConvLoader
     __device__ __forceinline__ void load (int it, float4 (&v)[R])
     {
         aspen_hip_ktab_t e;
-        if (slices_per_tap)
+        if (TABLE)
         {
-            // channel counts that are multiples of the slice width (every layer but a network's first):
-            // the whole slice belongs to one tap, found with a few scalar operations.  Fetching the table
-            // entry instead puts a dependent memory access in front of the operand loads of every slice.
+            typedef unsigned int uintx2 __attribute__ ((ext_vector_type (2)));
+            const uintx2 raw = *(const uintx2 __attribute__ ((address_space (1))) *)(ktab + it * 8 + chunk);
+            e.offset = (int32_t)raw[0]; e.kh = (uint16_t)(raw[1] & 0xffffu); e.kw = (uint16_t)(raw[1] >> 16);
+        }
+        else
+        {
             // Slices are asked for in ascending order from the one init was told, so the position is stepped, not
             // divided out, and `it` is not looked at.  (The K loops ask for the last slice once more than they need
             // and drop the answer: that request is one step past the K axis, where a tap either lies inside the
@@ -325,12 +337,6 @@ template <int ROWS, int COH> struct ConvLoader
             e.kh = (uint16_t)kh; e.kw = (uint16_t)kw;
             c += GEMM_BK;
             if (c == slices_per_tap * GEMM_BK) { c = 0; if (++kw == KW) { kw = 0; ++kh; } }
-        }
-        else
-        {
-            typedef unsigned int uintx2 __attribute__ ((ext_vector_type (2)));
-            const uintx2 raw = *(const uintx2 __attribute__ ((address_space (1))) *)(ktab + it * 8 + chunk);
-            e.offset = (int32_t)raw[0]; e.kh = (uint16_t)(raw[1] & 0xffffu); e.kw = (uint16_t)(raw[1] >> 16);
         }
         #pragma unroll
         for (int i = 0; i < R; i++)
@@ -793,9 +799,18 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
             if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
             else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
         }
+        else if (TM * TN == 1 && L.IC % GEMM_BK != 0)
+        {
+            if constexpr (TM * TN == 1)
+            {
+                ConvLoader<BN, COH, true> bl;
+                bl.init (L, in, n0, tid, kbase);
+                gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
+            }
+        }
         else
         {
-            ConvLoader<BN, COH> bl;
+            ConvLoader<BN, COH, false> bl;
             bl.init (L, in, n0, tid, kbase);
             if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
             else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);

@@ -289,6 +289,16 @@ int aspen_layer_dense3 (const aspen_layer_t *L)
         && getenv ("ASPEN_GPU_NO_DENSE3") == NULL;
 }
 
+/* A contraction layer whose channel count is not a multiple of the K slice width (32): a slice straddles taps, so
+   the kernels resolve its K axis through the k-chunk table, which only the 64 x 64 tile shape can do. */
+int aspen_layer_table_operand (const aspen_layer_t *L)
+{
+    const unsigned int *p = L->params;
+    if (L->type != CONV_LAYER && L->type != FC_LAYER && L->type != MATMUL_LAYER) return 0;
+    if (aspen_layer_dense3 (L)) return 0;
+    return (L->type == MATMUL_LAYER ? p[MAT_K] : p[IN_C]) % 32 != 0;
+}
+
 /* padded K of the device layout / 32 (must agree with aspen_layer_to_device) */
 unsigned int aspen_layer_kiters (const aspen_layer_t *L)
 {

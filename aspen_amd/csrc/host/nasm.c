@@ -114,6 +114,7 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
         if (cdiv (M, bm[v]) * cdiv (N, bn[v]) < want || (N <= 64 && v == ASPEN_HIP_GEMM_WIDE)) v = ASPEN_HIP_GEMM_SMALL;
         if (nasm->small_tiles_only) v = ASPEN_HIP_GEMM_SMALL;      /* graphs bound by their dependency chains, see create_nasm */
         if (nasm->kiters_cap && aspen_layer_kiters (L) > nasm->kiters_cap) v = ASPEN_HIP_GEMM_SMALL;   /* only the small shape is cut along K */
+        if (aspen_layer_table_operand (L)) v = ASPEN_HIP_GEMM_SMALL;
         ld->variant = v;
         ld->tile_dims[OUT_H] = bm[v]; ld->tile_dims[OUT_W] = bn[v];
     }
