@@ -138,6 +138,34 @@ def test_first_layer_over_three_channels_matches_oracle(gpu, mode, filters, size
         net.close()
 
 
+@pytest.mark.parametrize("mode", [api.MODE_LAYERS, api.MODE_DATAFLOW], ids=["layers", "dataflow"])
+def test_channel_counts_off_the_slice_width_in_a_graph_of_large_tiles(gpu, mode):
+    """Layers whose K axis goes through the k-chunk table (48 and 40 input channels: a K slice of 32 straddles taps)
+    next to layers that step through their taps, in a graph wide enough for the large tile shapes: the table layers
+    run on 64 x 64 tiles, their neighbours on 128 x 64 / 64 x 128, all against the oracle's convolution."""
+    from oracle import cpu
+    cfg = ("[net]\nheight=48\nwidth=48\nchannels=48\n\n"
+           "[convolutional]\nfilters=128\nsize=3\nstride=1\npad=1\nactivation=relu\n\n"
+           "[convolutional]\nfilters=128\nsize=3\nstride=1\npad=1\nactivation=leaky\n\n"
+           "[convolutional]\nfilters=40\nsize=1\nstride=1\npad=0\nactivation=relu\n\n"
+           "[convolutional]\nfilters=128\nsize=1\nstride=1\npad=0\nactivation=relu\n\n")
+    layers = M.parse_cfg(cfg)
+    tens = M.synth_weights(layers, 47, "he")
+    batch = 32
+    x = (M.synth_input(layers, 47, batch, 0, "token_ids") * 2.0 - 1.0).astype(np.float32)
+    outs = cpu.run_network(layers, tens, x, batch, 0)
+    net = H.GpuNet(cfg, tens, batch, 0, min_ninst=16, mode=mode)
+    try:
+        net.run(x)
+        shapes = [(net.nasm.info(l)["tile_H"], net.nasm.info(l)["tile_W"]) for l in range(1, 5)]
+        assert shapes[0] == (64, 64) and shapes[3] == (64, 64) and shapes[1] == (128, 64) and shapes[2] == (64, 128), shapes
+        for l in range(1, net.nasm.num_ldata):
+            err = H.rel_l2(net.layer(l), outs[l])
+            assert err <= H.REL_L2_TOL, f"layer {l}: rel L2 {err:.3g}"
+    finally:
+        net.close()
+
+
 def test_results_in_the_callers_dimension_order(gpu):
     """dse_get_ldata_result permutes a layer's native tensor into the order the caller names (reference
     get_ldata_output, src/apu.c:227-297): matrices of a transformer are (BATCH, MAT_N, MAT_M), attention

@@ -275,6 +275,36 @@ def test_three_channel_first_layer_contracts_a_dense_k_axis():
     assert first_conv_slices(96, 7) == 7 and first_conv_slices(128, 3) == 2
 
 
+def test_layers_cut_along_k_or_resolved_through_the_table_take_the_small_tile_shape():
+    """Only the 64 x 64 kernels hold split-K and k-chunk-table code: a layer cut along K, and a layer whose channel
+    count is not a multiple of the K slice width (so that a slice straddles taps), get that shape whatever the tile
+    count asks for; their neighbours with 32-multiple channel counts keep the large shapes."""
+    import ctypes
+    shp = (ctypes.c_uint32 * 9)()
+    api.lib().aspen_hip_tile_shapes(shp)
+    shp = list(shp)
+    cfg = ("[net]\nheight=64\nwidth=64\nchannels=48\n\n"
+           "[convolutional]\nfilters=128\nsize=3\nstride=1\npad=1\nactivation=relu\n\n"      # 48 channels in: table
+           "[convolutional]\nfilters=128\nsize=3\nstride=1\npad=1\nactivation=relu\n\n"      # 128 channels in: stepping
+           "[convolutional]\nfilters=40\nsize=1\nstride=1\npad=0\nactivation=relu\n\n"       # few rows: wide shape
+           "[convolutional]\nfilters=128\nsize=1\nstride=1\npad=0\nactivation=relu\n\n")     # 40 channels in: table
+    d = api.Dnn(cfg, None)
+    n = api.Nasm(d, 32, 0, 1)               # one tile per layer wanted: nothing but the rules above asks for small tiles
+    infos = [n.info(l) for l in range(n.num_ldata)]
+    n.destroy()
+    small = (shp[4], shp[5])
+    assert (infos[1]["tile_H"], infos[1]["tile_W"]) == small
+    assert (infos[2]["tile_H"], infos[2]["tile_W"]) == (shp[0], shp[1])
+    assert (infos[3]["tile_H"], infos[3]["tile_W"]) == (shp[2], shp[3])
+    assert (infos[4]["tile_H"], infos[4]["tile_W"]) == small
+    assert all(i["splits"] == 1 for i in infos)
+    n = api.Nasm(d, 32, 0, 8192)            # many tiles wanted: the K axis of the 3x3 layers is cut, on small tiles
+    infos = [n.info(l) for l in range(n.num_ldata)]
+    n.destroy(); d.destroy()
+    assert infos[2]["splits"] > 1
+    assert all((i["tile_H"], i["tile_W"]) == small for i in infos[1:] if i["splits"] > 1)
+
+
 def test_min_ninst_raises_tile_count():
     case = H.micro_cases()["resnet_mini_b2"]
     counts = []
