@@ -1330,11 +1330,14 @@ __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, ui
         ActRowLoader<BN, COH> bl; bl.init (Q, b * S + q0, b * S + S - 1, L.ld0, h * L.hd, tid);
         gemm_core<BM, BN, WM, WN, 1> (al, bl, 0, kiters, smem, acc);
     };
-    // exponential of one score; reference order of operations: mask with -1e10, scale, exp, no max subtraction
+    // exponential of one score; reference order of operations: mask with -1e10, scale, exp, no max subtraction.
+    // The hardware exponential (2^(x log2 e), about 1e-6 relative for scores of a few units against libm's expf, two
+    // orders inside the parity tolerance; exactly 0 for the masked -1e10): the tile is bound by this arithmetic,
+    // 32 exponentials per lane and key block, and expf costs five times the instructions.
     auto weight = [&] (float sc, uint32_t key, uint32_t q) -> float
     {
         if (L.masked && key > q) sc = -1e10f;
-        return (key < S && q < S) ? expf (sc * scale) : 0.f;
+        return (key < S && q < S) ? __expf (sc * scale) : 0.f;
     };
 
     float part[TN][16];
@@ -1391,15 +1394,15 @@ __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, ui
         for (uint32_t r = tid / C4; r < nq; r += STEP)
         {
             const uint32_t key = k0 + c, o = obase + (q0 + r) * L.ld + key;
-            const float sum = rowsum[r];
+            const float inv = 1.0f / rowsum[r];             // one division per piece, then products (within an ulp of the quotients)
             if (key + 4 <= S)
             {
                 float4 p = out.ld4 (o);
-                p.x /= sum; p.y /= sum; p.z /= sum; p.w /= sum;
+                p.x *= inv; p.y *= inv; p.z *= inv; p.w *= inv;
                 out.st4 (o, p);
             }
             else
-                for (uint32_t e = key; e < S; e++) out.st1 (o + e - key, out.ld1 (o + e - key) / sum);
+                for (uint32_t e = key; e < S; e++) out.st1 (o + e - key, out.ld1 (o + e - key) * inv);
         }
     // key blocks that are masked for every query of the tile
     for (uint32_t k0 = (kend + BM - 1) / BM * BM; k0 < S; k0 += BM)
