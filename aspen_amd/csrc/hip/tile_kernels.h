@@ -38,9 +38,12 @@ __device__ void tile_phase_lap (int which);
 #define VAR1_BN 128
 #define VAR2_BM 64
 #define VAR2_BN 64
-// K slices in flight from memory per tile shape (see gemm_core).  Two for the small shape, whose tiles are the
-// short ones of layers cut along K; with two the larger shapes run out of registers (measured: ResNet-50 batch 32
-// 2.81 -> 2.89 ms, VGG-16 7.90 -> 8.83 ms).
+// K slices in flight from memory per tile shape (see gemm_core).  With two the larger shapes run out of registers
+// (measured: ResNet-50 batch 32 2.81 -> 2.89 ms, VGG-16 7.90 -> 8.83 ms).  The small shape takes two for the matmul
+// layers of transformer graphs, which run one or two workgroups per compute unit with nothing else to hide a slice's
+// memory latency (BERT-base 2.45 -> 2.24 ms), and one in the kernels for convolutional networks: there four workgroups
+// per compute unit hide it, and the second set of requests only lengthens the memory queues every tile's set-up
+// waits in (YOLO-v3 batch 8 4.90 -> 4.84 ms, ResNet-50 batch 1 with one launch per layer 0.62 -> 0.60).
 #define VAR0_DEPTH 1
 #define VAR1_DEPTH 1
 #define VAR2_DEPTH 2
@@ -1551,7 +1554,14 @@ __device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, boo
         c4_log2 = 4; bn = VAR2_BN;
         if ((FEAT & TILES_LARGE) && L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, VAR0_DEPTH, COH, FEAT> (L, descriptor, tn, tm, -1, smem, pre); c4_log2 = 5; bn = VAR0_BN; }
         else if ((FEAT & TILES_WIDE) && L.variant == ASPEN_HIP_GEMM_WIDE) { contraction_mainloop<VAR1_BM, VAR1_BN, 2, 2, VAR1_DEPTH, COH, FEAT> (L, descriptor, tn, tm, -1, smem, pre); bn = VAR1_BN; }
-        else if (FEAT & TILES_SMALL) contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, VAR2_DEPTH, COH, FEAT> (L, descriptor, tn, tm, slice, smem, pre);
+        else if (FEAT & TILES_SMALL)
+        {
+            // two K slices in flight for the matmul layers of transformers, one for convolutional networks (see VAR2_DEPTH)
+            bool deep = false;
+            if constexpr ((FEAT & TILES_NORM) != 0) deep = (FEAT & TILES_GATHER) == 0 || L.type == MATMUL_LAYER;
+            if constexpr ((FEAT & TILES_NORM) != 0) { if (deep) contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, VAR2_DEPTH, COH, FEAT> (L, descriptor, tn, tm, slice, smem, pre); }
+            if constexpr ((FEAT & TILES_GATHER) != 0) { if (!deep) contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, 1, COH, FEAT> (L, descriptor, tn, tm, slice, smem, pre); }
+        }
         
         const aspen_hip_layer_t E = descriptor ();
         if (slice >= 0)
