@@ -33,7 +33,7 @@ __device__ void tile_phase_lap (int which);
 #define VAR0_BM 128
 #define VAR0_BN 64
 #define WG_PER_CU 4
-#define KATTN_BN 64
+#define KATTN_BN 32            // queries per K-attention tile
 #define VAR1_BM 64
 #define VAR1_BN 128
 #define VAR2_BM 64
@@ -1295,7 +1295,10 @@ __device__ __forceinline__ void tile_softmax (const aspen_hip_layer_t &L, uint32
 
 // ---------------------------------------------------------------------------------------------
 // Attention tiles.
-// K tile: one (batch, head) x KATTN_BN queries x all keys.  scores = K.Q on the matrix cores, 128 keys at
+// K tile: one (batch, head) x KATTN_BN queries x all keys.  (32 queries, four wavefronts side by side along the keys: a
+// tile works through its key blocks one after the other, and with 64 queries a long sequence has few tiles that each
+// take long; GPT-2 at 512 tokens 3.95 -> 3.83 ms, one launch per layer 4.43 -> 4.17; BERT at 128 tokens 2.24 -> 2.26
+// and 2.40 -> 2.32.  Both sizes in one kernel, chosen per layer, cost BERT 5 % through the register allocation.)  scores = K.Q on the matrix cores, 128 keys at
 // a time; causal mask (-1e10 before the 1/sqrt(hd) scale), exp without max subtraction; every block's
 // exponentials are stored (staged through LDS for 16-byte stores) while the queries' sums accumulate,
 // then a sweep over the tile's own output divides by the sums.  Key blocks the causal mask zeroes for
@@ -1305,7 +1308,7 @@ __device__ __forceinline__ void tile_softmax (const aspen_hip_layer_t &L, uint32
 template <int COH>
 __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, uint32_t tn, float *smem)
 {
-    constexpr int BM = 128, BN = KATTN_BN, WM = 2, WN = 2, TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int BM = 128, BN = KATTN_BN, WM = BN == 32 ? 4 : 2, WN = BN == 32 ? 1 : 2, TM = BM / WM / 32, TN = BN / WN / 32;
     constexpr int TROW = BM + 8;            // staging row of one query: (4 * TROW) % 64 == 32, see the contraction epilogue
     static_assert (BN * TROW <= GEMM_SMEM_FLOATS, "probability staging fits the GEMM stage");
     __shared__ float rowsum[BN];

@@ -166,6 +166,29 @@ def test_channel_counts_off_the_slice_width_in_a_graph_of_large_tiles(gpu, mode)
         net.close()
 
 
+@pytest.mark.parametrize("mode", [api.MODE_LAYERS, api.MODE_DATAFLOW], ids=["layers", "dataflow"])
+@pytest.mark.parametrize("masked", [True, False], ids=["causal", "full"])
+def test_attention_over_a_long_ragged_sequence_matches_oracle(gpu, mode, masked):
+    """A sequence that is a multiple of neither tile extent of the attention layers: 272 tokens = 8 x 32 + 16 queries and
+    2 x 128 + 16 keys per (batch, head), with and without the causal mask, every layer against the oracle."""
+    from oracle import cpu
+    cfg = M.gpt2_cfg(2, 64, 2, 128) if masked else M.bert_cfg(2, 64, 2, 128)
+    layers = M.parse_cfg(cfg)
+    tens = M.synth_weights(layers, 53, "gpt")
+    batch, seq = 2, 272
+    x = M.synth_input(layers, 53, batch, seq, "token_ids" if masked else "embeddings")
+    outs = cpu.run_network(layers, tens, x, batch, seq)
+    net = H.GpuNet(cfg, tens, batch, seq, min_ninst=32, mode=mode)
+    try:
+        net.run(x)
+        for l in range(1, net.nasm.num_ldata):
+            if net.nasm.info(l)["num_ninst"] == 0 and layers[l]["type"] != "residual": continue
+            err = H.rel_l2(net.layer(l), outs[l])
+            assert err <= H.REL_L2_TOL, f"layer {l} ({layers[l]['type']}): rel L2 {err:.3g}"
+    finally:
+        net.close()
+
+
 def test_results_in_the_callers_dimension_order(gpu):
     """dse_get_ldata_result permutes a layer's native tensor into the order the caller names (reference
     get_ldata_output, src/apu.c:227-297): matrices of a transformer are (BATCH, MAT_N, MAT_M), attention

@@ -96,16 +96,14 @@ def needed_regions(L, layers, c0, c1, r0, r1, batch, seq):
         out = []
         for c in cols:
             b, h, q = c // (Hn * seq), (c // seq) % Hn, c % seq
+            # the first parent holds the queries (only token q is read), the second the keys (every token of b):
+            # reference cfg order, parent = Query, from = Key
             out.append((p0, {b * seq + q}, h * hd, (h + 1) * hd))
-            out.append((p1, {b * seq + q}, h * hd, (h + 1) * hd))
-            # one parent holds the queries (only token q needed), the other the keys (every token of b);
-            # which is which is the cfg's business: require the union, accept it on both
-            out.append((p0, set(), 0, 0))
         keys = {(c // (Hn * seq)) for c in cols}
         heads = {((c // seq) % Hn) for c in cols}
         for b in keys:
             for h in heads:
-                out.append(("either", {b * seq + s for s in range(seq)}, h * hd, (h + 1) * hd))
+                out.append((p1, {b * seq + s for s in range(seq)}, h * hd, (h + 1) * hd))
         return out
     if t == "attn_v":       # column = token (b, s); rows = h*hd + d;  p0 = probabilities, p1 = values
         Hn, hd = L["n_head"], L["n_embd"] // L["n_head"]
@@ -121,11 +119,14 @@ def needed_regions(L, layers, c0, c1, r0, r1, batch, seq):
 @pytest.mark.parametrize("fuse", [True, False], ids=["fused", "unfused"])
 @pytest.mark.parametrize("name,min_ninst", [("custom_b3", 16), ("resnet_mini_b2", 64), ("resnet_mini_b2", 1024),
                                             ("vgg_mini_b5", 32), ("bert_mini_b2_s24", 16), ("gpt_mini_b2_s20", 256),
-                                            ("yolo_mini_b2", 16), ("yolo_mini_b2", 512)])
+                                            ("yolo_mini_b2", 16), ("yolo_mini_b2", 512), ("gpt_long_b1_s272", 64)])
 def test_tile_graph_against_brute_force(name, min_ninst, fuse, monkeypatch):
     if not fuse:
         monkeypatch.setenv("ASPEN_GPU_NO_FUSE", "1")
-    layers, d, n, batch, seq = make(H.micro_cases()[name], min_ninst)
+    cases = dict(H.micro_cases())
+    # several query tiles per sequence, ragged against both attention tile extents (272 = 8 x 32 + 16 = 2 x 128 + 16)
+    cases["gpt_long_b1_s272"] = (M.gpt2_cfg(1, 64, 2, 128), "gpt", 1, 272, 13, "token_ids")
+    layers, d, n, batch, seq = make(cases[name], min_ninst)
     tl, npar, off, idx = n.graph()
     T = n.num_ninst
     infos = [n.info(l) for l in range(n.num_ldata)]
