@@ -512,7 +512,7 @@ extern "C" const char *aspen_hip_last_error (void) { return g_err; }
 extern "C" void aspen_hip_tile_shapes (uint32_t shapes[9])
 {
     shapes[0] = VAR0_BM; shapes[1] = VAR0_BN; shapes[2] = VAR1_BM; shapes[3] = VAR1_BN; shapes[4] = VAR2_BM; shapes[5] = VAR2_BN;
-    shapes[6] = KATTN_BN; shapes[7] = 128; shapes[8] = WG_PER_CU;
+    shapes[6] = KATTN_BN; shapes[7] = VATTN_BN; shapes[8] = WG_PER_CU;
 }
 
 extern "C" int aspen_hip_device_info (int *num_cu, int *clock_khz, size_t *mem_bytes, char *name, int name_len)
@@ -762,7 +762,7 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
     else if (L.type == V_ATTENTION_LAYER)
     {
         if (!L.in1 || L.hd == 0 || L.heads == 0 || L.seq == 0) why = "attention geometry";
-        else if (L.tile_n != 128 || L.tile_m > 64 || L.hd % L.tile_m) why = "V-attention tiles are 128 queries x <=64 channels of one head";
+        else if (L.tile_n != VATTN_BN || L.tile_m > 64 || L.hd % L.tile_m) why = "V-attention tile extent (queries x <=64 channels of one head)";
         else if (L.ld0 % GEMM_BK || L.ld0 < L.seq) why = "probability stride must be a multiple of 32 covering seq";
     }
     else if (L.type == MAXPOOL_LAYER || L.type == AVGPOOL_LAYER)

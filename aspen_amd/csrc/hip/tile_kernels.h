@@ -34,6 +34,7 @@ __device__ void tile_phase_lap (int which);
 #define VAR0_BN 64
 #define WG_PER_CU 4
 #define KATTN_BN 32            // queries per K-attention tile
+#define VATTN_BN 64            // queries per V-attention tile
 #define VAR1_BM 64
 #define VAR1_BN 128
 #define VAR2_BM 64
@@ -1421,13 +1422,13 @@ __device__ __forceinline__ void tile_k_attention (const aspen_hip_layer_t &L, ui
     __syncthreads ();
 }
 
-// V tile: one (batch, head-slice of <= 64 channels) x 128 queries:
+// V tile: one (batch, head-slice of <= 64 channels) x VATTN_BN queries:
 // out[b*S + q][h*hd + j] = sum_s P[(b*H + h)*S + q][s] * V[b*S + s][h*hd + j].
 // in0 = probabilities (K-attention output), in1 = Value matrix.
 template <int COH>
 __device__ __forceinline__ void tile_v_attention (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, float *smem)
 {
-    constexpr int BM = 64, BN = 128, WM = 2, WN = 2, TM = 1, TN = 2;
+    constexpr int BM = 64, BN = VATTN_BN, WM = 2, WN = 2, TM = 1, TN = BN / WN / 32;
     const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
     const uint32_t S = L.seq, qtiles = (S + BN - 1) / BN;
     const uint32_t b = tn / qtiles, q0 = (tn - b * qtiles) * BN;

@@ -134,8 +134,10 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
         const unsigned int S = nasm->tr_seq_len, hd = L->params[NUM_HIDDEN] / L->params[NUM_HEAD];
         if (hd * L->params[NUM_HEAD] != M || (hd > 64 && hd % 64 != 0) || hd % 4 != 0)
         { ERROR_PRTF ("layer %u: unsupported head geometry (M %u, heads %u)\n", L->layer_idx, M, L->params[NUM_HEAD]); return -1; }
-        ld->tile_dims[OUT_H] = umin (hd, 64); ld->tile_dims[OUT_W] = 128;
-        ld->tiles_h = M / ld->tile_dims[OUT_H]; ld->tiles_w = (N / S) * cdiv (S, 128);
+        uint32_t shp[9];
+        aspen_hip_tile_shapes (shp);
+        ld->tile_dims[OUT_H] = umin (hd, 64); ld->tile_dims[OUT_W] = shp[7];
+        ld->tiles_h = M / ld->tile_dims[OUT_H]; ld->tiles_w = (N / S) * cdiv (S, shp[7]);
         ld->num_ninst = ld->tiles_h * ld->tiles_w;
         return 0;
     }
