@@ -97,6 +97,7 @@ def lib() -> C.CDLL:
         "aspen_rpool_profile_layers": (C.c_int, [_vp, C.c_uint, _fp]),
         "aspen_rpool_dataflow_profile": (C.c_int, [_vp, C.POINTER(C.c_uint64), C.c_int]),
         "aspen_rpool_dataflow_trace": (C.c_int, [_vp, _vp]),
+        "aspen_rpool_debug_set_epoch": (C.c_int, [_vp, C.c_uint32]),
         # aspen_hip.h
         "aspen_hip_init": (C.c_int, []),
         "aspen_hip_last_error": (C.c_char_p, []),
@@ -259,6 +260,10 @@ class RPool:
             raise RuntimeError("no dataflow run to report on")
         return {"executed": a.value, "double_runs": b.value, "aborted": c.value}
 
+    def debug_set_epoch(self, epoch: int):
+        if lib().aspen_rpool_debug_set_epoch(self.h, epoch):
+            raise RuntimeError("the pool has no device graph yet")
+
     def dataflow_profile(self, reset: bool = True) -> dict:
         """Summed workgroup time of dataflow runs since the last reset, in seconds (profile flag 4)."""
         t = (C.c_uint64 * 16)()
@@ -318,6 +323,11 @@ class DseGroup:
     @staticmethod
     def wait(nasm: Nasm):
         lib().dse_wait_for_nasm_completion(nasm.h)
+
+    @staticmethod
+    def check(nasm: Nasm) -> bool:
+        """``dse_check_nasm_completion``: True once THIS nasm has finished, whatever the pool's others do."""
+        return lib().dse_check_nasm_completion(nasm.h) == 1
 
     def destroy(self):
         if self.h:

@@ -31,6 +31,12 @@ typedef unsigned long long qentry_t;      // ready-queue entry / child-record en
 #define ST_QHEAD(q) (192u + 64u * (q))      // pop tickets of queue q
 #define ST_QTAIL(q) (224u + 64u * (q))      // push cursor of queue q
 #define ST_WORDS (192u + 64u * NUM_QUEUES)
+// Co-scheduled networks ("groups", aspen_hip_layer_t.graph_id): each counts its finished tiles without children on a
+// line of its own behind the state words; ST_SINKS counts the groups that have finished.
+#define MAX_GROUPS 64u
+#define ST_GROUP(g) (ST_WORDS + 32u * (g))
+#define ST_ALL_WORDS (ST_WORDS + 32u * MAX_GROUPS)
+#define HOST_DONE_WORD 16u      // pinned host block: [0] abort flag, [HOST_DONE_WORD + g] = serial of the last run group g finished in
 #define NUM_EVENTS 16
 #define DEFAULT_SPIN_LIMIT (1ull << 26)
 
@@ -53,8 +59,14 @@ struct aspen_hip_graph_t
     uint32_t *d_ran;        // per-tile execution count (sanity: every tile exactly once)
     uint32_t *d_arrivals;   // split-K arrival counters, see run_tile
     uint32_t num_sinks;     // tiles without children
+    uint32_t num_groups;    // co-scheduled networks (largest graph_id + 1)
+    uint32_t live_groups;   // those of them that have tiles
+    uint32_t *d_group_sinks;    // per group: its tiles without children
+    uint32_t run_serial;    // number of the last dataflow run (never 0): what a group's host word holds once it has finished in that run
+    int last_run_dataflow;  // the host words describe the last run
     unsigned features;      // TILES_* bits of the tile kinds the graph contains: picks the persistent kernel's variant
-    uint32_t epoch;         // tag of the last run's queue entries, cycles 1..255
+    uint32_t epoch;         // tag of the last run's queue entries, cycles 1..EPOCH_MAX
+    uint32_t queue_config;  // grid, flags and queue grouping of the last run (they decide which queue slots a run rewrites), see run_dataflow
     unsigned long long *d_prof;
     uint32_t default_workgroups;    // grid of a dataflow run when the caller names none, see graph_parallelism
     double parallelism;             // average parallelism of the tile graph, see graph_parallelism
@@ -64,6 +76,7 @@ struct aspen_hip_graph_t
 };
 
 static hipStream_t g_stream = nullptr;
+static hipStream_t g_side_stream = nullptr;       // read-outs that must not queue behind a running persistent kernel
 static hipEvent_t g_events[NUM_EVENTS];
 static int g_inited = 0;
 static int g_num_cu = 0;
@@ -103,16 +116,22 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) finish_kernel (const a
 }
 
 // Re-arm: counters back to the parent counts, queues seeded with the roots.  A queue entry is 64 bits:
-// tile [31:0], layer [47:32], the run's epoch [63:56] (a child record's entries carry the child's home queue in [55:48]).  An entry left over from an earlier run never
-// matches the current epoch, so the queues need no clearing and a poll can never mistake an old
-// entry for a new one; carrying the layer saves the consumer a dependent lookup.  All writes are
-// device-scope (write-through) stores, the same path the persistent kernel's polls and atomics use.
+// tile [31:0], layer [47:32], the run's epoch [63:48] (a child record's entries carry the child's home queue in [55:48] instead).
+// An entry left over from an earlier run does not match the current epoch, so a poll cannot mistake an old entry for
+// a new one and a run does not clear the queues.  Which slots a run rewrites depends on its grid, its flags and the
+// queue grouping (kept tiles never enter a queue), so a slot may keep an old entry over many runs: the host clears
+// all queues whenever the epoch wraps around and whenever one of those settings differs from the graph's previous
+// run (clear_queue_kernel), which is what makes "an old entry never matches" hold.  Carrying the layer saves the
+// consumer a dependent lookup.  All writes are device-scope (write-through) stores, the same path the persistent
+// kernel's polls and atomics use.
+#define EPOCH_SHIFT 48
+#define EPOCH_MAX 0xffffu
 #define QUEUE_ID_BITS 24
 #define QUEUE_ID_MASK ((1u << QUEUE_ID_BITS) - 1u)
 #define MAX_GRAPH_LAYERS 65535u
 __device__ __forceinline__ qentry_t make_entry (uint32_t epoch, uint32_t layer, uint32_t tile)
 {
-    return ((qentry_t)epoch << 56) | ((qentry_t)layer << 32) | tile;
+    return ((qentry_t)epoch << EPOCH_SHIFT) | ((qentry_t)layer << 32) | tile;
 }
 // Ticket t of a queue lives in that queue's entry (t % QUEUE_LANES) * row + t / QUEUE_LANES, row >= QUEUE_MIN_ROW
 // entries: the workgroups that wait hold consecutive tickets and each polls its entry, so neighbouring tickets
@@ -133,6 +152,14 @@ static uint32_t queue_row (uint32_t capacity)
 }
 
 struct queue_counts_t { uint32_t n[NUM_QUEUES]; };
+
+// every entry of every queue back to "no run's" (epoch 0), see make_entry
+__global__ void clear_queue_kernel (qentry_t *queue, size_t entries)
+{
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < entries; i += step)
+        __hip_atomic_store (&queue[i], (qentry_t)0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 // nq_mask = number of queues in use - 1 (7 or 0); root_pos / counts describe the 8-queue seeding
 __global__ void arm_kernel (uint32_t *dep, const uint32_t *num_parents, qentry_t *queue, uint32_t *ran,
@@ -164,22 +191,25 @@ __global__ void arm_kernel (uint32_t *dep, const uint32_t *num_parents, qentry_t
         __hip_atomic_store (&state[ST_TWICE], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store (&state[ST_SINKS], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    if (i < MAX_GROUPS) __hip_atomic_store (&state[ST_GROUP (i)], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 struct dataflow_args_t
 {
     const aspen_hip_layer_t *layers;
     const uint32_t *ninst_layer, *ninst_home, *child_off, *child_idx;
-    const qentry_t *child_rec;      // [num_ninst][CHILD_REC]: [0] = number of children, then the first CHILD_REC-1 as (home << 48 | layer << 32 | tile)
+    const qentry_t *child_rec;      // [num_ninst][CHILD_REC]: [0] = number of children | the tile's group << 32, then the first CHILD_REC-1 as (home << 48 | layer << 32 | tile)
     qentry_t *queue;
     uint32_t *dep, *state, *ran;
     uint32_t *arrivals;             // per split-K group (at its first tile's index): slices that have finished, see run_tile
-    uint32_t *host_abort;
+    uint32_t *host_abort;           // pinned host block, see HOST_DONE_WORD
+    const uint32_t *group_sinks;    // per co-scheduled network: its tiles without children
+    uint32_t num_groups, run_serial;
     unsigned long long *trace;      // per-tile start / end time stamps when ASPEN_HIP_FLAG_TRACE is set
     unsigned long long *prof;       // 8 counters of summed 100 MHz ticks, see aspen_hip_dataflow_profile
     uint32_t num_ninst;
     uint32_t num_sinks;             // tiles without children: when all of them have finished, so has every tile
-    uint32_t epoch;                 // 1..255, tag of this run's queue entries
+    uint32_t epoch;                 // 1..EPOCH_MAX, tag of this run's queue entries
     uint32_t flags;                 // ASPEN_HIP_FLAG_*
     uint32_t queue_row;             // see queue_slot
     uint32_t queue_cap;             // tickets a queue can hold
@@ -203,7 +233,7 @@ __device__ __forceinline__ qentry_t wait_for_slot (const dataflow_args_t &a, uin
     for (;;)
     {
         const qentry_t e = __hip_atomic_load (&a.queue[queue_slot (q, ticket, a.queue_row)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if ((uint32_t)(e >> 56) == a.epoch) return e;
+        if ((uint32_t)(e >> EPOCH_SHIFT) == a.epoch) return e;
         ++spins;
         if ((spins & 63) == 0 && __hip_atomic_load (&a.state[ST_ABORT], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return QENTRY_EMPTY;
         if (spins > a.spin_limit)
@@ -352,8 +382,19 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
         if (listed == 0u)
         {
             // a tile without children (no hand-off, so wavefront 1 is popping meanwhile): was it the run's last?
+            // Its network's last?  Then that network is complete (every tile has a descendant without children, and this
+            // tile's stores were acknowledged above): the host word of the network is raised, the counterpart of the
+            // reference's per-nasm completion signal (src/dse.c:94-105).  The network that completes last ends the run.
             uint32_t last = 0;
-            if (lane == 0) last = __hip_atomic_fetch_add (&a.state[ST_SINKS], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u == a.num_sinks;
+            if (lane == 0)
+            {
+                const uint32_t grp = (uint32_t)(rec >> 32);
+                if (__hip_atomic_fetch_add (&a.state[ST_GROUP (grp)], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u == a.group_sinks[grp])
+                {
+                    __hip_atomic_store (a.host_abort + HOST_DONE_WORD + grp, a.run_serial, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    last = __hip_atomic_fetch_add (&a.state[ST_SINKS], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u == a.num_groups;
+                }
+            }
             if (__shfl (last, 0, 64))
             {
                 // the run is over and nothing will be pushed any more: tell everyone who waits, this workgroup's
@@ -490,6 +531,7 @@ extern "C" int aspen_hip_init (void)
     CHECK (hipGetDeviceProperties (&prop, 0));
     g_num_cu = prop.multiProcessorCount;
     CHECK (hipStreamCreate (&g_stream));
+    CHECK (hipStreamCreate (&g_side_stream));
     for (int i = 0; i < NUM_EVENTS; i++) CHECK (hipEventCreate (&g_events[i]));
     CHECK (hipFuncSetAttribute ((const void *)layer_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
     CHECK (hipFuncSetAttribute ((const void *)sgemm_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
@@ -893,7 +935,18 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     g->cached_loads = lines_have_one_producer (layers, num_layers) && getenv ("ASPEN_GPU_COHERENT_LOADS") == nullptr;
     g->num_layers = num_layers; g->num_ninst = num_ninst; g->num_roots = num_roots; g->num_edges = num_edges;
     g->features = graph_features (layers, num_layers);
-    for (uint32_t t = 0; t < num_ninst; t++) g->num_sinks += child_off[t + 1] == child_off[t];
+    uint32_t group_sinks[MAX_GROUPS] = {0};
+    for (uint32_t l = 0; l < num_layers; l++)
+    {
+        if (layers[l].graph_id >= MAX_GROUPS) { snprintf (g_err, sizeof (g_err), "layer %u: graph_id %u, at most %u networks share a run", l, layers[l].graph_id, MAX_GROUPS); free (g); return nullptr; }
+        if (layers[l].graph_id + 1 > g->num_groups) g->num_groups = layers[l].graph_id + 1;
+    }
+    for (uint32_t t = 0; t < num_ninst; t++)
+        if (child_off[t + 1] == child_off[t]) { g->num_sinks++; group_sinks[layers[ninst_layer[t]].graph_id]++; }
+    // (a group without tiles would never report: it counts as finished from the start)
+    uint32_t live_groups = 0;
+    for (uint32_t i = 0; i < g->num_groups; i++) live_groups += group_sinks[i] != 0;
+    g->d_group_sinks = upload (group_sinks, MAX_GROUPS);
     {
         // default grid: a whole number of workgroups per compute unit, no more than the graph can keep busy
         const double par = graph_parallelism (layers, ninst_layer, child_off, child_idx, num_ninst);
@@ -940,7 +993,7 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
             for (uint32_t t = 0; t < num_ninst; t++)
             {
                 const uint32_t c0 = child_off[t], n = child_off[t + 1] - c0;
-                rec[(size_t)t * CHILD_REC] = n;
+                rec[(size_t)t * CHILD_REC] = n | ((qentry_t)layers[ninst_layer[t]].graph_id << 32);
                 for (uint32_t c = 0; c < n && c < CHILD_REC - 1; c++)
                 {
                     const uint32_t ch = child_idx[c0 + c];
@@ -954,12 +1007,13 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
         free (home); free (pos); free (rec);
     }
     g->d_ran = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
-    g->d_state = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * ST_WORDS);
+    g->d_state = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * ST_ALL_WORDS);
     g->d_arrivals = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * (num_ninst + 1));
     g->d_prof = (unsigned long long *)aspen_hip_alloc (sizeof (unsigned long long) * 16);
-    if (hipHostMalloc ((void **)&g->h_abort, 64, hipHostMallocDefault) != hipSuccess) g->h_abort = nullptr;
-    else *g->h_abort = 0;
-    if (!g->h_abort || !g->d_layers || !g->d_ninst_layer || !g->d_num_parents || !g->d_child_off || !g->d_child_idx || !g->d_roots
+    if (hipHostMalloc ((void **)&g->h_abort, sizeof (uint32_t) * (HOST_DONE_WORD + MAX_GROUPS), hipHostMallocDefault) != hipSuccess) g->h_abort = nullptr;
+    else memset (g->h_abort, 0, sizeof (uint32_t) * (HOST_DONE_WORD + MAX_GROUPS));
+    g->live_groups = live_groups;
+    if (!g->h_abort || !g->d_group_sinks || !g->d_layers || !g->d_ninst_layer || !g->d_num_parents || !g->d_child_off || !g->d_child_idx || !g->d_roots
         || !g->d_dep || !g->d_queue || !g->d_ran || !g->d_state || !g->d_child_rec || !g->d_ninst_home || !g->d_root_pos || !g->d_arrivals || !g->d_prof)
     {
         aspen_hip_graph_destroy (g);
@@ -974,7 +1028,7 @@ extern "C" void aspen_hip_graph_destroy (aspen_hip_graph_t *g)
     (void)hipStreamSynchronize (g_stream);
     aspen_hip_free (g->d_layers); aspen_hip_free (g->d_ninst_layer); aspen_hip_free (g->d_num_parents);
     aspen_hip_free (g->d_child_off); aspen_hip_free (g->d_child_idx); aspen_hip_free (g->d_roots); aspen_hip_free (g->d_ninst_home); aspen_hip_free (g->d_root_pos);
-    aspen_hip_free (g->d_child_rec); aspen_hip_free (g->d_dep); aspen_hip_free (g->d_queue); aspen_hip_free (g->d_ran); aspen_hip_free (g->d_arrivals); aspen_hip_free (g->d_state); aspen_hip_free (g->d_prof); aspen_hip_free (g->d_trace);
+    aspen_hip_free (g->d_child_rec); aspen_hip_free (g->d_dep); aspen_hip_free (g->d_queue); aspen_hip_free (g->d_ran); aspen_hip_free (g->d_arrivals); aspen_hip_free (g->d_state); aspen_hip_free (g->d_prof); aspen_hip_free (g->d_trace); aspen_hip_free (g->d_group_sinks);
     if (g->h_abort) (void)hipHostFree (g->h_abort);
     free (g->h_layers);
     free (g);
@@ -997,6 +1051,7 @@ static void launch_layer (const aspen_hip_graph_t *g, uint32_t l)
 extern "C" int aspen_hip_run_layers (aspen_hip_graph_t *g, uint32_t first_layer, uint32_t last_layer)
 {
     if (!g || first_layer > last_layer || last_layer >= g->num_layers) { snprintf (g_err, sizeof (g_err), "run_layers: bad range"); return -1; }
+    g->last_run_dataflow = 0;
     for (uint32_t l = first_layer; l <= last_layer; l++)
     {
         const aspen_hip_layer_t &L = g->h_layers[l];
@@ -1013,7 +1068,7 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     if (g->num_ninst == 0) return 0;
     if (workgroups == 0) workgroups = g->default_workgroups;
     if (workgroups > QUEUE_SLACK) workgroups = QUEUE_SLACK;         // every waiting workgroup must find a "leave" entry within its queue
-    g->epoch = g->epoch % 255u + 1u;
+    g->epoch = g->epoch % EPOCH_MAX + 1u;
     // one queue per XCD on request, when every XCD gets the same number of workgroups (workgroup b runs on XCD b % 8)
     static const bool xcd_queues_env = getenv ("ASPEN_GPU_XCD_QUEUES") != nullptr;
     const bool xcd_queues = xcd_queues_env || (g_flags & ASPEN_HIP_FLAG_XCD_QUEUES);
@@ -1035,6 +1090,19 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
         g->root_shift = nq_shift;
     }
     for (uint32_t q = 0; q < NUM_QUEUES; q++) counts.n[q] = g->root_count[q];
+    {
+        // The slots a run rewrites depend on the grid (leave entries), the hand-off (kept tiles take no slot) and the
+        // queue grouping.  A slot an earlier run with other settings wrote could otherwise survive until the epoch
+        // comes round again and be taken for an entry of that run.
+        const uint32_t config = workgroups ^ (nq_mask << 16) ^ (nq_shift << 20) ^ ((g_flags & (ASPEN_HIP_FLAG_NO_HANDOFF | ASPEN_HIP_FLAG_XCD_QUEUES | ASPEN_HIP_FLAG_SKIP_TILES)) << 24);
+        if (g->epoch == 1u || config != g->queue_config)
+        {
+            const size_t entries = (size_t)NUM_QUEUES * QUEUE_LANES * g->queue_row;
+            hipLaunchKernelGGL (clear_queue_kernel, dim3 (stream_grid (entries)), dim3 (WG_THREADS), 0, g_stream, g->d_queue, entries);
+            CHECK (hipGetLastError ());
+        }
+        g->queue_config = config;
+    }
     hipLaunchKernelGGL (arm_kernel, dim3 ((g->num_ninst + 255) / 256), dim3 (256), 0, g_stream,
         g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->d_ninst_layer, g->d_ninst_home, g->d_root_pos, counts,
         g->num_ninst, g->num_roots, g->d_state, g->epoch, g->queue_row, nq_mask, nq_shift, g->d_arrivals);
@@ -1042,6 +1110,9 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     dataflow_args_t a;
     a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.ninst_home = g->d_ninst_home; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx; a.child_rec = g->d_child_rec;
     a.dep = g->d_dep; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran; a.arrivals = g->d_arrivals; a.prof = g->d_prof; a.host_abort = g->h_abort;
+    g->run_serial = g->run_serial + 1u ? g->run_serial + 1u : 1u;
+    g->last_run_dataflow = 1;
+    a.group_sinks = g->d_group_sinks; a.num_groups = g->live_groups; a.run_serial = g->run_serial;
     if ((g_flags & ASPEN_HIP_FLAG_TRACE) && !g->d_trace)
     {
         g->d_trace = (unsigned long long *)aspen_hip_alloc (sizeof (unsigned long long) * 2 * (size_t)g->num_ninst);
@@ -1106,6 +1177,39 @@ extern "C" int aspen_hip_graph_sync (aspen_hip_graph_t *g)
     }
     return 0;
 }
+
+extern "C" int aspen_hip_graph_group_done (aspen_hip_graph_t *g, uint32_t group)
+{
+    if (!g || group >= g->num_groups || !g->last_run_dataflow) return -1;
+    return __atomic_load_n (&g->h_abort[HOST_DONE_WORD + group], __ATOMIC_ACQUIRE) == g->run_serial ? 1 : 0;
+}
+
+extern "C" int aspen_hip_graph_wait_group (aspen_hip_graph_t *g, uint32_t group)
+{
+    if (aspen_hip_init ()) return -1;
+    if (!g || group >= g->num_groups || !g->last_run_dataflow) return -1;
+    for (;;)
+    {
+        // the word is written by the device into pinned host memory: a few hundred polls between two looks at the stream
+        for (int spin = 0; spin < 256; spin++)
+        {
+            if (__atomic_load_n (&g->h_abort[HOST_DONE_WORD + group], __ATOMIC_ACQUIRE) == g->run_serial) return 0;
+            __builtin_ia32_pause ();
+        }
+        if (__atomic_load_n (&g->h_abort[0], __ATOMIC_ACQUIRE) != 0) return 0;      // given up: aspen_hip_graph_sync reports it
+        if (hipStreamQuery (g_stream) == hipSuccess) return 0;                       // the run is over (a group without tiles never reports)
+    }
+}
+
+extern "C" int aspen_hip_d2h_side (void *dst, const void *src, size_t bytes)
+{
+    if (aspen_hip_init ()) return -1;
+    CHECK (hipMemcpyAsync (dst, src, bytes, hipMemcpyDeviceToHost, g_side_stream));
+    CHECK (hipStreamSynchronize (g_side_stream));
+    return 0;
+}
+
+extern "C" void aspen_hip_graph_debug_set_epoch (aspen_hip_graph_t *g, uint32_t epoch) { if (g) g->epoch = epoch % EPOCH_MAX; }
 
 extern "C" int aspen_hip_idle (void)
 {

@@ -82,6 +82,13 @@ int aspen_rpool_dataflow_trace (rpool_t *rp, uint64_t *start_end)
     return aspen_hip_dataflow_trace (rp->graph, start_end, aspen_rpool_num_ninst (rp));
 }
 
+int aspen_rpool_debug_set_epoch (rpool_t *rp, uint32_t epoch)
+{
+    if (rp == NULL || rp->graph == NULL) return -1;
+    aspen_hip_graph_debug_set_epoch (rp->graph, epoch);
+    return 0;
+}
+
 unsigned int aspen_dnn_device_generation (aspen_dnn_t *dnn) { return dnn ? dnn->dev_generation : 0; }
 
 unsigned int aspen_rpool_num_ninst (rpool_t *rp)

@@ -103,6 +103,7 @@ struct nasm_t
     size_t arena_floats;
     float *d_arena;
     rpool_t *rpool;                          /* pool this nasm is attached to */
+    unsigned int pool_slot;                  /* its number among the pool's nasms in the merged device graph (aspen_hip_layer_t.graph_id) */
     int armed;                               /* input present and counters to be re-armed at the next run */
     int completed;                           /* 0 not run, 1 completed, 2 in flight, 3 the run failed (stall, launch error) */
 };
@@ -140,7 +141,7 @@ int aspen_layer_table_operand (const aspen_layer_t *layer);     /* K axis throug
 unsigned int aspen_layer_kiters (const aspen_layer_t *layer);   /* K slices of 32 of a contraction layer's device layout */
 /* nasm.c */
 int aspen_nasm_to_device (nasm_t *nasm);
-int aspen_nasm_fill_device_layers (nasm_t *nasm, aspen_hip_layer_t *dst, uint32_t ninst_base);
+int aspen_nasm_fill_device_layers (nasm_t *nasm, aspen_hip_layer_t *dst, uint32_t ninst_base, uint32_t graph_id);
 unsigned int aspen_ld_for_rows (unsigned int rows);
 
 int aspen_keep_layer_outputs_enabled (void);   /* ext.c: see aspen_keep_layer_outputs */

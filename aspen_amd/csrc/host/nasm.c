@@ -708,8 +708,9 @@ int aspen_nasm_to_device (nasm_t *nasm)
     return 0;
 }
 
-/* Device descriptors of all layers, tile indices shifted by ninst_base (position inside a merged graph). */
-int aspen_nasm_fill_device_layers (nasm_t *nasm, aspen_hip_layer_t *dst, uint32_t ninst_base)
+/* Device descriptors of all layers, tile indices shifted by ninst_base (position inside a merged graph);
+   graph_id = which of the merged graphs this one is (the engine reports each one's completion separately). */
+int aspen_nasm_fill_device_layers (nasm_t *nasm, aspen_hip_layer_t *dst, uint32_t ninst_base, uint32_t graph_id)
 {
     for (unsigned int l = 0; l < nasm->num_ldata; l++)
     {
@@ -719,6 +720,7 @@ int aspen_nasm_fill_device_layers (nasm_t *nasm, aspen_hip_layer_t *dst, uint32_
         aspen_hip_layer_t *d = &dst[l];
         memset (d, 0, sizeof (*d));
         d->type = L->type; d->act = L->activation; d->variant = ld->variant;
+        d->graph_id = graph_id;
         d->M = ld->out_mat_dims[OUT_H]; d->N = ld->out_mat_dims[OUT_W]; d->ld = ld->out_mat_stride;
         d->tile_m = ld->tile_dims[OUT_H]; d->tile_n = ld->tile_dims[OUT_W];
         d->tiles_m = ld->tiles_h; d->tiles_n = ld->tiles_w;

@@ -160,7 +160,8 @@ static int rebuild_graph (rpool_t *rp)
     {
         nasm_t *g = rp->nasms[i];
         if (aspen_nasm_to_device (g)) { rc = -1; break; }
-        aspen_nasm_fill_device_layers (g, L + lbase, nbase);
+        g->pool_slot = i;
+        aspen_nasm_fill_device_layers (g, L + lbase, nbase, i);
         for (uint32_t t = 0; t < g->num_ninst; t++)
         {
             nl[nbase + t] = lbase + g->ninst_ldata[t];
@@ -288,16 +289,38 @@ void dse_group_stop (dse_group_t *dse_group)
     finish (dse_group->rpool);
 }
 
+/* Per-nasm completion (reference src/dse.c:94-105: the thread that finishes a nasm's last layer sets
+   nasm->completed and signals that nasm's waiter, whatever the other nasms of the pool are doing; waiter
+   :279-289).  In a dataflow run the tile that finishes a nasm raises a host word for it, so a nasm can be
+   waited for and read out while the persistent kernel is still working on the others.  One launch per layer
+   has no such signal: there a nasm is complete when the stream has drained. */
+static int nasm_done_on_device (const nasm_t *nasm)
+{
+    const rpool_t *rp = nasm->rpool;
+    return rp != NULL && rp->running && rp->graph != NULL && aspen_hip_graph_group_done (rp->graph, nasm->pool_slot) == 1;
+}
+
 void dse_wait_for_nasm_completion (nasm_t *nasm)
 {
     if (nasm == NULL) return;
-    if (nasm->completed == 2) finish (nasm->rpool);
+    if (nasm->completed != 2) return;
+    rpool_t *rp = nasm->rpool;
+    if (rp != NULL && rp->running && rp->graph != NULL && aspen_hip_graph_wait_group (rp->graph, nasm->pool_slot) == 0 && nasm_done_on_device (nasm))
+    {
+        nasm->completed = 1;        /* the others stay in flight; dse_group_stop (or a wait for them) drains the run */
+        return;
+    }
+    finish (rp);
 }
 
 unsigned int dse_check_nasm_completion (nasm_t *nasm)
 {
     if (nasm == NULL) return 0;
-    if (nasm->completed == 2 && aspen_hip_idle () == 1) finish (nasm->rpool);
+    if (nasm->completed == 2)
+    {
+        if (aspen_hip_idle () == 1) finish (nasm->rpool);
+        else if (nasm_done_on_device (nasm)) nasm->completed = 1;
+    }
     return nasm->completed == 1;
 }
 
@@ -352,7 +375,7 @@ static ssize_t get_ldata_output (nasm_t *nasm, unsigned int ldata_idx, LAYER_PAR
     if (nasm == NULL || ldata_idx >= nasm->num_ldata) { ERROR_PRTF ("Error in get_ldata_output: ldata is NULL.\n"); return -1; }
     if (out_ptr == NULL) { ERROR_PRTF ("Error in get_ldata_output: out_ptr is NULL.\n"); return -1; }
     if (nasm->d_arena == NULL) { ERROR_PRTF ("Error in get_ldata_output: nasm has not been run.\n"); return -1; }
-    if (nasm->completed == 2) finish (nasm->rpool);
+    if (nasm->completed == 2) dse_wait_for_nasm_completion (nasm);
     if (nasm->completed == 3 && ldata_idx != 0)
     {
         ERROR_PRTF ("Error in get_ldata_output: the last run of this nasm failed; its layers hold no valid result.\n");
@@ -369,8 +392,24 @@ static ssize_t get_ldata_output (nasm_t *nasm, unsigned int ldata_idx, LAYER_PAR
     const size_t H = ld->out_mat_dims[OUT_H], W = ld->out_mat_dims[OUT_W];
     float *dense = malloc (H * W * sizeof (float));
     if (dense == NULL) return -1;
-    /* padding rows stripped on the device, one contiguous transfer */
-    if (aspen_hip_dense_device_to_host (dense, nasm->d_arena + ld->out_mat_offset, ld->out_mat_stride, (uint32_t)H, W))
+    int rc;
+    if (nasm->rpool != NULL && nasm->rpool->running && aspen_hip_idle () != 1)
+    {
+        /* this nasm has finished but the persistent kernel is still running others: anything enqueued on its stream
+           (also the kernel that strips the padding rows) would wait for the whole run.  The matrix is copied as it is
+           on a second stream and the padding stripped here. */
+        const size_t ldm = ld->out_mat_stride;
+        float *raw = ldm == H ? dense : malloc (W * ldm * sizeof (float));
+        rc = raw == NULL ? -1 : aspen_hip_d2h_side (raw, nasm->d_arena + ld->out_mat_offset, W * ldm * sizeof (float));
+        if (raw != NULL && raw != dense)
+        {
+            for (size_t c = 0; c < W && !rc; c++) memcpy (dense + c * H, raw + c * ldm, H * sizeof (float));
+            free (raw);
+        }
+    }
+    else    /* padding rows stripped on the device, one contiguous transfer */
+        rc = aspen_hip_dense_device_to_host (dense, nasm->d_arena + ld->out_mat_offset, ld->out_mat_stride, (uint32_t)H, W);
+    if (rc)
     {
         ERROR_PRTF ("Error in get_ldata_output: download failed: %s\n", aspen_hip_last_error ());
         free (dense);

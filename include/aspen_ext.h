@@ -69,6 +69,9 @@ int aspen_rpool_dataflow_profile (rpool_t *rpool, uint64_t ticks[16], int reset)
 /* start / end time stamps (100 MHz) of every tile of the pool's last run made with ASPEN_HIP_FLAG_TRACE;
    start_end holds 2 * aspen_rpool_num_ninst values, tiles in pool order (nasms in attachment order) */
 int aspen_rpool_dataflow_trace (rpool_t *rpool, uint64_t *start_end);
+/* Test hook: the tag the pool's next dataflow run derives its queue-entry tag from (aspen_hip_graph_debug_set_epoch);
+   returns -1 when the pool has no device graph yet. */
+int aspen_rpool_debug_set_epoch (rpool_t *rpool, uint32_t epoch);
 /* tiles in the pool's merged graph */
 unsigned int aspen_rpool_num_ninst (rpool_t *rpool);
 

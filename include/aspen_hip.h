@@ -81,6 +81,8 @@ typedef struct aspen_hip_layer_t
        the bias, activates and writes the output; only it releases the group's children */
     uint32_t splits, kiters_per_split;
     uint32_t fuse_discard;   /* 1 (only with fuse_out): the layer's own, pre-shortcut matrix `out` is not written */
+    uint32_t graph_id;       /* which of the co-scheduled networks of one engine run the layer belongs to (0 .. 63): the run
+                                reports each network's completion separately, see aspen_hip_graph_group_done */
     float *partial;
     float *out;
     const float *in0;        /* PARENT_0 */
@@ -197,6 +199,23 @@ int aspen_hip_sync (void);
 int aspen_hip_graph_sync (aspen_hip_graph_t *graph);
 /* 1 when everything enqueued so far has finished, 0 when still running */
 int aspen_hip_idle (void);
+/* Completion of ONE of the networks co-scheduled in a dataflow run (the layers with graph_id == group), the
+   counterpart of the reference marking a nasm completed when its own last layer has finished while other
+   nasms are still running (reference src/dse.c:94-105, waiter :279-289).  The tile that finishes a network
+   (its last tile without children) raises a pinned host word, so neither call touches the stream.
+   group_done: 1 = finished in the graph's last dataflow run, 0 = not yet, -1 = unknown (no such group, or the
+   last run was one launch per layer: ask aspen_hip_idle / aspen_hip_graph_sync).
+   wait_group blocks until the group has finished, the whole run has ended, or the run was given up; it returns 0,
+   or -1 for an unknown group (the caller still learns of a stalled run from aspen_hip_graph_sync). */
+int aspen_hip_graph_group_done (aspen_hip_graph_t *graph, uint32_t group);
+int aspen_hip_graph_wait_group (aspen_hip_graph_t *graph, uint32_t group);
+/* aspen_hip_d2h on a second stream: does not wait for work enqueued on the library's main stream, so a network
+   that has finished can be read out while the persistent kernel still runs the others.  Only memory whose
+   producers have finished may be read this way (tiles write through to memory before they are published). */
+int aspen_hip_d2h_side (void *dst, const void *src, size_t bytes);
+/* Test hook: sets the tag the graph's next dataflow run derives its queue-entry tag from (tags cycle through
+   1 .. 65535 and the queues are cleared when they wrap). */
+void aspen_hip_graph_debug_set_epoch (aspen_hip_graph_t *graph, uint32_t epoch);
 /* Counters of the last dataflow run (kept under ASPEN_HIP_FLAG_COUNT_TILES): tiles executed, tiles executed
    more than once, and the abort flag.  That no tile starts before its parents have ended is checked from
    the time stamps of a traced run (ASPEN_HIP_FLAG_TRACE), not counted on the device. */

@@ -260,6 +260,42 @@ def test_engine_rearm_many_runs(gpu):
         net.close()
 
 
+def test_queue_entries_of_earlier_runs_are_never_taken(gpu):
+    """Which queue slots a run rewrites depends on its flags (hand-off, per-XCD queues) and its grid, and entries carry
+    a 16-bit run tag: a slot written under one setting must not be taken for a fresh entry when the tag comes round
+    again.  Runs alternate the settings for several hundred runs, then cross the tag's wrap-around; every run executes
+    every tile once and reproduces the first run bit for bit."""
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()["gpt_mini_b2_s20"])
+    net = H.GpuNet(cfg, tens, batch, seq, min_ninst=64, mode=api.MODE_DATAFLOW)
+    L = api.lib()
+    try:
+        first = None
+        settings = [(0, 0), (16, 0), (32, 256), (0, 64), (32 | 16, 512)]
+
+        def run_and_check(rep):
+            nonlocal first
+            flags, wgs = settings[rep % len(settings)]
+            L.aspen_hip_set_flags(2 | flags)
+            L.aspen_dse_group_set_workgroups(net.dse.h, wgs)
+            net.run(x if first is None else None)
+            st = net.rpool.run_stats()
+            assert st == {"executed": net.nasm.num_ninst, "double_runs": 0, "aborted": 0}, (rep, flags, wgs, st)
+            out = net.layer(net.nasm.num_ldata - 1)
+            if first is None:
+                first = out
+            assert np.array_equal(first, out), f"run {rep} (flags {flags}, {wgs} workgroups) differs from run 0"
+
+        for rep in range(300):
+            run_and_check(rep)
+        # one run with per-XCD queues right before the wrap, plain runs across it, the same setting again after it
+        net.rpool.debug_set_epoch(65533)
+        for rep in (2, 0, 0, 0, 2, 1, 4, 3):
+            run_and_check(rep)
+    finally:
+        L.aspen_hip_set_flags(2)
+        net.close()
+
+
 FULL = ["resnet50_b1", "resnet50_b32", "vgg16_b32", "bert_base_b8_s128", "gpt2_b4_s512", "yolov3_b1"]
 
 
@@ -409,6 +445,31 @@ def test_co_inference_resnet50_vgg16_b16(gpu):
         for _, net, _ in nets:
             dse.wait(net.nasm)
         dse.stop()
+        # Completion is per nasm (reference src/dse.c:94-105, waiter :279-289): in a second run the wait for ResNet-50
+        # (a quarter of the work) returns while the persistent kernel is still running VGG-16, and ResNet-50's result,
+        # read at that moment, is already the final one.
+        pool.reset_queue()
+        for _, net, _ in nets:
+            pool.reset_nasm(net.nasm)
+        import time
+        t0 = time.perf_counter()
+        dse.run()
+        resnet, vgg = nets[0][1].nasm, nets[1][1].nasm
+        assert not dse.check(resnet)
+        dse.wait(resnet)
+        t_resnet = time.perf_counter() - t0
+        still_running = api.lib().aspen_hip_idle() == 0
+        assert dse.check(resnet)
+        early = resnet.result()
+        running_after_readout = api.lib().aspen_hip_idle() == 0
+        dse.wait(vgg)
+        t_vgg = time.perf_counter() - t0
+        dse.stop()
+        print(f"ResNet-50 B16 complete after {t_resnet * 1e3:.2f} ms (kernel still running: {still_running}, after the read-out: "
+              f"{running_after_readout}), VGG-16 B16 after {t_vgg * 1e3:.2f} ms", flush=True)
+        assert still_running, "ResNet-50's completion was only reported when the whole run was over"
+        assert t_resnet < t_vgg
+        assert np.array_equal(early, resnet.result()), "the result read while the kernel was running differs from the final one"
         st = pool.run_stats()
         assert st == {"executed": sum(n.nasm.num_ninst for _, n, _ in nets), "double_runs": 0, "aborted": 0}, st
         for name, net, layers in nets:
