@@ -79,6 +79,7 @@ def lib() -> C.CDLL:
         # aspen_ext.h
         "aspen_dse_group_set_mode": (None, [_vp, C.c_int]),
         "aspen_dse_group_last_mode": (C.c_int, [_vp]),
+        "aspen_dse_group_last_run_ordered": (C.c_int, [_vp]),
         "aspen_dse_group_set_spin_limit": (None, [_vp, C.c_uint64]),
         "aspen_dse_group_set_workgroups": (None, [_vp, C.c_uint]),
         "aspen_keep_layer_outputs": (None, [C.c_int]),
@@ -98,6 +99,7 @@ def lib() -> C.CDLL:
         "aspen_rpool_dataflow_profile": (C.c_int, [_vp, C.POINTER(C.c_uint64), C.c_int]),
         "aspen_rpool_dataflow_trace": (C.c_int, [_vp, _vp]),
         "aspen_rpool_debug_set_epoch": (C.c_int, [_vp, C.c_uint32]),
+        "aspen_rpool_dataflow_trace_phases": (C.c_int, [_vp, _vp]),
         # aspen_hip.h
         "aspen_hip_init": (C.c_int, []),
         "aspen_hip_last_error": (C.c_char_p, []),
@@ -283,6 +285,14 @@ class RPool:
             raise RuntimeError("no dataflow trace: " + lib().aspen_hip_last_error().decode())
         return t
 
+    def dataflow_trace_phases(self) -> np.ndarray:
+        """[tiles][2] end-of-K-loop / stores-issued stamps of the contraction tiles of the same traced run."""
+        n = lib().aspen_rpool_num_ninst(self.h)
+        t = np.zeros((n, 2), dtype=np.uint64)
+        if lib().aspen_rpool_dataflow_trace_phases(self.h, t.ctypes.data):
+            raise RuntimeError("no dataflow trace: " + lib().aspen_hip_last_error().decode())
+        return t
+
     def profile_layers(self, num_layers: int, iters: int = 5) -> np.ndarray:
         """Per-layer kernel time in ms (layer-launch mode, HIP events); the pool must have run once."""
         ms = np.zeros(num_layers, dtype=np.float32)
@@ -310,6 +320,9 @@ class DseGroup:
     def last_mode(self) -> int:
         """The engine the last run() used: MODE_LAYERS or MODE_DATAFLOW (-1 before the first run)."""
         return lib().aspen_dse_group_last_mode(self.h)
+
+    def last_run_ordered(self) -> bool:
+        return lib().aspen_dse_group_last_run_ordered(self.h) == 1
 
     def set_rpool(self, rpool: RPool):
         lib().dse_group_set_rpool(self.h, rpool.h)

@@ -39,6 +39,7 @@ typedef unsigned long long qentry_t;      // ready-queue entry / child-record en
 #define HOST_DONE_WORD 16u      // pinned host block: [0] abort flag, [HOST_DONE_WORD + g] = serial of the last run group g finished in
 #define NUM_EVENTS 16
 #define DEFAULT_SPIN_LIMIT (1ull << 26)
+#define ORDERED_BELOW 128.0     // average parallelism (tiles) under which a dataflow run takes its tiles in index order
 
 struct aspen_hip_graph_t
 {
@@ -52,6 +53,8 @@ struct aspen_hip_graph_t
     uint32_t root_shift;            // the XCD grouping (see nq_shift) d_root_pos / root_count were computed for
     uint32_t queue_row, queue_cap;  // see queue_slot
     uint32_t *d_dep;        // remaining-parent counters, re-armed before every dataflow run
+    uint32_t *d_dep_spread; // the same, one per cache line, for ordered runs (allocated at the first one), see dep_slot
+    uint32_t dep_stride;
     qentry_t *d_queue;      // ready queue: slot t is written once, by whoever makes a tile ready
     qentry_t *d_child_rec;  // per tile: child count + its first CHILD_REC-1 children with their layers
     uint32_t *d_state;      // one counter per 128-byte line: [ST_QHEAD (q)] pop tickets, [ST_QTAIL (q)] push cursor of queue q, [ST_DONE] tiles done,
@@ -64,6 +67,8 @@ struct aspen_hip_graph_t
     uint32_t *d_group_sinks;    // per group: its tiles without children
     uint32_t run_serial;    // number of the last dataflow run (never 0): what a group's host word holds once it has finished in that run
     int last_run_dataflow;  // the host words describe the last run
+    int last_run_ordered;   // the last dataflow run took its tiles in index order (no ready queue)
+    int prefer_ordered;     // -1: decided from the graph's parallelism; 0 / 1: the caller's choice, see aspen_hip_graph_set_ordered
     unsigned features;      // TILES_* bits of the tile kinds the graph contains: picks the persistent kernel's variant
     uint32_t epoch;         // tag of the last run's queue entries, cycles 1..EPOCH_MAX
     uint32_t queue_config;  // grid, flags and queue grouping of the last run (they decide which queue slots a run rewrites), see run_dataflow
@@ -153,6 +158,16 @@ static uint32_t queue_row (uint32_t capacity)
 
 struct queue_counts_t { uint32_t n[NUM_QUEUES]; };
 
+// Where tile id's dependency counter lives.  stride = 0: dep[id] (the counters of a layer's tiles share cache lines, which
+// is what the countdowns of a full device like best).  Ordered mode gives every counter a 128-byte line of its own and
+// puts neighbouring tiles' counters `stride` words (at least 4 KiB) apart: there a workgroup POLLS its tile's counter
+// while the tile's parents count it down, and the polls of a level's hundreds of tiles would otherwise all land on
+// the two or three memory channels that hold the level's lines, in front of the very countdowns they wait for.
+__host__ __device__ __forceinline__ size_t dep_slot (uint32_t id, uint32_t stride)
+{
+    return stride ? (size_t)(id & 31u) * stride + (size_t)(id >> 5) * 32u : (size_t)id;
+}
+
 // every entry of every queue back to "no run's" (epoch 0), see make_entry
 __global__ void clear_queue_kernel (qentry_t *queue, size_t entries)
 {
@@ -165,12 +180,12 @@ __global__ void clear_queue_kernel (qentry_t *queue, size_t entries)
 __global__ void arm_kernel (uint32_t *dep, const uint32_t *num_parents, qentry_t *queue, uint32_t *ran,
     const uint32_t *roots, const uint32_t *ninst_layer, const uint32_t *ninst_home, const uint32_t *root_pos, queue_counts_t counts,
     uint32_t num_ninst, uint32_t num_roots, uint32_t *state, uint32_t epoch, uint32_t qrow, uint32_t nq_mask, uint32_t nq_shift,
-    uint32_t *arrivals)
+    uint32_t *arrivals, uint32_t dep_stride)
 {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < num_ninst)
     {
-        __hip_atomic_store (&dep[i], num_parents[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store (&dep[dep_slot (i, dep_stride)], num_parents[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (i < num_roots)
         {
             const uint32_t r = roots[i], q = (ninst_home[r] >> nq_shift) & nq_mask, pos = nq_mask ? root_pos[i] : i;
@@ -205,6 +220,7 @@ struct dataflow_args_t
     uint32_t *host_abort;           // pinned host block, see HOST_DONE_WORD
     const uint32_t *group_sinks;    // per co-scheduled network: its tiles without children
     uint32_t num_groups, run_serial;
+    uint32_t dep_stride;            // ordered mode: see dep_slot (0: counters packed)
     unsigned long long *trace;      // per-tile start / end time stamps when ASPEN_HIP_FLAG_TRACE is set
     unsigned long long *prof;       // 8 counters of summed 100 MHz ticks, see aspen_hip_dataflow_profile
     uint32_t num_ninst;
@@ -255,6 +271,7 @@ struct sched_lds_t
     uint32_t complete;                   // 0: the tile just run was a split-K slice that did not finish its group
     uint32_t may_keep;                   // the tile just run releases children, one of which this workgroup may run next
     uint32_t my_queue;                   // the ready queue this workgroup serves
+    uint32_t next_ordered;               // ordered mode: the tile this workgroup takes next
     unsigned long long t0, ticks[6];     // profiling: last time stamp; tile / drain / scheduling / publish / ticket / slot-wait ticks
     unsigned long long p0, phase[5];     // profiling of contraction tiles: last phase stamp; set-up / K loop / epilogue / split-K ticks
 };
@@ -276,6 +293,9 @@ __device__ void tile_phase_lap (int which)
         const unsigned long long t = wall_clock64 ();
         s_sched.phase[which - 8] += t - s_sched.p0; s_sched.p0 = t;
     }
+    // traced runs also stamp a contraction tile's end of the K loop (9) and end of the epilogue's stores (10, 11)
+    if ((s_sched.a.flags & ASPEN_HIP_FLAG_TRACE) && threadIdx.x == 0 && which >= 9 && which <= 11)
+        s_sched.a.trace[2 * (size_t)s_sched.a.num_ninst + 2 * (size_t)s_sched.tile + (which == 9 ? 0 : 1)] = wall_clock64 ();
 }
 
 // Puts a tile that has become ready into the queue.
@@ -305,11 +325,26 @@ __device__ __forceinline__ void push_ready (const dataflow_args_t &a, uint32_t c
 // workgroup holds at most one ticket, so these are all the slots anyone can still be waiting for.
 // The pop half of a scheduling step, run by one wavefront: draws a ticket and waits for its slot.
 // kept != QUEUE_EMPTY: the tile to run is already known.
+template <bool ORDERED>
 __device__ __forceinline__ void pop_next (const dataflow_args_t &a, uint32_t lane, uint32_t kept, uint32_t kept_layer, bool prof)
 {
     if (lane == 0)
     {
         if (kept != QUEUE_EMPTY) { s_sched.tile = kept; s_sched.layer = kept_layer; }
+        else if (ORDERED)
+        {
+            // ordered mode: workgroup b runs tiles b, b + grid, b + 2 grid, ... (tiles are numbered parents first); whether
+            // a tile is ready is found out by the tile itself, see wait_until_ready.  A fixed assignment, no ticket
+            // counter: with a grid of two workgroups per compute unit the two tiles a compute unit holds are a grid
+            // apart, i.e. in neighbouring dependency levels, so one of them computes while the other is being
+            // prepared, and no two tiles of one level share a matrix pipeline while other units idle.  (Every workgroup
+            // of the grid must be resident: the host clamps the grid to what fits.)
+            const uint32_t ticket = s_sched.next_ordered;
+            s_sched.next_ordered = ticket + gridDim.x;
+            const bool live = ticket < a.num_ninst && __hip_atomic_load (&a.state[ST_ABORT], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0;
+            s_sched.tile = live ? ticket : QUEUE_EMPTY;
+            s_sched.layer = live ? a.ninst_layer[ticket] : 0u;
+        }
         else
         {
             // a ticket is drawn only now, when this workgroup is free.  Drawing it earlier would hide the
@@ -326,6 +361,7 @@ __device__ __forceinline__ void pop_next (const dataflow_args_t &a, uint32_t lan
     }
 }
 
+template <bool ORDERED>
 __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
 {
     const dataflow_args_t &a = s_sched.a;
@@ -336,7 +372,7 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
         // a tile that releases children may keep one of them: then the pop waits for the outcome of the
         // countdown; otherwise wavefront 1 pops while wavefront 0 does the accounting
         if (threadIdx.x == 0)
-            s_sched.may_keep = s_sched.complete && (uint32_t)rec != 0u && !(a.flags & ASPEN_HIP_FLAG_NO_HANDOFF);
+            s_sched.may_keep = !ORDERED && s_sched.complete && (uint32_t)rec != 0u && !(a.flags & ASPEN_HIP_FLAG_NO_HANDOFF);
         // every wave waits until its (write-through, device-coherent) stores have been acknowledged.
         // An explicit wait: a workgroup-scope fence does not have to wait for global stores.
         asm volatile ("s_waitcnt vmcnt(0)" ::: "memory");
@@ -355,7 +391,7 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
         const uint32_t child = (uint32_t)rec, layer = (uint32_t)(rec >> 32) & 0xffffu, home = (uint32_t)(rec >> 48) & 0xffu;
         bool ready = false;
         if (lane >= 1 && lane <= count)
-            ready = __hip_atomic_fetch_sub (&a.dep[child], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 1u;
+            ready = __hip_atomic_fetch_sub (&a.dep[dep_slot (child, ORDERED ? a.dep_stride : 0u)], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 1u;
         if (may_keep)
         {
             // only a child at home in this workgroup's queue is kept
@@ -368,7 +404,7 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
                 ready = ready && (int)lane != keeper;
             }
         }
-        if (ready) push_ready (a, child, layer, home);
+        if (ready && !ORDERED) push_ready (a, child, layer, home);
         if (count > CHILD_REC - 1)
         {
             // more children than the record holds: the rest comes from the CSR lists and goes through the queue
@@ -376,7 +412,7 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
             for (uint32_t c = c0 + lane; c < c1; c += 64)
             {
                 const uint32_t ch = a.child_idx[c];
-                if (__hip_atomic_fetch_sub (&a.dep[ch], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 1u) push_ready (a, ch, a.ninst_layer[ch], a.ninst_home[ch]);
+                if (__hip_atomic_fetch_sub (&a.dep[dep_slot (ch, ORDERED ? a.dep_stride : 0u)], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 1u && !ORDERED) push_ready (a, ch, a.ninst_layer[ch], a.ninst_home[ch]);
             }
         }
         if (listed == 0u)
@@ -395,7 +431,7 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
                     last = __hip_atomic_fetch_add (&a.state[ST_SINKS], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u == a.num_groups;
                 }
             }
-            if (__shfl (last, 0, 64))
+            if (__shfl (last, 0, 64) && !ORDERED)
             {
                 // the run is over and nothing will be pushed any more: tell everyone who waits, this workgroup's
                 // own popping wavefront included
@@ -413,9 +449,9 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
             atomicAdd (&a.state[ST_DONE], 1u);
         }
         if (prof) s_sched.ticks[3] += wall_clock64 () - tp;
-        if (may_keep) pop_next (a, lane, kept, kept_layer, prof);
+        if (may_keep) pop_next<ORDERED> (a, lane, kept, kept_layer, prof);
     }
-    else if (wave == 1 && !may_keep) pop_next (a, lane, QUEUE_EMPTY, 0, prof);
+    else if (wave == 1 && !may_keep) pop_next<ORDERED> (a, lane, QUEUE_EMPTY, 0, prof);
     __syncthreads ();
     const uint32_t next = s_sched.tile;
     prof_lap (2);
@@ -426,7 +462,40 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
 // No cache write-back / invalidate is needed anywhere: tiles store activations with device-scope
 // write-through instructions and load them either coherently (COH = 1) or, when the host has checked
 // that no cache line is shared between producer tiles, through the caches (COH = 2); see ActView.
-template <int COH, unsigned FEAT>
+// Ordered mode: waits until every parent of the tile this workgroup holds has finished (its dependency counter has
+// been counted down to zero).  Called from inside the tile, after the set-up that needs no activation.  Every
+// wavefront polls for itself (one request per poll, the word is the same for all lanes); a wait that exceeds the
+// run's spin limit gives the run up like a wait on a queue slot does: the tile then runs on whatever its parents have
+// written so far, inside its own buffers, and the next scheduling step ends the workgroup.
+__device__ __forceinline__ void wait_until_ready ()
+{
+    const dataflow_args_t &a = s_sched.a;
+    const uint32_t id = __builtin_amdgcn_readfirstlane (s_sched.tile);
+    // one wavefront polls, the others wait at the barrier: every poll is a trip to memory, and a thousand wavefronts
+    // polling at once slow down the very countdowns they are waiting for
+    if (threadIdx.x < 64)
+    {
+        unsigned long long spins = 0;
+        const uint32_t *counter = &a.dep[dep_slot (id, a.dep_stride)];
+        while (__builtin_amdgcn_readfirstlane (__hip_atomic_load (counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) != 0u)
+        {
+            ++spins;
+            if ((spins & 63) == 0 && __hip_atomic_load (&a.state[ST_ABORT], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+            if (spins > a.spin_limit)
+            {
+                __hip_atomic_store (&a.state[ST_ABORT], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store (a.host_abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                break;
+            }
+            __builtin_amdgcn_s_sleep (1);
+        }
+    }
+    __syncthreads ();
+    if ((a.flags & ASPEN_HIP_FLAG_TRACE) && threadIdx.x == 0) a.trace[2 * (size_t)id] = wall_clock64 ();      // a tile "starts" when it may touch its operands
+    if ((a.flags & ASPEN_HIP_FLAG_PROFILE) && threadIdx.x == 0) { const unsigned long long t = wall_clock64 (); s_sched.ticks[5] += t - s_sched.p0; s_sched.p0 = t; }
+}
+
+template <int COH, unsigned FEAT, bool ORDERED = false>
 __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataflow_args_t args)
 {
     extern __shared__ __align__ (16) float smem[];
@@ -438,6 +507,7 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
         for (int i = 0; i < 5; i++) s_sched.phase[i] = 0;
         s_sched.may_keep = 0;
         s_sched.my_queue = ((blockIdx.x & (NUM_QUEUES - 1u)) >> args.nq_shift) & args.nq_mask;
+        s_sched.next_ordered = blockIdx.x;
     }
     __syncthreads ();
     __builtin_amdgcn_s_setprio (TILE_PRIO);
@@ -446,7 +516,7 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
     qentry_t rec = 0;
     for (;;)
     {
-        id = __builtin_amdgcn_readfirstlane (schedule_step (id, rec));
+        id = __builtin_amdgcn_readfirstlane (schedule_step<ORDERED> (id, rec));
         if (id == QUEUE_EMPTY) break;           // all tickets taken, or aborted
         // wavefront 0 requests this tile's child record now; it arrives while the tile runs
         // (a global, not a flat load: a flat one would also count as LDS traffic the tile's first fragment wait sits out)
@@ -458,11 +528,13 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
         // and by all workgroups, so it sits in the scalar cache or in L2)
         const auto descriptor = [] () { return scalar_layer (s_sched.a.layers + s_sched.layer); };
         bool complete;
+        const auto ready = [] () { if constexpr (ORDERED) wait_until_ready (); };
         if (!(s_sched.a.flags & ASPEN_HIP_FLAG_SKIP_TILES))
-            complete = run_tile<COH, FEAT> (descriptor, id, true, smem, [] () { return s_sched.a.arrivals; });
+            complete = run_tile<COH, FEAT, ORDERED ? NARROW_PF_SLICES : 0> (descriptor, id, true, smem, [] () { return s_sched.a.arrivals; }, ready);
         else
         {
             // scheduler-only run: the split-K groups still elect the member that releases the children
+            ready ();
             const aspen_hip_layer_t L = descriptor ();
             const uint32_t t = id - L.ninst_start;
             complete = L.splits <= 1 || splitk_arrived_last (&s_sched.a.arrivals[id - t % L.splits], L.splits, smem);
@@ -492,6 +564,13 @@ static const void *const dataflow_kernels[NUM_KERNEL_VARIANTS][2] = {
     {(const void *)dataflow_kernel<1, TILES_CONVNET | TILES_YOLO>, (const void *)dataflow_kernel<2, TILES_CONVNET | TILES_YOLO>},
     {(const void *)dataflow_kernel<1, TILES_ALL>, (const void *)dataflow_kernel<2, TILES_ALL>}};
 
+// Ordered mode (see aspen_hip_run_dataflow), cached loads only: for convolutional networks, and with every tile kind.
+#define NUM_ORDERED_VARIANTS 2
+#define ORDERED_SMEM_BYTES CMAX (GEMM_SMEM_BYTES, NARROW_PF_SMEM_BYTES)       // the narrow tiles' weight prefetch buffers
+static const unsigned ordered_variant_tiles[NUM_ORDERED_VARIANTS] = {TILES_CONVNET | TILES_YOLO | TILES_NARROW, TILES_ALL};
+static const void *const ordered_kernels[NUM_ORDERED_VARIANTS] = {
+    (const void *)dataflow_kernel<2, TILES_CONVNET | TILES_YOLO | TILES_NARROW, true>, (const void *)dataflow_kernel<2, TILES_ALL, true>};
+
 // The tile kinds a graph contains, as TILES_* bits.
 static unsigned graph_features (const aspen_hip_layer_t *layers, uint32_t num_layers)
 {
@@ -503,6 +582,7 @@ static unsigned graph_features (const aspen_hip_layer_t *layers, uint32_t num_la
         switch (L.type)
         {
         case CONV_LAYER: case FC_LAYER: case MATMUL_LAYER:
+            if (L.variant == ASPEN_HIP_GEMM_NARROW) { f |= TILES_NARROW; break; }      // (brings its own operand loaders)
             f |= L.variant == ASPEN_HIP_GEMM_LARGE ? TILES_LARGE : L.variant == ASPEN_HIP_GEMM_WIDE ? TILES_WIDE : TILES_SMALL;
             if (L.direct != ASPEN_HIP_OPERAND_DIRECT) f |= TILES_GATHER;
             break;
@@ -538,6 +618,8 @@ extern "C" int aspen_hip_init (void)
     for (int v = 0; v < NUM_KERNEL_VARIANTS; v++)
         for (int coh = 0; coh < 2; coh++)
             CHECK (hipFuncSetAttribute (dataflow_kernels[v][coh], hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
+    for (int v = 0; v < NUM_ORDERED_VARIANTS; v++)
+        CHECK (hipFuncSetAttribute (ordered_kernels[v], hipFuncAttributeMaxDynamicSharedMemorySize, ORDERED_SMEM_BYTES));
     // how many persistent workgroups really fit a compute unit (registers, LDS): the default grid
     int occ1 = 0, occ2 = 0;
     CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&occ1, dataflow_kernel<1, TILES_ALL>, WG_THREADS, GEMM_SMEM_BYTES));
@@ -551,10 +633,10 @@ extern "C" int aspen_hip_init (void)
 
 extern "C" const char *aspen_hip_last_error (void) { return g_err; }
 
-extern "C" void aspen_hip_tile_shapes (uint32_t shapes[9])
+extern "C" void aspen_hip_tile_shapes (uint32_t shapes[11])
 {
     shapes[0] = VAR0_BM; shapes[1] = VAR0_BN; shapes[2] = VAR1_BM; shapes[3] = VAR1_BN; shapes[4] = VAR2_BM; shapes[5] = VAR2_BN;
-    shapes[6] = KATTN_BN; shapes[7] = VATTN_BN; shapes[8] = WG_PER_CU;
+    shapes[6] = KATTN_BN; shapes[7] = VATTN_BN; shapes[8] = WG_PER_CU; shapes[9] = VAR3_BM; shapes[10] = VAR3_BN;
 }
 
 extern "C" int aspen_hip_device_info (int *num_cu, int *clock_khz, size_t *mem_bytes, char *name, int name_len)
@@ -761,7 +843,7 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
     const char *why = nullptr;
     // buffer descriptors carry 32-bit sizes: this holds for every matrix, also one no tile of its own layer writes
     if ((uint64_t)L.N * L.ld * 4 >= 0xffffff00ull
-        || (L.splits > 1 && (uint64_t)L.splits * L.tiles_m * L.tiles_n * SPLITK_TILE_FLOATS * 4 >= 0xffffff00ull))
+        || (L.splits > 1 && (uint64_t)L.splits * L.tiles_m * L.tiles_n * L.tile_m * L.tile_n * 4 >= 0xffffff00ull))
     {
         snprintf (g_err, sizeof (g_err), "layer %u rejected: matrix larger than 4 GiB", idx);
         fprintf (stderr, "aspen_hip: %s\n", g_err);
@@ -773,15 +855,16 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
     else if (L.tiles_m == 0 || L.tiles_n == 0 || L.splits == 0
         || L.num_ninst != L.tiles_m * L.tiles_n * L.splits) why = "tile grid";
     else if (L.splits > 1 && (!L.partial || L.kiters_per_split == 0 || (uint64_t)L.splits * L.kiters_per_split * GEMM_BK < L.Kp
-        || !(L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER) || L.variant != ASPEN_HIP_GEMM_SMALL)) why = "split-K geometry";
+        || !(L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER) || (L.variant != ASPEN_HIP_GEMM_SMALL && L.variant != ASPEN_HIP_GEMM_NARROW))) why = "split-K geometry";
     else if ((L.type == CONV_LAYER || L.type == MAXPOOL_LAYER || L.type == AVGPOOL_LAYER)
         && (L.stride == 0 || L.KH == 0 || L.KW == 0 || L.IH == 0 || L.IW == 0 || L.OH == 0 || L.OW == 0 || L.N % (L.OH * L.OW))) why = "window geometry";
     else if (L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER)
     {
-        uint32_t shp[9];
+        uint32_t shp[11];
         aspen_hip_tile_shapes (shp);
         if (L.variant < 0 || L.variant >= ASPEN_HIP_NUM_GEMM_VARIANTS) { snprintf (g_err, sizeof (g_err), "layer %u rejected: GEMM variant", idx); return -1; }
-        const uint32_t bm = shp[2 * L.variant], bn = shp[2 * L.variant + 1];
+        const bool narrow = L.variant == ASPEN_HIP_GEMM_NARROW;
+        const uint32_t bm = narrow ? shp[9] : shp[2 * L.variant], bn = narrow ? shp[10] : shp[2 * L.variant + 1];
         if (!L.weight) why = "missing weight";
         else if ((uint64_t)((L.M + 127) / 128 * 128) * L.Kp * 4 >= 0xffffff00ull) why = "weight matrix larger than 4 GiB";
         else if (L.Kp == 0 || L.Kp % GEMM_BK) why = "Kp must be a positive multiple of 32";
@@ -794,6 +877,7 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
         else if (L.direct < 0 || L.direct > ASPEN_HIP_OPERAND_DENSE3) why = "operand kind";
         else if (L.direct == ASPEN_HIP_OPERAND_TABLE && L.IC % GEMM_BK != 0 && L.variant != ASPEN_HIP_GEMM_SMALL) why = "a K axis that needs the k-chunk table takes 64 x 64 tiles";
         else if (L.direct == ASPEN_HIP_OPERAND_TABLE && L.IC == 0) why = "channel count";
+        else if (narrow && (L.direct == ASPEN_HIP_OPERAND_DENSE3 || (L.direct == ASPEN_HIP_OPERAND_TABLE && L.IC % GEMM_BK != 0))) why = "the 32 x 32 tile reads its operand in place or steps through taps of whole K slices";
     }
     else if (L.type == K_ATTENTION_LAYER)
     {
@@ -880,6 +964,7 @@ static double graph_parallelism (const aspen_hip_layer_t *layers, const uint32_t
         if (L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER)
         {
             cost = 8.f + (float)(L.splits > 1 ? L.kiters_per_split : L.Kp / GEMM_BK);
+            if (L.variant == ASPEN_HIP_GEMM_NARROW) cost = 8.f + 0.25f * (float)(L.splits > 1 ? L.kiters_per_split : L.Kp / GEMM_BK);     // a quarter of the work, a quarter of the K axis per wavefront
         }
         else if (L.type == K_ATTENTION_LAYER || L.type == V_ATTENTION_LAYER) cost = 16.f;
         dist[t] += cost;
@@ -932,6 +1017,7 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
     }
     aspen_hip_graph_t *g = (aspen_hip_graph_t *)calloc (1, sizeof (aspen_hip_graph_t));
     if (!g) { snprintf (g_err, sizeof (g_err), "out of host memory"); return nullptr; }
+    g->prefer_ordered = -1;
     g->cached_loads = lines_have_one_producer (layers, num_layers) && getenv ("ASPEN_GPU_COHERENT_LOADS") == nullptr;
     g->num_layers = num_layers; g->num_ninst = num_ninst; g->num_roots = num_roots; g->num_edges = num_edges;
     g->features = graph_features (layers, num_layers);
@@ -1028,7 +1114,7 @@ extern "C" void aspen_hip_graph_destroy (aspen_hip_graph_t *g)
     (void)hipStreamSynchronize (g_stream);
     aspen_hip_free (g->d_layers); aspen_hip_free (g->d_ninst_layer); aspen_hip_free (g->d_num_parents);
     aspen_hip_free (g->d_child_off); aspen_hip_free (g->d_child_idx); aspen_hip_free (g->d_roots); aspen_hip_free (g->d_ninst_home); aspen_hip_free (g->d_root_pos);
-    aspen_hip_free (g->d_child_rec); aspen_hip_free (g->d_dep); aspen_hip_free (g->d_queue); aspen_hip_free (g->d_ran); aspen_hip_free (g->d_arrivals); aspen_hip_free (g->d_state); aspen_hip_free (g->d_prof); aspen_hip_free (g->d_trace); aspen_hip_free (g->d_group_sinks);
+    aspen_hip_free (g->d_child_rec); aspen_hip_free (g->d_dep); aspen_hip_free (g->d_queue); aspen_hip_free (g->d_ran); aspen_hip_free (g->d_arrivals); aspen_hip_free (g->d_state); aspen_hip_free (g->d_prof); aspen_hip_free (g->d_trace); aspen_hip_free (g->d_group_sinks); aspen_hip_free (g->d_dep_spread);
     if (g->h_abort) (void)hipHostFree (g->h_abort);
     free (g->h_layers);
     free (g);
@@ -1066,6 +1152,7 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
 {
     if (!g) { snprintf (g_err, sizeof (g_err), "run_dataflow: null graph"); return -1; }
     if (g->num_ninst == 0) return 0;
+    const uint32_t workgroups_requested = workgroups;
     if (workgroups == 0) workgroups = g->default_workgroups;
     if (workgroups > QUEUE_SLACK) workgroups = QUEUE_SLACK;         // every waiting workgroup must find a "leave" entry within its queue
     g->epoch = g->epoch % EPOCH_MAX + 1u;
@@ -1074,6 +1161,40 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     const bool xcd_queues = xcd_queues_env || (g_flags & ASPEN_HIP_FLAG_XCD_QUEUES);
     static const uint32_t shift_env = getenv ("ASPEN_GPU_XCD_QUEUE_SHIFT") ? (uint32_t)atoi (getenv ("ASPEN_GPU_XCD_QUEUE_SHIFT")) : 0u;
     const uint32_t nq_shift = shift_env > 2u ? 2u : shift_env;
+    // Ordered mode for graphs that can never keep the device busy (one image through a deep network): no ready queue,
+    // workgroups take the tiles in index order (parents first), set each one up and request its first weights BEFORE it
+    // is ready, and wait on the tile's own dependency counter.  With far more workgroups than ready tiles nothing is
+    // lost by binding a workgroup to a tile early, and a dependency level no longer pays for descriptor fetch, index
+    // arithmetic, the weights' memory latency and two queue round trips after its parents have finished.
+    static const char *ordered_env = getenv ("ASPEN_GPU_ORDERED");
+    bool ordered = ordered_env ? atoi (ordered_env) != 0 : g->prefer_ordered >= 0 ? g->prefer_ordered != 0 : g->parallelism < ORDERED_BELOW;
+    if (g_flags & ASPEN_HIP_FLAG_ORDERED) ordered = true;
+    if (g_flags & ASPEN_HIP_FLAG_NO_ORDERED) ordered = false;
+    if (!g->cached_loads || xcd_queues || g->num_ninst > (1u << 20)) ordered = false;
+    if (ordered)
+    {
+        // tiles are assigned to workgroups beforehand: every workgroup of the grid must be running
+        static int fit = -1;
+        if (fit < 0)
+        {
+            int o0 = 0, o1 = 0;
+            CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&o0, ordered_kernels[0], WG_THREADS, ORDERED_SMEM_BYTES));
+            CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&o1, ordered_kernels[1], WG_THREADS, ORDERED_SMEM_BYTES));
+            fit = (o0 < o1 ? o0 : o1) * g_num_cu;
+        }
+        if (fit < 1) ordered = false;
+        else
+        {
+            if (workgroups_requested == 0) workgroups = (uint32_t)fit;         // two per compute unit: one tile computes, the next is prepared
+            if (workgroups > (uint32_t)fit) workgroups = (uint32_t)fit;
+        }
+    }
+    if (ordered && !g->d_dep_spread)
+    {
+        g->dep_stride = (g->num_ninst + 31u) / 32u * 32u + 1024u;
+        g->d_dep_spread = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * 32u * (size_t)g->dep_stride);
+        if (!g->d_dep_spread) return -1;
+    }
     const uint32_t nq_mask = (xcd_queues && workgroups % NUM_QUEUES == 0) ? (NUM_QUEUES >> nq_shift) - 1u : 0u;
     queue_counts_t counts;
     if (nq_mask && g->root_shift != nq_shift)
@@ -1094,7 +1215,7 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
         // The slots a run rewrites depend on the grid (leave entries), the hand-off (kept tiles take no slot) and the
         // queue grouping.  A slot an earlier run with other settings wrote could otherwise survive until the epoch
         // comes round again and be taken for an entry of that run.
-        const uint32_t config = workgroups ^ (nq_mask << 16) ^ (nq_shift << 20) ^ ((g_flags & (ASPEN_HIP_FLAG_NO_HANDOFF | ASPEN_HIP_FLAG_XCD_QUEUES | ASPEN_HIP_FLAG_SKIP_TILES)) << 24);
+        const uint32_t config = workgroups ^ ((uint32_t)ordered << 15) ^ (nq_mask << 16) ^ (nq_shift << 20) ^ ((g_flags & (ASPEN_HIP_FLAG_NO_HANDOFF | ASPEN_HIP_FLAG_XCD_QUEUES | ASPEN_HIP_FLAG_SKIP_TILES)) << 24);
         if (g->epoch == 1u || config != g->queue_config)
         {
             const size_t entries = (size_t)NUM_QUEUES * QUEUE_LANES * g->queue_row;
@@ -1104,18 +1225,18 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
         g->queue_config = config;
     }
     hipLaunchKernelGGL (arm_kernel, dim3 ((g->num_ninst + 255) / 256), dim3 (256), 0, g_stream,
-        g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->d_ninst_layer, g->d_ninst_home, g->d_root_pos, counts,
-        g->num_ninst, g->num_roots, g->d_state, g->epoch, g->queue_row, nq_mask, nq_shift, g->d_arrivals);
+        ordered ? g->d_dep_spread : g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->d_ninst_layer, g->d_ninst_home, g->d_root_pos, counts,
+        g->num_ninst, g->num_roots, g->d_state, g->epoch, g->queue_row, nq_mask, nq_shift, g->d_arrivals, ordered ? g->dep_stride : 0u);
     CHECK (hipGetLastError ());
     dataflow_args_t a;
     a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.ninst_home = g->d_ninst_home; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx; a.child_rec = g->d_child_rec;
-    a.dep = g->d_dep; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran; a.arrivals = g->d_arrivals; a.prof = g->d_prof; a.host_abort = g->h_abort;
+    a.dep = ordered ? g->d_dep_spread : g->d_dep; a.dep_stride = ordered ? g->dep_stride : 0u; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran; a.arrivals = g->d_arrivals; a.prof = g->d_prof; a.host_abort = g->h_abort;
     g->run_serial = g->run_serial + 1u ? g->run_serial + 1u : 1u;
     g->last_run_dataflow = 1;
     a.group_sinks = g->d_group_sinks; a.num_groups = g->live_groups; a.run_serial = g->run_serial;
     if ((g_flags & ASPEN_HIP_FLAG_TRACE) && !g->d_trace)
     {
-        g->d_trace = (unsigned long long *)aspen_hip_alloc (sizeof (unsigned long long) * 2 * (size_t)g->num_ninst);
+        g->d_trace = (unsigned long long *)aspen_hip_alloc (sizeof (unsigned long long) * 4 * (size_t)g->num_ninst);     // start / end, then K loop / epilogue stamps
         if (!g->d_trace) return -1;
     }
     a.trace = g->d_trace;
@@ -1125,13 +1246,19 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
         static const bool all_tiles = getenv ("ASPEN_GPU_ONE_KERNEL") != nullptr;       // comparisons: always the variant with every tile kind
         int v = NUM_KERNEL_VARIANTS - 1;
         for (int i = NUM_KERNEL_VARIANTS - 2; i >= 0 && !all_tiles; i--) if ((g->features & ~kernel_variant_tiles[i]) == 0) v = i;
+        const void *kernel = dataflow_kernels[v][g->cached_loads ? 1 : 0];
+        if (ordered) kernel = ordered_kernels[(g->features & ~ordered_variant_tiles[0]) == 0 ? 0 : 1];
+        g->last_run_ordered = ordered;
         void *kernel_args[] = {&a};
-        CHECK (hipLaunchKernel (dataflow_kernels[v][g->cached_loads ? 1 : 0], dim3 (workgroups), dim3 (WG_THREADS), kernel_args, GEMM_SMEM_BYTES, g_stream));
+        CHECK (hipLaunchKernel (kernel, dim3 (workgroups), dim3 (WG_THREADS), kernel_args, ordered ? ORDERED_SMEM_BYTES : GEMM_SMEM_BYTES, g_stream));
     }
     CHECK (hipGetLastError ());
     CHECK (hipEventRecord (g_events[NUM_EVENTS - 1], g_stream));
     return 0;
 }
+
+extern "C" void aspen_hip_graph_set_ordered (aspen_hip_graph_t *g, int ordered) { if (g) g->prefer_ordered = ordered < 0 ? -1 : ordered != 0; }
+extern "C" int aspen_hip_graph_last_run_ordered (const aspen_hip_graph_t *g) { return g ? g->last_run_ordered : 0; }
 
 extern "C" double aspen_hip_graph_parallelism (const aspen_hip_graph_t *g) { return g ? g->parallelism : 0.0; }
 
@@ -1243,6 +1370,13 @@ extern "C" int aspen_hip_dataflow_trace (aspen_hip_graph_t *g, uint64_t *start_e
     if (!g || !start_end || !g->d_trace || num_ninst != g->num_ninst)
     { snprintf (g_err, sizeof (g_err), "dataflow_trace: no traced run, or wrong tile count"); return -1; }
     return aspen_hip_d2h (start_end, g->d_trace, sizeof (uint64_t) * 2 * (size_t)num_ninst);
+}
+
+extern "C" int aspen_hip_dataflow_trace_phases (aspen_hip_graph_t *g, uint64_t *kloop_epilogue, uint32_t num_ninst)
+{
+    if (!g || !kloop_epilogue || !g->d_trace || num_ninst != g->num_ninst)
+    { snprintf (g_err, sizeof (g_err), "dataflow_trace_phases: no traced run, or wrong tile count"); return -1; }
+    return aspen_hip_d2h (kloop_epilogue, g->d_trace + 2 * (size_t)num_ninst, sizeof (uint64_t) * 2 * (size_t)num_ninst);
 }
 
 extern "C" int aspen_hip_event_record (int slot)

@@ -11,6 +11,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 #include "aspen.h"
 #include "aspen_hip.h"
 
@@ -495,15 +496,19 @@ enum : unsigned
     TILES_LARGE = 2u, TILES_WIDE = 4u, TILES_SMALL = 8u,       // contraction tile shapes
     TILES_ATTENTION = 16u, TILES_NORM = 32u /* layernorm, softmax */, TILES_POOL = 64u, TILES_YOLO = 128u /* yolo, append */,
     TILES_RESIDUAL = 256u,
-    TILES_ALL = 511u,
+    TILES_NARROW = 512u,        // the 32 x 32 contraction tile of latency-bound graphs
+    TILES_ALL = 1023u,
     TILES_CONVNET = TILES_GATHER | TILES_LARGE | TILES_WIDE | TILES_SMALL | TILES_POOL | TILES_RESIDUAL,
     TILES_TRANSFORMER = TILES_SMALL | TILES_ATTENTION | TILES_NORM | TILES_RESIDUAL
 };
 // `before_last_slice` runs right before the MFMAs of the last K slice: the place to request what the epilogue
 // will need from memory, with the operand registers free and a whole slice of arithmetic to hide the latency.
-template <int BM, int BN, int WM, int WN, int DEPTH, class ALoader, class BLoader, class Hook = NoHook>
+// `ready` runs between the first request for the weight operand and the first request for the activation operand: a
+// kernel that starts tiles before their parents have finished (see the ordered mode of the persistent kernel) waits
+// there, with the tile's set-up done and its first weights on their way.
+template <int BM, int BN, int WM, int WN, int DEPTH, class ALoader, class BLoader, class Hook = NoHook, class Ready = NoHook>
 __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, int kiters, float *smem,
-    floatx16 (&acc)[BN / WN / 32][BM / WM / 32], bool phases = false, Hook before_last_slice = Hook ())
+    floatx16 (&acc)[BN / WN / 32][BM / WM / 32], bool phases = false, Hook before_last_slice = Hook (), Ready ready = Ready ())
 {
     static_assert (DEPTH == 1 || DEPTH == 2, "one or two register sets");
     if (phases) tile_phase_lap (12);
@@ -553,7 +558,7 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
 
     // register set s holds slice it with (it - first) % DEPTH == s
     float4 areg[DEPTH][ALoader::R], breg[DEPTH][BLoader::R];
-    al.load (kbase, areg[0]); bl.load (kbase, breg[0]);
+    al.load (kbase, areg[0]); ready (); bl.load (kbase, breg[0]);
     if (DEPTH == 2 && kiters > 1) { al.load (kbase + 1, areg[DEPTH - 1]); bl.load (kbase + 1, breg[DEPTH - 1]); }
     al.store (smem, areg[0]); bl.store (smem + BM * LDS_ROW, breg[0]);
     if (kiters > DEPTH) { al.load (kbase + DEPTH, areg[0]); bl.load (kbase + DEPTH, breg[0]); }
@@ -643,9 +648,9 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
 // Mij = MFMA on K pair j of sub-step i; X = barrier "everyone holds this slice's fragments", wA / wB = next
 // slice registers -> LDS, gA / gB = requests for the slice DEPTH ahead, Y = barrier "refill visible",
 // ri = fragments of sub-step i of the next slice (its buffer was released by Mi3).
-template <int DEPTH, class ALoader, class BLoader, class Hook = NoHook>
+template <int DEPTH, class ALoader, class BLoader, class Hook = NoHook, class Ready = NoHook>
 __device__ __forceinline__ void gemm_core_single_block (ALoader &al, BLoader &bl, int kbase, int kiters, float *smem,
-    floatx16 (&accs)[1][1], bool phases = false, Hook before_last_slice = Hook ())
+    floatx16 (&accs)[1][1], bool phases = false, Hook before_last_slice = Hook (), Ready ready = Ready ())
 {
     static_assert (DEPTH == 1 || DEPTH == 2, "one or two register sets");
     static_assert (ALoader::R == 2 && BLoader::R == 2 && GEMM_BK == 32, "64 x 64 tile, four sub-steps");
@@ -663,7 +668,7 @@ __device__ __forceinline__ void gemm_core_single_block (ALoader &al, BLoader &bl
 #define RD(i) do { fa[i] = ld4 (afrag + (i) * 8); fb[i] = ld4 (bfrag + (i) * 8); SB; } while (0)
 #define MF(i, c) do { acc = __builtin_amdgcn_mfma_f32_32x32x2f32 (fb[i].c, fa[i].c, acc, 0, 0, 0); SB; } while (0)
     float4 areg[DEPTH][2], breg[DEPTH][2];
-    al.load (kbase, areg[0]); bl.load (kbase, breg[0]);
+    al.load (kbase, areg[0]); ready (); bl.load (kbase, breg[0]);
     if (DEPTH == 2 && kiters > 1) { al.load (kbase + 1, areg[DEPTH - 1]); bl.load (kbase + 1, breg[DEPTH - 1]); }
     al.store (smem, areg[0]); bl.store (smem + BM * LDS_ROW, breg[0]);
     if (kiters > DEPTH) { al.load (kbase + DEPTH, areg[0]); bl.load (kbase + DEPTH, breg[0]); }
@@ -745,8 +750,8 @@ __device__ __forceinline__ void fused_shortcut (const aspen_hip_layer_t &L, cons
 // of the thread's pieces of a fused shortcut's operand (a tile has at most 128 columns: 8 pieces per thread)
 struct shortcut_prefetch_t { float4 s[8]; float4 bias; bool have, have_shortcut; };
 
-template <int BM, int BN, int WM, int WN, int DEPTH, int COH, unsigned FEAT, class Descriptor>
-__device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L, Descriptor descriptor, uint32_t tn, uint32_t tm, int slice, float *smem, shortcut_prefetch_t &pre)
+template <int BM, int BN, int WM, int WN, int DEPTH, int COH, unsigned FEAT, class Descriptor, class Ready>
+__device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L, Descriptor descriptor, uint32_t tn, uint32_t tm, int slice, float *smem, shortcut_prefetch_t &pre, Ready ready)
 {
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
@@ -790,8 +795,8 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
     {
         ActRowLoader<BN, COH> bl;
         bl.init (in, n0, L.N - 1, L.ld0, 0, tid);
-        if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
-        else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
+        if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
+        else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
     }
     else if constexpr ((FEAT & TILES_GATHER) != 0)
     {
@@ -800,8 +805,8 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
         {
             Dense3Loader<BN, COH> bl;
             bl.init (L, in, n0, tid);
-            if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
-            else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
+            if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
+            else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
         }
         else if (TM * TN == 1 && L.IC % GEMM_BK != 0)
         {
@@ -809,15 +814,15 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
             {
                 ConvLoader<BN, COH, true> bl;
                 bl.init (L, in, n0, tid, kbase);
-                gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
+                gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
             }
         }
         else
         {
             ConvLoader<BN, COH, false> bl;
             bl.init (L, in, n0, tid, kbase);
-            if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
-            else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut);
+            if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
+            else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
         }
     }
     if (COH) tile_phase_lap (9);
@@ -1513,12 +1518,327 @@ __device__ __forceinline__ bool splitk_arrived_last (uint32_t *counter, uint32_t
     return before % splits == splits - 1;
 }
 
+// ---------------------------------------------------------------------------------------------
+// The narrow contraction tile: 32 channels x 32 columns, the four wavefronts of the workgroup splitting the K axis
+// between them.  For graphs that are bound by the latency of their dependency chains (one image through a deep
+// network): a layer of a few dozen 64 x 64 tiles with long K loops becomes a few hundred short ones, so that a
+// dependency level keeps every compute unit busy for one or two microseconds instead of a quarter of them for
+// eight.  Throughput per workgroup does not matter here, so there is nothing to share between wavefronts and
+// nothing is staged through LDS: a lane reads its operands from memory in the layout the matrix instruction wants
+// (row = lane % 32, four consecutive K values at (lane / 32) * 4 of every 8: v_mfma_f32_32x32x2_f32 pairs the two
+// half-waves' values, and both operands use the same pairing, so the K order inside a slice is immaterial), the
+// K loop has no barrier, and the four partial sums meet in LDS once.  A layer can additionally be cut along K across
+// workgroups (`slice` >= 0) exactly like the 64 x 64 shape, with blocks of 32 x 32 sums in the threads' own order.
+// Operands: weights [.][Kp]; activations read in place (DIRECT) or gathered by stepping through the taps (a
+// convolution or FC layer over channels that are a multiple of the slice width).
+// ---------------------------------------------------------------------------------------------
+#define VAR3_BM 32
+#define VAR3_BN 32
+#define NARROW_TILE_FLOATS (VAR3_BM * VAR3_BN)
+#define NARROW_ROW 36          // floats per staged row of a wavefront's partial sums
+
+// what a thread of a narrow tile owns after the four wavefronts' sums have met: channels c .. c+3 of column n
+struct narrow_piece_t { uint32_t n, c; };
+__device__ __forceinline__ narrow_piece_t narrow_piece (uint32_t tid) { return {tid >> 3, (tid & 7u) * 4u}; }
+
+// bias, activation, store and fused shortcut of one thread's piece; `sc` = the shortcut operand's piece when `have_sc`
+template <int COH>
+__device__ __forceinline__ void narrow_finish_piece (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, uint32_t tid, float4 v, float4 bias, bool have_bias,
+    float4 sc, bool have_sc)
+{
+    const narrow_piece_t pc = narrow_piece (tid);
+    const uint32_t n = tn * VAR3_BN + pc.n, m = tm * VAR3_BM + pc.c;
+    if (n >= L.N || m >= L.M) return;
+    const uint32_t left = L.M - m;
+    ActView<COH> out;
+    out.init (L.out, L.N, L.ld);
+    if (!have_bias && L.bias)
+    {
+        bias.x = gld1 (L.bias + m);
+        if (left > 1) bias.y = gld1 (L.bias + m + 1);
+        if (left > 2) bias.z = gld1 (L.bias + m + 2);
+        if (left > 3) bias.w = gld1 (L.bias + m + 3);
+    }
+    v.x += bias.x; v.y += bias.y; v.z += bias.z; v.w += bias.w;
+    v = act4 (v, L.act);
+    const bool fuse = L.fuse_out != nullptr, keep = !(fuse && L.fuse_discard);
+    const uint32_t o = n * L.ld + m;
+    if (left >= 4)
+    {
+        if (keep) out.st4 (o, v);
+        if (fuse)
+        {
+            ActView<COH> fout;
+            fout.init (L.fuse_out, L.N, L.ld);
+            if (!have_sc) { ActView<COH> fin; fin.init (L.fuse_in, L.N, L.fuse_ld_in); sc = fin.ld4 (n * L.fuse_ld_in + m); }
+            v.x += sc.x; v.y += sc.y; v.z += sc.z; v.w += sc.w;
+            fout.st4 (o, act4 (v, L.fuse_act));
+        }
+    }
+    else
+    {
+        if (keep) { out.st1 (o, v.x); if (left > 1) out.st1 (o + 1, v.y); if (left > 2) out.st1 (o + 2, v.z); }
+        if (fuse)
+        {
+            ActView<COH> fin, fout;
+            fin.init (L.fuse_in, L.N, L.fuse_ld_in); fout.init (L.fuse_out, L.N, L.ld);
+            fused_shortcut<COH> (L, fin, fout, v, n, m, left);
+        }
+    }
+}
+
+// sum of the slices' blocks of output tile t (in slice order, whoever runs it), then the tile's epilogue
+template <int COH>
+__device__ __forceinline__ void narrow_gather_finish (const aspen_hip_layer_t &L, uint32_t t, uint32_t tn, uint32_t tm)
+{
+    const uint32_t tid = tile_thread ();
+    const uint32_t tiles = L.tiles_m * L.tiles_n, sstride = tiles * NARROW_TILE_FLOATS, last = L.splits - 1;
+    ActView<COH> part;
+    part.init (L.partial, L.splits * tiles, NARROW_TILE_FLOATS);
+    const uint32_t base = t * NARROW_TILE_FLOATS + tid * 4;
+    float4 v = make_float4 (0.f, 0.f, 0.f, 0.f);
+    constexpr uint32_t BATCH = 8;       // requests in flight per thread: the blocks come from other compute units' tiles
+    for (uint32_t s0 = 0; s0 < L.splits; s0 += BATCH)
+    {
+        float4 p[BATCH];
+        #pragma unroll
+        for (uint32_t j = 0; j < BATCH; j++) p[j] = part.ld4 (base + min (s0 + j, last) * sstride);
+        #pragma unroll
+        for (uint32_t j = 0; j < BATCH; j++)
+        {
+            const bool use = s0 + j <= last;
+            v.x += use ? p[j].x : 0.f; v.y += use ? p[j].y : 0.f; v.z += use ? p[j].z : 0.f; v.w += use ? p[j].w : 0.f;
+        }
+    }
+    narrow_finish_piece<COH> (L, tn, tm, tid, v, make_float4 (0.f, 0.f, 0.f, 0.f), false, make_float4 (0.f, 0.f, 0.f, 0.f), false);
+}
+
+// Returns the thread's piece of the tile's sums over the K slices [kbase, kbase + kiters).
+// PF > 0 (kernels that start a tile before its parents have finished, with PF * 16 KB of LDS per workgroup): the
+// weights of a wavefront's first PF slices are requested BEFORE `ready ()`, straight from memory into LDS
+// (buffer_load ... lds: lane l's 16 bytes land at block + 16 l, so a lane later reads back exactly the fragment it
+// asked for; LDS serves as a per-lane buffer that costs no registers), and the activations of the first NARROW_B_WINDOW
+// of them are all requested together right after it, the rest as the window's registers come free: a tile of up to PF
+// slices per wavefront pays for one trip to memory after its parents have finished.  Slices beyond PF (and all slices when PF = 0) go through registers, two in flight.
+#define NARROW_PF_SLICES 4
+#define NARROW_B_WINDOW 4           // slices of activations in flight in registers
+#define NARROW_PF_SMEM_BYTES (4 * NARROW_PF_SLICES * 4 * 1024)
+template <int COH, int PF, class Descriptor, class Ready>
+__device__ __forceinline__ float4 narrow_mainloop (const aspen_hip_layer_t &L, Descriptor descriptor, uint32_t tn, uint32_t tm, int kbase, int kiters,
+    float *smem, Ready ready)
+{
+    const uint32_t tid = tile_thread (), lane = tid & 63, wave = __builtin_amdgcn_readfirstlane (tid >> 6);
+    const uint32_t row = lane & 31, khalf = (lane >> 5) * 4;
+    // this wavefront's share of the slices: a contiguous quarter
+    const int per = (kiters + 3) >> 2, w0 = min ((int)wave * per, kiters), cnt = min (per, kiters - w0), first = kbase + w0;
+    // weights: one uniform base, 32-bit byte offsets
+    const float *wptr = descriptor ().weight;
+    const char __attribute__ ((address_space (1))) *wbase = (const char __attribute__ ((address_space (1))) *)wptr;
+    const uint32_t aoff = (((tm * VAR3_BM + row) * L.Kp) + (uint32_t)first * GEMM_BK + khalf) * 4u;
+    ActView<COH> in;
+    in.init (descriptor ().in0, L.in0_columns, L.ld0);
+    const bool direct = L.direct == ASPEN_HIP_OPERAND_DIRECT;
+    uint32_t n = tn * VAR3_BN + row;
+    n = n < L.N ? n : L.N - 1;
+    // activation operand: DIRECT = the parent's column; else the top-left input pixel of output position n and the
+    // tap / channel the first slice starts at (stepped from there, as ConvLoader does)
+    int32_t bbase, ih0 = 0, iw0 = 0;
+    uint32_t kh = 0, kw = 0, c = 0;
+    const uint32_t spt = direct ? 1u : L.IC / GEMM_BK;
+    if (direct) bbase = (int32_t)(n * L.ld0 + (uint32_t)first * GEMM_BK + khalf);
+    else
+    {
+        const uint32_t ohw = L.OH * L.OW;
+        const uint32_t b = fast_div (n, L.div_ohw), rem = n - b * ohw, oh = fast_div (rem, L.div_ow), ow = rem - oh * L.OW;
+        ih0 = (int32_t)(oh * L.stride) - (int32_t)L.pad;
+        iw0 = (int32_t)(ow * L.stride) - (int32_t)L.pad;
+        bbase = ((int32_t)(b * L.IH) + ih0) * (int32_t)L.IW * (int32_t)L.ld0 + iw0 * (int32_t)L.ld0 + (int32_t)khalf;
+        const uint32_t tap = (uint32_t)first / spt;
+        c = ((uint32_t)first - tap * spt) * GEMM_BK;
+        kh = tap / L.KW; kw = tap - kh * L.KW;
+    }
+    const uint32_t IH = L.IH, IW = L.IW, KW = L.KW, ld0 = L.ld0;
+    auto load_a = [&] (int i, float4 (&a)[4])
+    {
+        #pragma unroll
+        for (int sub = 0; sub < 4; sub++)
+        {
+            const floatx4 x = *(const floatx4 __attribute__ ((address_space (1))) *)(wbase + (aoff + (uint32_t)i * (GEMM_BK * 4u) + (uint32_t)sub * 32u));
+            a[sub] = make_float4 (x[0], x[1], x[2], x[3]);
+        }
+    };
+    // slices are asked for in ascending order: the tap position is stepped
+    auto load_b = [&] (int i, float4 (&bv)[4])
+    {
+        if (direct)
+        {
+            #pragma unroll
+            for (int sub = 0; sub < 4; sub++) bv[sub] = in.ld4 ((uint32_t)(bbase + i * GEMM_BK + sub * 8));
+        }
+        else
+        {
+            const int32_t off = (int32_t)((kh * IW + kw) * ld0 + c);
+            const bool ok = (uint32_t)(ih0 + (int32_t)kh) < IH && (uint32_t)(iw0 + (int32_t)kw) < IW;
+            #pragma unroll
+            for (int sub = 0; sub < 4; sub++) bv[sub] = in.ld4_if ((uint32_t)(bbase + off + sub * 8), ok);
+            c += GEMM_BK;
+            if (c == spt * GEMM_BK) { c = 0; if (++kw == KW) { kw = 0; ++kh; } }
+        }
+    };
+    floatx16 acc;
+    #pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = 0.f;
+    auto mfmas = [&] (const float4 (&a)[4], const float4 (&bv)[4])
+    {
+        #pragma unroll
+        for (int sub = 0; sub < 4; sub++)
+        {
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32 (bv[sub].x, a[sub].x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32 (bv[sub].y, a[sub].y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32 (bv[sub].z, a[sub].z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32 (bv[sub].w, a[sub].w, acc, 0, 0, 0);
+        }
+    };
+    constexpr uint32_t REGION = PF > 0 ? PF * 1024u : (uint32_t)(VAR3_BN * NARROW_ROW);     // floats of LDS per wavefront
+    float *mine = smem + wave * REGION;
+    int done = 0;       // slices of this wavefront's share that are finished
+    float4 a0[4], a1[4], b0[4], b1[4];
+    if constexpr (PF > 0)
+    {
+        const uint32_t Mp = (L.M + 127u) / 128u * 128u;
+        const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc ((void *)wptr, 0, (int)(Mp * L.Kp * 4u), 0x00020000);
+        #pragma unroll
+        for (int i = 0; i < PF; i++)
+            if (i < cnt)
+            {
+                #pragma unroll
+                for (int sub = 0; sub < 4; sub++)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds (wr, (__attribute__ ((address_space (3))) void *)(mine + (i * 4 + sub) * 256), 16,
+                        (int)(aoff + (uint32_t)i * (GEMM_BK * 4u) + (uint32_t)sub * 32u), 0, 0, 0);
+            }
+        ready ();
+        // one straight-line body per number of prefetched slices (wave-uniform): every activation request is issued
+        // before the first fragment is read back, so the slices' trips to memory overlap
+        auto body = [&] (auto count)
+        {
+            constexpr int C = decltype (count)::value, W = C < NARROW_B_WINDOW ? C : NARROW_B_WINDOW;
+            float4 bq[W][4];
+            #pragma unroll
+            for (int i = 0; i < W; i++) load_b (i, bq[i]);
+            #pragma unroll
+            for (int i = 0; i < C; i++)
+            {
+                float4 af[4];
+                #pragma unroll
+                for (int sub = 0; sub < 4; sub++) af[sub] = ld4 (mine + (i * 4 + sub) * 256 + lane * 4);
+                mfmas (af, bq[i % W]);
+                if (i + W < C) load_b (i + W, bq[i % W]);       // the window moves on: this slice's registers take the slice W ahead
+            }
+        };
+        static_assert (PF == 4, "one case per prefetched slice count");
+        const int pre = __builtin_amdgcn_readfirstlane (min (cnt, PF));
+        if (pre == 4) body (std::integral_constant<int, 4> ());
+        else if (pre == 3) body (std::integral_constant<int, 3> ());
+        else if (pre == 2) body (std::integral_constant<int, 2> ());
+        else if (pre == 1) body (std::integral_constant<int, 1> ());
+        done = min (cnt, PF);
+        if (done < cnt) { load_a (done, a0); load_b (done, b0); }
+        if (done + 1 < cnt) { load_a (done + 1, a1); load_b (done + 1, b1); }
+    }
+    else
+    {
+        // two slices in flight: set 0 holds the even, set 1 the odd ones of this wavefront's share
+        if (cnt > 0) load_a (0, a0);
+        if (cnt > 1) load_a (1, a1);
+        ready ();
+        if (cnt > 0) load_b (0, b0);
+        if (cnt > 1) load_b (1, b1);
+    }
+    for (int i = done; i < cnt; i += 2)
+    {
+        mfmas (a0, b0);
+        if (i + 2 < cnt) { load_a (i + 2, a0); load_b (i + 2, b0); }
+        if (i + 1 < cnt)
+        {
+            mfmas (a1, b1);
+            if (i + 3 < cnt) { load_a (i + 3, a1); load_b (i + 3, b1); }
+        }
+    }
+    // the four wavefronts' sums meet in LDS: [wave][column][NARROW_ROW] (a wavefront's own region, which it has read empty)
+    #pragma unroll
+    for (int v = 0; v < 16; v++) mine[ACC_N (0, 0, v, lane) * NARROW_ROW + row] = acc[v];
+    __syncthreads ();
+    const narrow_piece_t pc = narrow_piece (tid);
+    float4 sum = ld4 (smem + pc.n * NARROW_ROW + pc.c);
+    #pragma unroll
+    for (int w = 1; w < 4; w++)
+    {
+        const float4 x = ld4 (smem + w * REGION + pc.n * NARROW_ROW + pc.c);
+        sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
+    }
+    return sum;
+}
+
+// One narrow tile; returns false for a split-K member that was not the last of its group.
+template <int COH, int PF, class Descriptor, class Arrivals, class Ready>
+__device__ __forceinline__ bool narrow_tile (const aspen_hip_layer_t &L, Descriptor descriptor, uint32_t t, uint32_t tn, uint32_t tm, int slice, uint32_t group,
+    float *smem, Arrivals arrivals, Ready ready)
+{
+    const uint32_t tid = tile_thread ();
+    int kbase = 0, kiters = (int)(L.Kp / GEMM_BK);
+    if (slice >= 0)
+    {
+        kbase = slice * (int)L.kiters_per_split;
+        kiters = min ((int)L.kiters_per_split, kiters - kbase);
+    }
+    // the bias is a weight: requested before the wait for the parents
+    const narrow_piece_t pc = narrow_piece (tid);
+    const uint32_t m = tm * VAR3_BM + pc.c, n = tn * VAR3_BN + pc.n;
+    const bool whole = slice < 0 && m + 4 <= L.M && n < L.N;
+    float4 bias = make_float4 (0.f, 0.f, 0.f, 0.f), sc = bias;
+    if (whole && L.bias) bias = gld4 (L.bias + m);
+    bool have_sc = false;
+    const auto ready_then_shortcut = [&] ()
+    {
+        ready ();
+        // an unsplit tile's shortcut operand is an activation its dependency counter covers: requested with the first slice
+        if (whole && L.fuse_out != nullptr)
+        {
+            ActView<COH> fin;
+            fin.init (L.fuse_in, L.N, L.fuse_ld_in);
+            sc = fin.ld4 (n * L.fuse_ld_in + m);
+            have_sc = true;
+        }
+    };
+    const float4 sum = narrow_mainloop<COH, PF> (L, descriptor, tn, tm, kbase, kiters, smem, ready_then_shortcut);
+    if (COH) tile_phase_lap (9);
+    if (slice < 0)
+    {
+        narrow_finish_piece<COH> (L, tn, tm, tid, sum, bias, whole, sc, have_sc);
+        if (COH) tile_phase_lap (10);
+        return true;
+    }
+    {
+        const uint32_t tiles = L.tiles_m * L.tiles_n;
+        ActView<COH> part;
+        part.init (L.partial, L.splits * tiles, NARROW_TILE_FLOATS);
+        part.st4 (((uint32_t)slice * tiles + t) * NARROW_TILE_FLOATS + tid * 4, sum);
+    }
+    if (COH) tile_phase_lap (10);
+    uint32_t *counters = arrivals ();
+    if (counters == nullptr || !splitk_arrived_last (counters + group, L.splits, smem)) { if (COH) tile_phase_lap (11); return false; }
+    narrow_gather_finish<COH> (L, t, tn, tm);
+    if (COH) tile_phase_lap (11);
+    return true;
+}
+
 // Split-K reduction of output tile t of the layer as a tile of its own (launch-per-layer mode).
 template <int COH>
 __device__ __forceinline__ void finish_tile (const aspen_hip_layer_t &L, uint32_t t, float *smem)
 {
     t = __builtin_amdgcn_readfirstlane (t);
     const uint32_t tn = fast_div (t, L.div_tiles_m);
+    if (L.variant == ASPEN_HIP_GEMM_NARROW) { narrow_gather_finish<COH> (L, t, tn, t - tn * L.tiles_m); return; }
     shortcut_prefetch_t pre;
     pre.have = pre.have_shortcut = false;
     splitk_gather<COH> (L, t, smem);
@@ -1532,8 +1852,11 @@ __device__ __forceinline__ void finish_tile (const aspen_hip_layer_t &L, uint32_
 // fetched where it is needed instead of occupying registers while the tile runs.  Returns false for
 // a split-K partial tile that was not the last of its group to finish: the output tile is not
 // complete yet and nothing may be released.
-template <int COH, unsigned FEAT = TILES_ALL, class Descriptor, class Arrivals>
-__device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, bool t_counts_from_graph_start, float *smem, Arrivals arrivals)
+// `ready ()` returns once the tile's parents have finished; it is called after whatever set-up does not touch an
+// activation (contraction tiles: descriptor, index arithmetic, first weight requests), right before the first
+// activation is requested.  Kernels that only start tiles whose parents have finished pass nothing.
+template <int COH, unsigned FEAT = TILES_ALL, int NARROW_PF = 0, class Descriptor, class Arrivals, class Ready = NoHook>
+__device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, bool t_counts_from_graph_start, float *smem, Arrivals arrivals, Ready ready = Ready ())
 {
     const aspen_hip_layer_t L = descriptor ();
     t = __builtin_amdgcn_readfirstlane (t);
@@ -1556,15 +1879,19 @@ __device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, boo
         shortcut_prefetch_t pre;
         pre.have = pre.have_shortcut = false;
         c4_log2 = 4; bn = VAR2_BN;
-        if ((FEAT & TILES_LARGE) && L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, VAR0_DEPTH, COH, FEAT> (L, descriptor, tn, tm, -1, smem, pre); c4_log2 = 5; bn = VAR0_BN; }
-        else if ((FEAT & TILES_WIDE) && L.variant == ASPEN_HIP_GEMM_WIDE) { contraction_mainloop<VAR1_BM, VAR1_BN, 2, 2, VAR1_DEPTH, COH, FEAT> (L, descriptor, tn, tm, -1, smem, pre); bn = VAR1_BN; }
+        if constexpr ((FEAT & TILES_NARROW) != 0)
+        {
+            if (L.variant == ASPEN_HIP_GEMM_NARROW) return narrow_tile<COH, NARROW_PF> (L, descriptor, t, tn, tm, slice, group, smem, arrivals, ready);
+        }
+        if ((FEAT & TILES_LARGE) && L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, VAR0_DEPTH, COH, FEAT> (L, descriptor, tn, tm, -1, smem, pre, ready); c4_log2 = 5; bn = VAR0_BN; }
+        else if ((FEAT & TILES_WIDE) && L.variant == ASPEN_HIP_GEMM_WIDE) { contraction_mainloop<VAR1_BM, VAR1_BN, 2, 2, VAR1_DEPTH, COH, FEAT> (L, descriptor, tn, tm, -1, smem, pre, ready); bn = VAR1_BN; }
         else if (FEAT & TILES_SMALL)
         {
             // two K slices in flight for the matmul layers of transformers, one for convolutional networks (see VAR2_DEPTH)
             bool deep = false;
             if constexpr ((FEAT & TILES_NORM) != 0) deep = (FEAT & TILES_GATHER) == 0 || L.type == MATMUL_LAYER;
-            if constexpr ((FEAT & TILES_NORM) != 0) { if (deep) contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, VAR2_DEPTH, COH, FEAT> (L, descriptor, tn, tm, slice, smem, pre); }
-            if constexpr ((FEAT & TILES_GATHER) != 0) { if (!deep) contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, 1, COH, FEAT> (L, descriptor, tn, tm, slice, smem, pre); }
+            if constexpr ((FEAT & TILES_NORM) != 0) { if (deep) contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, VAR2_DEPTH, COH, FEAT> (L, descriptor, tn, tm, slice, smem, pre, ready); }
+            if constexpr ((FEAT & TILES_GATHER) != 0) { if (!deep) contraction_mainloop<VAR2_BM, VAR2_BN, 2, 2, 1, COH, FEAT> (L, descriptor, tn, tm, slice, smem, pre, ready); }
         }
         
         const aspen_hip_layer_t E = descriptor ();
@@ -1582,15 +1909,15 @@ __device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, boo
         if (COH) tile_phase_lap (slice >= 0 ? 11 : 10);
         break;
     }
-    case RESIDUAL_LAYER:    if constexpr ((FEAT & TILES_RESIDUAL) != 0) tile_residual<COH> (L, tn); break;
-    case MAXPOOL_LAYER:     if constexpr ((FEAT & TILES_POOL) != 0) tile_pool<true, COH> (L, tn, tm); break;
-    case AVGPOOL_LAYER:     if constexpr ((FEAT & TILES_POOL) != 0) tile_pool<false, COH> (L, tn, tm); break;
-    case YOLO_LAYER:        if constexpr ((FEAT & TILES_YOLO) != 0) tile_yolo<COH> (L, tn); break;
-    case APPEND_LAYER:      if constexpr ((FEAT & TILES_YOLO) != 0) tile_append<COH> (L, tn); break;
-    case LAYERNORM_LAYER:   if constexpr ((FEAT & TILES_NORM) != 0) tile_layernorm<COH> (L, tn); break;
-    case SOFTMAX_LAYER:     if constexpr ((FEAT & TILES_NORM) != 0) tile_softmax<COH> (L, tn); break;
-    case K_ATTENTION_LAYER: if constexpr ((FEAT & TILES_ATTENTION) != 0) tile_k_attention<COH> (L, tn, smem); break;
-    case V_ATTENTION_LAYER: if constexpr ((FEAT & TILES_ATTENTION) != 0) tile_v_attention<COH> (L, tn, tm, smem); break;
+    case RESIDUAL_LAYER:    if constexpr ((FEAT & TILES_RESIDUAL) != 0) { ready (); tile_residual<COH> (L, tn); } break;
+    case MAXPOOL_LAYER:     if constexpr ((FEAT & TILES_POOL) != 0) { ready (); tile_pool<true, COH> (L, tn, tm); } break;
+    case AVGPOOL_LAYER:     if constexpr ((FEAT & TILES_POOL) != 0) { ready (); tile_pool<false, COH> (L, tn, tm); } break;
+    case YOLO_LAYER:        if constexpr ((FEAT & TILES_YOLO) != 0) { ready (); tile_yolo<COH> (L, tn); } break;
+    case APPEND_LAYER:      if constexpr ((FEAT & TILES_YOLO) != 0) { ready (); tile_append<COH> (L, tn); } break;
+    case LAYERNORM_LAYER:   if constexpr ((FEAT & TILES_NORM) != 0) { ready (); tile_layernorm<COH> (L, tn); } break;
+    case SOFTMAX_LAYER:     if constexpr ((FEAT & TILES_NORM) != 0) { ready (); tile_softmax<COH> (L, tn); } break;
+    case K_ATTENTION_LAYER: if constexpr ((FEAT & TILES_ATTENTION) != 0) { ready (); tile_k_attention<COH> (L, tn, smem); } break;
+    case V_ATTENTION_LAYER: if constexpr ((FEAT & TILES_ATTENTION) != 0) { ready (); tile_v_attention<COH> (L, tn, tm, smem); } break;
     default: break;
     }
     return true;

@@ -285,8 +285,11 @@ static unsigned int round_up (unsigned int v, unsigned int to) { return (v + to 
    device: K = taps * 3 instead of taps * 4, see ASPEN_HIP_OPERAND_DENSE3.  (The stem of ResNet-50: 160 instead of 224.) */
 int aspen_layer_dense3 (const aspen_layer_t *L)
 {
+    /* read once: the K layout, the table layout and the operand kind of a layer all follow from this answer and must agree */
+    static int disabled = -1;
+    if (disabled < 0) disabled = getenv ("ASPEN_GPU_NO_DENSE3") != NULL;
     return L->type == CONV_LAYER && L->params[IN_C] == 3 && L->params[WEIGHT_H] * L->params[WEIGHT_W] * 3 <= 508 && L->gemm_m <= 64
-        && getenv ("ASPEN_GPU_NO_DENSE3") == NULL;
+        && !disabled;
 }
 
 /* A contraction layer whose channel count is not a multiple of the K slice width (32): a slice straddles taps, so

@@ -7,6 +7,10 @@ void aspen_nasm_tile_range_internal (const nasm_ldata_t *ld, unsigned int t, uns
 
 void aspen_dse_group_set_mode (dse_group_t *g, int mode) { if (g) g->mode = mode < 0 || mode > 2 ? 2 : mode; }
 int aspen_dse_group_last_mode (dse_group_t *g) { return g ? g->last_mode : -1; }
+int aspen_dse_group_last_run_ordered (dse_group_t *g)
+{
+    return g != NULL && g->last_mode == 1 && g->rpool != NULL && g->rpool->graph != NULL && aspen_hip_graph_last_run_ordered (g->rpool->graph);
+}
 void aspen_dse_group_set_spin_limit (dse_group_t *g, uint64_t polls) { if (g) g->spin_limit = polls; }
 void aspen_dse_group_set_workgroups (dse_group_t *g, unsigned int w) { if (g) g->workgroups = w; }
 
@@ -80,6 +84,12 @@ int aspen_rpool_dataflow_trace (rpool_t *rp, uint64_t *start_end)
 {
     if (rp == NULL || rp->graph == NULL) return -1;
     return aspen_hip_dataflow_trace (rp->graph, start_end, aspen_rpool_num_ninst (rp));
+}
+
+int aspen_rpool_dataflow_trace_phases (rpool_t *rp, uint64_t *kloop_epilogue)
+{
+    if (rp == NULL || rp->graph == NULL) return -1;
+    return aspen_hip_dataflow_trace_phases (rp->graph, kloop_epilogue, aspen_rpool_num_ninst (rp));
 }
 
 int aspen_rpool_debug_set_epoch (rpool_t *rp, uint32_t epoch)

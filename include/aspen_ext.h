@@ -21,12 +21,14 @@ void apu_load_dnn_data_from_file (aspen_dnn_t *dnn, char *input_path);
 unsigned int aspen_dnn_device_generation (aspen_dnn_t *dnn);
 
 /* 0: one kernel launch per layer (layer-synchronous); 1: persistent dataflow kernel; 2 (default): the
-   persistent kernel unless the graph's average parallelism is below half a tile per compute unit (a
-   single image through a deep network), where one launch per layer is faster.
+   persistent kernel, unless the graph came from apu_generate_nasm and its timing found one launch per layer faster.
    The environment variable ASPEN_GPU_MODE=layers|dataflow|auto sets the initial value. */
 void aspen_dse_group_set_mode (dse_group_t *dse_group, int mode);
 /* the mode the last dse_group_run used: 0 or 1 (-1 before the first run) */
 int aspen_dse_group_last_mode (dse_group_t *dse_group);
+/* 1 when that run was a dataflow run in ordered mode (tiles taken in index order and prepared before they are ready,
+   no ready queue: what graphs built for one image through a deep network run in) */
+int aspen_dse_group_last_run_ordered (dse_group_t *dse_group);
 /* Watchdog of the persistent kernel: polls a workgroup may spend waiting for one ready tile before the
    run is given up (every workgroup then leaves, the run reports ASPEN_HIP_ERR_STALLED and the next run
    starts from re-armed state).  0 = the library's default (2^26 polls, minutes). */
@@ -69,6 +71,8 @@ int aspen_rpool_dataflow_profile (rpool_t *rpool, uint64_t ticks[16], int reset)
 /* start / end time stamps (100 MHz) of every tile of the pool's last run made with ASPEN_HIP_FLAG_TRACE;
    start_end holds 2 * aspen_rpool_num_ninst values, tiles in pool order (nasms in attachment order) */
 int aspen_rpool_dataflow_trace (rpool_t *rpool, uint64_t *start_end);
+/* the K-loop / epilogue stamps of the same run (aspen_hip_dataflow_trace_phases), same order */
+int aspen_rpool_dataflow_trace_phases (rpool_t *rpool, uint64_t *kloop_epilogue);
 /* Test hook: the tag the pool's next dataflow run derives its queue-entry tag from (aspen_hip_graph_debug_set_epoch);
    returns -1 when the pool has no device graph yet. */
 int aspen_rpool_debug_set_epoch (rpool_t *rpool, uint32_t epoch);

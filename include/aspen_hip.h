@@ -46,13 +46,15 @@ typedef struct aspen_hip_ktab_t
 enum { ASPEN_HIP_OPERAND_TABLE = 0, ASPEN_HIP_OPERAND_DIRECT = 1, ASPEN_HIP_OPERAND_DENSE3 = 2 };
 
 /* GEMM tile shapes (rows of the weight matrix x activation columns per workgroup): LARGE = the
-   biggest shape of the build (128 x 64 by default), WIDE = 64 x 128, SMALL = 64 x 64.  The graph
-   builder asks aspen_hip_tile_shapes for the numbers instead of assuming them. */
-enum { ASPEN_HIP_GEMM_LARGE = 0, ASPEN_HIP_GEMM_WIDE = 1, ASPEN_HIP_GEMM_SMALL = 2, ASPEN_HIP_NUM_GEMM_VARIANTS };
-/* shapes[2*v] = rows, shapes[2*v+1] = columns of GEMM variant v; shapes[6] = queries per K-attention
+   biggest shape of the build (128 x 64 by default), WIDE = 64 x 128, SMALL = 64 x 64, NARROW = 32 x 32 with the
+   workgroup's four wavefronts splitting the K axis (for graphs bound by the latency of their dependency
+   chains; operands DIRECT or TABLE with IC % 32 == 0 only).  The graph builder asks aspen_hip_tile_shapes for
+   the numbers instead of assuming them. */
+enum { ASPEN_HIP_GEMM_LARGE = 0, ASPEN_HIP_GEMM_WIDE = 1, ASPEN_HIP_GEMM_SMALL = 2, ASPEN_HIP_GEMM_NARROW = 3, ASPEN_HIP_NUM_GEMM_VARIANTS };
+/* shapes[2*v] = rows, shapes[2*v+1] = columns of GEMM variant v = 0..2; shapes[6] = queries per K-attention
    tile; shapes[7] = queries per V-attention tile; shapes[8] = workgroups per compute unit the
-   kernels are built for.  Pure constants: callable without a GPU. */
-void aspen_hip_tile_shapes (uint32_t shapes[9]);
+   kernels are built for; shapes[9], shapes[10] = rows, columns of variant 3.  Pure constants: callable without a GPU. */
+void aspen_hip_tile_shapes (uint32_t shapes[11]);
 
 /* Per-layer descriptor: everything one tile needs, so a tile is (layer, tile index).
    Replaces the fields the reference's tiled_* read through ninst->ldata->layer
@@ -76,7 +78,7 @@ typedef struct aspen_hip_layer_t
     /* split-K (contraction layers): the layer has T*splits tiles, T = tiles_m*tiles_n; tile
        (tile*splits + slice) computes the partial products over kiters_per_split K slices and writes
        them to `partial` ([splits][T] blocks of tile_m*tile_n floats in the kernel's own register order;
-       64 x 64 tiles only).  The `splits` tiles of one output tile form a group: the
+       64 x 64 and 32 x 32 tiles only).  The `splits` tiles of one output tile form a group: the
        member that finishes last (an arrival counter decides) sums the slices in slice order, adds
        the bias, activates and writes the output; only it releases the group's children */
     uint32_t splits, kiters_per_split;
@@ -189,7 +191,18 @@ int aspen_hip_dataflow_profile (aspen_hip_graph_t *graph, uint64_t ticks[16], in
    by ASPEN_GPU_XCD_QUEUES in the environment; ASPEN_GPU_XCD_QUEUE_SHIFT = 1 / 2 groups the XCDs in pairs / fours (4 / 2
    queues).  Needs a grid that is a multiple of 8 workgroups (else ignored). */
 #define ASPEN_HIP_FLAG_XCD_QUEUES 32u
+/* ORDERED / NO_ORDERED force or forbid the ordered mode of the persistent kernel, which a run otherwise takes when
+   the graph's average parallelism is below 128 tiles (one image through a deep network): no ready queue; workgroups
+   take the tiles in index order (parents first), prepare each one and request its first weights before it is ready,
+   then wait on the tile's own dependency counter.  Also ASPEN_GPU_ORDERED=0|1 in the environment. */
+void aspen_hip_graph_set_ordered (aspen_hip_graph_t *graph, int ordered);     /* 1 / 0: this graph's dataflow runs use / do not use the ordered mode; -1: decided from its parallelism */
+int aspen_hip_graph_last_run_ordered (const aspen_hip_graph_t *graph);          /* 1 when the graph's last dataflow run was an ordered one */
+#define ASPEN_HIP_FLAG_ORDERED 64u
+#define ASPEN_HIP_FLAG_NO_ORDERED 128u
 int aspen_hip_dataflow_trace (aspen_hip_graph_t *graph, uint64_t *start_end, uint32_t num_ninst);
+/* Two more stamps per contraction tile of the same traced run: kloop_epilogue[2*i] = end of tile i's K loop,
+   [2*i+1] = its epilogue's (or, for a split-K member, its partial sums') stores issued; 0 for other tiles. */
+int aspen_hip_dataflow_trace_phases (aspen_hip_graph_t *graph, uint64_t *kloop_epilogue, uint32_t num_ninst);
 void aspen_hip_set_flags (uint32_t flags);
 /* Waits for everything enqueued on the library's stream.  Reports device errors only; whether a dataflow
    run was given up is a property of its graph, see aspen_hip_graph_sync. */

@@ -50,6 +50,8 @@ def lib():
         L.refglue_result.restype = C.c_long
         L.refglue_save_dnn.argtypes = [C.c_void_p, C.c_char_p]
         L.refglue_save_nasm.argtypes = [C.c_void_p, C.c_uint, C.c_uint, C.c_uint, C.c_char_p]
+        L.refglue_time_dse.argtypes = [C.c_void_p, C.c_uint, C.c_uint, C.c_uint, _fp, C.c_int, C.c_int, C.c_int, _fp, C.c_long]
+        L.refglue_time_dse.restype = C.c_double
         L.refglue_close.argtypes = [C.c_void_p]
         _lib = L
     return _lib
@@ -115,6 +117,18 @@ class RefNet:
 
     def time_forward(self, iters: int) -> float:
         return float(lib().refglue_time_forward(self.h, iters))
+
+    def time_dse(self, x: np.ndarray, batch: int, seq: int, min_ninst: int, num_dse: int, warmup: int, iters: int):
+        """The reference's own scheduler: apu_create_nasm (full dependency search) + the run loop of its main.c on
+        num_dse DSE threads.  Returns (seconds per inference, final layer as [columns][rows])."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        i = self.info(self.num_layers - 1)
+        out = np.zeros((i["W"], i["H"]), dtype=np.float32)
+        sec = float(lib().refglue_time_dse(self.h, batch, seq, min_ninst, x.ctypes.data_as(_fp), num_dse, warmup, iters,
+                                           out.ctypes.data_as(_fp), out.size))
+        if sec < 0:
+            raise RuntimeError("the reference could not build the graph")
+        return sec, out
 
     def close(self):
         if self.h:

@@ -194,6 +194,51 @@ int refglue_save_nasm (void *h, unsigned int batch, unsigned int seq, unsigned i
     return n;
 }
 
+/* The reference's own run loop (main.c:105-123) with its own scheduler: a graph with the full tile-dependency
+   search (apu_create_nasm: seconds at batch 1, minutes at batch 32), num_dse DSE pthreads on one ready pool,
+   `warmup` + `iters` times { rpool_reset_queue; rpool_reset_nasm; dse_group_run; dse_wait_for_nasm_completion;
+   dse_group_stop }.  Returns seconds per iteration (< 0 on failure); the final layer of the last iteration goes to
+   `result` (dense, W columns of H floats, at most max_floats) through dse_get_nasm_result when result != NULL. */
+double refglue_time_dse (void *h, unsigned int batch, unsigned int seq, unsigned int min_ninst_per_ldata, float *dense_input,
+    int num_dse, int warmup, int iters, float *result, long max_floats)
+{
+    refglue_t *g = h;
+    nasm_t *nasm = seq ? apu_create_transformer_nasm (g->dnn, min_ninst_per_ldata, batch, seq)
+                       : apu_create_nasm (g->dnn, min_ninst_per_ldata, batch);
+    if (nasm == NULL)
+        return -1.0;
+    rpool_t *rpool = rpool_init ();
+    dse_group_t *dse_group = dse_group_init (num_dse);
+    dse_group_set_rpool (dse_group, rpool);
+    rpool_add_nasm_raw_input (rpool, nasm, dense_input);
+    double t0 = 0.0;
+    for (int i = 0; i < warmup + iters; i++)
+    {
+        if (i == warmup)
+            t0 = omp_get_wtime ();
+        if (i > 0)
+        {
+            rpool_reset_queue (rpool);
+            rpool_reset_nasm (rpool, nasm);
+        }
+        dse_group_run (dse_group);
+        dse_wait_for_nasm_completion (nasm);
+        dse_group_stop (dse_group);
+    }
+    const double sec = (omp_get_wtime () - t0) / (iters > 0 ? iters : 1);
+    if (result != NULL)
+    {
+        nasm_ldata_t *last = &nasm->ldata_arr[nasm->num_ldata - 1];
+        const long n = (long)last->out_mat_dims[OUT_H] * last->out_mat_dims[OUT_W];
+        if (n <= max_floats && last->out_mat != NULL)
+            copy_ldata_out_mat_to_buffer (last, result);
+    }
+    dse_group_destroy (dse_group);
+    rpool_destroy (rpool);
+    apu_destroy_nasm (nasm);
+    return sec;
+}
+
 void refglue_close (void *h)
 {
     refglue_t *g = h;

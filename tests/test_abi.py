@@ -58,7 +58,7 @@ def test_reference_api_names_present():
 
 
 def test_tile_shapes_are_constants():
-    s = (ctypes.c_uint32 * 9)()
+    s = (ctypes.c_uint32 * 11)()
     api.lib().aspen_hip_tile_shapes(s)
     shapes = list(s)
     for v in range(3):

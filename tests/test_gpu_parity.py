@@ -11,10 +11,25 @@ from tests import helpers as H
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("mode", [api.MODE_LAYERS, api.MODE_DATAFLOW], ids=["layers", "dataflow"])
+# engine variants of the persistent kernel: ready queue (flag 128 forbids the ordered mode small graphs take by default)
+# and ordered mode (flag 64 forces it)
+QUEUE, ORDERED = 128, 64
+
+
+@pytest.fixture
+def engine_flags():
+    """Sets the engine flags for one test (2 = count executed tiles) and restores the default afterwards."""
+    def set_flags(flags):
+        api.lib().aspen_hip_set_flags(2 | flags)
+    yield set_flags
+    api.lib().aspen_hip_set_flags(2)
+
+
+@pytest.mark.parametrize("mode,flags", [(api.MODE_LAYERS, 0), (api.MODE_DATAFLOW, QUEUE), (api.MODE_DATAFLOW, ORDERED)], ids=["layers", "dataflow", "ordered"])
 @pytest.mark.parametrize("name", list(H.micro_cases()))
-def test_micro_nets_match_reference_fixture(gpu, name, mode):
+def test_micro_nets_match_reference_fixture(gpu, engine_flags, name, mode, flags):
     """Full per-layer tensors of small nets, as produced by the compiled reference."""
+    engine_flags(flags)
     cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()[name])
     gold = np.load(os.path.join(H.GOLDEN, f"micro_{name}.npz"))
     net = H.GpuNet(cfg, tens, batch, seq, min_ninst=8, mode=mode)
@@ -35,17 +50,19 @@ def test_micro_nets_match_reference_fixture(gpu, name, mode):
         net.close()
 
 
-@pytest.mark.parametrize("loads", ["cached", "coherent", "unfused"])
+@pytest.mark.parametrize("loads", ["cached", "coherent", "unfused", "ordered"])
 @pytest.mark.parametrize("name", list(H.micro_cases()))
-def test_micro_nets_match_oracle(gpu, name, loads, monkeypatch):
+def test_micro_nets_match_oracle(gpu, engine_flags, name, loads, monkeypatch):
     """Same nets against the CPU oracle (full tensors), dataflow engine with few workgroups so that
     tiles of several layers are in flight together.  The graph is re-armed and re-run with a
     DIFFERENT input each time: a tile that read a stale (cached) copy of its parent's previous
     output would not match the oracle of the new input.  Both load policies of the persistent kernel
     run: activations through the caches (the default when the layout allows it) and device-coherent;
     a third variant keeps the shortcut layers as tiles of their own instead of fusing them into the
-    producing contraction tile."""
+    producing contraction tile; a fourth runs the ordered mode (tiles taken in index order and prepared
+    before they are ready) instead of the ready queue."""
     from oracle import cpu
+    engine_flags(ORDERED if loads == "ordered" else QUEUE)
     if loads == "coherent":
         monkeypatch.setenv("ASPEN_GPU_COHERENT_LOADS", "1")      # read when the device graph is built (first run)
     if loads == "unfused":
@@ -239,9 +256,11 @@ def test_results_in_the_callers_dimension_order(gpu):
         net.close()
 
 
-def test_engine_rearm_many_runs(gpu):
+@pytest.mark.parametrize("flags", [QUEUE, ORDERED], ids=["queue", "ordered"])
+def test_engine_rearm_many_runs(gpu, engine_flags, flags):
     """Re-arm and re-run one graph many times: every run must execute each tile exactly once, never
     stall, and reproduce the first run bit for bit (tiles are deterministic; only their order varies)."""
+    engine_flags(flags)
     cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()["gpt_mini_b2_s20"])
     net = H.GpuNet(cfg, tens, batch, seq, min_ninst=64, mode=api.MODE_DATAFLOW)
     print(f"tiles {net.nasm.num_ninst}", flush=True)
@@ -270,7 +289,7 @@ def test_queue_entries_of_earlier_runs_are_never_taken(gpu):
     L = api.lib()
     try:
         first = None
-        settings = [(0, 0), (16, 0), (32, 256), (0, 64), (32 | 16, 512)]
+        settings = [(QUEUE, 0), (QUEUE | 16, 0), (QUEUE | 32, 256), (QUEUE, 64), (QUEUE | 32 | 16, 512), (ORDERED, 0)]
 
         def run_and_check(rep):
             nonlocal first
@@ -289,7 +308,7 @@ def test_queue_entries_of_earlier_runs_are_never_taken(gpu):
             run_and_check(rep)
         # one run with per-XCD queues right before the wrap, plain runs across it, the same setting again after it
         net.rpool.debug_set_epoch(65533)
-        for rep in (2, 0, 0, 0, 2, 1, 4, 3):
+        for rep in (2, 0, 5, 0, 2, 1, 4, 3):
             run_and_check(rep)
     finally:
         L.aspen_hip_set_flags(2)
@@ -741,7 +760,9 @@ def test_reference_main_call_sequence(gpu, tmp_path):
 @pytest.mark.parametrize("name,min_ninst,workgroups,flags", [("resnet_mini_b2", 1024, 0, 0), ("gpt_mini_b2_s20", 64, 16, 0), ("yolo_mini_b2", 16, 0, 0),
                                                             ("resnet50_b1", 128, 0, 0), ("bert_base_b8_s128", 192, 0, 0),
                                                             ("resnet_mini_b2", 1024, 0, 32), ("gpt_mini_b2_s20", 64, 16, 32),
-                                                            ("resnet50_b1", 128, 0, 32), ("resnet_mini_b2", 1024, 0, 16)],
+                                                            ("resnet50_b1", 128, 0, 32), ("resnet_mini_b2", 1024, 0, 16),
+                                                            ("resnet_mini_b2", 1024, 0, ORDERED), ("gpt_mini_b2_s20", 64, 16, ORDERED),
+                                                            ("yolo_mini_b2", 16, 0, ORDERED), ("resnet50_b1", 128, 0, ORDERED)],
                          ids=lambda v: str(v))
 def test_no_tile_starts_before_its_parents_have_ended(gpu, name, min_ninst, workgroups, flags):
     """The scheduler's invariant (reference src/dse.c:32-38, 311-317: a ninst runs only once all its parents are
@@ -749,20 +770,21 @@ def test_no_tile_starts_before_its_parents_have_ended(gpu, name, min_ninst, work
     every dependency edge the child's start stamp is not earlier than the parent's end stamp, which is taken
     after the parent's stores were acknowledged.  The members of a split-K group release their children
     together, through whichever member finishes last: a child waits for the group's last end.
-    flags: 0 = the default engine, 32 = one ready queue per XCD, 16 = no parent -> child hand-off; the final layer must
-    come out bit-identical to the default engine's in every variant (tiles do the same arithmetic wherever they run)."""
+    flags: 0 = the ready queue, 32 = one ready queue per XCD, 16 = no parent -> child hand-off, 64 = ordered mode (no
+    queue; a tile's start stamp is taken when its wait for the parents is over); the final layer must come out
+    bit-identical to the default engine's in every variant (tiles do the same arithmetic wherever they run)."""
     micro = name in H.micro_cases()
     cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()[name]) if micro else H.full_config(name)
     expected = None
     if flags:
-        api.lib().aspen_hip_set_flags(2)
+        api.lib().aspen_hip_set_flags(2 | QUEUE)
         plain = H.GpuNet(cfg, tens, batch, seq, min_ninst=min_ninst, mode=api.MODE_DATAFLOW, workgroups=workgroups)
         try:
             plain.run(x)
             expected = plain.nasm.layer_output(plain.nasm.num_ldata - 1).copy()
         finally:
             plain.close()
-    api.lib().aspen_hip_set_flags(2 | 8 | flags)
+    api.lib().aspen_hip_set_flags(2 | 8 | (flags if flags & ORDERED else flags | QUEUE))
     net = H.GpuNet(cfg, tens, batch, seq, min_ninst=min_ninst, mode=api.MODE_DATAFLOW, workgroups=workgroups)
     try:
         for rep in range(2):                                     # also on a re-armed graph
