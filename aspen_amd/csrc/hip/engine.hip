@@ -889,6 +889,11 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
     {
         if (!L.in1 || L.hd == 0 || L.heads == 0 || L.seq == 0) why = "attention geometry";
         else if (L.tile_n != VATTN_BN || L.tile_m > 64 || L.hd % L.tile_m) why = "V-attention tile extent (queries x <=64 channels of one head)";
+        else if (L.direct == ASPEN_HIP_ATTENTION_FUSED)
+        {
+            if (!L.fuse_in || L.fuse_ld_in % 4 || L.hd > 64 || L.hd % GEMM_BK || L.tile_m != L.hd || L.ld0 < L.heads * L.hd || L.ld1 < L.heads * L.hd || L.fuse_ld_in < L.heads * L.hd)
+                why = "fused attention takes whole heads of 32 or 64 channels and Query / Key / Value matrices";
+        }
         else if (L.ld0 % GEMM_BK || L.ld0 < L.seq) why = "probability stride must be a multiple of 32 covering seq";
     }
     else if (L.type == MAXPOOL_LAYER || L.type == AVGPOOL_LAYER)
@@ -929,7 +934,7 @@ static bool lines_have_one_producer (const aspen_hip_layer_t *layers, uint32_t n
         const aspen_hip_layer_t &P = layers[l];
         if (P.type == INPUT_LAYER || P.num_ninst == 0) continue;      // written by the host before the launch
         bool is_read = false;
-        for (uint32_t c = 0; c < num_layers && !is_read; c++) is_read = layers[c].in0 == P.out || layers[c].in1 == P.out || layers[c].fuse_in == P.out;
+        for (uint32_t c = 0; c < num_layers && !is_read; c++) is_read = layers[c].num_ninst != 0 && (layers[c].in0 == P.out || layers[c].in1 == P.out || layers[c].fuse_in == P.out);
         const bool aligned = (uintptr_t)P.out % 128 == 0 && ((size_t)P.ld * 4) % 128 == 0 && (P.tiles_m == 1 || (P.tile_m * 4) % 128 == 0);
         const bool ok = !(is_read && !aligned) && !(P.splits > 1 && ((uintptr_t)P.partial % 128 != 0 || !aligned))
             && !(P.fuse_out && ((uintptr_t)P.fuse_out % 128 != 0 || !aligned));

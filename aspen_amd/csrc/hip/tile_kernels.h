@@ -1458,6 +1458,106 @@ __device__ __forceinline__ void tile_v_attention (const aspen_hip_layer_t &L, ui
             }
 }
 
+// Fused attention tile: one (batch, head) x VATTN_BN queries, scores and weighted values in one pass, the S x S
+// probability matrix never leaves the chip (reference: tiled_k_attention followed by tiled_v_attention,
+// src/tiled_kernels.c:784-1037, which round-trip it through memory).  Per block of 64 keys:
+//   e[q][key] = exp (scale * (key > q && masked ? -1e10 : K[key] . Q[q]))      (the reference's order of operations,
+//                                                                               no max subtraction)
+//   rowsum[q] += sum_key e[q][key];   O[q][ch] += sum_key e[q][key] * V[key][ch]
+// and at the end O[q][ch] / rowsum[q].  The reference divides the probabilities first and multiplies then; dividing
+// the sum of products instead differs by rounding only (1e-7 relative).  The exponentials of a key block go to LDS in
+// the layout of an activation operand (row = query, K axis = key), the transposed values are staged next to them.
+// in0 = Query, in1 = Key, fuse_in = Value (stride fuse_ld_in); one head of at most 64 channels per tile.
+// Used when nothing but the V-attention layer reads the probabilities and their matrix need not be kept.
+// ---------------------------------------------------------------------------------------------
+template <int COH>
+__device__ __forceinline__ void tile_fused_attention (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, float *smem)
+{
+    constexpr int BQ = VATTN_BN, BKEY = 64, EROW = BKEY + 4;
+    static_assert (BQ == 64, "four wavefronts, one 32 x 32 block each");
+    static_assert ((64 + BQ) * LDS_ROW + BQ * EROW <= GEMM_SMEM_FLOATS, "operand stage and exponentials fit the tile's LDS");
+    __shared__ float qsum[BQ];
+    const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
+    const uint32_t S = L.seq, qtiles = (S + BQ - 1) / BQ;
+    const uint32_t b = tn / qtiles, q0 = (tn - b * qtiles) * BQ;
+    const uint32_t h = tm, hd = L.hd;
+    const uint32_t wm0 = (wave % 2) * 32, wn0 = (wave / 2) * 32;       // keys (phase 1) / channels (phase 2), queries
+    ActView<COH> Q, Kmat, V, out;
+    Q.init (L.in0, L.N, L.ld0); Kmat.init (L.in1, L.N, L.ld1); V.init (L.fuse_in, L.N, L.fuse_ld_in); out.init (L.out, L.N, L.ld);
+    const float scale = 1.0f / sqrtf ((float)hd);
+    const uint32_t kend = L.masked ? min (S, q0 + (uint32_t)BQ) : S;
+    const int kiters = (int)(hd / GEMM_BK);
+    float *ebuf = smem + (64 + BQ) * LDS_ROW;
+    if (tid < BQ) qsum[tid] = 0.f;                       // ordered before the atomics below by the barriers of the K loops
+    floatx16 oacc;
+    float part[16];
+    #pragma unroll
+    for (int v = 0; v < 16; v++) { oacc[v] = 0.f; part[v] = 0.f; }
+    for (uint32_t k0 = 0; k0 < kend; k0 += BKEY)
+    {
+        // scores of 64 keys x 64 queries: one 32 x 32 block per wavefront
+        floatx16 sacc[1][1];
+        {
+            ActRowLoader<64, COH> al; al.init (Kmat, b * S + k0, b * S + S - 1, L.ld1, h * hd, tid);
+            ActRowLoader<BQ, COH> bl; bl.init (Q, b * S + q0, b * S + S - 1, L.ld0, h * hd, tid);
+            gemm_core_single_block<1> (al, bl, 0, kiters, smem, sacc);          // ends with a barrier: the stage is free
+        }
+        #pragma unroll
+        for (int v = 0; v < 16; v++)
+        {
+            const uint32_t ql = ACC_N (wn0, 0, v, lane), key = k0 + wm0 + (lane & 31), q = q0 + ql;
+            float sc = sacc[0][0][v];
+            if (L.masked && key > q) sc = -1e10f;
+            const float e = (key < S && q < S) ? __expf (sc * scale) : 0.f;
+            part[v] += e;
+            ebuf[ql * EROW + wm0 + (lane & 31)] = e;
+        }
+        // weighted values: O[q][ch] += e[q][key] V[key][ch], two slices of 32 keys; V is read transposed through the stage
+        TransLoader64<COH> vl;
+        vl.init (V, (b * S + k0) * L.fuse_ld_in + h * hd, L.fuse_ld_in, hd, S - k0, tid);
+        float4 vreg[2];
+        vl.load (0, vreg);
+        #pragma unroll
+        for (int sl = 0; sl < BKEY / GEMM_BK; sl++)
+        {
+            vl.store (smem, vreg);
+            if (sl + 1 < BKEY / GEMM_BK) vl.load (sl + 1, vreg);
+            __syncthreads ();                            // the stage and (first slice) the exponentials are complete
+            const float *af = smem + (wm0 + (lane & 31)) * LDS_ROW + (lane >> 5) * 4;
+            const float *bf = ebuf + (wn0 + (lane & 31)) * EROW + sl * GEMM_BK + (lane >> 5) * 4;
+            #pragma unroll
+            for (int sub = 0; sub < 4; sub++)
+            {
+                const float4 a = ld4 (af + sub * 8), e4 = ld4 (bf + sub * 8);
+                oacc = __builtin_amdgcn_mfma_f32_32x32x2f32 (e4.x, a.x, oacc, 0, 0, 0);
+                oacc = __builtin_amdgcn_mfma_f32_32x32x2f32 (e4.y, a.y, oacc, 0, 0, 0);
+                oacc = __builtin_amdgcn_mfma_f32_32x32x2f32 (e4.z, a.z, oacc, 0, 0, 0);
+                oacc = __builtin_amdgcn_mfma_f32_32x32x2f32 (e4.w, a.w, oacc, 0, 0, 0);
+            }
+            __syncthreads ();                            // everyone has read the stage (and, last slice, the exponentials)
+        }
+    }
+    // row sums: the 32 lanes of a half-wave hold 32 keys of the same query; two wavefronts share a query block
+    #pragma unroll
+    for (int v = 0; v < 16; v++)
+    {
+        float t = part[v];
+        #pragma unroll
+        for (int o = 16; o > 0; o >>= 1) t += __shfl_xor (t, o, 64);
+        if ((lane & 31) == 0) atomicAdd (&qsum[ACC_N (wn0, 0, v, lane)], t);
+    }
+    __syncthreads ();
+    const uint32_t ch = wm0 + (lane & 31);
+    if (ch < hd)
+        #pragma unroll
+        for (int v = 0; v < 16; v++)
+        {
+            const uint32_t ql = ACC_N (wn0, 0, v, lane), q = q0 + ql;
+            if (q < S) out.st1 ((b * S + q) * L.ld + h * hd + ch, oacc[v] / qsum[ql]);
+        }
+    __syncthreads ();                                    // qsum is reused by the next tile of this workgroup
+}
+
 // ---------------------------------------------------------------------------------------------
 // Dispatch: the device-side counterpart of the switch in the reference's dse_schedule
 // (reference src/dse.c:39-79).  `t` = tile index inside the layer, row-tile fastest
@@ -1917,7 +2017,14 @@ __device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, boo
     case LAYERNORM_LAYER:   if constexpr ((FEAT & TILES_NORM) != 0) { ready (); tile_layernorm<COH> (L, tn); } break;
     case SOFTMAX_LAYER:     if constexpr ((FEAT & TILES_NORM) != 0) { ready (); tile_softmax<COH> (L, tn); } break;
     case K_ATTENTION_LAYER: if constexpr ((FEAT & TILES_ATTENTION) != 0) { ready (); tile_k_attention<COH> (L, tn, smem); } break;
-    case V_ATTENTION_LAYER: if constexpr ((FEAT & TILES_ATTENTION) != 0) { ready (); tile_v_attention<COH> (L, tn, tm, smem); } break;
+    case V_ATTENTION_LAYER:
+        if constexpr ((FEAT & TILES_ATTENTION) != 0)
+        {
+            ready ();
+            if (L.direct == ASPEN_HIP_ATTENTION_FUSED) tile_fused_attention<COH> (L, tn, tm, smem);
+            else tile_v_attention<COH> (L, tn, tm, smem);
+        }
+        break;
     default: break;
     }
     return true;

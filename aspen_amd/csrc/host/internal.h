@@ -79,6 +79,10 @@ struct nasm_ldata_t
        residual's); the residual then owns no tiles.  -1 = not fused */
     int fused_residual;                      /* contraction layer: index of the residual it also produces */
     int fused_into;                          /* residual layer: index of the contraction layer producing it */
+    /* attention fusion: a V-attention layer whose K-attention parent feeds nothing else computes scores, exponentials and
+       weighted values in one tile (the S x S probabilities stay on chip); the K-attention layer then owns no tiles and
+       its matrix is not written.  -1 = not fused */
+    int fused_attention;                     /* V-attention layer: index of the K-attention layer it absorbs */
     uint64_t flops;                          /* 2*M*N*K for contraction layers, 64-bit */
 };
 

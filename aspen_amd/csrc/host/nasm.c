@@ -372,7 +372,14 @@ static void find_parents (const nasm_t *nasm, const nasm_ldata_t *ld, unsigned i
     {
         const unsigned int H = p[NUM_HEAD], hd = p[NUM_HIDDEN] / H;
         const unsigned int b = c0 / S, h = r0 / hd, q0 = c0 % S, q1 = q0 + (c1 - c0);
-        add_parents (p0, (b * H + h) * S + q0, (b * H + h) * S + q1, 0, S, out); /* probability rows */
+        if (ld->fused_attention >= 0)
+        {
+            /* the tile computes its probabilities itself: it reads what the K-attention tile would have read */
+            const nasm_ldata_t *kl = &nasm->ldata_arr[ld->fused_attention];
+            add_parents (&nasm->ldata_arr[kl->parent_ldata_idx[PARENT_0]], b * S + q0, b * S + q1, h * hd, (h + 1) * hd, out);   /* its Queries */
+            add_parents (&nasm->ldata_arr[kl->parent_ldata_idx[PARENT_1]], b * S, (b + 1) * S, h * hd, (h + 1) * hd, out);       /* every Key */
+        }
+        else add_parents (p0, (b * H + h) * S + q0, (b * H + h) * S + q1, 0, S, out); /* probability rows */
         add_parents (p1, b * S, (b + 1) * S, r0, r1, out);                       /* every Value of the sequence */
         break;
     }
@@ -476,6 +483,35 @@ static void fuse_shortcuts (nasm_t *nasm)
     }
 }
 
+/* Attention fusion.  The reference computes the S x S probabilities of every (batch, head) in one layer and
+   multiplies them with the values in the next (tiled_k_attention / tiled_v_attention, src/tiled_kernels.c:784-1037),
+   through memory.  When nothing else reads the probabilities and their matrix need not be kept, the V-attention
+   layer's tiles compute both steps and the K-attention layer loses its tiles (its matrix is then not written, like
+   the pre-shortcut matrix of a fused shortcut). */
+static void fuse_attention (nasm_t *nasm)
+{
+    if (aspen_keep_layer_outputs_enabled () || getenv ("ASPEN_GPU_NO_FUSE_ATTENTION") != NULL) return;
+    for (unsigned int v = 0; v < nasm->num_ldata; v++)
+    {
+        nasm_ldata_t *vl = &nasm->ldata_arr[v];
+        if (vl->layer->type != V_ATTENTION_LAYER) continue;
+        const int k = vl->parent_ldata_idx[PARENT_0];
+        if (k < 0 || nasm->ldata_arr[k].layer->type != K_ATTENTION_LAYER) continue;
+        nasm_ldata_t *kl = &nasm->ldata_arr[k];
+        const unsigned int hd = vl->layer->params[NUM_HIDDEN] / vl->layer->params[NUM_HEAD];
+        if (hd > 64 || hd % 32 != 0 || vl->tile_dims[OUT_H] != hd) continue;
+        if (kl->layer->params[NUM_HEAD] != vl->layer->params[NUM_HEAD] || kl->layer->params[NUM_HIDDEN] != vl->layer->params[NUM_HIDDEN]) continue;
+        unsigned int consumers = 0;
+        for (unsigned int l = 0; l < nasm->num_ldata; l++)
+            for (int p = PARENT_0; p <= PARENT_1; p++)
+                consumers += nasm->ldata_arr[l].parent_ldata_idx[p] == k;
+        if (consumers != 1 || kl->parent_ldata_idx[PARENT_0] < 0 || kl->parent_ldata_idx[PARENT_1] < 0) continue;
+        vl->fused_attention = k;
+        kl->out_discarded = 1;
+        kl->num_ninst = 0; kl->tiles_h = kl->tiles_w = 0;
+    }
+}
+
 static nasm_t *build_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned int batch, unsigned int seq, unsigned int kiters_cap, int small_tiles_only, int narrow_tiles)
 {
     if (dnn == NULL) { ERROR_PRTF ("apu_create_nasm: dnn is NULL\n"); return NULL; }
@@ -499,7 +535,7 @@ static nasm_t *build_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned in
     {
         nasm_ldata_t *ld = &nasm->ldata_arr[l];
         ld->nasm = nasm; ld->layer = &dnn->layers[l];
-        ld->fused_residual = ld->fused_into = -1;
+        ld->fused_residual = ld->fused_into = ld->fused_attention = -1;
         ld->out_discarded = 0;
         for (int k = 0; k < NUM_PARENT_ELEMENTS; k++) ld->parent_ldata_idx[k] = ld->layer->parent_idx[k];
         if (set_out_mat (nasm, ld) || set_tiles (nasm, ld)) { bad = 1; break; }
@@ -513,6 +549,7 @@ static nasm_t *build_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned in
         }
     }
     if (!bad && getenv ("ASPEN_GPU_NO_FUSE") == NULL) fuse_shortcuts (nasm);
+    if (!bad) fuse_attention (nasm);
     for (unsigned int l = 0; l < nasm->num_ldata && !bad; l++)
     {
         nasm_ldata_t *ld = &nasm->ldata_arr[l];
@@ -789,6 +826,18 @@ int aspen_nasm_fill_device_layers (nasm_t *nasm, aspen_hip_layer_t *dst, uint32_
         if (L->type == K_ATTENTION_LAYER || L->type == V_ATTENTION_LAYER)
         {
             d->heads = p[NUM_HEAD]; d->seq = nasm->tr_seq_len; d->hd = p[NUM_HIDDEN] / p[NUM_HEAD]; d->masked = p[MASKED];
+        }
+        if (ld->fused_attention >= 0)
+        {
+            /* in0 = Query, in1 = Key (the K-attention layer's parents), fuse_in = Value */
+            const nasm_ldata_t *kl = &nasm->ldata_arr[ld->fused_attention];
+            const nasm_ldata_t *ql = &nasm->ldata_arr[kl->parent_ldata_idx[PARENT_0]], *keyl = &nasm->ldata_arr[kl->parent_ldata_idx[PARENT_1]];
+            const nasm_ldata_t *vl = &nasm->ldata_arr[ld->parent_ldata_idx[PARENT_1]];
+            d->direct = ASPEN_HIP_ATTENTION_FUSED;
+            d->in0 = nasm->d_arena + ql->out_mat_offset; d->ld0 = ql->out_mat_stride;
+            d->in1 = nasm->d_arena + keyl->out_mat_offset; d->ld1 = keyl->out_mat_stride;
+            d->fuse_in = nasm->d_arena + vl->out_mat_offset; d->fuse_ld_in = vl->out_mat_stride;
+            d->masked = kl->layer->params[MASKED];
         }
     }
     return 0;

@@ -386,6 +386,9 @@ WORKLOADS = {
     "resnet50_b1": (["resnet50_b1"], "img/s", 1, 256, "dataflow"),
     "vgg16_b32": (["vgg16_b32"], "img/s", 32, 1536, "dataflow"),
     "co_resnet50_vgg16_b16": (["resnet50_b16", "vgg16_b16"], "img/s", 32, 1536, "dataflow"),
+    # the two halves of the co-scheduled pair on their own: what back-to-back runs would take
+    "resnet50_b16": (["resnet50_b16"], "img/s", 16, 1536, "dataflow"),
+    "vgg16_b16": (["vgg16_b16"], "img/s", 16, 1536, "dataflow"),
     "bert_base_b8_s128": (["bert_base_b8_s128"], "tokens/s", 8 * 128, 192, "dataflow"),
     "gpt2_b4_s512": (["gpt2_b4_s512"], "tokens/s", 4 * 512, 384, "dataflow"),
     "yolov3_b1": (["yolov3_b1"], "img/s", 1, 768, "layers"),

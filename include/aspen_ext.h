@@ -51,7 +51,9 @@ uint64_t aspen_nasm_total_flops (nasm_t *nasm);
    parent0, parent1 (0xffffffff = none), first tile index, GEMM variant,
    [12] shortcut layers: index of the contraction layer whose tiles produce this layer (0xffffffff = own tiles),
    [13] contraction layers: index of the shortcut layer fused into the epilogue (0xffffffff = none),
-   [14] split-K slices, [15] row tiles, [16] K slices of 32 per split-K part, [17..19] reserved (0) */
+   [14] split-K slices, [15] row tiles, [16] K slices of 32 per split-K part,
+   [17] 1 when the layer's matrix is not written (nothing on the device reads it and outputs are not kept),
+   [18] V-attention layers: index of the K-attention layer whose work its tiles absorb (0xffffffff = none), [19] reserved (0) */
 void aspen_nasm_ldata_info (nasm_t *nasm, unsigned int ldata_idx, unsigned int *info);
 uint64_t aspen_nasm_ldata_flops (nasm_t *nasm, unsigned int ldata_idx);
 /* dependency graph in CSR form; pointers stay valid until the nasm is destroyed */

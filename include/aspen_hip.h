@@ -44,6 +44,11 @@ typedef struct aspen_hip_ktab_t
    the last 3 - c % 3 channels of tap 4c / 3 and the first c % 3 + 1 of the next tap; the table holds TWO entries per
    chunk, 2c for the first tap and 2c + 1 for the second, each with the offset of that pixel's channel 0. */
 enum { ASPEN_HIP_OPERAND_TABLE = 0, ASPEN_HIP_OPERAND_DIRECT = 1, ASPEN_HIP_OPERAND_DENSE3 = 2 };
+/* aspen_hip_layer_t.direct of a V-attention layer.  FUSED: the layer's tiles compute the scores, their exponentials
+   and the weighted values in one pass from in0 = Query, in1 = Key and fuse_in = Value (stride fuse_ld_in), with
+   `masked` as the K-attention layer has it; the K-attention layer in front of it then has no tiles and its S x S
+   matrix is not written (one head of hd <= 64, hd % 32 == 0, channels per tile).  0: in0 = probabilities, in1 = Value. */
+enum { ASPEN_HIP_ATTENTION_FUSED = 1 };
 
 /* GEMM tile shapes (rows of the weight matrix x activation columns per workgroup): LARGE = the
    biggest shape of the build (128 x 64 by default), WIDE = 64 x 128, SMALL = 64 x 64, NARROW = 32 x 32 with the

@@ -183,11 +183,23 @@ def test_channel_counts_off_the_slice_width_in_a_graph_of_large_tiles(gpu, mode)
         net.close()
 
 
+@pytest.mark.parametrize("fused", [False, True], ids=["two-layers", "fused"])
 @pytest.mark.parametrize("mode", [api.MODE_LAYERS, api.MODE_DATAFLOW], ids=["layers", "dataflow"])
 @pytest.mark.parametrize("masked", [True, False], ids=["causal", "full"])
-def test_attention_over_a_long_ragged_sequence_matches_oracle(gpu, mode, masked):
+def test_attention_over_a_long_ragged_sequence_matches_oracle(gpu, mode, masked, fused):
     """A sequence that is a multiple of neither tile extent of the attention layers: 272 tokens = 8 x 32 + 16 queries and
-    2 x 128 + 16 keys per (batch, head), with and without the causal mask, every layer against the oracle."""
+    2 x 128 + 16 keys per (batch, head) (4 x 64 + 16 of either for the fused tile), with and without the causal mask,
+    every layer against the oracle.  fused: layer outputs are not kept, so the V-attention tiles compute scores,
+    exponentials and weighted values in one pass and the probability matrix is never written."""
+    from oracle import cpu
+    api.lib().aspen_keep_layer_outputs(0 if fused else 1)
+    try:
+        _ragged_attention(mode, masked, fused)
+    finally:
+        api.lib().aspen_keep_layer_outputs(1)
+
+
+def _ragged_attention(mode, masked, fused):
     from oracle import cpu
     cfg = M.gpt2_cfg(2, 64, 2, 128) if masked else M.bert_cfg(2, 64, 2, 128)
     layers = M.parse_cfg(cfg)
@@ -198,12 +210,50 @@ def test_attention_over_a_long_ragged_sequence_matches_oracle(gpu, mode, masked)
     net = H.GpuNet(cfg, tens, batch, seq, min_ninst=32, mode=mode)
     try:
         net.run(x)
+        infos = [net.nasm.info(l) for l in range(net.nasm.num_ldata)]
+        assert fused == any(i["fused_attention"] >= 0 for i in infos)
         for l in range(1, net.nasm.num_ldata):
-            if net.nasm.info(l)["num_ninst"] == 0 and layers[l]["type"] != "residual": continue
+            if infos[l]["discarded"]:
+                with pytest.raises(RuntimeError):
+                    net.layer(l)
+                continue
+            if infos[l]["num_ninst"] == 0 and layers[l]["type"] != "residual": continue
             err = H.rel_l2(net.layer(l), outs[l])
             assert err <= H.REL_L2_TOL, f"layer {l} ({layers[l]['type']}): rel L2 {err:.3g}"
     finally:
         net.close()
+
+
+@pytest.mark.parametrize("mode,flags", [(api.MODE_LAYERS, 0), (api.MODE_DATAFLOW, QUEUE), (api.MODE_DATAFLOW, ORDERED)], ids=["layers", "dataflow", "ordered"])
+@pytest.mark.parametrize("name", ["bert_mini_b2_s24", "gpt_mini_b2_s20"])
+def test_fused_attention_matches_oracle(gpu, engine_flags, name, mode, flags):
+    """The default setting (layer outputs not kept): a V-attention layer whose probabilities nothing else reads computes
+    them in its own tiles (reference tiled_k_attention + tiled_v_attention, src/tiled_kernels.c:784-1037, in one pass).
+    Every layer that is written matches the oracle, on a re-armed graph with a second input as well; the
+    probability matrix is reported as not available."""
+    from oracle import cpu
+    engine_flags(flags)
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()[name])
+    api.lib().aspen_keep_layer_outputs(0)
+    try:
+        net = H.GpuNet(cfg, tens, batch, seq, min_ninst=32, mode=mode)
+        try:
+            infos = [net.nasm.info(l) for l in range(net.nasm.num_ldata)]
+            assert any(i["fused_attention"] >= 0 for i in infos)
+            for xin in (x, (x * 0.5 + 0.01).astype(np.float32) if name.startswith("bert") else x[::-1].copy()):
+                outs = cpu.run_network(layers, tens, xin, batch, seq)
+                net.run(xin)
+                for l in range(1, net.nasm.num_ldata):
+                    if infos[l]["discarded"]:
+                        with pytest.raises(RuntimeError):
+                            net.layer(l)
+                        continue
+                    err = H.rel_l2(net.layer(l), outs[l])
+                    assert err <= H.REL_L2_TOL, f"layer {l} ({layers[l]['type']}): rel L2 {err:.3g}"
+        finally:
+            net.close()
+    finally:
+        api.lib().aspen_keep_layer_outputs(1)
 
 
 def test_results_in_the_callers_dimension_order(gpu):
@@ -343,7 +393,8 @@ def test_full_config_matches_reference_summary(gpu, name, mode):
 
 
 @pytest.mark.timeout(900)
-@pytest.mark.parametrize("workload", list(M.WORKLOADS))
+# (the two batch-16 networks on their own are the same graphs as in the co-scheduled pair, which is checked as a pair)
+@pytest.mark.parametrize("workload", [w for w in M.WORKLOADS if w not in ("resnet50_b16", "vgg16_b16")])
 def test_timed_graphs_match_oracle_on_whole_tensors(gpu, workload):
     """Exactly the graphs bench.py times (models.WORKLOADS: same tile counts, same engine, one ready pool for the
     co-scheduled pair), first with the library's default of not writing matrices that only a fused shortcut
@@ -385,7 +436,7 @@ def test_timed_graphs_match_oracle_on_whole_tensors(gpu, workload):
                 for (name, _, layers, *_), net, outs in zip(cases, nets, want):
                     dropped = 0
                     for l in range(net.nasm.num_ldata):
-                        if keep == 0 and net.nasm.info(l)["fused_residual"] >= 0:
+                        if keep == 0 and net.nasm.info(l)["discarded"]:
                             with pytest.raises(RuntimeError):
                                 net.layer(l)
                             dropped += 1
@@ -397,7 +448,7 @@ def test_timed_graphs_match_oracle_on_whole_tensors(gpu, workload):
                         assert err <= H.REL_L2_TOL, f"{name} keep={keep} layer {l} ({layers[l]['type']}): rel L2 {err:.3g}"
                     last = net.nasm.num_ldata - 1
                     assert np.array_equal(net.layer(last).argmax(axis=1), outs[last].argmax(axis=1)), f"{name}: argmax differs"
-                    assert keep == 1 or dropped or not any(L["type"] == "residual" for L in layers)
+                    assert keep == 1 or dropped or not any(L["type"] in ("residual", "attn_k") for L in layers)
                 print(f"{workload} keep={keep}: worst rel L2 {worst:.3g}", flush=True)
             finally:
                 for net in nets:
@@ -662,11 +713,14 @@ def test_default_discards_outputs_only_a_fused_shortcut_reads(gpu):
 
 
 @pytest.mark.gpu
-def test_stalled_run_is_reported_and_the_next_runs_recover(gpu, capfd):
+@pytest.mark.parametrize("flags", [QUEUE, ORDERED], ids=["queue", "ordered"])
+def test_stalled_run_is_reported_and_the_next_runs_recover(gpu, engine_flags, capfd, flags):
     """The persistent kernel's watchdog, forced from the host with a spin limit of one poll: the first
-    workgroup that finds its queue slot still empty gives the run up, every workgroup leaves, the run
-    reports the stall.  The following runs (persistent kernel, then one launch per layer, whose split-K
-    groups count arrivals in the same counters) must be complete and correct again."""
+    workgroup that finds its queue slot still empty (ordered mode: its tile's dependency counter still
+    positive) gives the run up, every workgroup leaves, the run reports the stall.  The following runs
+    (persistent kernel, then one launch per layer, whose split-K groups count arrivals in the same counters)
+    must be complete and correct again."""
+    engine_flags(flags)
     name = "resnet_mini_b2"
     cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()[name])
     gold = np.load(os.path.join(H.GOLDEN, f"micro_{name}.npz"))
@@ -676,7 +730,9 @@ def test_stalled_run_is_reported_and_the_next_runs_recover(gpu, capfd):
         api.lib().aspen_dse_group_set_spin_limit(net.dse.h, 1)
         net.run(x)
         st = net.rpool.run_stats()
-        assert st["aborted"] == 1 and st["executed"] < net.nasm.num_ninst, st
+        # (in ordered mode every tile is already held by a workgroup when the run is given up, and is run through on
+        # whatever its parents have written so far: all tiles count as executed, the run is void all the same)
+        assert st["aborted"] == 1 and (flags == ORDERED or st["executed"] < net.nasm.num_ninst), st
         assert "stalled" in capfd.readouterr().err
         # a run that was given up does not count as completed and hands out no results
         assert api.lib().dse_check_nasm_completion(net.nasm.h) == 0

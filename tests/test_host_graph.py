@@ -193,6 +193,18 @@ def test_tile_graph_against_brute_force(name, min_ninst, fuse, monkeypatch):
                 shortcut_need = {int(v) for v in np.unique(owner[other][c0:c1, r0:r1])}
         need = set(shortcut_need)
         regions = needed_regions(L, layers, c0, c1, r0, r1, batch, seq)
+        if L["type"] == "attn_v" and layers[L["p0"]]["type"] == "attn_k" and infos[L["p0"]]["num_ninst"] == 0:
+            # attention fusion (the probabilities need not be kept): the V tile computes its probability columns itself,
+            # so it reads what the K-attention layer would have read for them
+            K = layers[L["p0"]]
+            fused = []
+            for (pp, cols, ra, rb) in regions:
+                if pp == L["p0"]:
+                    for c in sorted(cols):
+                        fused += needed_regions(K, layers, c, c + 1, 0, seq, batch, seq)
+                else:
+                    fused.append((pp, cols, ra, rb))
+            regions = fused
         pointwise = L["type"] == "matmul" or (L["type"] == "conv" and L["size"] == 1)
         if t in partials and pointwise:
             # a partial tile of a pointwise layer reads only the parent rows (= K indices) of its K slice
