@@ -55,6 +55,8 @@ struct aspen_hip_graph_t
     uint32_t *d_dep;        // remaining-parent counters, re-armed before every dataflow run
     uint32_t *d_dep_spread; // the same, one per cache line, for ordered runs (allocated at the first one), see dep_slot
     uint32_t dep_stride;
+    int spread_armed;       // an ordered run has left d_dep_spread and the sink counters armed for the next one (tiles set their own
+                            // counters back, see wait_until_ready): no arming pass is needed unless a run was given up since
     qentry_t *d_queue;      // ready queue: slot t is written once, by whoever makes a tile ready
     qentry_t *d_child_rec;  // per tile: child count + its first CHILD_REC-1 children with their layers
     uint32_t *d_state;      // one counter per 128-byte line: [ST_QHEAD (q)] pop tickets, [ST_QTAIL (q)] push cursor of queue q, [ST_DONE] tiles done,
@@ -70,6 +72,7 @@ struct aspen_hip_graph_t
     int last_run_ordered;   // the last dataflow run took its tiles in index order (no ready queue)
     int prefer_ordered;     // -1: decided from the graph's parallelism; 0 / 1: the caller's choice, see aspen_hip_graph_set_ordered
     unsigned features;      // TILES_* bits of the tile kinds the graph contains: picks the persistent kernel's variant
+    int variant;            // index into dataflow_kernels of the smallest variant that has all of them
     uint32_t epoch;         // tag of the last run's queue entries, cycles 1..EPOCH_MAX
     uint32_t queue_config;  // grid, flags and queue grouping of the last run (they decide which queue slots a run rewrites), see run_dataflow
     unsigned long long *d_prof;
@@ -85,7 +88,8 @@ static hipStream_t g_side_stream = nullptr;       // read-outs that must not que
 static hipEvent_t g_events[NUM_EVENTS];
 static int g_inited = 0;
 static int g_num_cu = 0;
-static int g_resident_wg = WG_PER_CU;     // workgroups of the dataflow kernel that fit one compute unit
+static int g_resident_wg = WG_PER_CU;     // workgroups of the dataflow kernel's largest variant that fit one compute unit
+static int g_variant_wg[8][2];            // the same per variant of the kernel ([variant][coherent / cached loads]), see dataflow_kernels
 static char g_err[512] = "";
 static uint32_t g_flags = 0;
 
@@ -221,6 +225,7 @@ struct dataflow_args_t
     const uint32_t *group_sinks;    // per co-scheduled network: its tiles without children
     uint32_t num_groups, run_serial;
     uint32_t dep_stride;            // ordered mode: see dep_slot (0: counters packed)
+    const uint32_t *num_parents;    // ordered mode: what a tile's counter is set back to once the tile has seen it reach zero
     unsigned long long *trace;      // per-tile start / end time stamps when ASPEN_HIP_FLAG_TRACE is set
     unsigned long long *prof;       // 8 counters of summed 100 MHz ticks, see aspen_hip_dataflow_profile
     uint32_t num_ninst;
@@ -429,6 +434,12 @@ __device__ __noinline__ uint32_t schedule_step (uint32_t done, qentry_t rec)
                 {
                     __hip_atomic_store (a.host_abort + HOST_DONE_WORD + grp, a.run_serial, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
                     last = __hip_atomic_fetch_add (&a.state[ST_SINKS], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u == a.num_groups;
+                    if (ORDERED)
+                    {
+                        // (these counters too are back at their start for the next ordered run: nobody adds to them any more)
+                        __hip_atomic_store (&a.state[ST_GROUP (grp)], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if (last) __hip_atomic_store (&a.state[ST_SINKS], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
                 }
             }
             if (__shfl (last, 0, 64) && !ORDERED)
@@ -476,19 +487,25 @@ __device__ __forceinline__ void wait_until_ready ()
     if (threadIdx.x < 64)
     {
         unsigned long long spins = 0;
-        const uint32_t *counter = &a.dep[dep_slot (id, a.dep_stride)];
+        uint32_t *counter = &a.dep[dep_slot (id, a.dep_stride)];
+        const uint32_t parents = a.num_parents[id];     // (requested before the wait)
+        bool seen_zero = true;
         while (__builtin_amdgcn_readfirstlane (__hip_atomic_load (counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) != 0u)
         {
             ++spins;
-            if ((spins & 63) == 0 && __hip_atomic_load (&a.state[ST_ABORT], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+            if ((spins & 63) == 0 && __hip_atomic_load (&a.state[ST_ABORT], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) { seen_zero = false; break; }
             if (spins > a.spin_limit)
             {
                 __hip_atomic_store (&a.state[ST_ABORT], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 __hip_atomic_store (a.host_abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                seen_zero = false;
                 break;
             }
             __builtin_amdgcn_s_sleep (1);
         }
+        // The counter has done its work for this run (every parent has counted down): it is set back right away, so
+        // that the next ordered run of the graph needs no arming pass in front of it.
+        if (seen_zero && threadIdx.x == 0) __hip_atomic_store (counter, parents, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads ();
     if ((a.flags & ASPEN_HIP_FLAG_TRACE) && threadIdx.x == 0) a.trace[2 * (size_t)id] = wall_clock64 ();      // a tile "starts" when it may touch its operands
@@ -620,12 +637,17 @@ extern "C" int aspen_hip_init (void)
             CHECK (hipFuncSetAttribute (dataflow_kernels[v][coh], hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_SMEM_BYTES));
     for (int v = 0; v < NUM_ORDERED_VARIANTS; v++)
         CHECK (hipFuncSetAttribute (ordered_kernels[v], hipFuncAttributeMaxDynamicSharedMemorySize, ORDERED_SMEM_BYTES));
-    // how many persistent workgroups really fit a compute unit (registers, LDS): the default grid
-    int occ1 = 0, occ2 = 0;
-    CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&occ1, dataflow_kernel<1, TILES_ALL>, WG_THREADS, GEMM_SMEM_BYTES));
-    CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&occ2, dataflow_kernel<2, TILES_ALL>, WG_THREADS, GEMM_SMEM_BYTES));
-    g_resident_wg = occ1 < occ2 ? occ1 : occ2;
-    if (g_resident_wg < 1) g_resident_wg = 1;
+    // how many persistent workgroups really fit a compute unit (registers, LDS), per variant: a graph's default grid
+    // follows the variant it runs on
+    g_resident_wg = WG_PER_CU;
+    for (int v = 0; v < NUM_KERNEL_VARIANTS; v++)
+        for (int coh = 0; coh < 2; coh++)
+        {
+            int occ = 0;
+            CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&occ, dataflow_kernels[v][coh], WG_THREADS, GEMM_SMEM_BYTES));
+            g_variant_wg[v][coh] = occ < 1 ? 1 : occ;
+            if (g_variant_wg[v][coh] < g_resident_wg) g_resident_wg = g_variant_wg[v][coh];
+        }
     if (getenv ("ASPEN_GPU_VERBOSE")) fprintf (stderr, "aspen_hip: %d resident dataflow workgroups per compute unit (built for %d)\n", g_resident_wg, WG_PER_CU);
     g_inited = 1;
     return 0;
@@ -776,12 +798,24 @@ extern "C" int aspen_hip_dense_device_to_host (float *dst_host, const float *src
     return 0;
 }
 
-// plain streaming copy, 16 bytes per lane per step; also the yardstick the HBM byte counters of a
-// profiler are calibrated with (its traffic is known: `bytes` read + `bytes` written)
+// plain streaming copy; also the yardstick the HBM byte counters of a profiler are calibrated with (its traffic is
+// known: `bytes` read + `bytes` written).  A workgroup moves contiguous pieces of COPY_UNROLL x 4 KB: every lane has
+// COPY_UNROLL 16-byte loads in flight before its first store (one load per lane per step leaves the memory pipeline
+// mostly empty: 4.5 of 8 TB/s against 5.7 this way), and the grid is what the device holds at once.
+#define COPY_UNROLL 8
 __global__ void __launch_bounds__ (WG_THREADS) copy_kernel (const float4 *__restrict__ src, float4 *__restrict__ dst, size_t n4)
 {
-    const size_t step = (size_t)gridDim.x * blockDim.x;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += step) dst[i] = src[i];
+    const size_t piece = (size_t)WG_THREADS * COPY_UNROLL, step = (size_t)gridDim.x * piece;
+    const floatx4 *s4 = reinterpret_cast<const floatx4 *> (src);
+    floatx4 *d4 = reinterpret_cast<floatx4 *> (dst);
+    for (size_t base = (size_t)blockIdx.x * piece + threadIdx.x; base < n4; base += step)
+    {
+        floatx4 v[COPY_UNROLL];
+        #pragma unroll
+        for (int u = 0; u < COPY_UNROLL; u++) if (base + (size_t)u * WG_THREADS < n4) v[u] = __builtin_nontemporal_load (&s4[base + (size_t)u * WG_THREADS]);
+        #pragma unroll
+        for (int u = 0; u < COPY_UNROLL; u++) if (base + (size_t)u * WG_THREADS < n4) __builtin_nontemporal_store (v[u], &d4[base + (size_t)u * WG_THREADS]);
+    }
 }
 extern "C" int aspen_hip_copy (void *dst, const void *src, size_t bytes)
 {
@@ -789,9 +823,16 @@ extern "C" int aspen_hip_copy (void *dst, const void *src, size_t bytes)
     if (bytes % 16 || ((uintptr_t)dst | (uintptr_t)src) % 16)
     { snprintf (g_err, sizeof (g_err), "copy: size and addresses must be multiples of 16 bytes"); return -1; }
     if (bytes == 0) return 0;
-    const size_t n4 = bytes / 16;
-    const size_t want = (n4 + WG_THREADS - 1) / WG_THREADS;
-    const unsigned grid = (unsigned)(want < (size_t)g_num_cu * 16 ? want : (size_t)g_num_cu * 16);
+    const size_t n4 = bytes / 16, piece = (size_t)WG_THREADS * COPY_UNROLL;
+    const size_t want = (n4 + piece - 1) / piece;
+    static int per_cu = 0;
+    if (per_cu == 0)
+    {
+        CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&per_cu, copy_kernel, WG_THREADS, 0));
+        if (per_cu < 1) per_cu = 1;
+    }
+    const size_t cap = (size_t)g_num_cu * (size_t)per_cu;
+    const unsigned grid = (unsigned)(want < cap ? want : cap);
     hipLaunchKernelGGL (copy_kernel, dim3 (grid), dim3 (WG_THREADS), 0, g_stream, (const float4 *)src, (float4 *)dst, n4);
     CHECK (hipGetLastError ());
     return 0;
@@ -1042,11 +1083,15 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
         // default grid: a whole number of workgroups per compute unit, no more than the graph can keep busy
         const double par = graph_parallelism (layers, ninst_layer, child_off, child_idx, num_ninst);
         g->parallelism = par;
-        uint32_t per_cu = (uint32_t)g_resident_wg;
+        static const bool all_tiles = getenv ("ASPEN_GPU_ONE_KERNEL") != nullptr;       // comparisons: always the variant with every tile kind
+        g->variant = NUM_KERNEL_VARIANTS - 1;
+        for (int i = NUM_KERNEL_VARIANTS - 2; i >= 0 && !all_tiles; i--) if ((g->features & ~kernel_variant_tiles[i]) == 0) g->variant = i;
+        const uint32_t resident = (uint32_t)g_variant_wg[g->variant][g->cached_loads ? 1 : 0];      // of the variant this graph runs on
+        uint32_t per_cu = resident;
         // measured on 256 compute units (ResNet-50 batch 1 / 32, VGG-16, BERT, GPT-2): one more workgroup per
         // unit pays once the average parallelism grows by another two tiles per unit
-        if (par < 2.0 * g_num_cu * g_resident_wg) per_cu = (uint32_t)(par / (2.0 * g_num_cu)) + 1;
-        if (per_cu > (uint32_t)g_resident_wg) per_cu = (uint32_t)g_resident_wg;
+        if (par < 2.0 * g_num_cu * resident) per_cu = (uint32_t)(par / (2.0 * g_num_cu)) + 1;
+        if (per_cu > resident) per_cu = resident;
         g->default_workgroups = per_cu * (uint32_t)g_num_cu;
         if (getenv ("ASPEN_GPU_VERBOSE"))
             fprintf (stderr, "aspen_hip: %u tiles, average parallelism %.0f: %u workgroups by default\n", num_ninst, par, g->default_workgroups);
@@ -1229,12 +1274,22 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
         }
         g->queue_config = config;
     }
-    hipLaunchKernelGGL (arm_kernel, dim3 ((g->num_ninst + 255) / 256), dim3 (256), 0, g_stream,
-        ordered ? g->d_dep_spread : g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->d_ninst_layer, g->d_ninst_home, g->d_root_pos, counts,
-        g->num_ninst, g->num_roots, g->d_state, g->epoch, g->queue_row, nq_mask, nq_shift, g->d_arrivals, ordered ? g->dep_stride : 0u);
-    CHECK (hipGetLastError ());
+    // An ordered run leaves its counters armed for the next one, so back-to-back ordered runs launch ONE kernel.  The
+    // arming pass runs in front of the first ordered run, after a run that was given up, and whenever the per-tile
+    // execution counts are kept (they are reset there).
+    if (*(volatile uint32_t *)g->h_abort != 0) g->spread_armed = 0;
+    const bool skip_arm = ordered && g->spread_armed && !(g_flags & (ASPEN_HIP_FLAG_COUNT_TILES | ASPEN_HIP_FLAG_SKIP_TILES));
+    if (!skip_arm)
+    {
+        hipLaunchKernelGGL (arm_kernel, dim3 ((g->num_ninst + 255) / 256), dim3 (256), 0, g_stream,
+            ordered ? g->d_dep_spread : g->d_dep, g->d_num_parents, g->d_queue, g->d_ran, g->d_roots, g->d_ninst_layer, g->d_ninst_home, g->d_root_pos, counts,
+            g->num_ninst, g->num_roots, g->d_state, g->epoch, g->queue_row, nq_mask, nq_shift, g->d_arrivals, ordered ? g->dep_stride : 0u);
+        CHECK (hipGetLastError ());
+    }
+    if (ordered) g->spread_armed = 1;
     dataflow_args_t a;
     a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.ninst_home = g->d_ninst_home; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx; a.child_rec = g->d_child_rec;
+    a.num_parents = g->d_num_parents;
     a.dep = ordered ? g->d_dep_spread : g->d_dep; a.dep_stride = ordered ? g->dep_stride : 0u; a.queue = g->d_queue; a.state = g->d_state; a.ran = g->d_ran; a.arrivals = g->d_arrivals; a.prof = g->d_prof; a.host_abort = g->h_abort;
     g->run_serial = g->run_serial + 1u ? g->run_serial + 1u : 1u;
     g->last_run_dataflow = 1;
@@ -1248,10 +1303,7 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     a.num_ninst = g->num_ninst; a.num_sinks = g->num_sinks; a.epoch = g->epoch; a.flags = g_flags; a.queue_row = g->queue_row; a.queue_cap = g->queue_cap; a.nq_mask = nq_mask; a.nq_shift = nq_shift; a.spin_limit = spin_limit ? spin_limit : DEFAULT_SPIN_LIMIT;
     CHECK (hipEventRecord (g_events[NUM_EVENTS - 2], g_stream));
     {
-        static const bool all_tiles = getenv ("ASPEN_GPU_ONE_KERNEL") != nullptr;       // comparisons: always the variant with every tile kind
-        int v = NUM_KERNEL_VARIANTS - 1;
-        for (int i = NUM_KERNEL_VARIANTS - 2; i >= 0 && !all_tiles; i--) if ((g->features & ~kernel_variant_tiles[i]) == 0) v = i;
-        const void *kernel = dataflow_kernels[v][g->cached_loads ? 1 : 0];
+        const void *kernel = dataflow_kernels[g->variant][g->cached_loads ? 1 : 0];
         if (ordered) kernel = ordered_kernels[(g->features & ~ordered_variant_tiles[0]) == 0 ? 0 : 1];
         g->last_run_ordered = ordered;
         void *kernel_args[] = {&a};
@@ -1303,6 +1355,7 @@ extern "C" int aspen_hip_graph_sync (aspen_hip_graph_t *g)
     if (g && *(volatile uint32_t *)g->h_abort != 0)
     {
         *g->h_abort = 0;
+        g->spread_armed = 0;
         snprintf (g_err, sizeof (g_err), "dataflow run stalled: a wait on the ready queue exceeded its spin limit and the run was aborted");
         fprintf (stderr, "aspen_hip: %s\n", g_err);
         return ASPEN_HIP_ERR_STALLED;
@@ -1429,8 +1482,9 @@ extern "C" int aspen_hip_sgemm (uint32_t M, uint32_t N, uint32_t K, const float 
 }
 
 // ------------------------------------------------------------------------------------------------
-// SGEMM that allocates nothing (for callers that cannot call hipMalloc: code under stream capture, tight
-// serving loops).  aspen_hip_sgemm stages A into a zero-padded copy it allocates and frees per call; here that
+// SGEMM that allocates nothing (for callers that cannot call hipMalloc: tight serving loops, harnesses that
+// forbid it).  It launches on the library's own stream, so it cannot join a caller's stream capture, and the first
+// call on a device performs the library's one-time initialisation (stream and event creation, kernel attributes).  aspen_hip_sgemm stages A into a zero-padded copy it allocates and frees per call; here that
 // staging copy lives in a file-scope device array, and the layer descriptor travels as a kernel argument.
 // Each device holds its own copy of the array at its own address: the address is looked up once per device
 // with hipGetSymbolAddress and only that pointer is ever handed to kernels.  Every call on a device shares the

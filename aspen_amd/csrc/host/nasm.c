@@ -14,6 +14,7 @@
 #include "internal.h"
 
 static unsigned int nasm_counter = 0;
+#define WEIGHT_STREAM_BYTES (16u << 20)      /* see set_tiles */
 
 static unsigned int cdiv (unsigned int a, unsigned int b) { return (a + b - 1) / b; }
 static unsigned int umin (unsigned int a, unsigned int b) { return a < b ? a : b; }
@@ -119,6 +120,13 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
            takes the 32 x 32 shape, whose four wavefronts split the K axis between them */
         if (nasm->narrow_tiles && v == ASPEN_HIP_GEMM_SMALL && !aspen_layer_table_operand (L) && !aspen_layer_dense3 (L)
             && 2 * cdiv (M, bm[v]) * cdiv (N, bn[v]) < want) v = ASPEN_HIP_GEMM_NARROW;
+        /* (Weight streaming with the 32 x 32 shape -- every wavefront reading its own rows and K range straight into
+           registers, for layers over a handful of columns with a large weight matrix -- was measured on the FC layers of
+           VGG-16 at batch 32 and is slower than the 64 x 64 shape with its operands staged through LDS: 411 MB in 148
+           instead of 118 us, 67 MB in 27.8 instead of 25.7 us; a lane pair per row and request makes poor use of the memory
+           pipeline.  ASPEN_GPU_WEIGHT_STREAM=1 switches it on for comparisons.) */
+        if (N <= bn[ASPEN_HIP_GEMM_NARROW] && (uint64_t)M * aspen_layer_kiters (L) * 32 * sizeof (float) >= WEIGHT_STREAM_BYTES
+            && !aspen_layer_table_operand (L) && !aspen_layer_dense3 (L) && getenv ("ASPEN_GPU_WEIGHT_STREAM") != NULL) v = ASPEN_HIP_GEMM_NARROW;
         ld->variant = v;
         ld->tile_dims[OUT_H] = bm[v]; ld->tile_dims[OUT_W] = bn[v];
     }

@@ -260,8 +260,10 @@ void aspen_hip_divider_for (uint32_t d, uint32_t out[2]);
 int aspen_hip_sgemm (uint32_t M, uint32_t N, uint32_t K, const float *A, uint32_t lda, const float *B,
     uint32_t ldb, float *C, uint32_t ldc, const float *bias, int act);
 
-/* The same SGEMM for callers that cannot allocate device memory (code under stream capture, tight serving
-   loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  It calls no hipMalloc / hipFree:
+/* The same SGEMM for callers that cannot allocate device memory (tight serving loops, harnesses that forbid
+   hipMalloc).  No counterpart in the reference.  It runs on the library's own stream (it cannot be recorded into a
+   caller's stream capture) and the first call initialises the library (stream, events, kernel attributes: call
+   aspen_hip_init beforehand where that matters).  It calls no hipMalloc / hipFree:
    the zero-padded staging copy of A that aspen_hip_sgemm allocates per call lives in a static device array of
    aspen_hip_sgemm_static_max_bytes () bytes (8 MiB per GPU, held until the process ends), so
    roundup (M, 128) * K * 4 must not exceed that; larger problems are refused with a message.  Asynchronous on

@@ -306,11 +306,17 @@ def test_results_in_the_callers_dimension_order(gpu):
         net.close()
 
 
-@pytest.mark.parametrize("flags", [QUEUE, ORDERED], ids=["queue", "ordered"])
+@pytest.mark.parametrize("flags", [QUEUE, ORDERED, -ORDERED], ids=["queue", "ordered", "ordered-armed-by-its-tiles"])
 def test_engine_rearm_many_runs(gpu, engine_flags, flags):
     """Re-arm and re-run one graph many times: every run must execute each tile exactly once, never
-    stall, and reproduce the first run bit for bit (tiles are deterministic; only their order varies)."""
+    stall, and reproduce the first run bit for bit (tiles are deterministic; only their order varies).
+    Third variant: ordered runs WITHOUT the per-tile execution counts, which is what production runs: there no arming
+    pass runs between two runs, every tile sets its own dependency counter back for the next run; different inputs
+    on the way check that no run saw another run's counters or data."""
+    counted = flags >= 0
     engine_flags(flags)
+    if not counted:
+        api.lib().aspen_hip_set_flags(ORDERED)           # no counts: runs after the first skip the arming pass
     cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()["gpt_mini_b2_s20"])
     net = H.GpuNet(cfg, tens, batch, seq, min_ninst=64, mode=api.MODE_DATAFLOW)
     print(f"tiles {net.nasm.num_ninst}", flush=True)
@@ -318,13 +324,24 @@ def test_engine_rearm_many_runs(gpu, engine_flags, flags):
         first = None
         for rep in range(40):
             net.run(x if rep == 0 else None)
-            st = net.rpool.run_stats()
-            assert st == {"executed": net.nasm.num_ninst, "double_runs": 0, "aborted": 0}, (rep, st)
+            if counted:
+                st = net.rpool.run_stats()
+                assert st == {"executed": net.nasm.num_ninst, "double_runs": 0, "aborted": 0}, (rep, st)
+            else:
+                assert net.dse.last_run_ordered()
             out = net.layer(net.nasm.num_ldata - 1)
             if first is None:
                 first = out
             else:
                 assert np.array_equal(first, out), f"run {rep} differs from run 0"
+        if not counted:
+            from oracle import cpu
+            for xin in ((x * 0.5).astype(np.float32), x[::-1].copy(), x):
+                want = cpu.run_network(layers, tens, xin, batch, seq)
+                net.run(xin)
+                for l in range(1, net.nasm.num_ldata):
+                    assert H.rel_l2(net.layer(l), want[l]) <= H.REL_L2_TOL, l
+            assert np.array_equal(first, net.layer(net.nasm.num_ldata - 1))
     finally:
         net.close()
 
