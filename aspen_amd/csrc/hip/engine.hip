@@ -573,11 +573,12 @@ __global__ void sgemm_kernel (const aspen_hip_layer_t L);       // defined with 
 
 // The persistent kernel's variants, smallest first: [variant][0] coherent loads, [1] cached loads.  A graph runs on the
 // first variant that has all its tile kinds, see graph_features.
-#define NUM_KERNEL_VARIANTS 4
-static const unsigned kernel_variant_tiles[NUM_KERNEL_VARIANTS] = {TILES_TRANSFORMER, TILES_CONVNET, TILES_CONVNET | TILES_YOLO, TILES_ALL};
+#define NUM_KERNEL_VARIANTS 5
+static const unsigned kernel_variant_tiles[NUM_KERNEL_VARIANTS] = {TILES_TRANSFORMER, TILES_CONVNET, TILES_CONVNET | TILES_TALL, TILES_CONVNET | TILES_YOLO, TILES_ALL};
 static const void *const dataflow_kernels[NUM_KERNEL_VARIANTS][2] = {
     {(const void *)dataflow_kernel<1, TILES_TRANSFORMER>, (const void *)dataflow_kernel<2, TILES_TRANSFORMER>},
     {(const void *)dataflow_kernel<1, TILES_CONVNET>, (const void *)dataflow_kernel<2, TILES_CONVNET>},
+    {(const void *)dataflow_kernel<1, TILES_CONVNET | TILES_TALL>, (const void *)dataflow_kernel<2, TILES_CONVNET | TILES_TALL>},
     {(const void *)dataflow_kernel<1, TILES_CONVNET | TILES_YOLO>, (const void *)dataflow_kernel<2, TILES_CONVNET | TILES_YOLO>},
     {(const void *)dataflow_kernel<1, TILES_ALL>, (const void *)dataflow_kernel<2, TILES_ALL>}};
 
@@ -600,7 +601,7 @@ static unsigned graph_features (const aspen_hip_layer_t *layers, uint32_t num_la
         {
         case CONV_LAYER: case FC_LAYER: case MATMUL_LAYER:
             if (L.variant == ASPEN_HIP_GEMM_NARROW) { f |= TILES_NARROW; break; }      // (brings its own operand loaders)
-            f |= L.variant == ASPEN_HIP_GEMM_LARGE ? TILES_LARGE : L.variant == ASPEN_HIP_GEMM_WIDE ? TILES_WIDE : TILES_SMALL;
+            f |= L.variant == ASPEN_HIP_GEMM_LARGE ? TILES_LARGE : L.variant == ASPEN_HIP_GEMM_WIDE ? TILES_WIDE : L.variant == ASPEN_HIP_GEMM_TALL ? TILES_TALL : TILES_SMALL;
             if (L.direct != ASPEN_HIP_OPERAND_DIRECT) f |= TILES_GATHER;
             break;
         case K_ATTENTION_LAYER: case V_ATTENTION_LAYER: f |= TILES_ATTENTION; break;
@@ -655,8 +656,9 @@ extern "C" int aspen_hip_init (void)
 
 extern "C" const char *aspen_hip_last_error (void) { return g_err; }
 
-extern "C" void aspen_hip_tile_shapes (uint32_t shapes[11])
+extern "C" void aspen_hip_tile_shapes (uint32_t shapes[13])
 {
+    shapes[11] = VAR4_BM; shapes[12] = VAR4_BN;
     shapes[0] = VAR0_BM; shapes[1] = VAR0_BN; shapes[2] = VAR1_BM; shapes[3] = VAR1_BN; shapes[4] = VAR2_BM; shapes[5] = VAR2_BN;
     shapes[6] = KATTN_BN; shapes[7] = VATTN_BN; shapes[8] = WG_PER_CU; shapes[9] = VAR3_BM; shapes[10] = VAR3_BN;
 }
@@ -896,16 +898,16 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
     else if (L.tiles_m == 0 || L.tiles_n == 0 || L.splits == 0
         || L.num_ninst != L.tiles_m * L.tiles_n * L.splits) why = "tile grid";
     else if (L.splits > 1 && (!L.partial || L.kiters_per_split == 0 || (uint64_t)L.splits * L.kiters_per_split * GEMM_BK < L.Kp
-        || !(L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER) || (L.variant != ASPEN_HIP_GEMM_SMALL && L.variant != ASPEN_HIP_GEMM_NARROW))) why = "split-K geometry";
+        || !(L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER) || (L.variant != ASPEN_HIP_GEMM_SMALL && L.variant != ASPEN_HIP_GEMM_NARROW && L.variant != ASPEN_HIP_GEMM_TALL))) why = "split-K geometry";
     else if ((L.type == CONV_LAYER || L.type == MAXPOOL_LAYER || L.type == AVGPOOL_LAYER)
         && (L.stride == 0 || L.KH == 0 || L.KW == 0 || L.IH == 0 || L.IW == 0 || L.OH == 0 || L.OW == 0 || L.N % (L.OH * L.OW))) why = "window geometry";
     else if (L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER)
     {
-        uint32_t shp[11];
+        uint32_t shp[13];
         aspen_hip_tile_shapes (shp);
         if (L.variant < 0 || L.variant >= ASPEN_HIP_NUM_GEMM_VARIANTS) { snprintf (g_err, sizeof (g_err), "layer %u rejected: GEMM variant", idx); return -1; }
-        const bool narrow = L.variant == ASPEN_HIP_GEMM_NARROW;
-        const uint32_t bm = narrow ? shp[9] : shp[2 * L.variant], bn = narrow ? shp[10] : shp[2 * L.variant + 1];
+        const bool narrow = L.variant == ASPEN_HIP_GEMM_NARROW, tall = L.variant == ASPEN_HIP_GEMM_TALL;
+        const uint32_t bm = narrow ? shp[9] : tall ? shp[11] : shp[2 * L.variant], bn = narrow ? shp[10] : tall ? shp[12] : shp[2 * L.variant + 1];
         if (!L.weight) why = "missing weight";
         else if ((uint64_t)((L.M + 127) / 128 * 128) * L.Kp * 4 >= 0xffffff00ull) why = "weight matrix larger than 4 GiB";
         else if (L.Kp == 0 || L.Kp % GEMM_BK) why = "Kp must be a positive multiple of 32";
@@ -918,6 +920,7 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
         else if (L.direct < 0 || L.direct > ASPEN_HIP_OPERAND_DENSE3) why = "operand kind";
         else if (L.direct == ASPEN_HIP_OPERAND_TABLE && L.IC % GEMM_BK != 0 && L.variant != ASPEN_HIP_GEMM_SMALL) why = "a K axis that needs the k-chunk table takes 64 x 64 tiles";
         else if (L.direct == ASPEN_HIP_OPERAND_TABLE && L.IC == 0) why = "channel count";
+        else if (tall && L.direct == ASPEN_HIP_OPERAND_DENSE3) why = "the dense three-channel operand takes 64-row tiles";
         else if (narrow && (L.direct == ASPEN_HIP_OPERAND_DENSE3 || (L.direct == ASPEN_HIP_OPERAND_TABLE && L.IC % GEMM_BK != 0))) why = "the 32 x 32 tile reads its operand in place or steps through taps of whole K slices";
     }
     else if (L.type == K_ATTENTION_LAYER)

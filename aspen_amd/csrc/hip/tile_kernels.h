@@ -40,6 +40,13 @@ __device__ void tile_phase_lap (int which);
 #define VAR1_BN 128
 #define VAR2_BM 64
 #define VAR2_BN 64
+// The tall shape, for layers that stream a large weight matrix past a handful of columns (a fully connected layer at
+// batch <= 32): four wavefronts, each 32 weight rows x the tile's 32 columns.  A 64 x 64 tile computes 32 columns of
+// padding there, which makes such a layer bound by the matrix pipeline at twice its useful work instead of by the
+// weights' trip from memory; this shape requests 16 KB of weights per K slice for the same number of MFMAs.
+#define VAR4_BM 128
+#define VAR4_BN 32
+#define VAR4_DEPTH 2            // two slices of weights in flight: memory latency is all such a tile waits for
 // K slices in flight from memory per tile shape (see gemm_core).  With two the larger shapes run out of registers
 // (measured: ResNet-50 batch 32 2.81 -> 2.89 ms, VGG-16 7.90 -> 8.83 ms).  The small shape takes two for the matmul
 // layers of transformer graphs, which run one or two workgroups per compute unit with nothing else to hide a slice's
@@ -49,7 +56,7 @@ __device__ void tile_phase_lap (int which);
 #define VAR0_DEPTH 1
 #define VAR1_DEPTH 1
 #define VAR2_DEPTH 2
-#define SPLITK_TILE_FLOATS (VAR2_BM * VAR2_BN)     // one slice's sums of one output tile: a block of its own in `partial`
+#define SPLITK_TILE_FLOATS (VAR2_BM * VAR2_BN)     // one slice's sums of one output tile: a block of its own in `partial` (the tall shape has as many)
 #define CMAX(a, b) ((a) > (b) ? (a) : (b))
 #define STAGE_FLOATS(bm, bn) (((bm) + (bn)) * LDS_ROW)
 #define EPI_FLOATS(bm, bn) ((bn) * ((bm) + 8))
@@ -497,7 +504,8 @@ enum : unsigned
     TILES_ATTENTION = 16u, TILES_NORM = 32u /* layernorm, softmax */, TILES_POOL = 64u, TILES_YOLO = 128u /* yolo, append */,
     TILES_RESIDUAL = 256u,
     TILES_NARROW = 512u,        // the 32 x 32 contraction tile of latency-bound graphs
-    TILES_ALL = 1023u,
+    TILES_TALL = 1024u,         // the 128 x 32 contraction tile of weight-streaming layers
+    TILES_ALL = 2047u,
     TILES_CONVNET = TILES_GATHER | TILES_LARGE | TILES_WIDE | TILES_SMALL | TILES_POOL | TILES_RESIDUAL,
     TILES_TRANSFORMER = TILES_SMALL | TILES_ATTENTION | TILES_NORM | TILES_RESIDUAL
 };
@@ -754,6 +762,7 @@ template <int BM, int BN, int WM, int WN, int DEPTH, int COH, unsigned FEAT, cla
 __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L, Descriptor descriptor, uint32_t tn, uint32_t tm, int slice, float *smem, shortcut_prefetch_t &pre, Ready ready)
 {
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr bool SINGLE = TM * TN == 1 && BM == VAR2_BM && BN == VAR2_BN;     // the hand-scheduled loop of the 64 x 64 shape
     const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
     const uint32_t m0 = tm * BM, n0 = tn * BN;
     floatx16 acc[TN][TM];
@@ -795,7 +804,7 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
     {
         ActRowLoader<BN, COH> bl;
         bl.init (in, n0, L.N - 1, L.ld0, 0, tid);
-        if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
+        if constexpr (SINGLE) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
         else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
     }
     else if constexpr ((FEAT & TILES_GATHER) != 0)
@@ -805,12 +814,12 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
         {
             Dense3Loader<BN, COH> bl;
             bl.init (L, in, n0, tid);
-            if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
+            if constexpr (SINGLE) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
             else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
         }
-        else if (TM * TN == 1 && L.IC % GEMM_BK != 0)
+        else if (SINGLE && L.IC % GEMM_BK != 0)
         {
-            if constexpr (TM * TN == 1)
+            if constexpr (SINGLE)
             {
                 ConvLoader<BN, COH, true> bl;
                 bl.init (L, in, n0, tid, kbase);
@@ -821,7 +830,7 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
         {
             ConvLoader<BN, COH, false> bl;
             bl.init (L, in, n0, tid, kbase);
-            if constexpr (TM * TN == 1) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
+            if constexpr (SINGLE) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
             else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
         }
     }
@@ -832,8 +841,8 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
         // split-K: the raw sums go straight from the accumulators to this slice's block of the output tile, in the
         // accumulators' own layout (splitk_gather reads them back the same way): four 16-byte stores per lane, each
         // instruction 1 KB in one piece; no bias, no activation, no bounds, nothing to stage through LDS.  Only the
-        // 64 x 64 shape is ever cut along K.
-        if constexpr (BM == VAR2_BM && BN == VAR2_BN)
+        // 64 x 64 and the 128 x 32 shape (one accumulator block per wavefront either way) are ever cut along K.
+        if constexpr (TM * TN == 1)
         {
             const aspen_hip_layer_t L = descriptor ();
             const uint32_t tiles = L.tiles_m * L.tiles_n;
@@ -953,7 +962,7 @@ __device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L
 // latencies overlap instead of adding up (the blocks come from other XCDs' tiles and miss this XCD's L2); a slice
 // index past the last one re-reads the last slice and is not added.
 template <int COH>
-__device__ __forceinline__ void splitk_gather (const aspen_hip_layer_t &L, uint32_t t, float *smem)
+__device__ __forceinline__ void splitk_gather (const aspen_hip_layer_t &L, uint32_t t, float *smem, bool tall = false)
 {
     const uint32_t tid = tile_thread (), lane = tid & 63, wave = tid >> 6;
     const uint32_t tiles = L.tiles_m * L.tiles_n, sstride = tiles * SPLITK_TILE_FLOATS, last = L.splits - 1;
@@ -980,8 +989,9 @@ __device__ __forceinline__ void splitk_gather (const aspen_hip_layer_t &L, uint3
             { v[q].x += use ? p[j][q].x : 0.f; v[q].y += use ? p[j][q].y : 0.f; v[q].z += use ? p[j][q].z : 0.f; v[q].w += use ? p[j][q].w : 0.f; }
         }
     }
-    constexpr int TROW = VAR2_BM + 8;
-    const uint32_t wm0 = (wave % 2) * 32, wn0 = (wave / 2) * 32, m = wm0 + (lane & 31);
+    // (tall: 128 channels x 32 columns, the four wavefronts' blocks below each other; else 2 x 2 blocks of 64 x 64)
+    const uint32_t TROW = (tall ? VAR4_BM : VAR2_BM) + 8;
+    const uint32_t wm0 = tall ? wave * 32 : (wave % 2) * 32, wn0 = tall ? 0u : (wave / 2) * 32, m = wm0 + (lane & 31);
     #pragma unroll
     for (int q = 0; q < 4; q++)
     {
@@ -1941,8 +1951,9 @@ __device__ __forceinline__ void finish_tile (const aspen_hip_layer_t &L, uint32_
     if (L.variant == ASPEN_HIP_GEMM_NARROW) { narrow_gather_finish<COH> (L, t, tn, t - tn * L.tiles_m); return; }
     shortcut_prefetch_t pre;
     pre.have = pre.have_shortcut = false;
-    splitk_gather<COH> (L, t, smem);
-    contraction_epilogue<COH> (L, tn, t - tn * L.tiles_m, smem, 4, VAR2_BN, pre);
+    const bool tall = L.variant == ASPEN_HIP_GEMM_TALL;
+    splitk_gather<COH> (L, t, smem, tall);
+    contraction_epilogue<COH> (L, tn, t - tn * L.tiles_m, smem, tall ? 5 : 4, tall ? VAR4_BN : VAR2_BN, pre);
 }
 
 // Runs tile t of the layer.  `descriptor ()` yields a wave-uniform copy of the layer's descriptor (scalar_layer /
@@ -1985,6 +1996,7 @@ __device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, boo
         }
         if ((FEAT & TILES_LARGE) && L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, VAR0_DEPTH, COH, FEAT> (L, descriptor, tn, tm, -1, smem, pre, ready); c4_log2 = 5; bn = VAR0_BN; }
         else if ((FEAT & TILES_WIDE) && L.variant == ASPEN_HIP_GEMM_WIDE) { contraction_mainloop<VAR1_BM, VAR1_BN, 2, 2, VAR1_DEPTH, COH, FEAT> (L, descriptor, tn, tm, -1, smem, pre, ready); bn = VAR1_BN; }
+        else if ((FEAT & TILES_TALL) && L.variant == ASPEN_HIP_GEMM_TALL) { contraction_mainloop<VAR4_BM, VAR4_BN, 4, 1, VAR4_DEPTH, COH, FEAT> (L, descriptor, tn, tm, slice, smem, pre, ready); c4_log2 = 5; bn = VAR4_BN; }
         else if (FEAT & TILES_SMALL)
         {
             // two K slices in flight for the matmul layers of transformers, one for convolutional networks (see VAR2_DEPTH)
@@ -2003,7 +2015,7 @@ __device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, boo
             if (COH) tile_phase_lap (10);
             uint32_t *counters = arrivals ();
             if (counters == nullptr || !splitk_arrived_last (counters + group, E.splits, smem)) { if (COH) tile_phase_lap (11); return false; }
-            splitk_gather<COH> (E, t, smem);
+            splitk_gather<COH> (E, t, smem, c4_log2 == 5);       // (of the shapes cut along K only the tall one has 128 channels)
         }
         contraction_epilogue<COH> (E, tn, tm, smem, c4_log2, bn, pre);
         if (COH) tile_phase_lap (slice >= 0 ? 11 : 10);

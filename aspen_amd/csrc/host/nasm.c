@@ -106,9 +106,9 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
     }
     if (is_contraction (L->type))
     {
-        uint32_t shp[11];
+        uint32_t shp[13];
         aspen_hip_tile_shapes (shp);
-        const unsigned int bm[ASPEN_HIP_NUM_GEMM_VARIANTS] = {shp[0], shp[2], shp[4], shp[9]}, bn[ASPEN_HIP_NUM_GEMM_VARIANTS] = {shp[1], shp[3], shp[5], shp[10]};
+        const unsigned int bm[ASPEN_HIP_NUM_GEMM_VARIANTS] = {shp[0], shp[2], shp[4], shp[9], shp[11]}, bn[ASPEN_HIP_NUM_GEMM_VARIANTS] = {shp[1], shp[3], shp[5], shp[10], shp[12]};
         /* few output rows: the wide shape; otherwise the large one; either falls back to the small
            shape when it would leave the layer with fewer tiles than wanted */
         int v = M <= 64 ? ASPEN_HIP_GEMM_WIDE : ASPEN_HIP_GEMM_LARGE;
@@ -120,13 +120,20 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
            takes the 32 x 32 shape, whose four wavefronts split the K axis between them */
         if (nasm->narrow_tiles && v == ASPEN_HIP_GEMM_SMALL && !aspen_layer_table_operand (L) && !aspen_layer_dense3 (L)
             && 2 * cdiv (M, bm[v]) * cdiv (N, bn[v]) < want) v = ASPEN_HIP_GEMM_NARROW;
-        /* (Weight streaming with the 32 x 32 shape -- every wavefront reading its own rows and K range straight into
-           registers, for layers over a handful of columns with a large weight matrix -- was measured on the FC layers of
-           VGG-16 at batch 32 and is slower than the 64 x 64 shape with its operands staged through LDS: 411 MB in 148
-           instead of 118 us, 67 MB in 27.8 instead of 25.7 us; a lane pair per row and request makes poor use of the memory
-           pipeline.  ASPEN_GPU_WEIGHT_STREAM=1 switches it on for comparisons.) */
-        if (N <= bn[ASPEN_HIP_GEMM_NARROW] && (uint64_t)M * aspen_layer_kiters (L) * 32 * sizeof (float) >= WEIGHT_STREAM_BYTES
-            && !aspen_layer_table_operand (L) && !aspen_layer_dense3 (L) && getenv ("ASPEN_GPU_WEIGHT_STREAM") != NULL) v = ASPEN_HIP_GEMM_NARROW;
+        /* A layer that streams a large weight matrix past at most 32 columns (the first FC layers of VGG-16 up to batch
+           32: 411 MB and 67 MB of weights) takes the tall shape, 128 weight rows x 32 columns.  With 64 x 64 tiles half of
+           every MFMA works on padding columns, and the layer is bound by the matrix pipeline at twice its useful work
+           (411 MB in 116 us = 3.5 TB/s, whatever the number of tiles and whether or not the weights lie in memory in tile
+           order -- both measured) instead of by the weights' trip from memory.  (The 32 x 32 shape, every wavefront
+           reading its own rows and K range straight into registers, is slower still: 148 us; a lane pair per row and
+           request makes poor use of the memory pipeline.  ASPEN_GPU_WEIGHT_STREAM=narrow / =off for comparisons.) */
+        const char *wsb = getenv ("ASPEN_GPU_WEIGHT_STREAM_BYTES");       /* (tests: the shape on small layers) */
+        if (N <= bn[ASPEN_HIP_GEMM_TALL] && (uint64_t)M * aspen_layer_kiters (L) * 32 * sizeof (float) >= (wsb ? strtoull (wsb, NULL, 10) : WEIGHT_STREAM_BYTES)
+            && !aspen_layer_table_operand (L) && !aspen_layer_dense3 (L))
+        {
+            const char *e = getenv ("ASPEN_GPU_WEIGHT_STREAM");
+            if (e == NULL || strcmp (e, "off") != 0) v = (e != NULL && strcmp (e, "narrow") == 0) ? ASPEN_HIP_GEMM_NARROW : ASPEN_HIP_GEMM_TALL;
+        }
         ld->variant = v;
         ld->tile_dims[OUT_H] = bm[v]; ld->tile_dims[OUT_W] = bn[v];
     }
@@ -134,7 +141,7 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
     {
         const unsigned int S = nasm->tr_seq_len, hd = L->params[NUM_HIDDEN] / L->params[NUM_HEAD];
         if (hd % 32 != 0) { ERROR_PRTF ("layer %u: head size %u must be a multiple of 32\n", L->layer_idx, hd); return -1; }
-        uint32_t shp[11];
+        uint32_t shp[13];
         aspen_hip_tile_shapes (shp);
         ld->tile_dims[OUT_H] = M; ld->tile_dims[OUT_W] = shp[6];
         ld->tiles_h = 1; ld->tiles_w = (N / S) * cdiv (S, shp[6]);
@@ -146,7 +153,7 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
         const unsigned int S = nasm->tr_seq_len, hd = L->params[NUM_HIDDEN] / L->params[NUM_HEAD];
         if (hd * L->params[NUM_HEAD] != M || (hd > 64 && hd % 64 != 0) || hd % 4 != 0)
         { ERROR_PRTF ("layer %u: unsupported head geometry (M %u, heads %u)\n", L->layer_idx, M, L->params[NUM_HEAD]); return -1; }
-        uint32_t shp[11];
+        uint32_t shp[13];
         aspen_hip_tile_shapes (shp);
         ld->tile_dims[OUT_H] = umin (hd, 64); ld->tile_dims[OUT_W] = shp[7];
         ld->tiles_h = M / ld->tile_dims[OUT_H]; ld->tiles_w = (N / S) * cdiv (S, shp[7]);
@@ -197,8 +204,12 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
         }
         else if ((T < want || (cap && kiters > cap)) && kiters >= 16 && getenv ("ASPEN_GPU_NO_SPLITK") == NULL)
         {
-            const char *e1 = getenv ("ASPEN_GPU_MAX_SPLITS"), *e2 = getenv ("ASPEN_GPU_MIN_KITERS");
-            const unsigned int max_splits = e1 ? (unsigned int)atoi (e1) : 8, min_kiters = e2 ? (unsigned int)atoi (e2) : 8;
+            /* (a tall tile's layer has few row tiles and a long K axis: up to 16 parts of at least 16 slices.  Measured on
+               VGG-16 batch 32, each layer launched alone: 4096 x 25088 in 87 / 85 / 97 us with 8 / 16 / 32 parts, 4096 x 4096
+               in 19.5 / 23.5 us with 8 / 16) */
+            const int tall = ld->variant == ASPEN_HIP_GEMM_TALL;
+            const char *e1 = getenv (tall ? "ASPEN_GPU_TALL_MAX_SPLITS" : "ASPEN_GPU_MAX_SPLITS"), *e2 = getenv (tall ? "ASPEN_GPU_TALL_MIN_KITERS" : "ASPEN_GPU_MIN_KITERS");
+            const unsigned int max_splits = e1 ? (unsigned int)atoi (e1) : tall ? 16 : 8, min_kiters = e2 ? (unsigned int)atoi (e2) : tall ? 16 : 8;
             unsigned int s = umin (umin (umax (cdiv (want, T), cap ? cdiv (kiters, cap) : 1), kiters / umax (min_kiters, 1)), umax (max_splits, 1));
             ld->kiters_per_split = cdiv (kiters, s);
             ld->splits = cdiv (kiters, ld->kiters_per_split);

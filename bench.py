@@ -171,11 +171,14 @@ def cpu_description():
     return {"model": model, "physical_cores": len(phys) or None, "hardware_threads": threads or (os.cpu_count() or 0)}
 
 
-def measure_workload(api, M, name, steps, warmup):
+def measure_workload(api, M, name, steps, warmup, flags=0):
     """One of the other benchmark configurations, in the same loop as the headline one: its tuned tile count and
-    engine (models.WORKLOADS), inputs resident, `warmup` untimed + `steps` timed steps, final layer checked
-    against the compiled reference's fixture afterwards.  Everything is torn down again."""
+    engine (models.WORKLOADS), inputs resident, `warmup` untimed + `steps` timed steps (more of both for steps of
+    under a millisecond, so that the timed region is tens of milliseconds long), final layer checked against the
+    compiled reference's fixture afterwards.  `flags`: engine flags for this workload's runs.  Everything is torn down
+    again."""
     L = api.lib()
+    L.aspen_hip_set_flags(flags)
     cfgs, unit, units_per_step, min_ninst, engine = WORKLOADS[name]
     pool = api.RPool()
     dse = api.DseGroup(1, api.MODE_DATAFLOW if engine == "dataflow" else api.MODE_LAYERS)
@@ -209,14 +212,39 @@ def measure_workload(api, M, name, steps, warmup):
         dse.stop()
 
     one(first=True)
+    L.aspen_hip_sync()
+    t0 = time.perf_counter()
     for _ in range(warmup):
         one()
     L.aspen_hip_sync()
+    estimate_ms = (time.perf_counter() - t0) / max(warmup, 1) * 1e3
+    if warmup and estimate_ms < 2.0:
+        # a step of a few hundred microseconds: the clock settles over many of them, and 20 would be a 10 ms sample
+        steps = max(steps, min(200, int(60.0 / estimate_ms)))
+        for _ in range(steps // 4):
+            one()
+        L.aspen_hip_sync()
     t0 = time.perf_counter()
     for _ in range(steps):
         one(timed=True)
     L.aspen_hip_sync()
     ms = (time.perf_counter() - t0) / steps * 1e3
+    weight_stream = None
+    if name == "vgg16_b32":
+        # the layer that streams the most weights past the fewest columns (FC1 of VGG-16: 411 MB of weights, 32 columns),
+        # launched alone five times: a memory-bound contraction, priced against the memory roofline
+        nasm = nets[0][2]
+        lms = pool.profile_layers(nasm.num_ldata, 5)
+        infos = [nasm.info(l) for l in range(nasm.num_ldata)]
+        fc = [l for l, i in enumerate(infos) if api.LAYER_TYPE_NAMES[i["type"]] == "fc"]
+        if fc:
+            l = max(fc, key=lambda l: infos[l]["flops"])
+            i = infos[l]
+            wbytes = i["flops"] / (2 * i["W"]) * 4          # rows x K floats
+            gbs = wbytes / (float(lms[l]) * 1e-3) / 1e9
+            weight_stream = {"layer": l, "rows": i["H"], "columns": i["W"], "tile": [i["tile_H"], i["tile_W"]], "tiles": i["num_ninst"],
+                             "weight_bytes": wbytes, "us": float(lms[l]) * 1e3,
+                             "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS}}
     checks = [verify_final_layer(cname, n) for cname, _, n in nets]
     have = [c for c in checks if c is not None]
     ach = flops / (ms * 1e-3) / 1e12
@@ -225,8 +253,12 @@ def measure_workload(api, M, name, steps, warmup):
            "frac_of_fp32_mfma_peak": ach / PEAK_FP32_MFMA_TFLOPS, "verified": all(c["ok"] for c in have) if have else None}
     if engine == "dataflow" and dse.last_run_ordered():
         out["engine"] = "dataflow-ordered"
+    out["steps"] = steps
+    if weight_stream:
+        out["weight_streaming_layer"] = weight_stream
     if len(nets) > 1:
         out["nasm_completion_ms"] = {cname: done_ms[i] / steps for i, (cname, _, _) in enumerate(nets)}
+    L.aspen_hip_set_flags(0)
     dse.destroy()
     for _, _, n in nets:
         n.destroy()

@@ -53,13 +53,16 @@ enum { ASPEN_HIP_ATTENTION_FUSED = 1 };
 /* GEMM tile shapes (rows of the weight matrix x activation columns per workgroup): LARGE = the
    biggest shape of the build (128 x 64 by default), WIDE = 64 x 128, SMALL = 64 x 64, NARROW = 32 x 32 with the
    workgroup's four wavefronts splitting the K axis (for graphs bound by the latency of their dependency
-   chains; operands DIRECT or TABLE with IC % 32 == 0 only).  The graph builder asks aspen_hip_tile_shapes for
-   the numbers instead of assuming them. */
-enum { ASPEN_HIP_GEMM_LARGE = 0, ASPEN_HIP_GEMM_WIDE = 1, ASPEN_HIP_GEMM_SMALL = 2, ASPEN_HIP_GEMM_NARROW = 3, ASPEN_HIP_NUM_GEMM_VARIANTS };
+   chains; operands DIRECT or TABLE with IC % 32 == 0 only), TALL = 128 x 32 for layers that stream a large weight
+   matrix past at most 32 columns (fully connected layers at small batch; not with the k-chunk table of a channel
+   count off the slice width, nor DENSE3).  SMALL, NARROW and TALL tiles may be cut along K (splits).  The graph
+   builder asks aspen_hip_tile_shapes for the numbers instead of assuming them. */
+enum { ASPEN_HIP_GEMM_LARGE = 0, ASPEN_HIP_GEMM_WIDE = 1, ASPEN_HIP_GEMM_SMALL = 2, ASPEN_HIP_GEMM_NARROW = 3, ASPEN_HIP_GEMM_TALL = 4, ASPEN_HIP_NUM_GEMM_VARIANTS };
 /* shapes[2*v] = rows, shapes[2*v+1] = columns of GEMM variant v = 0..2; shapes[6] = queries per K-attention
    tile; shapes[7] = queries per V-attention tile; shapes[8] = workgroups per compute unit the
-   kernels are built for; shapes[9], shapes[10] = rows, columns of variant 3.  Pure constants: callable without a GPU. */
-void aspen_hip_tile_shapes (uint32_t shapes[11]);
+   kernels are built for; shapes[9], shapes[10] = rows, columns of variant 3; shapes[11], shapes[12] = of variant 4.  Pure
+   constants: callable without a GPU. */
+void aspen_hip_tile_shapes (uint32_t shapes[13]);
 
 /* Per-layer descriptor: everything one tile needs, so a tile is (layer, tile index).
    Replaces the fields the reference's tiled_* read through ninst->ldata->layer

@@ -58,12 +58,13 @@ def test_reference_api_names_present():
 
 
 def test_tile_shapes_are_constants():
-    s = (ctypes.c_uint32 * 11)()
+    s = (ctypes.c_uint32 * 13)()
     api.lib().aspen_hip_tile_shapes(s)
     shapes = list(s)
     for v in range(3):
         assert shapes[2 * v] in (64, 128) and shapes[2 * v + 1] in (64, 128)
     assert shapes[6] in (32, 64, 128) and shapes[7] > 0 and shapes[8] in (2, 4)
+    assert (shapes[9], shapes[10]) == (32, 32) and (shapes[11], shapes[12]) == (128, 32)      # the narrow and the tall shape
 
 
 def test_bench_refuses_more_than_one_gpu():

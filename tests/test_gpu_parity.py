@@ -50,6 +50,33 @@ def test_micro_nets_match_reference_fixture(gpu, engine_flags, name, mode, flags
         net.close()
 
 
+@pytest.mark.parametrize("mode,flags", [(api.MODE_LAYERS, 0), (api.MODE_DATAFLOW, QUEUE), (api.MODE_DATAFLOW, ORDERED)], ids=["layers", "dataflow", "ordered"])
+@pytest.mark.parametrize("name,min_ninst", [("vgg_mini_b5", 8), ("vgg_mini_b5", 1), ("custom_b3", 8), ("resnet_mini_b2", 8)])
+def test_tall_tiles_of_weight_streaming_layers_match_reference_fixture(gpu, engine_flags, monkeypatch, name, min_ninst, mode, flags):
+    """Layers over at most 32 columns whose weight matrix is large take 128 x 32 tiles (the FC layers of VGG-16 at
+    batch 32); here the size limit is lowered so that the small networks' FC layers take them too: cut along K and
+    whole, with 128, 10 and 100 output rows."""
+    monkeypatch.setenv("ASPEN_GPU_WEIGHT_STREAM_BYTES", "0")
+    engine_flags(flags)
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()[name])
+    gold = np.load(os.path.join(H.GOLDEN, f"micro_{name}.npz"))
+    net = H.GpuNet(cfg, tens, batch, seq, min_ninst=min_ninst, mode=mode)
+    tall = [l for l in range(net.nasm.num_ldata) if net.nasm.info(l)["variant"] == 4 and layers[l]["type"] in ("fc", "conv", "matmul")]
+    print(f"case {name} mode {mode} tiles {net.nasm.num_ninst} tall layers {[(l, net.nasm.info(l)['splits']) for l in tall]}", flush=True)
+    assert tall, "no layer took the tall shape"
+    net.run(x)
+    try:
+        for l in range(net.nasm.num_ldata):
+            err = H.rel_l2(net.layer(l), gold[f"layer{l}"])
+            assert err <= H.REL_L2_TOL, f"layer {l} ({layers[l]['type']}): rel L2 {err:.3g}"
+        assert (net.layer(net.nasm.num_ldata - 1).argmax(1) == gold[f"layer{net.nasm.num_ldata - 1}"].argmax(1)).all()
+        if mode == api.MODE_DATAFLOW:
+            st = net.rpool.run_stats()
+            assert st == {"executed": net.nasm.num_ninst, "double_runs": 0, "aborted": 0}, st
+    finally:
+        net.close()
+
+
 @pytest.mark.parametrize("loads", ["cached", "coherent", "unfused", "ordered"])
 @pytest.mark.parametrize("name", list(H.micro_cases()))
 def test_micro_nets_match_oracle(gpu, engine_flags, name, loads, monkeypatch):
@@ -478,13 +505,14 @@ def test_timed_graphs_match_oracle_on_whole_tensors(gpu, workload):
         api.lib().aspen_keep_layer_outputs(1)
 
 
-@pytest.mark.parametrize("mode", [api.MODE_LAYERS, api.MODE_DATAFLOW], ids=["layers", "dataflow"])
-def test_two_nasms_of_one_dnn_share_a_pool(gpu, mode, tmp_path):
+@pytest.mark.parametrize("mode,flags", [(api.MODE_LAYERS, 0), (api.MODE_DATAFLOW, QUEUE), (api.MODE_DATAFLOW, ORDERED)], ids=["layers", "dataflow", "ordered"])
+def test_two_nasms_of_one_dnn_share_a_pool(gpu, engine_flags, mode, flags, tmp_path):
     """The reference's second example runs two graphs of ONE model side by side (reference
     examples/2. vgg16_example/aspen_execute.c:38-50): both share the model's device weights, each has its own
     activations and input.  Here with different batch sizes and inputs; then one graph is destroyed and the
     pool runs on with the other."""
     from oracle import cpu
+    engine_flags(flags)
     cfg, layers, tens, x3, _, _ = H.build_case(H.micro_cases()["custom_b3"])
     wp = str(tmp_path / "w.bin")
     M.write_aspen_data(wp, tens)
@@ -497,6 +525,8 @@ def test_two_nasms_of_one_dnn_share_a_pool(gpu, mode, tmp_path):
         pool.add_nasm_raw_input(na, x3)
         pool.add_nasm_raw_input(nb, x2)
         dse.run(); dse.wait(na); dse.wait(nb); dse.stop()
+        if mode == api.MODE_DATAFLOW:
+            assert pool.run_stats() == {"executed": na.num_ninst + nb.num_ninst, "double_runs": 0, "aborted": 0}, pool.run_stats()
         ref_a, ref_b = cpu.run_network(layers, tens, x3, 3, 0), cpu.run_network(layers, tens, x2, 2, 0)
         for l in range(na.num_ldata):
             assert H.rel_l2(na.layer_output(l), ref_a[l]) <= H.REL_L2_TOL, ("a", l)

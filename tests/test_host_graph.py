@@ -293,7 +293,7 @@ def test_layers_cut_along_k_or_resolved_through_the_table_take_the_small_tile_sh
     count is not a multiple of the K slice width (so that a slice straddles taps), get that shape whatever the tile
     count asks for; their neighbours with 32-multiple channel counts keep the large shapes."""
     import ctypes
-    shp = (ctypes.c_uint32 * 11)()
+    shp = (ctypes.c_uint32 * 13)()
     api.lib().aspen_hip_tile_shapes(shp)
     shp = list(shp)
     cfg = ("[net]\nheight=64\nwidth=64\nchannels=48\n\n"

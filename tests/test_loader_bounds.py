@@ -123,7 +123,7 @@ def walk_contraction(L, info, pinfo, batch, name, l):
                                     ok = (ih0 + kh >= 0) & (ih0 + kh < IH) & (iw0 + kw >= 0) & (iw0 + kw < IW)
                                     count += check(base + (kh * IW + kw) * g["ld0"] + c + sub * 8 + khalf, ok, in_size, f"{name} layer {l} narrow taps")
                 continue
-            depth = 2 if (L["type"] == "matmul" and bm == 64 and bn == 64) else 1
+            depth = 2 if (L["type"] == "matmul" and bm == 64 and bn == 64) or info["variant"] == 4 else 1      # (VAR2_DEPTH of the transformer kernels, VAR4_DEPTH)
             asked = slices_asked(kbase, kiters, depth)
             rows_b = np.arange(bn)
             # weights: RowLoader<BM>, rows padded to a multiple of 128
@@ -250,6 +250,15 @@ def walk_network(name, cfg, batch, seq, min_ninst):
 @pytest.mark.parametrize("min_ninst", [8, 32, 1024])
 @pytest.mark.parametrize("name", list(H.micro_cases()))
 def test_every_requested_operand_offset_lies_inside_its_matrix(name, min_ninst):
+    cfg, style, batch, seq, seed, kind = H.micro_cases()[name]
+    assert walk_network(name, cfg, batch, seq, min_ninst) > 0
+
+
+@pytest.mark.parametrize("min_ninst", [1, 8])
+@pytest.mark.parametrize("name", ["vgg_mini_b5", "custom_b3", "resnet_mini_b2"])
+def test_tall_tiles_stay_inside_their_matrices(name, min_ninst, monkeypatch):
+    """The same walk with the 128 x 32 shape on every layer of at most 32 columns (the size limit lowered)."""
+    monkeypatch.setenv("ASPEN_GPU_WEIGHT_STREAM_BYTES", "0")
     cfg, style, batch, seq, seed, kind = H.micro_cases()[name]
     assert walk_network(name, cfg, batch, seq, min_ninst) > 0
 
