@@ -1223,7 +1223,9 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     bool ordered = ordered_env ? atoi (ordered_env) != 0 : g->prefer_ordered >= 0 ? g->prefer_ordered != 0 : g->parallelism < ORDERED_BELOW;
     if (g_flags & ASPEN_HIP_FLAG_ORDERED) ordered = true;
     if (g_flags & ASPEN_HIP_FLAG_NO_ORDERED) ordered = false;
-    if (!g->cached_loads || xcd_queues || g->num_ninst > (1u << 20)) ordered = false;
+    // (a static assignment in index order only terminates when every tile's parents have smaller indices: graph_parallelism
+    // reports 1e30 for a graph that is not listed that way)
+    if (!g->cached_loads || xcd_queues || g->num_ninst > (1u << 20) || g->parallelism > 1e29) ordered = false;
     if (ordered)
     {
         // tiles are assigned to workgroups beforehand: every workgroup of the grid must be running
