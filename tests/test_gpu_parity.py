@@ -409,7 +409,7 @@ def test_queue_entries_of_earlier_runs_are_never_taken(gpu):
         net.close()
 
 
-FULL = ["resnet50_b1", "resnet50_b32", "vgg16_b32", "bert_base_b8_s128", "gpt2_b4_s512", "yolov3_b1"]
+FULL = ["resnet50_b1", "resnet50_b32", "vgg16_b32", "bert_base_b8_s128", "gpt2_b4_s512", "yolov3_b1", "yolov3_b8"]
 
 
 # every configuration on the persistent kernel; the small-batch ones also as one launch per layer (what the
