@@ -292,6 +292,11 @@ template <int ROWS, int COH> struct ActRowLoader
 // slice belongs to one tap, found with a few scalar operations: fetching the table entry instead puts a dependent
 // memory access in front of the operand loads of every slice.  Two loaders, not one with a branch: with both
 // paths in one K loop the compiler waits for ALL outstanding loads wherever they join.
+// K order of the stepping form (the host packs the weights to match): (channel block of 32, kh, kw, channel in block),
+// i.e. consecutive slices walk the TAPS of one block of 32 channels.  The windows of neighbouring taps overlap, so a
+// slice mostly re-reads what the previous one or the one KW before it fetched, while it is still in the caches; with
+// the taps outermost (the reference's order) a tap's data came round again only after a whole pass over the channels,
+// by which time a busy L2 had replaced it, and a 3 x 3 layer fetched its input up to nine times over the fabric.
 template <int ROWS, int COH, bool TABLE> struct ConvLoader
 {
     static constexpr int R = ROWS / 32;
@@ -299,7 +304,7 @@ template <int ROWS, int COH, bool TABLE> struct ConvLoader
     const aspen_hip_ktab_t *ktab;
     int32_t base[R], ih0[R], iw0[R];
     uint32_t IH, IW, chunk, row0;
-    uint32_t slices_per_tap, KW, ld0;
+    uint32_t KH, KW, ld0;
     uint32_t kh, kw, c;                     // tap and channel the next slice asked for starts at (!TABLE)
     // first_it: the first K slice that will be asked for
     __device__ __forceinline__ void init (const aspen_hip_layer_t &L, const ActView<COH> &v, uint32_t first_row, uint32_t tid, int first_it)
@@ -309,12 +314,12 @@ template <int ROWS, int COH, bool TABLE> struct ConvLoader
         if (TABLE) ktab = L.ktab;
         else
         {
-            slices_per_tap = L.IC / GEMM_BK; KW = L.KW; ld0 = L.ld0;
+            KH = L.KH; KW = L.KW; ld0 = L.ld0;
             kh = kw = c = 0;
             if (first_it)
             {
-                const uint32_t tap = (uint32_t)first_it / slices_per_tap;
-                c = ((uint32_t)first_it - tap * slices_per_tap) * GEMM_BK;
+                const uint32_t taps = KH * KW, block = (uint32_t)first_it / taps, tap = (uint32_t)first_it - block * taps;
+                c = block * GEMM_BK;
                 kh = tap / KW; kw = tap - kh * KW;
             }
         }
@@ -343,12 +348,12 @@ template <int ROWS, int COH, bool TABLE> struct ConvLoader
         {
             // Slices are asked for in ascending order from the one init was told, so the position is stepped, not
             // divided out, and `it` is not looked at.  (The K loops ask for the last slice once more than they need
-            // and drop the answer: that request is one step past the K axis, where a tap either lies inside the
-            // image, so the address exists, or fails the bounds test below and nothing is loaded.)
+            // and drop the answer: that request is one step past the K axis, i.e. the first tap again at the channels
+            // behind the last block: the 128 bytes that follow the pixel's channel run, which exist for every pixel
+            // but the matrix's last, where they lie in the slack behind the allocation.)
             e.offset = (int32_t)((kh * IW + kw) * ld0 + c + chunk * 4);
             e.kh = (uint16_t)kh; e.kw = (uint16_t)kw;
-            c += GEMM_BK;
-            if (c == slices_per_tap * GEMM_BK) { c = 0; if (++kw == KW) { kw = 0; ++kh; } }
+            if (++kw == KW) { kw = 0; if (++kh == KH) { kh = 0; c += GEMM_BK; } }
         }
         #pragma unroll
         for (int i = 0; i < R; i++)
@@ -1754,7 +1759,6 @@ __device__ __forceinline__ float4 narrow_mainloop (const aspen_hip_layer_t &L, D
     // tap / channel the first slice starts at (stepped from there, as ConvLoader does)
     int32_t bbase, ih0 = 0, iw0 = 0;
     uint32_t kh = 0, kw = 0, c = 0;
-    const uint32_t spt = direct ? 1u : L.IC / GEMM_BK;
     if (direct) bbase = (int32_t)(n * L.ld0 + (uint32_t)first * GEMM_BK + khalf);
     else
     {
@@ -1763,11 +1767,12 @@ __device__ __forceinline__ float4 narrow_mainloop (const aspen_hip_layer_t &L, D
         ih0 = (int32_t)(oh * L.stride) - (int32_t)L.pad;
         iw0 = (int32_t)(ow * L.stride) - (int32_t)L.pad;
         bbase = ((int32_t)(b * L.IH) + ih0) * (int32_t)L.IW * (int32_t)L.ld0 + iw0 * (int32_t)L.ld0 + (int32_t)khalf;
-        const uint32_t tap = (uint32_t)first / spt;
-        c = ((uint32_t)first - tap * spt) * GEMM_BK;
+        // (K order: channel block, kh, kw, channel in block; see ConvLoader)
+        const uint32_t taps = L.KH * L.KW, block = (uint32_t)first / taps, tap = (uint32_t)first - block * taps;
+        c = block * GEMM_BK;
         kh = tap / L.KW; kw = tap - kh * L.KW;
     }
-    const uint32_t IH = L.IH, IW = L.IW, KW = L.KW, ld0 = L.ld0;
+    const uint32_t IH = L.IH, IW = L.IW, KH = L.KH, KW = L.KW, ld0 = L.ld0;
     auto load_a = [&] (int i, float4 (&a)[4])
     {
         #pragma unroll
@@ -1791,8 +1796,7 @@ __device__ __forceinline__ float4 narrow_mainloop (const aspen_hip_layer_t &L, D
             const bool ok = (uint32_t)(ih0 + (int32_t)kh) < IH && (uint32_t)(iw0 + (int32_t)kw) < IW;
             #pragma unroll
             for (int sub = 0; sub < 4; sub++) bv[sub] = in.ld4_if ((uint32_t)(bbase + off + sub * 8), ok);
-            c += GEMM_BK;
-            if (c == spt * GEMM_BK) { c = 0; if (++kw == KW) { kw = 0; ++kh; } }
+            if (++kw == KW) { kw = 0; if (++kh == KH) { kh = 0; c += GEMM_BK; } }
         }
     };
     floatx16 acc;

@@ -302,6 +302,17 @@ int aspen_layer_table_operand (const aspen_layer_t *L)
     return (L->type == MATMUL_LAYER ? p[MAT_K] : p[IN_C]) % 32 != 0;
 }
 
+/* A convolution / FC layer whose K axis is laid out as (channel block of 32, tap, channel in block) on the device: every
+   layer the kernels read with the stepping loader, i.e. channel count a multiple of 32 and more than one tap (with one
+   tap the two orders are the same). */
+int aspen_layer_block_major_k (const aspen_layer_t *L)
+{
+    const unsigned int *p = L->params;
+    if (L->type != CONV_LAYER && L->type != FC_LAYER) return 0;
+    if (aspen_layer_dense3 (L) || p[IN_C] % 32 != 0) return 0;
+    return (L->type == CONV_LAYER ? p[WEIGHT_H] * p[WEIGHT_W] : p[IN_H] * p[IN_W]) > 1;
+}
+
 /* padded K of the device layout / 32 (must agree with aspen_layer_to_device) */
 unsigned int aspen_layer_kiters (const aspen_layer_t *L)
 {
@@ -348,9 +359,19 @@ int aspen_layer_to_device (aspen_layer_t *L, unsigned int parent_ld)
     const unsigned int mp = round_up (L->gemm_m, 128);
     float *staged = calloc ((size_t)mp * kp, sizeof (float));
     if (staged == NULL) return -1;
+    /* K order on the device.  Channel counts that are multiples of the K slice width: (channel block of 32, tap, channel
+       in block), the order the kernels' stepping loader walks (consecutive slices are the taps of one channel block, whose
+       windows overlap in the caches).  Otherwise the reference's (tap, channel), each tap's run padded to icp. */
+    const int block_major = aspen_layer_block_major_k (L);
     for (unsigned int m = 0; m < L->gemm_m; m++)
         for (unsigned int t = 0; t < taps; t++)
-            memcpy (staged + (size_t)m * kp + (size_t)t * icp, L->weight.data + (size_t)m * L->gemm_k + (size_t)t * ic, ic * sizeof (float));
+        {
+            const float *src = L->weight.data + (size_t)m * L->gemm_k + (size_t)t * ic;
+            if (!block_major) memcpy (staged + (size_t)m * kp + (size_t)t * icp, src, ic * sizeof (float));
+            else
+                for (unsigned int c = 0; c < ic; c += 32)
+                    memcpy (staged + (size_t)m * kp + ((size_t)(c / 32) * taps + t) * 32, src + c, 32 * sizeof (float));
+        }
     L->d_weight = aspen_hip_alloc ((size_t)mp * kp * sizeof (float));
     int rc = L->d_weight ? aspen_hip_h2d (L->d_weight, staged, (size_t)mp * kp * sizeof (float)) : -1;
     free (staged);

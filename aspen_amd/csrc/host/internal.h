@@ -144,6 +144,7 @@ int aspen_layer_to_device (aspen_layer_t *layer, unsigned int parent_ld);
 int aspen_load_weight_file (aspen_dnn_t *dnn, const char *path);
 int aspen_layer_dense3 (const aspen_layer_t *layer);            /* three input channels: dense K axis on the device */
 int aspen_layer_table_operand (const aspen_layer_t *layer);     /* K axis through the k-chunk table: 64 x 64 tiles only */
+int aspen_layer_block_major_k (const aspen_layer_t *layer);     /* device K order (channel block, tap, channel in block) */
 unsigned int aspen_layer_kiters (const aspen_layer_t *layer);   /* K slices of 32 of a contraction layer's device layout */
 /* nasm.c */
 int aspen_nasm_to_device (nasm_t *nasm);

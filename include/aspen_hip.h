@@ -97,7 +97,10 @@ typedef struct aspen_hip_layer_t
     float *out;
     const float *in0;        /* PARENT_0 */
     const float *in1;        /* PARENT_1 */
-    const float *weight;     /* [roundup(M,128)][Kp] row-major, zero padded; layernorm: gamma[M] */
+    const float *weight;     /* [roundup(M,128)][Kp] row-major, zero padded; layernorm: gamma[M].  K order of a convolution /
+                                FC operand that is neither DIRECT nor DENSE3: IC % 32 == 0 (the kernels step through it):
+                                (channel block of 32, kh, kw, channel in block); else (kh, kw, channel padded to 4), the
+                                order the k-chunk table describes */
     const float *bias;       /* [M] or NULL */
     const aspen_hip_ktab_t *ktab; /* Kp/4 entries (Kp/2 for DENSE3), NULL when direct */
     /* fused shortcut (contraction layers; reference tiled_residual, src/tiled_kernels.c:613-638, run in

@@ -115,8 +115,8 @@ def walk_contraction(L, info, pinfo, batch, name, l):
                                 if g["direct"]:
                                     count += check(n * g["ld0"] + k, np.ones(32, bool), in_size, f"{name} layer {l} narrow direct")
                                 else:
-                                    spt = g["ic"] // BK
-                                    tap, c = (first + i) // spt, ((first + i) % spt) * BK
+                                    block, tap = (first + i) // g["taps"], (first + i) % g["taps"]
+                                    c = block * BK
                                     kh, kw = tap // g["kw_count"], tap % g["kw_count"]
                                     b, ih0, iw0, IH, IW = conv_rows(L, 32, N, n0)
                                     base = ((b * IH + ih0) * IW + iw0) * g["ld0"]
@@ -169,11 +169,13 @@ def walk_contraction(L, info, pinfo, batch, name, l):
                         count += check(base + off, ok, in_size, f"{name} layer {l} table")
             else:
                 # ConvLoader stepping: the position advances by one slice per request, whatever `it` says; the
-                # repeated request of a two-deep loop therefore lands one step past the K axis
-                spt = g["ic"] // BK
+                # repeated requests of a two-deep loop therefore land one and two steps past the K axis.  K order:
+                # (channel block of 32, kh, kw, channel in block), so a step past the end is the first taps again at
+                # the 32 channels BEHIND the pixel's run
                 pos = kbase
                 for _ in asked:
-                    tap, c = pos // spt, (pos % spt) * BK
+                    block, tap = pos // g["taps"], pos % g["taps"]
+                    c = block * BK
                     kh, kw = tap // g["kw_count"], tap % g["kw_count"]
                     ok = (ih0 + kh >= 0) & (ih0 + kh < IH) & (iw0 + kw >= 0) & (iw0 + kw < IW)
                     o = (base + (kh * IW + kw) * g["ld0"] + c)[:, None] + chunk[None, :] * 4
