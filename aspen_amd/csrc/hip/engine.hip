@@ -1210,10 +1210,13 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     if (workgroups > QUEUE_SLACK) workgroups = QUEUE_SLACK;         // every waiting workgroup must find a "leave" entry within its queue
     g->epoch = g->epoch % EPOCH_MAX + 1u;
     // one queue per XCD on request, when every XCD gets the same number of workgroups (workgroup b runs on XCD b % 8)
-    static const bool xcd_queues_env = getenv ("ASPEN_GPU_XCD_QUEUES") != nullptr;
-    const bool xcd_queues = xcd_queues_env || (g_flags & ASPEN_HIP_FLAG_XCD_QUEUES);
+    // (ASPEN_GPU_XCD_QUEUES=0: always one queue; any other value: one queue per XCD, in groups of 2 / 4 XCDs with
+    // ASPEN_GPU_XCD_QUEUE_SHIFT = 1 / 2)
+    static const char *xcd_queues_env = getenv ("ASPEN_GPU_XCD_QUEUES");
+    static const bool one_queue_env = xcd_queues_env != nullptr && strcmp (xcd_queues_env, "0") == 0;
+    const bool xcd_queues = (xcd_queues_env != nullptr && !one_queue_env) || (g_flags & ASPEN_HIP_FLAG_XCD_QUEUES);
     static const uint32_t shift_env = getenv ("ASPEN_GPU_XCD_QUEUE_SHIFT") ? (uint32_t)atoi (getenv ("ASPEN_GPU_XCD_QUEUE_SHIFT")) : 0u;
-    const uint32_t nq_shift = shift_env > 2u ? 2u : shift_env;
+    uint32_t nq_shift = shift_env > 2u ? 2u : shift_env;
     // Ordered mode for graphs that can never keep the device busy (one image through a deep network): no ready queue,
     // workgroups take the tiles in index order (parents first), set each one up and request its first weights BEFORE it
     // is ready, and wait on the tile's own dependency counter.  With far more workgroups than ready tiles nothing is
@@ -1250,7 +1253,15 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
         g->d_dep_spread = (uint32_t *)aspen_hip_alloc (sizeof (uint32_t) * 32u * (size_t)g->dep_stride);
         if (!g->d_dep_spread) return -1;
     }
-    const uint32_t nq_mask = (xcd_queues && workgroups % NUM_QUEUES == 0) ? (NUM_QUEUES >> nq_shift) - 1u : 0u;
+    uint32_t nq_mask = (xcd_queues && workgroups % NUM_QUEUES == 0) ? (NUM_QUEUES >> nq_shift) - 1u : 0u;
+    // By default a graph that fills the device (every compute unit holds as many workgroups as fit) runs on TWO queues,
+    // one per half of the XCDs: tiles that read the same activations then meet in one of four L2s instead of eight (a
+    // tenth less memory traffic on the convolutional networks), and two pools of 512 workgroups balance as well as one of
+    // 1024 (same run time; four and eight queues cost 1 % and 3 %).  Smaller grids keep one queue: their runs are bound by
+    // dependency chains, and every restriction on who may take a ready tile lengthens those.
+    if (!xcd_queues && !one_queue_env && !ordered && workgroups % NUM_QUEUES == 0
+        && workgroups >= (uint32_t)g_variant_wg[g->variant][g->cached_loads ? 1 : 0] * (uint32_t)g_num_cu)
+    { nq_shift = 2u; nq_mask = (NUM_QUEUES >> nq_shift) - 1u; }
     queue_counts_t counts;
     if (nq_mask && g->root_shift != nq_shift)
     {

@@ -200,7 +200,9 @@ int aspen_hip_dataflow_profile (aspen_hip_graph_t *graph, uint64_t ticks[16], in
    columns), so that tiles reading the same activations share an L2: about 40 % less memory traffic on the
    convolutional networks, but free workgroups cannot help another XCD and runs take 0-11 % longer.  Also switched on
    by ASPEN_GPU_XCD_QUEUES in the environment; ASPEN_GPU_XCD_QUEUE_SHIFT = 1 / 2 groups the XCDs in pairs / fours (4 / 2
-   queues).  Needs a grid that is a multiple of 8 workgroups (else ignored). */
+   queues).  Needs a grid that is a multiple of 8 workgroups (else ignored).  Without the flag a run whose grid fills the
+   device takes TWO queues (one per half of the XCDs: same run time as one queue, a tenth less memory traffic) and every
+   other run one; ASPEN_GPU_XCD_QUEUES=0 forces one queue everywhere. */
 #define ASPEN_HIP_FLAG_XCD_QUEUES 32u
 /* ORDERED / NO_ORDERED force or forbid the ordered mode of the persistent kernel, which a run otherwise takes when
    the graph's average parallelism is below 128 tiles (one image through a deep network): no ready queue; workgroups
