@@ -1127,6 +1127,16 @@ extern "C" aspen_hip_graph_t *aspen_hip_graph_create (const aspen_hip_layer_t *l
                 const aspen_hip_layer_t &L = layers[ninst_layer[t]];
                 const uint64_t in_layer = t >= L.ninst_start ? t - L.ninst_start : 0;
                 home[t] = L.num_ninst ? (uint32_t)(in_layer * NUM_QUEUES / L.num_ninst) % NUM_QUEUES : 0u;
+                // a contraction layer whose weight matrix is larger than its input (the last stage of a deep convolutional
+                // network: megabytes of weights, a few hundred columns) is divided by weight rows and K parts instead, so
+                // that the tiles which read the same weights meet in the same caches
+                const bool contraction = L.type == CONV_LAYER || L.type == FC_LAYER || L.type == MATMUL_LAYER;
+                static const bool by_weights = getenv ("ASPEN_GPU_NO_WEIGHT_HOMES") == nullptr;
+                if (contraction && by_weights && L.num_ninst && (uint64_t)L.M * L.Kp > (uint64_t)L.ld0 * g->h_layers[ninst_layer[t]].in0_columns)
+                {
+                    const uint64_t per_column_tile = (uint64_t)L.tiles_m * (L.splits ? L.splits : 1u);
+                    home[t] = (uint32_t)((in_layer % per_column_tile) * NUM_QUEUES / per_column_tile) % NUM_QUEUES;
+                }
             }
             for (uint32_t r = 0; r < num_roots; r++) pos[r] = g->root_count[home[roots[r]]]++;
             for (uint32_t t = 0; t < num_ninst; t++)
