@@ -47,6 +47,37 @@ def gemm_flops(nasm, api):
     return total
 
 
+def compulsory_bytes(nasm, api):
+    """What one inference must move if every matrix is read once by each layer that consumes it and written once, and
+    every weight matrix is read once: the yardstick for the measured traffic (which adds re-reads by several XCDs,
+    window overlaps that have left the caches, and split-K partial sums).  Follows the graph as built: a matrix that
+    is never written (the pre-shortcut sums of a fused shortcut, the probabilities of a fused attention) counts
+    neither as output nor as input."""
+    infos = [nasm.info(l) for l in range(nasm.num_ldata)]
+    size = lambda i: 4 * i["H"] * i["W"]
+    contraction = (api.CONV_LAYER, api.FC_LAYER, api.MATMUL_LAYER)
+    total = 0
+    for i in infos:
+        t = i["type"]
+        if t == api.INPUT_LAYER:
+            continue
+        no_tiles = i["num_ninst"] == 0
+        if t == api.K_ATTENTION_LAYER and no_tiles:
+            continue                                    # fused into the V-attention tiles: nothing written, nothing read here
+        if not i.get("discarded"):
+            total += size(i)
+        parents = [infos[p] for p in (i["p0"], i["p1"]) if 0 <= p < len(infos)]
+        if t == api.RESIDUAL_LAYER and no_tiles:
+            parents = parents[1:]                       # computed in its producer's epilogue: only the other operand is read
+        if t == api.V_ATTENTION_LAYER and parents and parents[0]["type"] == api.K_ATTENTION_LAYER and parents[0]["num_ninst"] == 0:
+            k = parents[0]
+            parents = [infos[p] for p in (k["p0"], k["p1"]) if 0 <= p < len(infos)] + parents[1:]     # Query, Key, Value
+        total += sum(size(p) for p in parents)
+        if t in contraction and i["flops"]:
+            total += 4 * i["flops"] // (2 * i["W"])     # rows x K weights
+    return total
+
+
 def cpu_baseline(cfgname, budget_s=20.0):
     """Reference tile kernels (oracle/_ref, compiled from the reference's sources) timed on this host's
     cores; falls back to the oracle port when that library is absent.  Bounded sample of the workload."""
@@ -248,7 +279,10 @@ def measure_workload(api, M, name, steps, warmup, flags=0):
     checks = [verify_final_layer(cname, n) for cname, _, n in nets]
     have = [c for c in checks if c is not None]
     ach = flops / (ms * 1e-3) / 1e12
+    traffic = MEASURED_TRAFFIC_BYTES.get((name, engine, min_ninst))
+    compulsory = sum(compulsory_bytes(n, api) for _, _, n in nets)
     out = {"ms_per_step": ms, "value": units_per_step / (ms * 1e-3), "unit": unit, "engine": engine, "min_ninst_per_ldata": min_ninst,
+           "traffic": traffic, "compulsory_bytes": compulsory, "traffic_over_compulsory": traffic / compulsory if traffic else None,
            "tiles_per_step": sum(n.num_ninst for _, _, n in nets), "flops_per_step": flops,
            "frac_of_fp32_mfma_peak": ach / PEAK_FP32_MFMA_TFLOPS, "verified": all(c["ok"] for c in have) if have else None}
     if engine == "dataflow" and dse.last_run_ordered():
@@ -406,6 +440,9 @@ def main():
                            "unit": "TFLOP/s", "frac": ach / PEAK_FP32_MFMA_TFLOPS,
                            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, args.mode, args.min_ninst)),
                            "flops_per_launch": flops, "kernel_ms": k_ms}
+        out["roofline"]["compulsory_bytes"] = sum(compulsory_bytes(n, api) for _, _, n, _ in nets)
+        if out["roofline"]["traffic"]:
+            out["roofline"]["traffic_over_compulsory"] = out["roofline"]["traffic"] / out["roofline"]["compulsory_bytes"]
     else:
         ach = flops / (ms_per_step * 1e-3) / 1e12
         out["roofline"] = {"bound": "mfma", "kernel": "layer_kernel (all layers of one step)", "achieved": ach,
