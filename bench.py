@@ -328,6 +328,9 @@ def main():
     ap.add_argument("--min-ninst", type=int, default=0, help="tiles wanted per layer (0: the workload's tuned value)")
     ap.add_argument("--workgroups", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-baseline-dse", default="", metavar="CONFIG",
+                    help="also time the reference's own scheduler (apu_create_nasm + dse_group_run, through oracle/_ref) on this configuration; "
+                         "its dependency search takes minutes beyond batch 1 (bert_base_b8_s128: about 2.5 minutes), so it is not part of the default run")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="skip the `workloads` section (the other benchmark configurations, measured after the headline one)")
     ap.add_argument("--skip-tiles", action="store_true", help="scheduler-only run: dependency protocol with empty tiles")
@@ -554,6 +557,8 @@ def main():
             b1 = cpu_baseline_dse("resnet50_b1")
             if b1 is not None:
                 out["cpu_baseline_b1"] = b1
+    if args.cpu_baseline_dse:
+        out["cpu_baseline_dse"] = cpu_baseline_dse(args.cpu_baseline_dse, iters=5)
     emit(json.dumps(out))
     if out.get("verified") is False:
         print("bench.py: the timed graph's output does not match the reference fixture", file=sys.stderr)
