@@ -113,7 +113,13 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) layer_kernel (const as
     const uint32_t nt = gridDim.x, bid = blockIdx.x;
     const uint32_t xcd = bid & 7, local = bid >> 3, chunk = nt >> 3, rem = nt & 7;
     const uint32_t t = first_tile + xcd * chunk + (xcd < rem ? xcd : rem) + local;
-    run_tile<0> ([=] () { return scalar_layer (layers + l); }, t, false, smem, [=] () { return arrivals; });
+    bool more_rows;
+    uint32_t row_rep = 0;
+    do
+    {
+        more_rows = false;
+        run_tile<0> ([=] () { return scalar_layer (layers + l); }, t, false, smem, [=] () { return arrivals; }, NoHook (), row_rep++, &more_rows);
+    } while (more_rows);
 }
 
 // Second launch of a split-K layer in launch-per-layer mode: one workgroup per output tile adds the slices up.
@@ -530,24 +536,28 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
     __builtin_amdgcn_s_setprio (TILE_PRIO);
     const unsigned long long t_begin = wall_clock64 (), c_begin = clock64 ();
     uint32_t id = QUEUE_EMPTY;
+    uint32_t row_rep = 0;           // which row tile of a row group comes next (see run_tile); 0: a new tile
     qentry_t rec = 0;
     for (;;)
     {
-        id = __builtin_amdgcn_readfirstlane (schedule_step<ORDERED> (id, rec));
-        if (id == QUEUE_EMPTY) break;           // all tickets taken, or aborted
-        // wavefront 0 requests this tile's child record now; it arrives while the tile runs
-        // (a global, not a flat load: a flat one would also count as LDS traffic the tile's first fragment wait sits out)
-        if (threadIdx.x < CHILD_REC)
-            rec = *(const qentry_t __attribute__ ((address_space (1))) *)(s_sched.a.child_rec + (size_t)id * CHILD_REC + threadIdx.x);
-        if ((s_sched.a.flags & ASPEN_HIP_FLAG_TRACE) && threadIdx.x == 0) s_sched.a.trace[2 * (size_t)id] = wall_clock64 ();
-        if ((s_sched.a.flags & ASPEN_HIP_FLAG_PROFILE) && threadIdx.x == 0) s_sched.p0 = wall_clock64 ();
+        if (row_rep == 0)
+        {
+            id = __builtin_amdgcn_readfirstlane (schedule_step<ORDERED> (id, rec));
+            if (id == QUEUE_EMPTY) break;           // all tickets taken, or aborted
+            // wavefront 0 requests this tile's child record now; it arrives while the tile runs
+            // (a global, not a flat load: a flat one would also count as LDS traffic the tile's first fragment wait sits out)
+            if (threadIdx.x < CHILD_REC)
+                rec = *(const qentry_t __attribute__ ((address_space (1))) *)(s_sched.a.child_rec + (size_t)id * CHILD_REC + threadIdx.x);
+            if ((s_sched.a.flags & ASPEN_HIP_FLAG_TRACE) && threadIdx.x == 0) s_sched.a.trace[2 * (size_t)id] = wall_clock64 ();
+            if ((s_sched.a.flags & ASPEN_HIP_FLAG_PROFILE) && threadIdx.x == 0) s_sched.p0 = wall_clock64 ();
+        }
         // the layer's descriptor goes from memory into scalar registers (it is shared by all tiles of the layer
         // and by all workgroups, so it sits in the scalar cache or in L2)
         const auto descriptor = [] () { return scalar_layer (s_sched.a.layers + s_sched.layer); };
-        bool complete;
+        bool complete, more_rows = false;
         const auto ready = [] () { if constexpr (ORDERED) wait_until_ready (); };
         if (!(s_sched.a.flags & ASPEN_HIP_FLAG_SKIP_TILES))
-            complete = run_tile<COH, FEAT, ORDERED ? NARROW_PF_SLICES : 0> (descriptor, id, true, smem, [] () { return s_sched.a.arrivals; }, ready);
+            complete = run_tile<COH, FEAT, ORDERED ? NARROW_PF_SLICES : 0> (descriptor, id, true, smem, [] () { return s_sched.a.arrivals; }, ready, row_rep, &more_rows);
         else
         {
             // scheduler-only run: the split-K groups still elect the member that releases the children
@@ -556,6 +566,7 @@ __global__ void __launch_bounds__ (WG_THREADS, WG_PER_CU) dataflow_kernel (dataf
             const uint32_t t = id - L.ninst_start;
             complete = L.splits <= 1 || splitk_arrived_last (&s_sched.a.arrivals[id - t % L.splits], L.splits, smem);
         }
+        row_rep = __builtin_amdgcn_readfirstlane (more_rows ? row_rep + 1u : 0u);
         if (threadIdx.x == 0) s_sched.complete = complete;      // read by schedule_step behind its barrier
     }
     if ((s_sched.a.flags & ASPEN_HIP_FLAG_PROFILE) && threadIdx.x == 0)
@@ -911,8 +922,9 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
         if (!L.weight) why = "missing weight";
         else if ((uint64_t)((L.M + 127) / 128 * 128) * L.Kp * 4 >= 0xffffff00ull) why = "weight matrix larger than 4 GiB";
         else if (L.Kp == 0 || L.Kp % GEMM_BK) why = "Kp must be a positive multiple of 32";
-        else if (L.tile_m != bm || L.tile_n != bn) why = "tile extent does not match the GEMM variant";
-        else if ((uint64_t)L.tiles_m * bm < L.M || (uint64_t)L.tiles_n * bn < L.N) why = "tile grid does not cover the matrix";
+        else if (L.tile_n != bn || (L.tile_m != bm && !(L.variant == ASPEN_HIP_GEMM_LARGE && L.splits == 1 && (L.tile_m == 2 * bm || L.tile_m == 4 * bm))))
+            why = "tile extent does not match the GEMM variant";         // (the large shape may cover two or four row tiles per workgroup)
+        else if ((uint64_t)L.tiles_m * L.tile_m < L.M || (uint64_t)L.tiles_n * bn < L.N) why = "tile grid does not cover the matrix";
         else if (L.direct != ASPEN_HIP_OPERAND_DIRECT && !L.ktab) why = "missing k-chunk table";
         else if (L.fuse_out && (!L.fuse_in || L.fuse_ld_in % 4 || L.fuse_ld_in < L.M)) why = "fused shortcut operand";
         else if (L.direct == ASPEN_HIP_OPERAND_DIRECT && (L.ld0 < L.Kp)) why = "direct operand shorter than Kp";

@@ -1970,8 +1970,15 @@ __device__ __forceinline__ void finish_tile (const aspen_hip_layer_t &L, uint32_
 // `ready ()` returns once the tile's parents have finished; it is called after whatever set-up does not touch an
 // activation (contraction tiles: descriptor, index arithmetic, first weight requests), right before the first
 // activation is requested.  Kernels that only start tiles whose parents have finished pass nothing.
+// Row groups: under the large shape a layer with a short K axis may give a workgroup SEVERAL row tiles of one column
+// block (tile_m = 2 or 4 times the shape's 128 rows): such tiles are all set-up, first fetch and epilogue, and a
+// workgroup that works through its column block's row tiles pays one scheduling step for all of them and finds the
+// activation block in its caches from the second one on.  The caller runs the tile once per row tile, row_rep = 0, 1, ...
+// while *more_rows comes back true (the tile code itself stays one straight pass: a loop around it here made the
+// compiler duplicate and spill the persistent kernel's K loops).
 template <int COH, unsigned FEAT = TILES_ALL, int NARROW_PF = 0, class Descriptor, class Arrivals, class Ready = NoHook>
-__device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, bool t_counts_from_graph_start, float *smem, Arrivals arrivals, Ready ready = Ready ())
+__device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, bool t_counts_from_graph_start, float *smem, Arrivals arrivals, Ready ready = Ready (),
+    uint32_t row_rep = 0, bool *more_rows = nullptr)
 {
     const aspen_hip_layer_t L = descriptor ();
     t = __builtin_amdgcn_readfirstlane (t);
@@ -1985,7 +1992,8 @@ __device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, boo
         group = L.ninst_start + t - (uint32_t)slice;
         t = q;
     }
-    const uint32_t tn = fast_div (t, L.div_tiles_m), tm = t - tn * L.tiles_m;
+    const uint32_t tn = fast_div (t, L.div_tiles_m);
+    uint32_t tm = t - tn * L.tiles_m;
     switch (L.type)
     {
     case CONV_LAYER: case FC_LAYER: case MATMUL_LAYER:
@@ -1998,7 +2006,19 @@ __device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, boo
         {
             if (L.variant == ASPEN_HIP_GEMM_NARROW) return narrow_tile<COH, NARROW_PF> (L, descriptor, t, tn, tm, slice, group, smem, arrivals, ready);
         }
-        if ((FEAT & TILES_LARGE) && L.variant == ASPEN_HIP_GEMM_LARGE) { contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, VAR0_DEPTH, COH, FEAT> (L, descriptor, tn, tm, -1, smem, pre, ready); c4_log2 = 5; bn = VAR0_BN; }
+        if ((FEAT & TILES_LARGE) && L.variant == ASPEN_HIP_GEMM_LARGE)
+        {
+            const uint32_t reps = L.tile_m / VAR0_BM;
+            if (reps > 1)
+            {
+                if (row_rep) __syncthreads ();      // the previous row tile's epilogue has read the stage this one refills
+                tm = tm * reps + row_rep;
+                if (more_rows) *more_rows = row_rep + 1 < reps;
+            }
+            const auto ready_first = [&] () { if (row_rep == 0) ready (); };
+            contraction_mainloop<VAR0_BM, VAR0_BN, 2, 2, VAR0_DEPTH, COH, FEAT> (L, descriptor, tn, tm, -1, smem, pre, ready_first);
+            c4_log2 = 5; bn = VAR0_BN;
+        }
         else if ((FEAT & TILES_WIDE) && L.variant == ASPEN_HIP_GEMM_WIDE) { contraction_mainloop<VAR1_BM, VAR1_BN, 2, 2, VAR1_DEPTH, COH, FEAT> (L, descriptor, tn, tm, -1, smem, pre, ready); bn = VAR1_BN; }
         else if ((FEAT & TILES_TALL) && L.variant == ASPEN_HIP_GEMM_TALL) { contraction_mainloop<VAR4_BM, VAR4_BN, 4, 1, VAR4_DEPTH, COH, FEAT> (L, descriptor, tn, tm, slice, smem, pre, ready); c4_log2 = 5; bn = VAR4_BN; }
         else if (FEAT & TILES_SMALL)

@@ -136,6 +136,16 @@ static int set_tiles (nasm_t *nasm, nasm_ldata_t *ld)
         }
         ld->variant = v;
         ld->tile_dims[OUT_H] = bm[v]; ld->tile_dims[OUT_W] = bn[v];
+        /* A short K axis (up to four slices) under the large shape: a tile is mostly set-up, first fetch and epilogue, so a
+           workgroup takes two or four row tiles of its column block at a time while that still leaves the layer the tiles
+           it wants (the 64 -> 256 channel layers of ResNet-50's first stage: 1568 tiles of 256 x 64 instead of 3136 of
+           128 x 64). */
+        if (v == ASPEN_HIP_GEMM_LARGE && aspen_layer_kiters (L) <= 4 && getenv ("ASPEN_GPU_NO_ROW_GROUPS") == NULL)
+        {
+            unsigned int r = 1;
+            while (r < 4 && M >= bm[v] * 2 * r && cdiv (M, bm[v] * 2 * r) * cdiv (N, bn[v]) >= want) r *= 2;
+            ld->tile_dims[OUT_H] = bm[v] * r;
+        }
     }
     else if (L->type == K_ATTENTION_LAYER)
     {

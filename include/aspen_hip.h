@@ -75,7 +75,9 @@ typedef struct aspen_hip_layer_t
     int32_t direct;          /* how the B operand is found, ASPEN_HIP_OPERAND_*: 0 k-chunk table, 1 read in place (1x1 stride-1
                                 conv / matmul, K % 32 == 0), 2 dense three-channel table */
     uint32_t M, N, ld;       /* output rows, columns, stride */
-    uint32_t tile_m, tile_n; /* tile extent in rows / columns */
+    uint32_t tile_m, tile_n; /* tile extent in rows / columns: the GEMM variant's shape; an uncut (splits == 1) layer of the LARGE
+                                shape may also have tile_m = 2 or 4 times the shape's rows (one workgroup runs those row tiles of
+                                its column block one after the other) */
     uint32_t tiles_m, tiles_n;
     uint32_t ninst_start;    /* engine-wide index of this layer's first tile */
     uint32_t num_ninst;

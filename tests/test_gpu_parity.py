@@ -210,6 +210,42 @@ def test_channel_counts_off_the_slice_width_in_a_graph_of_large_tiles(gpu, mode)
         net.close()
 
 
+@pytest.mark.parametrize("mode,flags", [(api.MODE_LAYERS, 0), (api.MODE_DATAFLOW, QUEUE), (api.MODE_DATAFLOW, ORDERED)], ids=["layers", "dataflow", "ordered"])
+@pytest.mark.parametrize("min_ninst,rows_per_tile", [(2048, 512), (4096, 256), (8192, 128)])
+def test_short_k_layers_take_several_row_tiles_per_workgroup(gpu, engine_flags, mode, flags, min_ninst, rows_per_tile):
+    """A 1 x 1 convolution with a short K axis (64 channels in) and many output channels under the 128 x 64 shape: a
+    workgroup works through two or four row tiles of its column block while the layer still has the tiles it wants;
+    one such layer on its own, one with a shortcut fused into its epilogue, one with 448 rows (a last row tile that is
+    only half there), all against the oracle."""
+    from oracle import cpu
+    engine_flags(flags)
+    cfg = ("[net]\nheight=64\nwidth=64\nchannels=64\n\n"
+           "[convolutional]\nfilters=512\nsize=1\nstride=1\npad=0\nactivation=relu\n\n"
+           "[convolutional]\nfilters=64\nsize=1\nstride=1\npad=0\nactivation=relu\n\n"
+           "[convolutional]\nfilters=512\nsize=1\nstride=1\npad=0\nactivation=linear\n\n"
+           "[shortcut]\nfrom=-3\nactivation=relu\n\n"
+           "[convolutional]\nfilters=96\nsize=1\nstride=1\npad=0\nactivation=relu\n\n"
+           "[convolutional]\nfilters=448\nsize=1\nstride=1\npad=0\nactivation=leaky\n\n")
+    layers = M.parse_cfg(cfg)
+    tens = M.synth_weights(layers, 61, "he")
+    batch = 32
+    x = (M.synth_input(layers, 61, batch, 0, "token_ids") * 2.0 - 1.0).astype(np.float32)
+    outs = cpu.run_network(layers, tens, x, batch, 0)
+    net = H.GpuNet(cfg, tens, batch, 0, min_ninst=min_ninst, mode=mode)
+    try:
+        net.run(x)
+        info = [net.nasm.info(l) for l in range(net.nasm.num_ldata)]
+        assert info[1]["tile_H"] == rows_per_tile and info[3]["tile_H"] == rows_per_tile, [(i["tile_H"], i["tile_W"], i["num_ninst"]) for i in info]
+        assert info[6]["tile_H"] == min(rows_per_tile, 256) or rows_per_tile == 128, [(i["tile_H"], i["tile_W"], i["num_ninst"]) for i in info]
+        for l in range(1, net.nasm.num_ldata):
+            err = H.rel_l2(net.layer(l), outs[l])
+            assert err <= H.REL_L2_TOL, f"layer {l}: rel L2 {err:.3g}"
+        if mode == api.MODE_DATAFLOW:
+            assert net.rpool.run_stats() == {"executed": net.nasm.num_ninst, "double_runs": 0, "aborted": 0}
+    finally:
+        net.close()
+
+
 @pytest.mark.parametrize("fused", [False, True], ids=["two-layers", "fused"])
 @pytest.mark.parametrize("mode", [api.MODE_LAYERS, api.MODE_DATAFLOW], ids=["layers", "dataflow"])
 @pytest.mark.parametrize("masked", [True, False], ids=["causal", "full"])
