@@ -1510,6 +1510,12 @@ __device__ __forceinline__ void tile_fused_attention (const aspen_hip_layer_t &L
     for (int v = 0; v < 16; v++) { oacc[v] = 0.f; part[v] = 0.f; }
     for (uint32_t k0 = 0; k0 < kend; k0 += BKEY)
     {
+        // the block's first 32 rows of V are requested before the scores are computed (they do not depend on them): one
+        // trip to memory less on the path of a tile whose key blocks run one after the other
+        TransLoader64<COH> vl;
+        vl.init (V, (b * S + k0) * L.fuse_ld_in + h * hd, L.fuse_ld_in, hd, S - k0, tid);
+        float4 vreg[2];
+        vl.load (0, vreg);
         // scores of 64 keys x 64 queries: one 32 x 32 block per wavefront
         floatx16 sacc[1][1];
         {
@@ -1528,10 +1534,6 @@ __device__ __forceinline__ void tile_fused_attention (const aspen_hip_layer_t &L
             ebuf[ql * EROW + wm0 + (lane & 31)] = e;
         }
         // weighted values: O[q][ch] += e[q][key] V[key][ch], two slices of 32 keys; V is read transposed through the stage
-        TransLoader64<COH> vl;
-        vl.init (V, (b * S + k0) * L.fuse_ld_in + h * hd, L.fuse_ld_in, hd, S - k0, tid);
-        float4 vreg[2];
-        vl.load (0, vreg);
         #pragma unroll
         for (int sl = 0; sl < BKEY / GEMM_BK; sl++)
         {
