@@ -522,8 +522,8 @@ template <int COH, unsigned FEAT, bool ORDERED = false>
 // (The variant for transformer graphs is built for three workgroups per compute unit instead of four: those graphs never
 // fill the device (256 to 768 workgroups), and 168 instead of 128 registers per lane spare their attention and matmul loops
 // the spills the tighter budget forces.)
-#define DATAFLOW_WG_PER_CU(feat) ((feat) == TILES_TRANSFORMER ? WG_PER_CU - 1 : WG_PER_CU)
-__global__ void __launch_bounds__ (WG_THREADS, DATAFLOW_WG_PER_CU (FEAT)) dataflow_kernel (dataflow_args_t args)
+#define DATAFLOW_WG_PER_CU(feat, ordered) ((ordered) ? 2 : (feat) == TILES_TRANSFORMER ? WG_PER_CU - 1 : WG_PER_CU)
+__global__ void __launch_bounds__ (WG_THREADS, DATAFLOW_WG_PER_CU (FEAT, ORDERED)) dataflow_kernel (dataflow_args_t args)
 {
     extern __shared__ __align__ (16) float smem[];
     if (threadIdx.x == 0)
