@@ -80,6 +80,7 @@ def lib() -> C.CDLL:
         "aspen_dse_group_set_mode": (None, [_vp, C.c_int]),
         "aspen_dse_group_last_mode": (C.c_int, [_vp]),
         "aspen_dse_group_last_run_ordered": (C.c_int, [_vp]),
+        "aspen_nasm_set_ordered": (None, [_vp, C.c_int]),
         "aspen_dse_group_set_spin_limit": (None, [_vp, C.c_uint64]),
         "aspen_dse_group_set_workgroups": (None, [_vp, C.c_uint]),
         "aspen_keep_layer_outputs": (None, [C.c_int]),
@@ -203,6 +204,10 @@ class Nasm:
             d[k] = -1 if d[k] == 0xffffffff else d[k]
         d["flops"] = int(lib().aspen_nasm_ldata_flops(self.h, l))
         return d
+
+    def set_ordered(self, ordered: int):
+        """1 / 0: runs on the persistent kernel use / do not use its ordered mode; -1: the engine decides."""
+        lib().aspen_nasm_set_ordered(self.h, ordered)
 
     def graph(self):
         """(tile -> layer, parent counts, child offsets, child indices) as numpy copies."""

@@ -11,6 +11,12 @@ int aspen_dse_group_last_run_ordered (dse_group_t *g)
 {
     return g != NULL && g->last_mode == 1 && g->rpool != NULL && g->rpool->graph != NULL && aspen_hip_graph_last_run_ordered (g->rpool->graph);
 }
+void aspen_nasm_set_ordered (nasm_t *nasm, int ordered)
+{
+    if (nasm == NULL) return;
+    nasm->ordered_pref = ordered < 0 ? -1 : ordered != 0;
+    if (nasm->rpool != NULL) nasm->rpool->graph_dirty = 1;        /* the pool's device graph carries the setting: rebuilt at the next run */
+}
 void aspen_dse_group_set_spin_limit (dse_group_t *g, uint64_t polls) { if (g) g->spin_limit = polls; }
 void aspen_dse_group_set_workgroups (dse_group_t *g, unsigned int w) { if (g) g->workgroups = w; }
 

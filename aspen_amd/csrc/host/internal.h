@@ -95,7 +95,8 @@ struct nasm_t
     unsigned int kiters_cap;                 /* 0, or the longest K loop (in slices of 32) a contraction tile may have, see create_nasm */
     int small_tiles_only;                    /* every contraction layer uses the small tile shape, see create_nasm */
     int narrow_tiles;                        /* layers short of tiles use the 32 x 32 shape, see create_nasm */
-    int latency_bound;                       /* built for the engine's ordered mode (one image through a deep network), see create_nasm */
+    int ordered_pref;                        /* persistent kernel in its ordered mode (no ready queue): 1 yes (graphs bound by latency, see create_nasm;
+                                                the tuner; aspen_nasm_set_ordered), 0 no, -1 the engine decides from the graph's parallelism */
     nasm_ldata_t *ldata_arr;
     unsigned int num_ldata;
     unsigned int num_ninst;

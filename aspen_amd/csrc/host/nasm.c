@@ -551,6 +551,7 @@ static nasm_t *build_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned in
     nasm->small_tiles_only = small_tiles_only;
     nasm->narrow_tiles = narrow_tiles;
     nasm->preferred_mode = -1;
+    nasm->ordered_pref = -1;
     nasm->dnn = dnn; nasm->nasm_id = nasm_counter++;
     nasm->batch_size = batch > 0 ? batch : 1;
     nasm->tr_seq_len = seq; nasm->min_ninst_per_ldata = min_ninst;
@@ -642,6 +643,7 @@ static double nasm_parallelism (const nasm_t *nasm)
 #define CHAIN_BOUND_CAP_FROM 400.0
 #define CHAIN_BOUND_KITERS_CAP 48
 #define LATENCY_BOUND_BELOW 128.0
+#define ORDERED_VISION_BELOW 300.0
 static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned int batch, unsigned int seq)
 {
     const char *e = getenv ("ASPEN_GPU_MAX_KITERS");            /* experiments: fixed cap, 0 = none */
@@ -649,6 +651,7 @@ static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned i
     nasm_t *nasm = build_nasm (dnn, min_ninst, batch, seq, 0, 0, 0);
     if (nasm == NULL) return nasm;
     const double parallelism = nasm_parallelism (nasm);
+    if (getenv ("ASPEN_GPU_VERBOSE")) fprintf (stderr, "aspen: graph of %u tiles, average parallelism %.0f\n", nasm->num_ninst, parallelism);
     if (parallelism >= CHAIN_BOUND_BELOW) return nasm;
     /* bound by the LATENCY of its chains (one image through a deep network; the engine runs such a graph in its ordered
        mode): layers short of tiles take the 32 x 32 shape */
@@ -656,7 +659,13 @@ static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned i
     const int narrow = nt != NULL ? atoi (nt) != 0 : parallelism < LATENCY_BOUND_BELOW;
     nasm_t *rebuilt = build_nasm (dnn, min_ninst, batch, seq, parallelism >= CHAIN_BOUND_CAP_FROM ? CHAIN_BOUND_KITERS_CAP : 0, 1, narrow);
     if (rebuilt == NULL) return nasm;
-    rebuilt->latency_bound = parallelism < LATENCY_BOUND_BELOW;
+    /* The ordered mode itself pays further up than the 32 x 32 tiles do, for convolutional networks: measured against the
+       ready queue on ResNet-50 at batch 1 / 2 / 4 (parallelism 95 / 175 / 276: 0.45 / 0.62 / 0.76 ms against 0.64 / 0.73 /
+       0.87), VGG-16 at batch 1 (316: 0.58 against 0.62) and YOLO-v3 at batch 1 (251: 1.46 against 1.48); from about 350 on
+       the queue wins more often than not (YOLO-v3 batch 2, 329: 2.09 against 2.00), and the transformer graphs lose with
+       it at every size (their long, uniform tiles want the queue's balancing: BERT-base, 265: 2.9 against 2.2 ms).  Where
+       it matters, apu_generate_nasm times both. */
+    if (parallelism < LATENCY_BOUND_BELOW || (seq == 0 && parallelism < ORDERED_VISION_BELOW)) rebuilt->ordered_pref = 1;
     apu_destroy_nasm (nasm);
     return rebuilt;
 }
@@ -718,28 +727,34 @@ static nasm_t *generate_nasm (aspen_dnn_t *dnn, unsigned int batch, unsigned int
 {
     const unsigned int ncand = sizeof (tuner_candidates) / sizeof (tuner_candidates[0]);
     if (num_iter == 0 || aspen_hip_init () != 0) return create_nasm (dnn, DEFAULT_MIN_NINST, batch, seq);
+    static const char *const engine_name[3] = {"one launch per layer", "persistent kernel, ready queue", "persistent kernel, ordered"};
     unsigned int best = DEFAULT_MIN_NINST;
-    int best_mode = 1;
+    int best_engine = 1;
     double best_time = -1.0;
-    /* every candidate on both engines: the persistent kernel (1) and one launch per layer (0) */
+    /* every candidate on the three engines: the persistent kernel with its ready queue (1) and in its ordered mode (2), one
+       launch per layer (0) */
     for (unsigned int c = 0; c < ncand && c <= num_iter; c++)
     {
         nasm_t *cand = create_nasm (dnn, tuner_candidates[c], batch, seq);
         if (cand == NULL) return NULL;
-        for (int mode = 1; mode >= 0; mode--)
+        for (int engine = 2; engine >= 0; engine--)
         {
-            const double t = test_nasm_time_sec (cand, 10, mode);
-            printf ("APU: min_ninst_per_ldata %u, %s: %u tiles, %f sec per inference\n", tuner_candidates[c],
-                mode ? "persistent kernel" : "one launch per layer", cand->num_ninst, t);
+            cand->ordered_pref = engine == 2;
+            const double t = test_nasm_time_sec (cand, 10, engine != 0);
+            printf ("APU: min_ninst_per_ldata %u, %s: %u tiles, %f sec per inference\n", tuner_candidates[c], engine_name[engine], cand->num_ninst, t);
             fflush (stdout);
-            if (t > 0 && (best_time < 0 || t < best_time)) { best_time = t; best = tuner_candidates[c]; best_mode = mode; }
+            if (t > 0 && (best_time < 0 || t < best_time)) { best_time = t; best = tuner_candidates[c]; best_engine = engine; }
         }
         apu_destroy_nasm (cand);
     }
-    printf ("APU: NASM with min_ninst_per_ldata %u, %s, time = %f sec selected.\n", best, best_mode ? "persistent kernel" : "one launch per layer", best_time);
+    printf ("APU: NASM with min_ninst_per_ldata %u, %s, time = %f sec selected.\n", best, engine_name[best_engine], best_time);
     fflush (stdout);
     nasm_t *nasm = create_nasm (dnn, best, batch, seq);
-    if (nasm != NULL) nasm->preferred_mode = best_mode;      /* what an engine group in mode "auto" will run it with */
+    if (nasm != NULL)
+    {
+        nasm->preferred_mode = best_engine != 0;        /* what an engine group in mode "auto" will run it with */
+        nasm->ordered_pref = best_engine == 2;
+    }
     return nasm;
 }
 

@@ -193,10 +193,12 @@ static int rebuild_graph (rpool_t *rp)
         if (rp->graph == NULL) rc = -1;
         else
         {
-            /* graphs built for latency (their tile grids were chosen for it) run the persistent kernel in its ordered mode */
-            int latency = rp->num_nasms > 0;
-            for (unsigned int i = 0; i < rp->num_nasms; i++) latency &= rp->nasms[i]->latency_bound;
-            if (latency) aspen_hip_graph_set_ordered (rp->graph, 1);
+            /* graphs bound by latency run the persistent kernel in its ordered mode: when every nasm of the pool asks for it;
+               a nasm that asks for the ready queue gets it; otherwise the engine decides from the merged graph */
+            int all_ordered = rp->num_nasms > 0, any_queue = 0;
+            for (unsigned int i = 0; i < rp->num_nasms; i++) { all_ordered &= rp->nasms[i]->ordered_pref == 1; any_queue |= rp->nasms[i]->ordered_pref == 0; }
+            if (all_ordered) aspen_hip_graph_set_ordered (rp->graph, 1);
+            else if (any_queue) aspen_hip_graph_set_ordered (rp->graph, 0);
         }
     }
     free (L); free (nl); free (np); free (co); free (ci); free (roots);

@@ -391,7 +391,8 @@ WORKLOADS = {
     "vgg16_b16": (["vgg16_b16"], "img/s", 16, 1536, "dataflow"),
     "bert_base_b8_s128": (["bert_base_b8_s128"], "tokens/s", 8 * 128, 192, "dataflow"),
     "gpt2_b4_s512": (["gpt2_b4_s512"], "tokens/s", 4 * 512, 384, "dataflow"),
-    "yolov3_b1": (["yolov3_b1"], "img/s", 1, 768, "layers"),
+    # (engine "dataflow-ordered": the persistent kernel, its ordered mode asked for with Nasm.set_ordered)
+    "yolov3_b1": (["yolov3_b1"], "img/s", 1, 768, "dataflow-ordered"),
     "yolov3_b8": (["yolov3_b8"], "img/s", 8, 1536, "dataflow"),
 }
 

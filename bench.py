@@ -212,7 +212,7 @@ def measure_workload(api, M, name, steps, warmup, flags=0):
     L.aspen_hip_set_flags(flags)
     cfgs, unit, units_per_step, min_ninst, engine = WORKLOADS[name]
     pool = api.RPool()
-    dse = api.DseGroup(1, api.MODE_DATAFLOW if engine == "dataflow" else api.MODE_LAYERS)
+    dse = api.DseGroup(1, api.MODE_DATAFLOW if engine.startswith("dataflow") else api.MODE_LAYERS)
     dse.set_rpool(pool)
     nets = []
     for cname in cfgs:
@@ -223,6 +223,8 @@ def measure_workload(api, M, name, steps, warmup, flags=0):
         os.unlink(wp)
         del tens
         nasm = api.Nasm(dnn, batch, seq, min_ninst)
+        if engine == "dataflow-ordered":
+            nasm.set_ordered(1)
         pool.add_nasm_raw_input(nasm, x)
         nets.append((cname, dnn, nasm))
     flops = sum(gemm_flops(n, api) for _, _, n in nets)
@@ -285,7 +287,7 @@ def measure_workload(api, M, name, steps, warmup, flags=0):
            "traffic": traffic, "compulsory_bytes": compulsory, "traffic_over_compulsory": traffic / compulsory if traffic else None,
            "tiles_per_step": sum(n.num_ninst for _, _, n in nets), "flops_per_step": flops,
            "frac_of_fp32_mfma_peak": ach / PEAK_FP32_MFMA_TFLOPS, "verified": all(c["ok"] for c in have) if have else None}
-    if engine == "dataflow" and dse.last_run_ordered():
+    if engine.startswith("dataflow") and dse.last_run_ordered():
         out["engine"] = "dataflow-ordered"
     out["steps"] = steps
     if weight_stream:
@@ -374,8 +376,9 @@ def main():
     cfgs, unit, units_per_step, tuned_min_ninst, tuned_engine = WORKLOADS[args.workload]
     if args.min_ninst <= 0:
         args.min_ninst = tuned_min_ninst
+    ask_ordered = False
     if args.mode == "auto":
-        args.mode = tuned_engine
+        args.mode, ask_ordered = tuned_engine.split("-")[0], tuned_engine == "dataflow-ordered"
 
     pool = api.RPool()
     dse = api.DseGroup(1, {"auto": api.MODE_AUTO, "dataflow": api.MODE_DATAFLOW, "layers": api.MODE_LAYERS}[args.mode], args.workgroups)
@@ -389,6 +392,8 @@ def main():
         os.unlink(wp)
         del tens
         nasm = api.Nasm(dnn, batch, seq, args.min_ninst)
+        if ask_ordered:
+            nasm.set_ordered(1)
         pool.add_nasm_raw_input(nasm, x)
         nets.append((name, dnn, nasm, layers))
     flops = sum(gemm_flops(n, api) for _, _, n, _ in nets)

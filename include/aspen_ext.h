@@ -29,6 +29,11 @@ int aspen_dse_group_last_mode (dse_group_t *dse_group);
 /* 1 when that run was a dataflow run in ordered mode (tiles taken in index order and prepared before they are ready,
    no ready queue: what graphs built for one image through a deep network run in) */
 int aspen_dse_group_last_run_ordered (dse_group_t *dse_group);
+/* Whether runs of this nasm on the persistent kernel use its ordered mode (no ready queue; tiles assigned to workgroups in
+   index order and prepared before their parents have finished): 1 / 0, -1 = the engine decides.  apu_create_nasm asks
+   for it on graphs bound by latency (a single image, small batches of convolutional networks), apu_generate_nasm times
+   it against the other engines; a pool runs ordered when all its nasms ask for it. */
+void aspen_nasm_set_ordered (nasm_t *nasm, int ordered);
 /* Watchdog of the persistent kernel: polls a workgroup may spend waiting for one ready tile before the
    run is given up (every workgroup then leaves, the run reports ASPEN_HIP_ERR_STALLED and the next run
    starts from re-armed state).  0 = the library's default (2^26 polls, minutes). */

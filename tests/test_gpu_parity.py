@@ -483,7 +483,7 @@ def test_timed_graphs_match_oracle_on_whole_tensors(gpu, workload):
     the final layer); a single wrong tile anywhere fails its layer."""
     from oracle import cpu
     cfgs, _, _, min_ninst, engine = M.WORKLOADS[workload]
-    mode = api.MODE_DATAFLOW if engine == "dataflow" else api.MODE_LAYERS
+    mode = api.MODE_DATAFLOW if engine.startswith("dataflow") else api.MODE_LAYERS
     cases, want = [], []
     for name in cfgs:
         cfg, layers, tens, x, batch, seq = H.full_config(name)
@@ -502,6 +502,8 @@ def test_timed_graphs_match_oracle_on_whole_tensors(gpu, workload):
                     net = H.GpuNet(cfg, tens, batch, seq, min_ninst=min_ninst, mode=mode)
                     net.rpool.destroy()
                     net.rpool = pool
+                    if engine == "dataflow-ordered":
+                        net.nasm.set_ordered(1)
                     pool.add_nasm_raw_input(net.nasm, x)
                     nets.append(net)
                 print(f"{workload} keep={keep}: {sum(n.nasm.num_ninst for n in nets)} tiles", flush=True)
@@ -512,6 +514,7 @@ def test_timed_graphs_match_oracle_on_whole_tensors(gpu, workload):
                 if mode == api.MODE_DATAFLOW:
                     st = pool.run_stats()
                     assert st == {"executed": sum(n.nasm.num_ninst for n in nets), "double_runs": 0, "aborted": 0}, st
+                    assert dse.last_run_ordered() or engine != "dataflow-ordered"
                 worst = 0.0
                 for (name, _, layers, *_), net, outs in zip(cases, nets, want):
                     dropped = 0
@@ -692,7 +695,8 @@ def test_generate_nasm_times_candidates(gpu, capfd):
     os.unlink(wp)
     nasm = api.Nasm(dnn, batch, seq, generate_iters=2)
     out = capfd.readouterr().out
-    assert out.count("sec per inference") == 6 and "selected" in out          # three candidates on both engines
+    assert out.count("sec per inference") == 9 and "selected" in out          # three candidates on three engines (ready queue, ordered, per layer)
+    assert out.count("persistent kernel, ordered:") == 3 and out.count("persistent kernel, ready queue:") == 3
     pool, dse = api.RPool(), api.DseGroup(1, api.MODE_DATAFLOW)
     dse.set_rpool(pool)
     pool.add_nasm_raw_input(nasm, x)
