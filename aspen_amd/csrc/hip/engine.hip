@@ -522,7 +522,7 @@ template <int COH, unsigned FEAT, bool ORDERED = false>
 // (The variant for transformer graphs is built for three workgroups per compute unit instead of four: those graphs never
 // fill the device (256 to 768 workgroups), and 168 instead of 128 registers per lane spare their attention and matmul loops
 // the spills the tighter budget forces.)
-#define DATAFLOW_WG_PER_CU(feat, ordered) ((ordered) ? 2 : (feat) == TILES_TRANSFORMER ? WG_PER_CU - 1 : WG_PER_CU)
+#define DATAFLOW_WG_PER_CU(feat, ordered) ((feat) == TILES_TRANSFORMER ? WG_PER_CU - 1 : WG_PER_CU)
 __global__ void __launch_bounds__ (WG_THREADS, DATAFLOW_WG_PER_CU (FEAT, ORDERED)) dataflow_kernel (dataflow_args_t args)
 {
     extern __shared__ __align__ (16) float smem[];
@@ -1255,21 +1255,30 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     // (a static assignment in index order only terminates when every tile's parents have smaller indices: graph_parallelism
     // reports 1e30 for a graph that is not listed that way)
     if (!g->cached_loads || xcd_queues || g->num_ninst > (1u << 20) || g->parallelism > 1e29) ordered = false;
+    size_t ordered_smem = ORDERED_SMEM_BYTES;
     if (ordered)
     {
         // tiles are assigned to workgroups beforehand: every workgroup of the grid must be running
-        static int fit = -1;
-        if (fit < 0)
+        // (graphs without 32 x 32 tiles need no weight prefetch buffers: their workgroups take the LDS of any other tile, and
+        // twice as many fit a compute unit)
+        static int fits[2] = {-1, -1};
+        const int small_lds = (g->features & TILES_NARROW) == 0;
+        if (fits[small_lds] < 0)
         {
             int o0 = 0, o1 = 0;
-            CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&o0, ordered_kernels[0], WG_THREADS, ORDERED_SMEM_BYTES));
-            CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&o1, ordered_kernels[1], WG_THREADS, ORDERED_SMEM_BYTES));
-            fit = (o0 < o1 ? o0 : o1) * g_num_cu;
+            const size_t smem = small_lds ? GEMM_SMEM_BYTES : ORDERED_SMEM_BYTES;
+            CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&o0, ordered_kernels[0], WG_THREADS, smem));
+            CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&o1, ordered_kernels[1], WG_THREADS, smem));
+            fits[small_lds] = (o0 < o1 ? o0 : o1) * g_num_cu;
         }
+        const int fit = fits[small_lds];
+        ordered_smem = small_lds ? GEMM_SMEM_BYTES : ORDERED_SMEM_BYTES;
         if (fit < 1) ordered = false;
         else
         {
-            if (workgroups_requested == 0) workgroups = (uint32_t)fit;         // two per compute unit: one tile computes, the next is prepared
+            // by default two per compute unit with the prefetch buffers (one tile computes, the next is prepared), three
+            // without (YOLO-v3 batch 1: 1.30 / 1.25 / 1.26 ms with two / three / four)
+            if (workgroups_requested == 0) workgroups = small_lds && fit > 3 * g_num_cu ? 3u * (uint32_t)g_num_cu : (uint32_t)fit;
             if (workgroups > (uint32_t)fit) workgroups = (uint32_t)fit;
         }
     }
@@ -1349,7 +1358,7 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
         if (ordered) kernel = ordered_kernels[(g->features & ~ordered_variant_tiles[0]) == 0 ? 0 : 1];
         g->last_run_ordered = ordered;
         void *kernel_args[] = {&a};
-        CHECK (hipLaunchKernel (kernel, dim3 (workgroups), dim3 (WG_THREADS), kernel_args, ordered ? ORDERED_SMEM_BYTES : GEMM_SMEM_BYTES, g_stream));
+        CHECK (hipLaunchKernel (kernel, dim3 (workgroups), dim3 (WG_THREADS), kernel_args, ordered ? ordered_smem : GEMM_SMEM_BYTES, g_stream));
     }
     CHECK (hipGetLastError ());
     CHECK (hipEventRecord (g_events[NUM_EVENTS - 1], g_stream));
