@@ -1056,6 +1056,43 @@ __device__ __forceinline__ void tile_pool (const aspen_hip_layer_t &L, uint32_t 
         if (m + 4 > L.M) { if (m + 0 >= L.M) r.x = 0.f; if (m + 1 >= L.M) r.y = 0.f; if (m + 2 >= L.M) r.z = 0.f; if (m + 3 >= L.M) r.w = 0.f; }
         out.st4 (n * L.ld + m, r);
     };
+    if (per_thread == 1 && L.KH == 2 && L.KW == 2)
+    {
+        // the 2x2 window of the VGG / Darknet pools: a thread requests the four inputs of two of its pieces together (clamped
+        // to the image where padding puts them outside, and then not used); combined in the order of the general loop below
+        for (uint32_t i0 = tile_thread (); i0 < total; i0 += 2 * WG_THREADS)
+        {
+            float4 x[2][4];
+            uint32_t nn[2], mm[2];
+            int ih0[2], iw0[2];
+            #pragma unroll
+            for (int u = 0; u < 2; u++)
+            {
+                const uint32_t i = min (i0 + u * WG_THREADS, total - 1);
+                const uint32_t c = i / M4, m = r0 + (i - c * M4) * 4, n = n0 + c;
+                const uint32_t b = n / ohw, rem = n - b * ohw, oh = rem / L.OW, ow = rem - oh * L.OW;
+                nn[u] = n; mm[u] = m;
+                ih0[u] = (int)(oh * L.stride) - (int)L.pad; iw0[u] = (int)(ow * L.stride) - (int)L.pad;
+                #pragma unroll
+                for (int q = 0; q < 4; q++)
+                {
+                    const uint32_t ihc = (uint32_t)min (max (ih0[u] + (q >> 1), 0), (int)L.IH - 1), iwc = (uint32_t)min (max (iw0[u] + (q & 1), 0), (int)L.IW - 1);
+                    x[u][q] = in.ld4 (((b * L.IH + ihc) * L.IW + iwc) * L.ld0 + m);
+                }
+            }
+            #pragma unroll
+            for (int u = 0; u < 2; u++)
+            {
+                if (u && i0 + WG_THREADS >= total) break;
+                float4 r = start;
+                #pragma unroll
+                for (int q = 0; q < 4; q++)
+                    if ((uint32_t)(ih0[u] + (q >> 1)) < L.IH && (uint32_t)(iw0[u] + (q & 1)) < L.IW) combine (r, x[u][q]);
+                finish (r, nn[u], mm[u]);
+            }
+        }
+        return;
+    }
     for (uint32_t i = tile_thread (); i < total; i += WG_THREADS)
     {
         const uint32_t c = i / M4, m = r0 + (i - c * M4) * 4, n = n0 + per_thread * c;

@@ -155,6 +155,35 @@ def test_every_activation_and_softmax_match_oracle(gpu, mode):
 
 
 @pytest.mark.parametrize("mode", [api.MODE_LAYERS, api.MODE_DATAFLOW], ids=["layers", "dataflow"])
+@pytest.mark.parametrize("height,width,pad", [(12, 8, 0), (11, 9, 1), (10, 8, 1), (7, 5, 0)])
+def test_two_by_two_pools_with_padding_and_odd_images_match_oracle(gpu, mode, height, width, pad):
+    """2x2 / stride-2 max and average pools (the window the VGG and Darknet pools use; its four inputs are
+    fetched together): windows that reach over the top / left padding, over the bottom / right one, and
+    images whose last row and column no window covers (reference tiled_maxpool2d / tiled_avgpool2d,
+    src/tiled_kernels.c:411-498: positions outside the image are skipped, the average still divides by 4)."""
+    from oracle import cpu
+    cfg = (f"[net]\nheight={height}\nwidth={width}\nchannels=3\n\n"
+           "[convolutional]\nfilters=40\nsize=3\nstride=1\npad=1\nactivation=linear\n\n"
+           f"[maxpool]\nsize=2\nstride=2\npad={pad}\n\n"
+           "[convolutional]\nfilters=24\nsize=1\nstride=1\npad=0\nactivation=linear\n\n"
+           f"[avgpool]\nsize=2\nstride=2\npad={pad}\n\n"
+           "[connected]\noutput=10\nactivation=linear\n\n")
+    layers = M.parse_cfg(cfg)
+    tens = M.synth_weights(layers, 33, "he")
+    batch = 5
+    x = (M.synth_input(layers, 33, batch, 0, "token_ids") * 2.0 - 1.0).astype(np.float32)
+    outs = cpu.run_network(layers, tens, x, batch, 0)
+    net = H.GpuNet(cfg, tens, batch, 0, min_ninst=16, mode=mode)
+    try:
+        net.run(x)
+        for l in range(net.nasm.num_ldata):
+            err = H.rel_l2(net.layer(l), outs[l])
+            assert err <= H.REL_L2_TOL, f"layer {l} ({layers[l]['type']}): rel L2 {err:.3g}"
+    finally:
+        net.close()
+
+
+@pytest.mark.parametrize("mode", [api.MODE_LAYERS, api.MODE_DATAFLOW], ids=["layers", "dataflow"])
 @pytest.mark.parametrize("filters,size,stride,pad,min_ninst", [(16, 7, 2, 3, 16), (64, 3, 1, 1, 16), (64, 5, 1, 0, 2048), (96, 3, 2, 1, 16), (8, 1, 1, 0, 16)])
 def test_first_layer_over_three_channels_matches_oracle(gpu, mode, filters, size, stride, pad, min_ninst):
     """A convolution over three input channels keeps its K axis dense on the device (K = 3 x taps, a chunk of four K
