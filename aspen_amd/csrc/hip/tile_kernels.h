@@ -1018,12 +1018,26 @@ __device__ __forceinline__ void tile_residual (const aspen_hip_layer_t &L, uint3
     const uint32_t total = (n1 - n0) * M4;
     ActView<COH> p0, p1, out;
     p0.init (L.in0, L.N, L.ld0); p1.init (L.in1, L.N, L.ld1); out.init (L.out, L.N, L.ld);
-    for (uint32_t i = tile_thread (); i < total; i += WG_THREADS)
+    // two pieces per thread and step: four loads in flight before the first store (the second piece of a thread's last
+    // step may lie past the end: it is then fetched from the last piece's address and not stored)
+    for (uint32_t i0 = tile_thread (); i0 < total; i0 += 2 * WG_THREADS)
     {
-        const uint32_t c = i / M4, m = (i - c * M4) * 4, n = n0 + c;
-        float4 a = p0.ld4 (n * L.ld0 + m), b = p1.ld4 (n * L.ld1 + m);
-        a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
-        out.st4 (n * L.ld + m, act4 (a, L.act));
+        float4 a[2], b[2];
+        uint32_t dst[2];
+        #pragma unroll
+        for (int u = 0; u < 2; u++)
+        {
+            const uint32_t i = min (i0 + u * WG_THREADS, total - 1), c = i / M4, m = (i - c * M4) * 4, n = n0 + c;
+            a[u] = p0.ld4 (n * L.ld0 + m); b[u] = p1.ld4 (n * L.ld1 + m);
+            dst[u] = n * L.ld + m;
+        }
+        #pragma unroll
+        for (int u = 0; u < 2; u++)
+        {
+            if (u && i0 + WG_THREADS >= total) break;
+            a[u].x += b[u].x; a[u].y += b[u].y; a[u].z += b[u].z; a[u].w += b[u].w;
+            out.st4 (dst[u], act4 (a[u], L.act));
+        }
     }
 }
 
@@ -1056,6 +1070,49 @@ __device__ __forceinline__ void tile_pool (const aspen_hip_layer_t &L, uint32_t 
         if (m + 4 > L.M) { if (m + 0 >= L.M) r.x = 0.f; if (m + 1 >= L.M) r.y = 0.f; if (m + 2 >= L.M) r.z = 0.f; if (m + 3 >= L.M) r.w = 0.f; }
         out.st4 (n * L.ld + m, r);
     };
+    if (per_thread == 1 && L.KH * L.KW >= 32)
+    {
+        // a wide window (global average pooling, 7x7 = 49 positions): eight neighbouring lanes share a piece, each
+        // requests every eighth position of the window (all of its up to eight at once), and the eight partial results
+        // meet through lane exchanges: one trip to memory per piece instead of one per window row.  (Sums are
+        // formed in a different order than row by row: equal up to rounding.)
+        const uint32_t sub = tile_thread () & 7u, P = L.KH * L.KW;
+        for (uint32_t i0 = tile_thread () >> 3; i0 < (total + WG_THREADS / 8 - 1) / (WG_THREADS / 8) * (WG_THREADS / 8); i0 += WG_THREADS / 8)
+        {
+            // (every lane of a wavefront takes part in the exchanges: a group past the end works on the last piece and stores nothing)
+            const uint32_t i = min (i0, total - 1);
+            const uint32_t c = i / M4, m = r0 + (i - c * M4) * 4, n = n0 + c;
+            const uint32_t b = n / ohw, rem = n - b * ohw, oh = rem / L.OW, ow = rem - oh * L.OW;
+            const int ih0 = (int)(oh * L.stride) - (int)L.pad, iw0 = (int)(ow * L.stride) - (int)L.pad;
+            float4 r = start;
+            for (uint32_t p0 = 0; p0 < P; p0 += 64)
+            {
+                float4 x[8];
+                #pragma unroll
+                for (uint32_t q = 0; q < 8; q++)
+                {
+                    const uint32_t pos = min (p0 + sub + 8 * q, P - 1), kh = pos / L.KW, kw = pos - kh * L.KW;
+                    const uint32_t ihc = (uint32_t)min (max (ih0 + (int)kh, 0), (int)L.IH - 1), iwc = (uint32_t)min (max (iw0 + (int)kw, 0), (int)L.IW - 1);
+                    x[q] = in.ld4 (((b * L.IH + ihc) * L.IW + iwc) * L.ld0 + m);
+                }
+                #pragma unroll
+                for (uint32_t q = 0; q < 8; q++)
+                {
+                    const uint32_t pos = p0 + sub + 8 * q, kh = pos / L.KW, kw = pos - kh * L.KW;
+                    if (pos < P && (uint32_t)(ih0 + (int)kh) < L.IH && (uint32_t)(iw0 + (int)kw) < L.IW) combine (r, x[q]);
+                }
+            }
+            #pragma unroll
+            for (int o = 1; o < 8; o <<= 1)
+            {
+                float4 y;
+                y.x = __shfl_xor (r.x, o, 64); y.y = __shfl_xor (r.y, o, 64); y.z = __shfl_xor (r.z, o, 64); y.w = __shfl_xor (r.w, o, 64);
+                combine (r, y);
+            }
+            if (sub == 0 && i0 < total) finish (r, n, m);
+        }
+        return;
+    }
     if (per_thread == 1 && L.KH == 2 && L.KW == 2)
     {
         // the 2x2 window of the VGG / Darknet pools: a thread requests the four inputs of two of its pieces together (clamped
@@ -1205,13 +1262,24 @@ __device__ __forceinline__ void tile_append (const aspen_hip_layer_t &L, uint32_
     if (((L.IC | L.M) & 3u) == 0)
     {
         const uint32_t M4 = L.M >> 2, total = (n1 - n0) * M4;
-        for (uint32_t i = tile_thread (); i < total; i += WG_THREADS)
+        // four pieces per thread and step, all requested before the first store (pieces past the end: fetched from the
+        // last piece's address and not stored)
+        for (uint32_t i0 = tile_thread (); i0 < total; i0 += 4 * WG_THREADS)
         {
-            const uint32_t c = i / M4, m = (i - c * M4) * 4, n = n0 + c;
-            const uint32_t b = n / ohw, rem = n - b * ohw, oh = rem / L.OW, ow = rem - oh * L.OW;
-            const float4 v = m < L.IC ? p0.ld4 (((b * ih + oh / L.stride) * iw + ow / L.stride) * L.ld0 + m)
-                                      : p1.ld4 (n * L.ld1 + (m - L.IC));
-            out.st4 (n * L.ld + m, v);
+            float4 v[4];
+            uint32_t dst[4];
+            #pragma unroll
+            for (int u = 0; u < 4; u++)
+            {
+                const uint32_t i = min (i0 + u * WG_THREADS, total - 1), c = i / M4, m = (i - c * M4) * 4, n = n0 + c;
+                const uint32_t b = n / ohw, rem = n - b * ohw, oh = rem / L.OW, ow = rem - oh * L.OW;
+                v[u] = m < L.IC ? p0.ld4 (((b * ih + oh / L.stride) * iw + ow / L.stride) * L.ld0 + m)
+                                : p1.ld4 (n * L.ld1 + (m - L.IC));
+                dst[u] = n * L.ld + m;
+            }
+            #pragma unroll
+            for (int u = 0; u < 4; u++)
+                if (i0 + u * WG_THREADS < total) out.st4 (dst[u], v[u]);
         }
         return;
     }
