@@ -1163,6 +1163,35 @@ __device__ __forceinline__ void tile_pool (const aspen_hip_layer_t &L, uint32_t 
             uint32_t bb = b, hh = oh, ww = ow;
             if (which) { ww = ow + 1; if (ww == L.OW) { ww = 0; if (++hh == L.OH) { hh = 0; ++bb; } } }
             float4 ra = start, rb = start;
+            if (same_row && L.KH == 3 && L.KW == 3 && L.stride == 2)
+            {
+                // two neighbouring 3x3 / stride-2 windows (the ResNet stem's pool): all fifteen inputs are requested
+                // together; clamped where padding puts them outside the image, and then not used
+                const int ih0 = (int)(hh * L.stride) - (int)L.pad, iw0 = (int)(ww * L.stride) - (int)L.pad;
+                float4 x[3][5];
+                #pragma unroll
+                for (int kh = 0; kh < 3; kh++)
+                {
+                    const uint32_t row = (bb * L.IH + (uint32_t)min (max (ih0 + kh, 0), (int)L.IH - 1)) * L.IW;
+                    #pragma unroll
+                    for (int q = 0; q < 5; q++) x[kh][q] = in.ld4 ((row + (uint32_t)min (max (iw0 + q, 0), (int)L.IW - 1)) * L.ld0 + m);
+                }
+                #pragma unroll
+                for (int kh = 0; kh < 3; kh++)
+                {
+                    if ((uint32_t)(ih0 + kh) >= L.IH) continue;
+                    #pragma unroll
+                    for (int q = 0; q < 5; q++)
+                    {
+                        if ((uint32_t)(iw0 + q) >= L.IW) continue;
+                        if (q < 3) combine (ra, x[kh][q]);
+                        if (q >= 2) combine (rb, x[kh][q]);
+                    }
+                }
+                finish (ra, nn, m);
+                finish (rb, nn + 1, m);
+                continue;
+            }
             for (uint32_t kh = 0; kh < L.KH; kh++)
             {
                 const int ih = (int)(hh * L.stride + kh) - (int)L.pad;
