@@ -1276,9 +1276,11 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
         if (fit < 1) ordered = false;
         else
         {
-            // by default two per compute unit with the prefetch buffers (one tile computes, the next is prepared), three
-            // without (YOLO-v3 batch 1: 1.30 / 1.25 / 1.26 ms with two / three / four)
-            if (workgroups_requested == 0) workgroups = small_lds && fit > 3 * g_num_cu ? 3u * (uint32_t)g_num_cu : (uint32_t)fit;
+            // by default two per compute unit (one tile computes, the next is prepared); without the prefetch buffers three
+            // from an estimated parallelism of 350 and four from 600 on (YOLO-v3 batch 1, 409: 1.30 / 1.25 / 1.26 ms with
+            // two / three / four; ResNet-50 batch 4, 335: 0.72 / 0.76 / 0.76; VGG-16 batch 4, 766: 1.51 / 1.40 / 1.34)
+            const uint32_t per_cu = !small_lds || g->parallelism < 350.0 ? 2u : g->parallelism < 600.0 ? 3u : 4u;
+            if (workgroups_requested == 0) workgroups = per_cu * (uint32_t)g_num_cu < (uint32_t)fit ? per_cu * (uint32_t)g_num_cu : (uint32_t)fit;
             if (workgroups > (uint32_t)fit) workgroups = (uint32_t)fit;
         }
     }
