@@ -597,12 +597,14 @@ static const void *const dataflow_kernels[NUM_KERNEL_VARIANTS][2] = {
     {(const void *)dataflow_kernel<1, TILES_CONVNET | TILES_YOLO>, (const void *)dataflow_kernel<2, TILES_CONVNET | TILES_YOLO>},
     {(const void *)dataflow_kernel<1, TILES_ALL>, (const void *)dataflow_kernel<2, TILES_ALL>}};
 
-// Ordered mode (see aspen_hip_run_dataflow), cached loads only: for convolutional networks, and with every tile kind.
-#define NUM_ORDERED_VARIANTS 2
+// Ordered mode (see aspen_hip_run_dataflow), cached loads only: for convolutional networks, for those with weight-streaming
+// layers (VGG-16 at small batches), and with every tile kind.
+#define NUM_ORDERED_VARIANTS 3
 #define ORDERED_SMEM_BYTES CMAX (GEMM_SMEM_BYTES, NARROW_PF_SMEM_BYTES)       // the narrow tiles' weight prefetch buffers
-static const unsigned ordered_variant_tiles[NUM_ORDERED_VARIANTS] = {TILES_CONVNET | TILES_YOLO | TILES_NARROW, TILES_ALL};
+static const unsigned ordered_variant_tiles[NUM_ORDERED_VARIANTS] = {TILES_CONVNET | TILES_YOLO | TILES_NARROW, TILES_CONVNET | TILES_TALL, TILES_ALL};
 static const void *const ordered_kernels[NUM_ORDERED_VARIANTS] = {
-    (const void *)dataflow_kernel<2, TILES_CONVNET | TILES_YOLO | TILES_NARROW, true>, (const void *)dataflow_kernel<2, TILES_ALL, true>};
+    (const void *)dataflow_kernel<2, TILES_CONVNET | TILES_YOLO | TILES_NARROW, true>, (const void *)dataflow_kernel<2, TILES_CONVNET | TILES_TALL, true>,
+    (const void *)dataflow_kernel<2, TILES_ALL, true>};
 
 // The tile kinds a graph contains, as TILES_* bits.
 static unsigned graph_features (const aspen_hip_layer_t *layers, uint32_t num_layers)
@@ -1265,11 +1267,15 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
         const int small_lds = (g->features & TILES_NARROW) == 0;
         if (fits[small_lds] < 0)
         {
-            int o0 = 0, o1 = 0;
+            int least = 1 << 30;
             const size_t smem = small_lds ? GEMM_SMEM_BYTES : ORDERED_SMEM_BYTES;
-            CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&o0, ordered_kernels[0], WG_THREADS, smem));
-            CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&o1, ordered_kernels[1], WG_THREADS, smem));
-            fits[small_lds] = (o0 < o1 ? o0 : o1) * g_num_cu;
+            for (int v = 0; v < NUM_ORDERED_VARIANTS; v++)
+            {
+                int o = 0;
+                CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&o, ordered_kernels[v], WG_THREADS, smem));
+                if (o < least) least = o;
+            }
+            fits[small_lds] = least * g_num_cu;
         }
         const int fit = fits[small_lds];
         ordered_smem = small_lds ? GEMM_SMEM_BYTES : ORDERED_SMEM_BYTES;
@@ -1339,7 +1345,7 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
             g->num_ninst, g->num_roots, g->d_state, g->epoch, g->queue_row, nq_mask, nq_shift, g->d_arrivals, ordered ? g->dep_stride : 0u);
         CHECK (hipGetLastError ());
     }
-    if (ordered) g->spread_armed = 1;
+    g->spread_armed = ordered ? 1 : 0;          // (a run on the ready queue leaves the shared counters at their final values)
     dataflow_args_t a;
     a.layers = g->d_layers; a.ninst_layer = g->d_ninst_layer; a.ninst_home = g->d_ninst_home; a.child_off = g->d_child_off; a.child_idx = g->d_child_idx; a.child_rec = g->d_child_rec;
     a.num_parents = g->d_num_parents;
@@ -1357,7 +1363,12 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
     CHECK (hipEventRecord (g_events[NUM_EVENTS - 2], g_stream));
     {
         const void *kernel = dataflow_kernels[g->variant][g->cached_loads ? 1 : 0];
-        if (ordered) kernel = ordered_kernels[(g->features & ~ordered_variant_tiles[0]) == 0 ? 0 : 1];
+        if (ordered)
+        {
+            int v = 0;
+            while (v + 1 < NUM_ORDERED_VARIANTS && (g->features & ~ordered_variant_tiles[v]) != 0) v++;
+            kernel = ordered_kernels[v];
+        }
         g->last_run_ordered = ordered;
         void *kernel_args[] = {&a};
         CHECK (hipLaunchKernel (kernel, dim3 (workgroups), dim3 (WG_THREADS), kernel_args, ordered ? ordered_smem : GEMM_SMEM_BYTES, g_stream));

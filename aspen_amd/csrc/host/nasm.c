@@ -643,7 +643,6 @@ static double nasm_parallelism (const nasm_t *nasm)
 #define CHAIN_BOUND_CAP_FROM 400.0
 #define CHAIN_BOUND_KITERS_CAP 48
 #define LATENCY_BOUND_BELOW 128.0
-#define ORDERED_TALL_BELOW 300.0
 static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned int batch, unsigned int seq)
 {
     const char *e = getenv ("ASPEN_GPU_MAX_KITERS");            /* experiments: fixed cap, 0 = none */
@@ -662,15 +661,11 @@ static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned i
     /* The ordered mode itself pays further up than the 32 x 32 tiles do, for convolutional networks.  Measured against the
        ready queue (ms, ordered / queue): ResNet-50 at batch 1 / 2 / 4 / 8 / 16 (parallelism 95 / 175 / 335 / 593 / 790):
        0.45 / 0.64, 0.62 / 0.74, 0.72 / 0.88, 0.99 / 1.08, 1.47 / 1.62; YOLO-v3 at batch 1 / 2 / 4 (409 / 691 / 942): 1.24 / 1.57,
-       1.71 / 1.94, 2.69 / 2.82.  Graphs that are not rebuilt here (1024 and up) are a tie or lose (YOLO-v3 batch 8, 1271:
-       4.76 / 4.68; ResNet-50 batch 32: 2.56 / 2.39).  A graph with weight-streaming (128 x 32) tiles runs the ordered mode
-       on the kernel built with every tile kind, which is slower: VGG-16 wins at batch 1 (316: 0.58 / 0.62) and loses from
-       batch 2 on (654: 0.90 / 0.84; 766: 1.34 / 1.31), so such graphs keep the old limit.  The transformer graphs lose at
-       every size (their long, uniform tiles want the queue's balancing: BERT-base, 265: 2.9 / 2.2 ms).  Where it matters,
-       apu_generate_nasm times both. */
-    int tall = 0;
-    for (unsigned int l = 0; l < rebuilt->num_ldata; l++) tall |= rebuilt->ldata_arr[l].variant == ASPEN_HIP_GEMM_TALL;
-    if (parallelism < LATENCY_BOUND_BELOW || (seq == 0 && parallelism < (tall ? ORDERED_TALL_BELOW : CHAIN_BOUND_BELOW))) rebuilt->ordered_pref = 1;
+       1.71 / 1.94, 2.69 / 2.82; VGG-16 at batch 1 / 2 / 4 / 8 (583 / 654 / 766 / 884): 0.54 / 0.64, 0.82 / 0.85, 1.24 / 1.31,
+       2.16 / 2.24.  Graphs that are not rebuilt here (1024 and up) are a tie or lose (YOLO-v3 batch 8, 1271: 4.76 / 4.68;
+       ResNet-50 batch 32: 2.56 / 2.39).  The transformer graphs lose at every size (their long, uniform tiles want the
+       queue's balancing: BERT-base, 265: 2.9 / 2.2 ms).  Where it matters, apu_generate_nasm times both. */
+    if (parallelism < LATENCY_BOUND_BELOW || seq == 0) rebuilt->ordered_pref = 1;
     apu_destroy_nasm (nasm);
     return rebuilt;
 }

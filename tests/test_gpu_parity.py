@@ -438,6 +438,27 @@ def test_engine_rearm_many_runs(gpu, engine_flags, flags):
         net.close()
 
 
+def test_ordered_and_queue_runs_alternate_on_one_graph(gpu):
+    """An ordered run leaves its counters armed for the next ordered run; a run on the ready queue in between leaves
+    the counters both engines share at their final values.  The ordered run after it has to arm again: engines
+    alternate on one graph, without per-tile counts (no arming pass of their own), and every run matches the oracle."""
+    from oracle import cpu
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()["resnet_mini_b2"])
+    want = cpu.run_network(layers, tens, x, batch, seq)
+    net = H.GpuNet(cfg, tens, batch, seq, min_ninst=64, mode=api.MODE_DATAFLOW)
+    try:
+        for rep, flags in enumerate((ORDERED, ORDERED, QUEUE, ORDERED, ORDERED, QUEUE, QUEUE, ORDERED)):
+            api.lib().aspen_hip_set_flags(flags)
+            net.run(x if rep == 0 else None)
+            assert net.dse.last_run_ordered() == (flags == ORDERED), rep
+            assert net.rpool.run_stats()["aborted"] == 0, rep
+            for l in range(1, net.nasm.num_ldata):
+                assert H.rel_l2(net.layer(l), want[l]) <= H.REL_L2_TOL, (rep, l)
+    finally:
+        api.lib().aspen_hip_set_flags(0)
+        net.close()
+
+
 def test_queue_entries_of_earlier_runs_are_never_taken(gpu):
     """Which queue slots a run rewrites depends on its flags (hand-off, per-XCD queues) and its grid, and entries carry
     a 16-bit run tag: a slot written under one setting must not be taken for a fresh entry when the tag comes round
