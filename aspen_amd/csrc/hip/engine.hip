@@ -598,13 +598,13 @@ static const void *const dataflow_kernels[NUM_KERNEL_VARIANTS][2] = {
     {(const void *)dataflow_kernel<1, TILES_ALL>, (const void *)dataflow_kernel<2, TILES_ALL>}};
 
 // Ordered mode (see aspen_hip_run_dataflow), cached loads only: for convolutional networks, for those with weight-streaming
-// layers (VGG-16 at small batches), and with every tile kind.
-#define NUM_ORDERED_VARIANTS 3
+// layers (VGG-16 at small batches), for transformer graphs, and with every tile kind.
+#define NUM_ORDERED_VARIANTS 4
 #define ORDERED_SMEM_BYTES CMAX (GEMM_SMEM_BYTES, NARROW_PF_SMEM_BYTES)       // the narrow tiles' weight prefetch buffers
-static const unsigned ordered_variant_tiles[NUM_ORDERED_VARIANTS] = {TILES_CONVNET | TILES_YOLO | TILES_NARROW, TILES_CONVNET | TILES_TALL, TILES_ALL};
+static const unsigned ordered_variant_tiles[NUM_ORDERED_VARIANTS] = {TILES_CONVNET | TILES_YOLO | TILES_NARROW, TILES_CONVNET | TILES_TALL, TILES_TRANSFORMER, TILES_ALL};
 static const void *const ordered_kernels[NUM_ORDERED_VARIANTS] = {
     (const void *)dataflow_kernel<2, TILES_CONVNET | TILES_YOLO | TILES_NARROW, true>, (const void *)dataflow_kernel<2, TILES_CONVNET | TILES_TALL, true>,
-    (const void *)dataflow_kernel<2, TILES_ALL, true>};
+    (const void *)dataflow_kernel<2, TILES_TRANSFORMER, true>, (const void *)dataflow_kernel<2, TILES_ALL, true>};
 
 // The tile kinds a graph contains, as TILES_* bits.
 static unsigned graph_features (const aspen_hip_layer_t *layers, uint32_t num_layers)
@@ -1285,7 +1285,10 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
             // by default two per compute unit (one tile computes, the next is prepared); without the prefetch buffers three
             // from an estimated parallelism of 350 and four from 600 on (YOLO-v3 batch 1, 409: 1.30 / 1.25 / 1.26 ms with
             // two / three / four; ResNet-50 batch 4, 335: 0.72 / 0.76 / 0.76; VGG-16 batch 4, 766: 1.51 / 1.40 / 1.34)
-            const uint32_t per_cu = !small_lds || g->parallelism < 350.0 ? 2u : g->parallelism < 600.0 ? 3u : 4u;
+            // (transformer graphs, whose kernel fits three times: two below 600; BERT-base 8 x 128, 519: 1.96 / 2.00 ms with
+            // two / three, 16 x 128, 1024: 3.49 / 3.33)
+            const double three_from = (g->features & TILES_ATTENTION) ? 600.0 : 350.0;
+            const uint32_t per_cu = !small_lds || g->parallelism < three_from ? 2u : g->parallelism < 600.0 ? 3u : 4u;
             if (workgroups_requested == 0) workgroups = per_cu * (uint32_t)g_num_cu < (uint32_t)fit ? per_cu * (uint32_t)g_num_cu : (uint32_t)fit;
             if (workgroups > (uint32_t)fit) workgroups = (uint32_t)fit;
         }

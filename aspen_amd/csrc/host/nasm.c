@@ -637,11 +637,13 @@ static double nasm_parallelism (const nasm_t *nasm)
      better than few long ones (the FFN layers of BERT as 768 tiles instead of 384: GPT-2 -2 %, BERT -0.5 %);
    - if it still offers work for a second workgroup per compute unit, with no tile longer than 48 K slices (more
      split-K): GPT-2 (average parallelism 529) -6 %.  With a single workgroup per compute unit the extra tiles only
-     queue up behind the others: BERT (265) is 2 % faster without the cap.
+     queue up behind the others: BERT (265) is 2 % faster without the cap on the ready queue (in the ordered mode, which
+     such transformer graphs now run, a cap of 24 pays: see create_nasm).
    Throughput-bound graphs (batch-32 vision nets) lose 2-3 % with either and keep their large, long tiles. */
 #define CHAIN_BOUND_BELOW 1024.0
 #define CHAIN_BOUND_CAP_FROM 400.0
 #define CHAIN_BOUND_KITERS_CAP 48
+#define ORDERED_KITERS_CAP 24
 #define LATENCY_BOUND_BELOW 128.0
 static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned int batch, unsigned int seq)
 {
@@ -656,16 +658,21 @@ static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned i
        mode): layers short of tiles take the 32 x 32 shape */
     const char *nt = getenv ("ASPEN_GPU_NARROW_TILES");
     const int narrow = nt != NULL ? atoi (nt) != 0 : parallelism < LATENCY_BOUND_BELOW;
-    nasm_t *rebuilt = build_nasm (dnn, min_ninst, batch, seq, parallelism >= CHAIN_BOUND_CAP_FROM ? CHAIN_BOUND_KITERS_CAP : 0, 1, narrow);
+    /* transformer graphs below the cap's limit run the ordered mode (below), where shorter tiles do pay: no tile longer
+       than 24 K slices, i.e. the second FFN layer of a BERT-base block in four parts */
+    const int tr_ordered = seq > 0 && parallelism < CHAIN_BOUND_CAP_FROM;
+    nasm_t *rebuilt = build_nasm (dnn, min_ninst, batch, seq, parallelism >= CHAIN_BOUND_CAP_FROM ? CHAIN_BOUND_KITERS_CAP : tr_ordered ? ORDERED_KITERS_CAP : 0, 1, narrow);
     if (rebuilt == NULL) return nasm;
     /* The ordered mode itself pays further up than the 32 x 32 tiles do, for convolutional networks.  Measured against the
        ready queue (ms, ordered / queue): ResNet-50 at batch 1 / 2 / 4 / 8 / 16 (parallelism 95 / 175 / 335 / 593 / 790):
        0.45 / 0.64, 0.62 / 0.74, 0.72 / 0.88, 0.99 / 1.08, 1.47 / 1.62; YOLO-v3 at batch 1 / 2 / 4 (409 / 691 / 942): 1.24 / 1.57,
        1.71 / 1.94, 2.69 / 2.82; VGG-16 at batch 1 / 2 / 4 / 8 (583 / 654 / 766 / 884): 0.54 / 0.64, 0.82 / 0.85, 1.24 / 1.31,
        2.16 / 2.24.  Graphs that are not rebuilt here (1024 and up) are a tie or lose (YOLO-v3 batch 8, 1271: 4.76 / 4.68;
-       ResNet-50 batch 32: 2.56 / 2.39).  The transformer graphs lose at every size (their long, uniform tiles want the
-       queue's balancing: BERT-base, 265: 2.9 / 2.2 ms).  Where it matters, apu_generate_nasm times both. */
-    if (parallelism < LATENCY_BOUND_BELOW || seq == 0) rebuilt->ordered_pref = 1;
+       ResNet-50 batch 32: 2.56 / 2.39).  Transformer graphs win with it below 400, together with the cap of 24 K slices
+       (BERT-base, batch x tokens 8 x 128 / 4 x 128 / 8 x 64 / 2 x 384: 2.00 / 2.15, 1.38 / 1.46, 1.34 / 1.39, 1.90 / 2.08;
+       GPT-2 1 x 512 / 2 x 256 / 8 x 128: 1.59 / 1.65, 1.43 / 1.50, 2.01 / 2.10) and tie above (GPT-2 4 x 512, 529: 3.54 / 3.52;
+       BERT-base 16 x 128: 3.33 / 3.38), where they keep the queue.  Where it matters, apu_generate_nasm times both. */
+    if (parallelism < LATENCY_BOUND_BELOW || seq == 0 || tr_ordered) rebuilt->ordered_pref = 1;
     apu_destroy_nasm (nasm);
     return rebuilt;
 }
