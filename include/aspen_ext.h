@@ -31,7 +31,8 @@ int aspen_dse_group_last_mode (dse_group_t *dse_group);
 int aspen_dse_group_last_run_ordered (dse_group_t *dse_group);
 /* Whether runs of this nasm on the persistent kernel use its ordered mode (no ready queue; tiles assigned to workgroups in
    index order and prepared before their parents have finished): 1 / 0, -1 = the engine decides.  apu_create_nasm asks
-   for it on graphs bound by latency (a single image, small batches of convolutional networks), apu_generate_nasm times
+   for it on graphs bound by their dependency chains (convolutional networks at small and medium batches, transformers
+   with up to about a thousand tokens), apu_generate_nasm times
    it against the other engines; a pool runs ordered when all its nasms ask for it. */
 void aspen_nasm_set_ordered (nasm_t *nasm, int ordered);
 /* Watchdog of the persistent kernel: polls a workgroup may spend waiting for one ready tile before the
