@@ -25,9 +25,9 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the persistent kernel, measured with rocprofv3 FETCH_SIZE / WRITE_SIZE passes
 # calibrated on the library's copy kernel (summaries: profiles/dataflow_kernel_resnet50_b32_hbm_traffic.txt and
 # profiles/dataflow_kernel_vgg16_co_inference_bert_gpt2_kernel_stats_hbm_traffic.txt); valid for these tuned configurations only
-MEASURED_TRAFFIC_BYTES = {("resnet50_b32", "dataflow", 1536): 8.77e9, ("vgg16_b32", "dataflow", 1536): 17.10e9,
-                          ("co_resnet50_vgg16_b16", "dataflow", 1536): 15.05e9, ("bert_base_b8_s128", "dataflow", 192): 7.53e9,
-                          ("gpt2_b4_s512", "dataflow", 384): 16.61e9, ("resnet50_b1", "dataflow", 256): 0.415e9}
+MEASURED_TRAFFIC_BYTES = {("resnet50_b32", "dataflow", 1536): 8.68e9, ("vgg16_b32", "dataflow", 1536): 17.36e9,
+                          ("co_resnet50_vgg16_b16", "dataflow", 1536): 15.00e9, ("bert_base_b8_s128", "dataflow", 192): 2.94e9,
+                          ("gpt2_b4_s512", "dataflow", 384): 15.72e9, ("resnet50_b1", "dataflow", 256): 0.414e9}
 
 # algorithmic GEMM-class flops per unit (2*M*N*K with the reference's K: padding taps counted, full
 # S x S attention): per image for the vision nets, per token for the transformers
