@@ -670,9 +670,12 @@ static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned i
        2.16 / 2.24.  Graphs that are not rebuilt here (1024 and up) are a tie or lose (YOLO-v3 batch 8, 1271: 4.76 / 4.68;
        ResNet-50 batch 32: 2.56 / 2.39).  Transformer graphs win with it below 400, together with the cap of 24 K slices
        (BERT-base, batch x tokens 8 x 128 / 4 x 128 / 8 x 64 / 2 x 384: 2.00 / 2.15, 1.38 / 1.46, 1.34 / 1.39, 1.90 / 2.08;
-       GPT-2 1 x 512 / 2 x 256 / 8 x 128: 1.59 / 1.65, 1.43 / 1.50, 2.01 / 2.10) and tie above (GPT-2 4 x 512, 529: 3.54 / 3.52;
-       BERT-base 16 x 128: 3.33 / 3.38), where they keep the queue.  Where it matters, apu_generate_nasm times both. */
-    if (parallelism < LATENCY_BOUND_BELOW || seq == 0 || tr_ordered) rebuilt->ordered_pref = 1;
+       GPT-2 1 x 512 / 2 x 256 / 8 x 128: 1.59 / 1.65, 1.43 / 1.50, 2.01 / 2.10); above, the times are within a percent or two
+       of each other either way (GPT-2 4 x 512, 529: 3.56 / 3.60 on one box, 3.57 / 3.52 on another; BERT-base 16 x 128:
+       3.34 / 3.38), and the ordered mode moves far less data: a tile's workgroup, and with it the XCD whose L2 its operands
+       pass through, is fixed by the tile's index, so every XCD keeps to an eighth of a layer's weight rows.  So every
+       rebuilt graph asks for the ordered mode.  Where it matters, apu_generate_nasm times both. */
+    rebuilt->ordered_pref = 1;
     apu_destroy_nasm (nasm);
     return rebuilt;
 }
