@@ -198,9 +198,9 @@ class Nasm:
         a = (C.c_uint * 20)()
         lib().aspen_nasm_ldata_info(self.h, l, a)
         keys = ["type", "act", "H", "W", "stride", "num_ninst", "tile_H", "tile_W", "p0", "p1", "ninst_start", "variant",
-                "fused_into", "fused_residual", "splits", "tiles_H", "kiters_per_split", "discarded", "fused_attention"]
+                "fused_into", "fused_residual", "splits", "tiles_H", "kiters_per_split", "discarded", "fused_attention", "folded_norm"]
         d = dict(zip(keys, [int(v) for v in a]))
-        for k in ("fused_into", "fused_residual", "fused_attention"):
+        for k in ("fused_into", "fused_residual", "fused_attention", "folded_norm"):
             d[k] = -1 if d[k] == 0xffffffff else d[k]
         d["flops"] = int(lib().aspen_nasm_ldata_flops(self.h, l))
         return d

@@ -934,6 +934,7 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
         else if (L.direct != ASPEN_HIP_OPERAND_DIRECT && !L.ktab) why = "missing k-chunk table";
         else if (L.fuse_out && (!L.fuse_in || L.fuse_ld_in % 4 || L.fuse_ld_in < L.M)) why = "fused shortcut operand";
         else if (L.direct == ASPEN_HIP_OPERAND_DIRECT && (L.ld0 < L.Kp)) why = "direct operand shorter than Kp";
+        else if (L.norm_fold && (L.type != MATMUL_LAYER || L.direct != ASPEN_HIP_OPERAND_DIRECT || L.variant != ASPEN_HIP_GEMM_SMALL || L.splits > 1 || !L.in1 || L.K % GEMM_BK)) why = "a folded layer norm needs a direct operand, 64 x 64 tiles and an uncut K axis";
         else if (L.direct == ASPEN_HIP_OPERAND_DENSE3 && (L.IC != 3 || L.Kp > 512 || L.Kp < 3 * L.KH * L.KW || L.ld0 < 4 || bm != 64)) why = "dense three-channel operand";
         else if (L.direct < 0 || L.direct > ASPEN_HIP_OPERAND_DENSE3) why = "operand kind";
         else if (L.direct == ASPEN_HIP_OPERAND_TABLE && L.IC % GEMM_BK != 0 && L.variant != ASPEN_HIP_GEMM_SMALL) why = "a K axis that needs the k-chunk table takes 64 x 64 tiles";

@@ -661,10 +661,58 @@ __device__ __forceinline__ void gemm_core (ALoader &al, BLoader &bl, int kbase, 
 // Mij = MFMA on K pair j of sub-step i; X = barrier "everyone holds this slice's fragments", wA / wB = next
 // slice registers -> LDS, gA / gB = requests for the slice DEPTH ahead, Y = barrier "refill visible",
 // ri = fragments of sub-step i of the next slice (its buffer was released by Mi3).
-template <int DEPTH, class ALoader, class BLoader, class Hook = NoHook, class Ready = NoHook>
-__device__ __forceinline__ void gemm_core_single_block (ALoader &al, BLoader &bl, int kbase, int kiters, float *smem,
-    floatx16 (&accs)[1][1], bool phases = false, Hook before_last_slice = Hook (), Ready ready = Ready ())
+// Accumulator register v of MFMA block (i, j) holds output (row n, channel m):
+//   n = wn0 + 32 i + 8 (v / 4) + 4 (lane / 32) + v % 4,   m = wm0 + 32 j + lane % 32
+#define ACC_N(wn0, i, v, lane) ((wn0) + 32 * (i) + 8 * ((v) >> 2) + 4 * ((lane) >> 5) + ((v) & 3))
+
+struct NoStats { __device__ __forceinline__ void operator() (const float4 (&)[2]) const {} };
+
+// A layer norm folded into a matmul tile (aspen_hip_layer_t.norm_fold), second half: the K loop has left every thread
+// the sum and the sum of squares of its eight-th of two columns' K axis (thread t: columns t / 8 and t / 8 + 32, the
+// ActRowLoader's assignment).  The eight threads of a column add up, one of them writes the column's mean and
+// 1 / sqrt (variance + eps) behind the stage in LDS, and every lane corrects its sixteen sums:
+// acc = rstd[n] * (acc - mean[n] * rowsum[m]).  Same arithmetic for mean and variance as tile_layernorm.
+#define NORM_FOLD_STATS_OFFSET (128 * LDS_ROW)      // floats: behind the two operand blocks of the stage
+__device__ __forceinline__ void norm_fold_finish (const aspen_hip_layer_t &L, floatx16 &acc, float (&cs)[2], float (&cq)[2], float *smem,
+    uint32_t tid, uint32_t m0, uint32_t wm0, uint32_t wn0)
 {
+    const uint32_t lane = tid & 63;
+    #pragma unroll
+    for (int o = 1; o < 8; o <<= 1)
+    {
+        #pragma unroll
+        for (int i = 0; i < 2; i++) { cs[i] += __shfl_xor (cs[i], o, 64); cq[i] += __shfl_xor (cq[i], o, 64); }
+    }
+    float *st = smem + NORM_FOLD_STATS_OFFSET;
+    if ((tid & 7u) == 0)
+    {
+        #pragma unroll
+        for (int i = 0; i < 2; i++)
+        {
+            const float mean = cs[i] / (float)L.K;
+            const float var = cq[i] / (float)L.K - mean * mean;
+            const uint32_t n = (tid >> 3) + 32 * i;
+            st[2 * n] = mean; st[2 * n + 1] = 1.0f / sqrtf (var + 1e-6f);
+        }
+    }
+    // (the row sums are weights: requested before the barrier)
+    const uint32_t m = min (m0 + wm0 + (lane & 31), L.M - 1);
+    const float rs = gld1 (L.in1 + m);
+    lds_barrier ();
+    #pragma unroll
+    for (int v = 0; v < 16; v++)
+    {
+        const uint32_t n = ACC_N (wn0, 0, v, lane);
+        acc[v] = st[2 * n + 1] * (acc[v] - st[2 * n] * rs);
+    }
+}
+
+template <int DEPTH, class ALoader, class BLoader, class Hook = NoHook, class Ready = NoHook, class Stats = NoStats>
+__device__ __forceinline__ void gemm_core_single_block (ALoader &al, BLoader &bl, int kbase, int kiters, float *smem,
+    floatx16 (&accs)[1][1], bool phases = false, Hook before_last_slice = Hook (), Ready ready = Ready (), Stats stats = Stats ())
+{
+    // `stats` sees every K slice of the activation operand once, as the registers it passes through on its way into LDS
+    // (a folded layer norm's column sums, see norm_fold_finish)
     static_assert (DEPTH == 1 || DEPTH == 2, "one or two register sets");
     static_assert (ALoader::R == 2 && BLoader::R == 2 && GEMM_BK == 32, "64 x 64 tile, four sub-steps");
     constexpr int BM = 64;
@@ -683,7 +731,7 @@ __device__ __forceinline__ void gemm_core_single_block (ALoader &al, BLoader &bl
     float4 areg[DEPTH][2], breg[DEPTH][2];
     al.load (kbase, areg[0]); ready (); bl.load (kbase, breg[0]);
     if (DEPTH == 2 && kiters > 1) { al.load (kbase + 1, areg[DEPTH - 1]); bl.load (kbase + 1, breg[DEPTH - 1]); }
-    al.store (smem, areg[0]); bl.store (smem + BM * LDS_ROW, breg[0]);
+    al.store (smem, areg[0]); bl.store (smem + BM * LDS_ROW, breg[0]); stats (breg[0]);
     if (kiters > DEPTH) { al.load (kbase + DEPTH, areg[0]); bl.load (kbase + DEPTH, breg[0]); }
     lds_barrier ();
     if (phases) tile_phase_lap (8);
@@ -698,7 +746,7 @@ __device__ __forceinline__ void gemm_core_single_block (ALoader &al, BLoader &bl
         SB; MF (0, x); MF (0, y); MF (0, z);
         lds_barrier (); SB;
         MF (0, w); al.store (smem, areg[set]); SB;
-        MF (1, x); bl.store (smem + BM * LDS_ROW, breg[set]); SB;
+        MF (1, x); bl.store (smem + BM * LDS_ROW, breg[set]); stats (breg[set]); SB;
         MF (1, y); if (DEPTH == 2 || it + 2 < kiters) al.load (nxt, areg[set]); SB;
         MF (1, z); if (DEPTH == 2 || it + 2 < kiters) bl.load (nxt, breg[set]); SB;
         MF (1, w); MF (2, x);
@@ -728,9 +776,6 @@ __device__ __forceinline__ void gemm_core_single_block (ALoader &al, BLoader &bl
     lds_barrier ();          // the caller reuses the stage (epilogue)
 }
 
-// Accumulator register v of MFMA block (i, j) holds output (row n, channel m):
-//   n = wn0 + 32 i + 8 (v / 4) + 4 (lane / 32) + v % 4,   m = wm0 + 32 j + lane % 32
-#define ACC_N(wn0, i, v, lane) ((wn0) + 32 * (i) + 8 * ((v) >> 2) + 4 * ((lane) >> 5) + ((v) & 3))
 
 // Shortcut fused into a contraction epilogue: fuse_out = fuse_act (v + fuse_in) for the (up to) four
 // channels m .. m+3 of column n; `left` = channels of the matrix from m on.  Same arithmetic, in the same
@@ -809,7 +854,24 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
     {
         ActRowLoader<BN, COH> bl;
         bl.init (in, n0, L.N - 1, L.ld0, 0, tid);
-        if constexpr (SINGLE) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
+        if constexpr (SINGLE && (FEAT & TILES_NORM) != 0)
+        {
+            // (kernels for transformer graphs: the column sums a folded layer norm needs are gathered in every such tile,
+            // sixteen additions and multiplications per K slice, and used where the layer asks for them)
+            float cs[2] = {0.f, 0.f}, cq[2] = {0.f, 0.f};
+            auto stats = [&] (const float4 (&b)[2])
+            {
+                #pragma unroll
+                for (int i = 0; i < 2; i++)
+                {
+                    cs[i] += (b[i].x + b[i].y) + (b[i].z + b[i].w);
+                    cq[i] += (b[i].x * b[i].x + b[i].y * b[i].y) + (b[i].z * b[i].z + b[i].w * b[i].w);
+                }
+            };
+            gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready, stats);
+            if (L.norm_fold) norm_fold_finish (L, acc[0][0], cs, cq, smem, tid, m0, (wave % 2) * 32, (wave / 2) * 32);
+        }
+        else if constexpr (SINGLE) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
         else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
     }
     else if constexpr ((FEAT & TILES_GATHER) != 0)

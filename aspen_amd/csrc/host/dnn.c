@@ -139,7 +139,18 @@ static void invalidate_device (aspen_layer_t *L)
     /* device graphs that were built from these buffers must not run again as they are */
     if ((L->d_weight || L->d_bias || L->d_ktab) && L->dnn != NULL) L->dnn->dev_generation++;
     aspen_hip_free (L->d_weight); aspen_hip_free (L->d_bias); aspen_hip_free (L->d_ktab);
+    aspen_hip_free (L->d_weight_ln); aspen_hip_free (L->d_bias_ln); aspen_hip_free (L->d_rowsum_ln);
     L->d_weight = NULL; L->d_bias = NULL; L->d_ktab = NULL;
+    L->d_weight_ln = NULL; L->d_bias_ln = NULL; L->d_rowsum_ln = NULL;
+    /* (a layer norm's parameters are part of what the matmul layers behind it hold folded in) */
+    if (L->type == LAYERNORM_LAYER && L->dnn != NULL)
+        for (unsigned int i = 0; i < L->dnn->num_layers; i++)
+        {
+            aspen_layer_t *C = &L->dnn->layers[i];
+            if (C->type != MATMUL_LAYER || C->parent_idx[PARENT_0] != (int)L->layer_idx || C->d_weight_ln == NULL) continue;
+            aspen_hip_free (C->d_weight_ln); aspen_hip_free (C->d_bias_ln); aspen_hip_free (C->d_rowsum_ln);
+            C->d_weight_ln = NULL; C->d_bias_ln = NULL; C->d_rowsum_ln = NULL;
+        }
 }
 
 int aspen_load_weight_file (aspen_dnn_t *dnn, const char *path)
@@ -415,5 +426,46 @@ int aspen_layer_to_device (aspen_layer_t *L, unsigned int parent_ld)
     rc = L->d_ktab ? aspen_hip_h2d (L->d_ktab, tab, kp / 4 * sizeof (aspen_hip_ktab_t)) : -1;
     free (tab);
     L->dev_kp = kp; L->dev_icp = icp; L->dev_in_ld = parent_ld;
+    return rc;
+}
+
+/* The device buffers of a matmul layer L that absorbs the layer norm `norm` in front of it (y = W LN (x) + b with
+   LN (x) = (x - mean) * rstd * gamma + beta, reference tiled_layernorm, src/tiled_kernels.c:743-782):
+     y[m] = rstd * (sum_k W[m][k] gamma[k] x[k]  -  mean * sum_k W[m][k] gamma[k])  +  (b[m] + sum_k W[m][k] beta[k]),
+   i.e. the product of the scaled weights with the RAW column, corrected with the column's statistics and the scaled
+   weights' row sums.  Sums in double.  Idempotent; dropped with the layer's other device buffers. */
+int aspen_layer_norm_fold_to_device (aspen_layer_t *L, const aspen_layer_t *norm)
+{
+    if (L->d_weight_ln != NULL) return 0;
+    if (L->type != MATMUL_LAYER || norm->type != LAYERNORM_LAYER || L->weight.data == NULL || norm->weight.data == NULL
+        || norm->gemm_m != L->gemm_k) return -1;
+    const unsigned int M = L->gemm_m, K = L->gemm_k, kp = round_up (K, 32), mp = round_up (M, 128);
+    float *staged = calloc ((size_t)mp * kp, sizeof (float)), *bias = calloc (M, sizeof (float)), *rowsum = calloc (M, sizeof (float));
+    int rc = -1;
+    if (staged != NULL && bias != NULL && rowsum != NULL)
+    {
+        const float *gamma = norm->weight.data, *beta = norm->bias.data;
+        for (unsigned int m = 0; m < M; m++)
+        {
+            const float *w = L->weight.data + (size_t)m * K;
+            double rs = 0.0, sh = 0.0;
+            for (unsigned int k = 0; k < K; k++)
+            {
+                const float scaled = w[k] * gamma[k];
+                staged[(size_t)m * kp + k] = scaled;
+                rs += (double)scaled;
+                if (beta != NULL) sh += (double)w[k] * (double)beta[k];
+            }
+            rowsum[m] = (float)rs;
+            bias[m] = (float)((L->bias.data != NULL ? (double)L->bias.data[m] : 0.0) + sh);
+        }
+        L->d_weight_ln = aspen_hip_alloc ((size_t)mp * kp * sizeof (float));
+        L->d_bias_ln = aspen_hip_alloc (M * sizeof (float));
+        L->d_rowsum_ln = aspen_hip_alloc (M * sizeof (float));
+        if (L->d_weight_ln && L->d_bias_ln && L->d_rowsum_ln)
+            rc = aspen_hip_h2d (L->d_weight_ln, staged, (size_t)mp * kp * sizeof (float))
+                || aspen_hip_h2d (L->d_bias_ln, bias, M * sizeof (float)) || aspen_hip_h2d (L->d_rowsum_ln, rowsum, M * sizeof (float));
+    }
+    free (staged); free (bias); free (rowsum);
     return rc;
 }

@@ -48,7 +48,7 @@ void aspen_nasm_ldata_info (nasm_t *n, unsigned int l, unsigned int *info)
     info[10] = ld->ninst_start; info[11] = (unsigned int)ld->variant;
     info[12] = (unsigned int)ld->fused_into; info[13] = (unsigned int)ld->fused_residual;
     info[14] = ld->splits; info[15] = ld->tiles_h; info[16] = ld->kiters_per_split;
-    info[17] = (unsigned int)ld->out_discarded; info[18] = (unsigned int)ld->fused_attention; info[19] = 0;
+    info[17] = (unsigned int)ld->out_discarded; info[18] = (unsigned int)ld->fused_attention; info[19] = (unsigned int)ld->folded_norm;
 }
 
 void aspen_nasm_graph (nasm_t *n, const uint32_t **ninst_ldata, const uint32_t **num_parents,

@@ -41,6 +41,10 @@ struct aspen_layer_t
     /* device copies, created on first use */
     float *d_weight, *d_bias;
     aspen_hip_ktab_t *d_ktab;
+    /* matmul layers whose parent is a layer norm that the engine folds into them (see fold_layernorms in nasm.c):
+       weights with the norm's scale multiplied into their K axis, bias plus the weights applied to the norm's shift,
+       and the row sums of the scaled weights */
+    float *d_weight_ln, *d_bias_ln, *d_rowsum_ln;
     unsigned int dev_kp, dev_icp, dev_in_ld;  /* padded K, padded channels per tap, parent stride assumed */
 };
 
@@ -83,6 +87,10 @@ struct nasm_ldata_t
        weighted values in one tile (the S x S probabilities stay on chip); the K-attention layer then owns no tiles and
        its matrix is not written.  -1 = not fused */
     int fused_attention;                     /* V-attention layer: index of the K-attention layer it absorbs */
+    /* layer-norm folding: the matmul layers behind a layer norm that nothing else reads take the norm's INPUT and
+       normalise it themselves (column statistics gathered in their K loops); the norm then owns no tiles and its matrix
+       is not written.  -1 = not folded */
+    int folded_norm;                         /* matmul layer: index of the layer norm it absorbs */
     uint64_t flops;                          /* 2*M*N*K for contraction layers, 64-bit */
 };
 
@@ -143,6 +151,7 @@ int aspen_layer_validate (aspen_dnn_t *dnn, aspen_layer_t *layer);
 /* dnn.c */
 int aspen_layer_to_device (aspen_layer_t *layer, unsigned int parent_ld);
 int aspen_load_weight_file (aspen_dnn_t *dnn, const char *path);
+int aspen_layer_norm_fold_to_device (aspen_layer_t *L, const aspen_layer_t *norm);
 int aspen_layer_dense3 (const aspen_layer_t *layer);            /* three input channels: dense K axis on the device */
 int aspen_layer_table_operand (const aspen_layer_t *layer);     /* K axis through the k-chunk table: 64 x 64 tiles only */
 int aspen_layer_block_major_k (const aspen_layer_t *layer);     /* device K order (channel block, tap, channel in block) */

@@ -93,6 +93,13 @@ typedef struct aspen_hip_layer_t
        the bias, activates and writes the output; only it releases the group's children */
     uint32_t splits, kiters_per_split;
     uint32_t fuse_discard;   /* 1 (only with fuse_out): the layer's own, pre-shortcut matrix `out` is not written */
+    /* 1 (matmul layers with a DIRECT operand, 64 x 64 tiles, K axis not cut, K a multiple of 32): a layer norm over the
+       K axis of the operand is folded into the layer (reference tiled_layernorm, src/tiled_kernels.c:743-782, eps 1e-6):
+       in0 is the norm's INPUT, `weight` holds W[m][k] * gamma[k], `bias` b[m] + sum_k W[m][k] * beta[k], in1 the row sums
+       of `weight` ([M]); a tile gathers sum and sum of squares of its columns in its K loop and computes
+       out = act (rstd[n] * (acc[m][n] - mean[n] * in1[m]) + bias[m]) */
+    uint32_t norm_fold;
+    uint32_t reserved0;
     uint32_t graph_id;       /* which of the co-scheduled networks of one engine run the layer belongs to (0 .. 63): the run
                                 reports each network's completion separately, see aspen_hip_graph_group_done */
     float *partial;

@@ -348,6 +348,45 @@ def test_fused_attention_matches_oracle(gpu, engine_flags, name, mode, flags):
         api.lib().aspen_keep_layer_outputs(1)
 
 
+@pytest.mark.parametrize("mode,flags", [(api.MODE_LAYERS, QUEUE), (api.MODE_DATAFLOW, QUEUE), (api.MODE_DATAFLOW, ORDERED)], ids=["layers", "dataflow", "dataflow-ordered"])
+@pytest.mark.parametrize("name", ["bert_mini_b2_s24", "gpt_mini_b2_s20"])
+def test_folded_layernorm_matches_oracle(gpu, engine_flags, monkeypatch, name, mode, flags):
+    """The default setting (layer outputs not kept): the matmul layers behind a layer norm that nothing else reads take
+    the norm's input and normalise it themselves (column sums gathered in the K loop, weights with the norm's scale
+    folded in): y = rstd * (W' x - mean * rowsum (W')) + b' must match W LN (x) + b (reference tiled_layernorm,
+    src/tiled_kernels.c:743-782, then matmul) to the tolerance of every other layer.  GPT-2's norms are folded and lose
+    their tiles; BERT's, which the block's shortcut reads as well, stay as they are.  Every layer that is written matches
+    the oracle, on a re-armed graph with a second input as well."""
+    from oracle import cpu
+    engine_flags(flags)
+    monkeypatch.setenv("ASPEN_GPU_NARROW_TILES", "0")        # graphs this small would take 32 x 32 tiles, which do not fold
+    cfg, layers, tens, x, batch, seq = H.build_case(H.micro_cases()[name])
+    api.lib().aspen_keep_layer_outputs(0)
+    try:
+        net = H.GpuNet(cfg, tens, batch, seq, min_ninst=32, mode=mode)
+        try:
+            infos = [net.nasm.info(l) for l in range(net.nasm.num_ldata)]
+            folded = sorted(set(i["folded_norm"] for i in infos if i["folded_norm"] >= 0))
+            norms = [l for l, i in enumerate(infos[:-1]) if layers[l]["type"] == "layernorm"]
+            if name.startswith("gpt"):
+                assert folded == norms and all(infos[l]["num_ninst"] == 0 and infos[l]["discarded"] for l in norms), (folded, norms)
+            else:
+                assert not folded and all(infos[l]["num_ninst"] > 0 for l in norms)
+            for xin in (x, (x * 0.5 + 0.01).astype(np.float32) if name.startswith("bert") else x[::-1].copy()):
+                outs = cpu.run_network(layers, tens, xin, batch, seq)
+                net.run(xin)
+                for l in range(1, net.nasm.num_ldata):
+                    if infos[l]["discarded"]:
+                        continue
+                    err = H.rel_l2(net.layer(l), outs[l])
+                    assert err <= H.REL_L2_TOL, f"layer {l} ({layers[l]['type']}): rel L2 {err:.3g}"
+                assert np.array_equal(net.layer(net.nasm.num_ldata - 1).argmax(axis=-1), outs[-1].argmax(axis=-1))
+        finally:
+            net.close()
+    finally:
+        api.lib().aspen_keep_layer_outputs(1)
+
+
 def test_results_in_the_callers_dimension_order(gpu):
     """dse_get_ldata_result permutes a layer's native tensor into the order the caller names (reference
     get_ldata_output, src/apu.c:227-297): matrices of a transformer are (BATCH, MAT_N, MAT_M), attention
