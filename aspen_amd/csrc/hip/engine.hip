@@ -934,6 +934,8 @@ static int check_layer (const aspen_hip_layer_t &L, uint32_t idx)
         else if (L.direct != ASPEN_HIP_OPERAND_DIRECT && !L.ktab) why = "missing k-chunk table";
         else if (L.fuse_out && (!L.fuse_in || L.fuse_ld_in % 4 || L.fuse_ld_in < L.M)) why = "fused shortcut operand";
         else if (L.direct == ASPEN_HIP_OPERAND_DIRECT && (L.ld0 < L.Kp)) why = "direct operand shorter than Kp";
+        else if (L.fuse_norm_stats && (!L.fuse_out || !L.fuse_norm_gamma || L.variant != ASPEN_HIP_GEMM_SMALL || L.M % 64)) why = "a normalised shortcut operand needs a fused shortcut, the norm's scale, 64 x 64 tiles and whole groups of 64 channels";
+        else if (L.norm_stats && !L.norm_fold) why = "column statistics are stored by a layer with a folded layer norm";
         else if (L.norm_fold && (L.type != MATMUL_LAYER || L.direct != ASPEN_HIP_OPERAND_DIRECT || L.variant != ASPEN_HIP_GEMM_SMALL || L.splits > 1 || !L.in1 || L.K % GEMM_BK)) why = "a folded layer norm needs a direct operand, 64 x 64 tiles and an uncut K axis";
         else if (L.direct == ASPEN_HIP_OPERAND_DENSE3 && (L.IC != 3 || L.Kp > 512 || L.Kp < 3 * L.KH * L.KW || L.ld0 < 4 || bm != 64)) why = "dense three-channel operand";
         else if (L.direct < 0 || L.direct > ASPEN_HIP_OPERAND_DENSE3) why = "operand kind";

@@ -673,8 +673,9 @@ struct NoStats { __device__ __forceinline__ void operator() (const float4 (&)[2]
 // 1 / sqrt (variance + eps) behind the stage in LDS, and every lane corrects its sixteen sums:
 // acc = rstd[n] * (acc - mean[n] * rowsum[m]).  Same arithmetic for mean and variance as tile_layernorm.
 #define NORM_FOLD_STATS_OFFSET (128 * LDS_ROW)      // floats: behind the two operand blocks of the stage
+template <int COH>
 __device__ __forceinline__ void norm_fold_finish (const aspen_hip_layer_t &L, floatx16 &acc, float (&cs)[2], float (&cq)[2], float *smem,
-    uint32_t tid, uint32_t m0, uint32_t wm0, uint32_t wn0)
+    uint32_t tid, uint32_t m0, uint32_t n0, uint32_t wm0, uint32_t wn0)
 {
     const uint32_t lane = tid & 63;
     #pragma unroll
@@ -692,7 +693,16 @@ __device__ __forceinline__ void norm_fold_finish (const aspen_hip_layer_t &L, fl
             const float mean = cs[i] / (float)L.K;
             const float var = cq[i] / (float)L.K - mean * mean;
             const uint32_t n = (tid >> 3) + 32 * i;
-            st[2 * n] = mean; st[2 * n + 1] = 1.0f / sqrtf (var + 1e-6f);
+            const float rstd = 1.0f / sqrtf (var + 1e-6f);
+            st[2 * n] = mean; st[2 * n + 1] = rstd;
+            // (row 0 of the layer that was asked to: the pairs go to memory as well, for a fused shortcut that needs the
+            // normalised matrix nobody writes any more)
+            if (L.norm_stats != nullptr && m0 == 0 && n0 + n < L.N)
+            {
+                ActView<COH> sv;
+                sv.init (L.norm_stats, L.N, 2);
+                sv.st1 (2 * (n0 + n), mean); sv.st1 (2 * (n0 + n) + 1, rstd);
+            }
         }
     }
     // (the row sums are weights: requested before the barrier)
@@ -869,7 +879,7 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
                 }
             };
             gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready, stats);
-            if (L.norm_fold) norm_fold_finish (L, acc[0][0], cs, cq, smem, tid, m0, (wave % 2) * 32, (wave / 2) * 32);
+            if (L.norm_fold) norm_fold_finish<COH> (L, acc[0][0], cs, cq, smem, tid, m0, n0, (wave % 2) * 32, (wave / 2) * 32);
         }
         else if constexpr (SINGLE) gemm_core_single_block<DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
         else gemm_core<BM, BN, WM, WN, DEPTH> (al, bl, kbase, kiters, smem, acc, COH != 0, fetch_shortcut, ready);
@@ -938,7 +948,7 @@ __device__ __forceinline__ void contraction_mainloop (const aspen_hip_layer_t &L
 // Second part of a contraction tile of BM = 4 << c4_log2 channels by BN columns, accumulators parked in
 // LDS as [column][BM + 8]: a rolled loop adds the bias, applies the activation and writes 128-bit pieces,
 // so a wavefront covers whole 512-byte (BM = 128) / 256-byte (BM = 64) runs of a column.
-template <int COH>
+template <int COH, bool NORM = false>
 __device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L, uint32_t tn, uint32_t tm, float *smem,
     uint32_t c4_log2, uint32_t BN, const shortcut_prefetch_t &pre)
 {
@@ -964,6 +974,17 @@ __device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L
         const bool keep = !(fuse && L.fuse_discard);        // the pre-shortcut sums are stored unless the host has no use for them
         ActView<COH> fin, fout;
         if (fuse) { fin.init (L.fuse_in, L.N, L.fuse_ld_in); fout.init (L.fuse_out, L.N, L.ld); }
+        // the shortcut's operand may be the input of a layer norm nobody runs as a layer any more: normalised here, with
+        // the arithmetic of tile_layernorm (see aspen_hip_layer_t.fuse_norm_stats)
+        const bool normed = NORM && fuse && L.fuse_norm_stats != nullptr;
+        ActView<COH> stv;
+        float4 gam = make_float4 (1.f, 1.f, 1.f, 1.f), bet = make_float4 (0.f, 0.f, 0.f, 0.f);
+        if (NORM && normed)
+        {
+            stv.init (L.fuse_norm_stats, L.N, 2);
+            gam = gld4 (L.fuse_norm_gamma + m0 + c);
+            if (L.fuse_norm_beta) bet = gld4 (L.fuse_norm_beta + m0 + c);
+        }
         const uint32_t STEP = WG_THREADS >> c4_log2;
         constexpr uint32_t U = 4;                              // 4 rows at a time: all 8 of the larger tiles measured slower (code size, registers)
         if (c + 4 <= mrem)
@@ -978,6 +999,7 @@ __device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L
                 const uint32_t r0 = (tid >> c4_log2) + g * U * STEP;
                 if (r0 >= rows) break;
                 float4 v[U], s[U];
+                float mu[U], rs[U];
                 #pragma unroll
                 for (uint32_t u = 0; u < U; u++)
                 {
@@ -986,6 +1008,7 @@ __device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L
                     {
                         v[u] = ld4 (smem + r * TROW + c);
                         if (fuse) s[u] = pre.have_shortcut ? pre.s[g * U + u] : fin.ld4 ((n0 + r) * L.fuse_ld_in + m0 + c);
+                        if (NORM && normed) { mu[u] = stv.ld1 (2 * (n0 + r)); rs[u] = stv.ld1 (2 * (n0 + r) + 1); }
                     }
                 }
                 #pragma unroll
@@ -1001,6 +1024,11 @@ __device__ __forceinline__ void contraction_epilogue (const aspen_hip_layer_t &L
                         if (keep) out.st4 (o, y);
                         if (fuse)
                         {
+                            if (NORM && normed)
+                            {
+                                s[u].x = (s[u].x - mu[u]) * rs[u] * gam.x + bet.x; s[u].y = (s[u].y - mu[u]) * rs[u] * gam.y + bet.y;
+                                s[u].z = (s[u].z - mu[u]) * rs[u] * gam.z + bet.z; s[u].w = (s[u].w - mu[u]) * rs[u] * gam.w + bet.w;
+                            }
                             y.x += s[u].x; y.y += s[u].y; y.z += s[u].z; y.w += s[u].w;
                             fout.st4 (o, act4 (y, L.fuse_act));
                         }
@@ -2155,7 +2183,7 @@ __device__ __forceinline__ void finish_tile (const aspen_hip_layer_t &L, uint32_
     pre.have = pre.have_shortcut = false;
     const bool tall = L.variant == ASPEN_HIP_GEMM_TALL;
     splitk_gather<COH> (L, t, smem, tall);
-    contraction_epilogue<COH> (L, tn, t - tn * L.tiles_m, smem, tall ? 5 : 4, tall ? VAR4_BN : VAR2_BN, pre);
+    contraction_epilogue<COH, true> (L, tn, t - tn * L.tiles_m, smem, tall ? 5 : 4, tall ? VAR4_BN : VAR2_BN, pre);
 }
 
 // Runs tile t of the layer.  `descriptor ()` yields a wave-uniform copy of the layer's descriptor (scalar_layer /
@@ -2239,7 +2267,7 @@ __device__ __forceinline__ bool run_tile (Descriptor descriptor, uint32_t t, boo
             if (counters == nullptr || !splitk_arrived_last (counters + group, E.splits, smem)) { if (COH) tile_phase_lap (11); return false; }
             splitk_gather<COH> (E, t, smem, c4_log2 == 5);       // (of the shapes cut along K only the tall one has 128 channels)
         }
-        contraction_epilogue<COH> (E, tn, tm, smem, c4_log2, bn, pre);
+        contraction_epilogue<COH, (FEAT & TILES_NORM) != 0> (E, tn, tm, smem, c4_log2, bn, pre);
         if (COH) tile_phase_lap (slice >= 0 ? 11 : 10);
         break;
     }

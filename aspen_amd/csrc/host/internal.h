@@ -91,6 +91,10 @@ struct nasm_ldata_t
        normalise it themselves (column statistics gathered in their K loops); the norm then owns no tiles and its matrix
        is not written.  -1 = not folded */
     int folded_norm;                         /* matmul layer: index of the layer norm it absorbs */
+    /* a folded norm whose matrix a fused shortcut reads as well: that shortcut's producer normalises the norm's input
+       itself, with the column statistics the row-0 tiles of ONE folding layer (stats_writer) store at stats_offset */
+    int stats_writer;                        /* layer norm: index of the folding layer that stores the statistics, -1 = none needed */
+    size_t stats_offset;                     /* floats into the arena: [columns][2] */
     uint64_t flops;                          /* 2*M*N*K for contraction layers, 64-bit */
 };
 

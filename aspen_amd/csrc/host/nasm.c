@@ -304,7 +304,15 @@ static void find_parents (const nasm_t *nasm, const nasm_ldata_t *ld, unsigned i
     if (ld->fused_residual >= 0)
     {
         const nasm_ldata_t *res = &nasm->ldata_arr[ld->fused_residual];
-        add_parents (&nasm->ldata_arr[res->parent_ldata_idx[PARENT_1]], c0, c1, r0, r1, out);
+        const nasm_ldata_t *other = &nasm->ldata_arr[res->parent_ldata_idx[PARENT_1]];
+        if (other->stats_writer >= 0)
+        {
+            /* a folded norm: the epilogue normalises the norm's input itself, with the statistics the row-0 tiles of the
+               norm's first folding layer have stored */
+            add_parents (&nasm->ldata_arr[other->parent_ldata_idx[PARENT_0]], c0, c1, r0, r1, out);
+            add_parents (&nasm->ldata_arr[other->stats_writer], c0, c1, 0, 1, out);
+        }
+        else add_parents (other, c0, c1, r0, r1, out);
     }
     /* A split-K partial tile of a pointwise layer (matmul, 1x1 convolution: the K index IS the parent's
        row index) reads only the parent rows of its K slice, so it waits only for the parent tiles
@@ -561,19 +569,31 @@ static void fold_layernorms (nasm_t *nasm)
         if (nl->layer->type != LAYERNORM_LAYER || nl->num_ninst == 0 || nl->parent_ldata_idx[PARENT_0] < 0) continue;
         const nasm_ldata_t *xl = &nasm->ldata_arr[nl->parent_ldata_idx[PARENT_0]];
         if (xl->out_mat_stride != nl->out_mat_stride || xl->out_mat_dims[OUT_H] != nl->out_mat_dims[OUT_H]) continue;
-        unsigned int consumers = 0, able = 0;
+        unsigned int consumers = 0, able = 0, shortcuts = 0;
+        int first_folding = -1;
         for (unsigned int l = 0; l < nasm->num_ldata; l++)
             for (int k = PARENT_0; k <= PARENT_1; k++)
             {
                 const nasm_ldata_t *cl = &nasm->ldata_arr[l];
                 if (cl->parent_ldata_idx[k] != (int)n) continue;
                 consumers++;
-                able += k == PARENT_0 && cl->layer->type == MATMUL_LAYER && cl->variant == ASPEN_HIP_GEMM_SMALL && cl->splits <= 1 && cl->num_ninst > 0
-                    && cl->layer->gemm_k == nl->out_mat_dims[OUT_H] && cl->layer->gemm_k % 32 == 0;
+                if (k == PARENT_0 && cl->layer->type == MATMUL_LAYER && cl->variant == ASPEN_HIP_GEMM_SMALL && cl->splits <= 1 && cl->num_ninst > 0
+                    && cl->layer->gemm_k == nl->out_mat_dims[OUT_H] && cl->layer->gemm_k % 32 == 0)
+                {
+                    able++;
+                    if (first_folding < 0) first_folding = (int)l;
+                }
+                /* a shortcut computed in its producer's epilogue (64 x 64 tiles over whole groups of 64 channels) can
+                   normalise the norm's input there, given the column statistics: see aspen_hip_layer_t.fuse_norm_stats */
+                else if (k == PARENT_1 && cl->layer->type == RESIDUAL_LAYER && cl->fused_into >= 0 && first_folding >= 0 && cl->fused_into > first_folding
+                    && nasm->ldata_arr[cl->fused_into].variant == ASPEN_HIP_GEMM_SMALL && cl->out_mat_dims[OUT_H] % 64 == 0
+                    && getenv ("ASPEN_GPU_NO_FOLD_SHORTCUT_NORM") == NULL)
+                    shortcuts++;
             }
-        if (consumers == 0 || consumers != able) continue;
+        if (able == 0 || consumers != able + shortcuts) continue;
         for (unsigned int l = 0; l < nasm->num_ldata; l++)
             if (nasm->ldata_arr[l].parent_ldata_idx[PARENT_0] == (int)n) nasm->ldata_arr[l].folded_norm = (int)n;
+        if (shortcuts) nl->stats_writer = first_folding;
         nl->out_discarded = 1;
         nl->num_ninst = 0; nl->tiles_h = nl->tiles_w = 0;
     }
@@ -603,7 +623,7 @@ static nasm_t *build_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned in
     {
         nasm_ldata_t *ld = &nasm->ldata_arr[l];
         ld->nasm = nasm; ld->layer = &dnn->layers[l];
-        ld->fused_residual = ld->fused_into = ld->fused_attention = ld->folded_norm = -1;
+        ld->fused_residual = ld->fused_into = ld->fused_attention = ld->folded_norm = ld->stats_writer = -1;
         ld->out_discarded = 0;
         for (int k = 0; k < NUM_PARENT_ELEMENTS; k++) ld->parent_ldata_idx[k] = ld->layer->parent_idx[k];
         if (set_out_mat (nasm, ld) || set_tiles (nasm, ld)) { bad = 1; break; }
@@ -629,6 +649,11 @@ static nasm_t *build_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned in
             ld->partial_offset = arena;
             /* one block of tile_m x tile_n sums per slice and output tile (edge tiles included whole) */
             arena += (size_t)ld->splits * ld->tiles_h * ld->tiles_w * ld->tile_dims[OUT_H] * ld->tile_dims[OUT_W];
+        }
+        if (ld->stats_writer >= 0)
+        {
+            ld->stats_offset = arena;
+            arena += ((size_t)2 * ld->out_mat_dims[OUT_W] + 63) / 64 * 64;
         }
         nasm->total_flops += ld->flops;
     }
@@ -918,6 +943,13 @@ int aspen_nasm_fill_device_layers (nasm_t *nasm, aspen_hip_layer_t *dst, uint32_
             const nasm_ldata_t *other = &nasm->ldata_arr[res->parent_ldata_idx[PARENT_1]];
             d->fuse_out = nasm->d_arena + res->out_mat_offset;
             d->fuse_in = nasm->d_arena + other->out_mat_offset; d->fuse_ld_in = other->out_mat_stride;
+            if (other->stats_writer >= 0)
+            {
+                const nasm_ldata_t *xl = &nasm->ldata_arr[other->parent_ldata_idx[PARENT_0]];
+                d->fuse_in = nasm->d_arena + xl->out_mat_offset; d->fuse_ld_in = xl->out_mat_stride;
+                d->fuse_norm_stats = nasm->d_arena + other->stats_offset;
+                d->fuse_norm_gamma = other->layer->d_weight; d->fuse_norm_beta = other->layer->d_bias;
+            }
             d->fuse_act = res->layer->activation;
             d->fuse_discard = ld->out_discarded;
         }
@@ -944,6 +976,7 @@ int aspen_nasm_fill_device_layers (nasm_t *nasm, aspen_hip_layer_t *dst, uint32_
             d->in0 = nasm->d_arena + xl->out_mat_offset; d->ld0 = xl->out_mat_stride;
             d->weight = L->d_weight_ln; d->bias = L->d_bias_ln; d->in1 = L->d_rowsum_ln; d->ld1 = 0;
             d->norm_fold = 1;
+            if (nl->stats_writer == (int)l) d->norm_stats = nasm->d_arena + nl->stats_offset;
         }
     }
     return 0;

@@ -100,6 +100,15 @@ typedef struct aspen_hip_layer_t
        out = act (rstd[n] * (acc[m][n] - mean[n] * in1[m]) + bias[m]) */
     uint32_t norm_fold;
     uint32_t reserved0;
+    /* Where the folded norm's matrix is still needed as a fused shortcut's operand (a post-norm transformer block), nobody
+       writes it either: the tiles of row 0 of ONE of the folding layers store their columns' mean and
+       1 / sqrt (variance + eps) to norm_stats ([N][2] floats; NULL: not stored), and the layer with the fused shortcut
+       gets the norm's INPUT as fuse_in together with fuse_norm_stats (those pairs), fuse_norm_gamma and
+       fuse_norm_beta ([M]; beta may be NULL): its epilogue normalises the operand piece by piece,
+       (x - mean[n]) * rstd[n] * gamma[m] + beta[m], before it adds it.  fuse_norm_stats == NULL: fuse_in is used as it
+       is.  64 x 64 tiles over a multiple of 64 channels only. */
+    float *norm_stats;
+    const float *fuse_norm_stats, *fuse_norm_gamma, *fuse_norm_beta;
     uint32_t graph_id;       /* which of the co-scheduled networks of one engine run the layer belongs to (0 .. 63): the run
                                 reports each network's completion separately, see aspen_hip_graph_group_done */
     float *partial;
