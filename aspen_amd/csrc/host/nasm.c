@@ -554,11 +554,15 @@ static void fuse_attention (nasm_t *nasm)
 /* Layer-norm folding.  y = W LN (x) + b is a product with the RAW column x, corrected afterwards with the column's mean
    and deviation (aspen_layer_norm_fold_to_device has the algebra).  A matmul layer in the 64 x 64 shape whose K axis is
    not cut reads every row of its columns in its K loop anyway and gathers the two sums on the way, so it need not wait
-   for the norm's tiles.  A norm ALL of whose consumers can do that (the norms of a pre-norm transformer block, GPT-2's)
-   is folded into them: it loses its tiles, its matrix is not written, and the graph is one dependency level shorter
-   per norm (GPT-2, 4 x 512 tokens: 3.70 -> 3.56 ms).  A norm that something else reads as well (the shortcut of a
-   post-norm block, BERT's) is left alone: its tiles would still have to run before that reader, and its matmul
-   consumers starting early gains nothing (measured: BERT-base 2.06 -> 2.07 ms).  Not when layer outputs are kept. */
+   for the norm's tiles.  A norm whose consumers can all do without its matrix is folded into them: it loses its tiles,
+   its matrix is not written, and the graph is one dependency level shorter per norm.  Consumers that can:
+   - such matmul layers (both norms of a pre-norm transformer block, GPT-2's: 4 x 512 tokens 3.70 -> 3.56 ms);
+   - a shortcut that is computed in its producer's epilogue (the norms of a post-norm block, BERT's, are the
+     shortcut's second operand): that epilogue normalises the norm's input itself, with the column statistics the
+     row-0 tiles of the norm's first folding layer store (BERT-base 8 x 128 tokens: 2.07 -> 2.01 ms).  Folding only the
+     matmul consumers and keeping the norm's tiles for the shortcut gains nothing (2.06 -> 2.07 ms: the tiles still
+     have to run before the shortcut's reader).
+   Not when layer outputs are kept. */
 static void fold_layernorms (nasm_t *nasm)
 {
     const char *e = getenv ("ASPEN_GPU_FOLD_LAYERNORM");
