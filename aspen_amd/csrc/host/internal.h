@@ -87,7 +87,7 @@ struct nasm_ldata_t
        weighted values in one tile (the S x S probabilities stay on chip); the K-attention layer then owns no tiles and
        its matrix is not written.  -1 = not fused */
     int fused_attention;                     /* V-attention layer: index of the K-attention layer it absorbs */
-    /* layer-norm folding: the matmul layers behind a layer norm that nothing else reads take the norm's INPUT and
+    /* layer-norm folding (fold_layernorms in nasm.c): the matmul layers behind a layer norm take the norm's INPUT and
        normalise it themselves (column statistics gathered in their K loops); the norm then owns no tiles and its matrix
        is not written.  -1 = not folded */
     int folded_norm;                         /* matmul layer: index of the layer norm it absorbs */
