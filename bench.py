@@ -26,7 +26,7 @@ PEAK_HBM_GBS = 8000.0
 # calibrated on the library's copy kernel (summaries: profiles/dataflow_kernel_resnet50_b32_hbm_traffic.txt and
 # profiles/dataflow_kernel_vgg16_co_inference_bert_gpt2_kernel_stats_hbm_traffic.txt); valid for these tuned configurations only
 MEASURED_TRAFFIC_BYTES = {("resnet50_b32", "dataflow", 1536): 8.68e9, ("vgg16_b32", "dataflow", 1536): 17.36e9,
-                          ("co_resnet50_vgg16_b16", "dataflow", 1536): 15.00e9, ("bert_base_b8_s128", "dataflow", 192): 2.94e9,
+                          ("co_resnet50_vgg16_b16", "dataflow", 1536): 15.00e9, ("bert_base_b8_s128", "dataflow", 192): 2.89e9,
                           ("gpt2_b4_s512", "dataflow", 384): 8.77e9, ("resnet50_b1", "dataflow", 256): 0.414e9}
 
 # algorithmic GEMM-class flops per unit (2*M*N*K with the reference's K: padding taps counted, full
