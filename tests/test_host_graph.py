@@ -273,6 +273,83 @@ def test_tile_graph_against_brute_force(name, min_ninst, fuse, monkeypatch):
     n.destroy(); d.destroy()
 
 
+@pytest.mark.parametrize("name", ["gpt_mini_b2_s20", "bert_mini_b2_s24"])
+def test_folded_layernorms_rewire_the_tile_graph(name, monkeypatch):
+    """Layer outputs not kept: a layer norm is folded into the matmul layers behind it (and, in a post-norm block, into
+    the epilogue that computes the block's shortcut).  The norm owns no tiles; a folding matmul tile waits for exactly
+    the tiles that write its columns of the norm's INPUT (all rows: it gathers their statistics); the tile that
+    computes a shortcut whose operand is such a norm waits for its piece of the norm's input and for the row-0 tile of
+    the norm's first folding layer, which stores the statistics of those columns."""
+    monkeypatch.setenv("ASPEN_GPU_NARROW_TILES", "0")        # graphs this small would take 32 x 32 tiles, which do not fold
+    api.lib().aspen_keep_layer_outputs(0)
+    try:
+        layers, d, n, batch, seq = make(H.micro_cases()[name], 32)
+        tl, npar, off, idx = n.graph()
+        T = n.num_ninst
+        infos = [n.info(l) for l in range(n.num_ldata)]
+        norms = [l for l, L in enumerate(layers[:-1]) if L["type"] == "layernorm"]
+        assert norms and all(infos[l]["num_ninst"] == 0 and infos[l]["discarded"] for l in norms)
+        assert sorted(set(i["folded_norm"] for i in infos if i["folded_norm"] >= 0)) == norms
+        # who writes which element: a layer's own tiles (a split-K group counts as its first member), or the tiles of the
+        # contraction layer that computes a fused shortcut
+        owner = {}
+        for l, i in enumerate(infos):
+            if i["num_ninst"] == 0:
+                continue
+            own = -np.ones((i["W"], i["H"]), dtype=np.int64)
+            for t in range(i["ninst_start"], i["ninst_start"] + i["num_ninst"], i["splits"]):
+                c0, c1, r0, r1 = n.tile_range(t)
+                own[c0:c1, r0:r1] = t
+            owner[l] = own
+        for l, i in enumerate(infos):
+            if i["fused_into"] >= 0:
+                owner[l] = owner[i["fused_into"]]
+        parents = [set() for _ in range(T)]
+        for l, i in enumerate(infos):
+            for t in range(i["ninst_start"], i["ninst_start"] + i["num_ninst"], i["splits"]):
+                for c in idx[off[t]:off[t + 1]]:
+                    parents[c].add(t)
+        checked_matmul = checked_shortcut = 0
+        for l, i in enumerate(infos):
+            for t in range(i["ninst_start"], i["ninst_start"] + i["num_ninst"]):
+                c0, c1, r0, r1 = n.tile_range(t)
+                if i["folded_norm"] >= 0:
+                    x = layers[i["folded_norm"]]["p0"]
+                    need = {int(v) for v in np.unique(owner[x][c0:c1, :])} if x in owner else set()
+                    assert parents[t] == need, (l, t)
+                    checked_matmul += 1
+                if i["fused_residual"] >= 0 and layers[i["fused_residual"]]["p1"] in norms:
+                    norm = layers[i["fused_residual"]]["p1"]
+                    x = layers[norm]["p0"]
+                    writer = min(c for c, ci in enumerate(infos) if ci["folded_norm"] == norm)
+                    need = {int(v) for v in np.unique(owner[x][c0:c1, r0:r1])} if x in owner else set()
+                    need |= {int(v) for v in np.unique(owner[writer][c0:c1, 0:1])}
+                    assert need <= parents[t], (l, t, sorted(need - parents[t]))
+                    checked_shortcut += 1
+        assert checked_matmul > 0 and (checked_shortcut > 0) == name.startswith("bert")
+        # executing by the counters still runs every tile exactly once
+        cnt = npar.copy().astype(np.int64)
+        ready = [t for t in range(T) if cnt[t] == 0]
+        ran, arrived = 0, {}
+        while ready:
+            t = ready.pop()
+            ran += 1
+            i = infos[int(tl[t])]
+            if i["splits"] > 1:
+                g = t - (t - i["ninst_start"]) % i["splits"]
+                arrived[g] = arrived.get(g, 0) + 1
+                if arrived[g] < i["splits"]:
+                    continue
+            for c in idx[off[t]:off[t + 1]]:
+                cnt[c] -= 1
+                if cnt[c] == 0:
+                    ready.append(int(c))
+        assert ran == T and (cnt == 0).all()
+        n.destroy(); d.destroy()
+    finally:
+        api.lib().aspen_keep_layer_outputs(1)
+
+
 def test_three_channel_first_layer_contracts_a_dense_k_axis():
     """K slices (of 32) of a network's first convolution: 3 x taps without padding for up to 64 output channels (the
     7x7 stem: 147 -> 160, five slices), taps x 4 as for every other layer beyond that."""
