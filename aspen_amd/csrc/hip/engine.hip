@@ -1266,21 +1266,19 @@ extern "C" int aspen_hip_run_dataflow (aspen_hip_graph_t *g, uint32_t workgroups
         // tiles are assigned to workgroups beforehand: every workgroup of the grid must be running
         // (graphs without 32 x 32 tiles need no weight prefetch buffers: their workgroups take the LDS of any other tile, and
         // twice as many fit a compute unit)
-        static int fits[2] = {-1, -1};
+        static int fits[NUM_ORDERED_VARIANTS][2];
+        static bool fits_known[NUM_ORDERED_VARIANTS][2];
         const int small_lds = (g->features & TILES_NARROW) == 0;
-        if (fits[small_lds] < 0)
+        int ov = 0;         // (the variant the launch below takes)
+        while (ov + 1 < NUM_ORDERED_VARIANTS && (g->features & ~ordered_variant_tiles[ov]) != 0) ov++;
+        if (!fits_known[ov][small_lds])
         {
-            int least = 1 << 30;
-            const size_t smem = small_lds ? GEMM_SMEM_BYTES : ORDERED_SMEM_BYTES;
-            for (int v = 0; v < NUM_ORDERED_VARIANTS; v++)
-            {
-                int o = 0;
-                CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&o, ordered_kernels[v], WG_THREADS, smem));
-                if (o < least) least = o;
-            }
-            fits[small_lds] = least * g_num_cu;
+            int o = 0;
+            CHECK (hipOccupancyMaxActiveBlocksPerMultiprocessor (&o, ordered_kernels[ov], WG_THREADS, small_lds ? GEMM_SMEM_BYTES : ORDERED_SMEM_BYTES));
+            fits[ov][small_lds] = o * g_num_cu;
+            fits_known[ov][small_lds] = true;
         }
-        const int fit = fits[small_lds];
+        const int fit = fits[ov][small_lds];
         ordered_smem = small_lds ? GEMM_SMEM_BYTES : ORDERED_SMEM_BYTES;
         if (fit < 1) ordered = false;
         else

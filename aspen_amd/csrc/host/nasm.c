@@ -717,6 +717,7 @@ static double nasm_parallelism (const nasm_t *nasm)
 #define CHAIN_BOUND_KITERS_CAP 48
 #define ORDERED_KITERS_CAP 24
 #define LATENCY_BOUND_BELOW 128.0
+#define ORDERED_VISION_BELOW 1250.0
 static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned int batch, unsigned int seq)
 {
     const char *e = getenv ("ASPEN_GPU_MAX_KITERS");            /* experiments: fixed cap, 0 = none */
@@ -725,7 +726,14 @@ static nasm_t *create_nasm (aspen_dnn_t *dnn, unsigned int min_ninst, unsigned i
     if (nasm == NULL) return nasm;
     const double parallelism = nasm_parallelism (nasm);
     if (getenv ("ASPEN_GPU_VERBOSE")) fprintf (stderr, "aspen: graph of %u tiles, average parallelism %.0f\n", nasm->num_ninst, parallelism);
-    if (parallelism >= CHAIN_BOUND_BELOW) return nasm;
+    if (parallelism >= CHAIN_BOUND_BELOW)
+    {
+        /* (convolutional graphs a little above the limit keep their tiles but still run better in the ordered mode,
+           ordered / queue in ms: ResNet-50 batch 16, 1162: 1.49 / 1.53; VGG-16 batch 2 / 4 / 16 at 1052 / 1220 / 1234:
+           0.80 / 0.91, 1.25 / 1.30, 3.94 / 4.09; from YOLO-v3 batch 8, 1271, on the queue wins: 4.76 / 4.68) */
+        if (seq == 0 && parallelism < ORDERED_VISION_BELOW) nasm->ordered_pref = 1;
+        return nasm;
+    }
     /* bound by the LATENCY of its chains (one image through a deep network; the engine runs such a graph in its ordered
        mode): layers short of tiles take the 32 x 32 shape */
     const char *nt = getenv ("ASPEN_GPU_NARROW_TILES");
